@@ -1,0 +1,217 @@
+/*
+ * ocnn_hip.h - C ABI of the MI355X (gfx950) octree sparse-convolution library.
+ *
+ * The reference (octree-nn/ocnn-pytorch) has no FFI: its hot path is Python
+ * calling torch ops and Triton kernels.  Each entry point below names the
+ * reference code it stands in for (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name starts with "h_";
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued, not awaited;
+ *   - the library never allocates device memory: outputs and workspaces are
+ *     supplied by the caller (sizes from the *_workspace_bytes queries);
+ *   - return value 0 = ok, negative = error (text from ocnn_last_error());
+ *   - feature matrices are row-major (rows, channels); neighbour tables are
+ *     row-major (rows, K) int32 with -1 for "no neighbour";
+ *   - dtype codes: 0 = float32, 1 = float16, 2 = bfloat16 (fp32 accumulation).
+ */
+#ifndef OCNN_HIP_H_
+#define OCNN_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OCNN_F32 0
+#define OCNN_F16 1
+#define OCNN_BF16 2
+
+#define OCNN_OK 0
+#define OCNN_ERR_ARG (-1)      /* bad argument / unsupported shape          */
+#define OCNN_ERR_HIP (-2)      /* a HIP call or launch failed               */
+#define OCNN_ERR_WORKSPACE (-3)/* workspace too small                       */
+
+const char* ocnn_last_error(void);
+int ocnn_abi_version(void);
+
+/* ---- Morton keys ------------------------------------------------------- */
+
+/* ocnn/octree/shuffled_key.py:60-90 (xyz2key).  b may be NULL. */
+int ocnn_xyz2key(const int64_t* x, const int64_t* y, const int64_t* z,
+                 const int64_t* b, int64_t n, int depth, int64_t* key,
+                 void* stream);
+
+/* ocnn/octree/shuffled_key.py:93-115 (key2xyz). */
+int ocnn_key2xyz(const int64_t* key, int64_t n, int depth, int64_t* x,
+                 int64_t* y, int64_t* z, int64_t* b, void* stream);
+
+/* ocnn/octree/points.py:223-244 (Points.normalize) fused with the key
+ * computation of ocnn/octree/octree.py:219-226: pts_out = (pts - bbmin) *
+ * factor in fp32 (no FMA contraction), key = xyz2key(trunc(pts_out), batch).
+ * batch (one id per point) may be NULL; batch_is_float selects float32 ids
+ * (as Points.merge_points makes them) or int64 ids.  h_bbmin: 3 host floats. */
+int ocnn_points2key(const float* pts, int64_t n, const float* h_bbmin,
+                    float factor, const void* batch, int batch_is_float,
+                    int depth, float* pts_out, int64_t* key, void* stream);
+
+/* Host-side evaluation of the bit arithmetic the two kernels above use, so
+ * that it can be checked without a GPU.  xyzb: 4 host int64. */
+int64_t ocnn_host_encode_key(int64_t x, int64_t y, int64_t z, int64_t b, int depth);
+void ocnn_host_decode_key(int64_t key, int depth, int64_t* h_xyzb);
+
+/* ---- octree build ------------------------------------------------------ */
+
+/* torch.unique(key, sorted, return_inverse, return_counts) as used by
+ * ocnn/octree/octree.py:227-228, plus the segment layout the leaf averaging
+ * needs.  key_bits = number of significant low bits of the Morton part
+ * (3*depth); batch ids live at bit 48 and up (batch_bits of them).
+ * Outputs (capacity n each unless noted): node_key, inverse (int64, per
+ * point), counts (int64), seg_start (int32, capacity n+1: first sorted
+ * position of each unique key, closed by n), perm (int32: sorted position ->
+ * point index, stable).  n_unique: one int64 on the device. */
+int64_t ocnn_sort_unique_workspace_bytes(int64_t n);
+int ocnn_sort_unique(const int64_t* key, int64_t n, int key_bits,
+                     int batch_bits, void* workspace, int64_t workspace_bytes,
+                     int64_t* node_key, int64_t* inverse, int64_t* counts,
+                     int32_t* seg_start, int32_t* perm, int64_t* n_unique,
+                     void* stream);
+
+/* One level of ocnn/octree/octree.py:235-259, in two steps because the node
+ * count of the level is data dependent.
+ * count: pidx[i] = ordinal of the parent of node_key[i] among the distinct
+ *        (node_key >> 3); n_parent (device int64) = their number.
+ * fill : keys[8*n_parent] = (parent_key << 3) + 0..7; children[8*n_parent] =
+ *        -1 except children[(pidx << 3) | (node_key & 7)] = i; next_key
+ *        [n_parent] = parent key with the batch id moved back to bit 48 when
+ *        batched != 0. */
+int64_t ocnn_build_level_workspace_bytes(int64_t n);
+int ocnn_build_level_count(const int64_t* node_key, int64_t n, void* workspace,
+                           int64_t workspace_bytes, int32_t* pidx,
+                           int64_t* n_parent, void* stream);
+int ocnn_build_level_fill(const int64_t* node_key, const int32_t* pidx,
+                          int64_t n, int64_t n_parent, int batched,
+                          int64_t* keys, int32_t* children, int64_t* next_key,
+                          void* stream);
+
+/* Per-leaf signal of ocnn/octree/octree.py:273-281: sequential fp32 sum of
+ * the leaf's points (in point order), then mode 0: divide by the count
+ * (points, features); mode 1: L2-normalise with eps 1e-12 (normals). */
+int ocnn_leaf_average(const float* src, int channels, const int32_t* perm,
+                      const int32_t* seg_start, int64_t n_leaf, int mode,
+                      float* out, void* stream);
+
+/* ---- neighbour search -------------------------------------------------- */
+
+/* ocnn/octree/octree.py:411-428: 27-neighbour table of a full layer,
+ * (batch * 8^depth, 27).  out64 or out32 may be NULL. */
+int ocnn_neigh_full(int depth, int batch, int64_t* out64, int32_t* out32,
+                    void* stream);
+
+/* ocnn/octree/octree.py:430-439: table of depth d from the table of depth
+ * d-1.  child_p: children[d-1] (n_p nodes); neigh_p: (n_p, 27) table of depth
+ * d-1; nempty_p: node index of each of the n_ne non-empty parents in order.
+ * Output rows 8c..8c+7 belong to parent ordinal c: (8*n_ne, 27). */
+int ocnn_neigh_from_parent(const int32_t* child_p, const int32_t* neigh_p,
+                           const int32_t* nempty_p, int64_t n_ne,
+                           int64_t* out64, int32_t* out32, void* stream);
+
+/* Host evaluation of the arithmetic that replaces the reference's lut_parent /
+ * lut_child tables (ocnn/octree/octree.py:87-95) inside the kernel above. */
+void ocnn_host_child_slot_lut(int j, int k, int* lut_parent, int* lut_child);
+
+/* ocnn/octree/octree.py:160-172 (nempty_index): index[children[q]] = q for
+ * children[q] >= 0.  index32 / index64 may be NULL. */
+int ocnn_nempty_index(const int32_t* children, int64_t n, int32_t* index32,
+                      int64_t* index64, void* stream);
+
+/* ocnn/octree/octree.py:188-199 and :490-523 (remap_nempty_neigh, get_neigh)
+ * in one pass: out[i][c] = remap(neigh[row(i)][cols[c]]) with
+ * row(i) = row_index[i] if row_index else i * row_stride, and
+ * remap(v) = v < 0 ? -1 : (children ? children[v] : v).
+ * h_cols: K host ints (column selection, NULL = identity over 27). */
+int ocnn_neigh_select(const int32_t* neigh, const int32_t* row_index,
+                      int row_stride, const int32_t* children,
+                      const int* h_cols, int K, int64_t rows, int64_t* out64,
+                      int32_t* out32, void* stream);
+
+/* Widening copy of a table (the public int64 view of an int32 table). */
+int ocnn_table_to_i64(const int32_t* in, int64_t n, int64_t* out, void* stream);
+int ocnn_table_to_i32(const int64_t* in, int64_t n, int32_t* out, void* stream);
+
+/* Inverse of a table: out (rows_in, K) with out[t[i][k]][k] = i, -1 elsewhere.
+ * Valid because every (input row, slot) has at most one producer.  Turns the
+ * scatter of ocnn/nn/octree_conv.py:160-166 (backward_gemm) into a gather. */
+int ocnn_table_transpose(const int32_t* table, int64_t rows, int K,
+                         int64_t rows_in, int32_t* out, void* stream);
+
+/* ---- convolution engine ------------------------------------------------ */
+
+/* Gather-GEMM: out[i][:] = sum_k [t[i][k] >= 0] in[t[i][k]][:] @ Wk (+ bias)
+ * where Wk = w[k'] (cin, cout) or its transpose, k' = k or K-1-k.
+ *   w_transposed = 0: w is (K, cin, cout)      (forward_gemm,
+ *                     ocnn/nn/octree_conv.py:115-143)
+ *   w_transposed = 1: w is (K, cout, cin)      (backward_gemm :145-168 in
+ *                     gather form; reverse_slots = 1 uses the mirrored slot of
+ *                     a centrally symmetric table instead of a transposed one,
+ *                     as ocnn/nn/kernels/conv_bwd_implicit_gemm.py:56 does)
+ * bias may be NULL.  Rows of `in` are addressed by table values only.
+ * workspace: ocnn_conv_workspace_bytes(K, cin, cout) bytes (packed weights). */
+int64_t ocnn_conv_workspace_bytes(int K, int cin, int cout);
+int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
+                     const int32_t* table, int64_t rows_out, int K,
+                     const void* w, int cin, int cout, int w_transposed,
+                     int reverse_slots, const void* bias, void* out,
+                     void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Selects how the MFMA weight-gradient kernel reads its LDS tiles: 1 (default)
+ * = transposing LDS loads, 0 = 16-bit loads.  Same results either way. */
+void ocnn_set_wgrad_transpose_load(int on);
+
+/* Weight gradient, ocnn/nn/octree_conv.py:170-202 (weight_gemm) and
+ * ocnn/nn/kernels/conv_bwd_implicit_gemm_splitk.py:94-184,294-306:
+ * gw[k][a][b] = sum_i [t[i][k] >= 0] x[t[i][k]][a] * g[i][b], computed as
+ * split-K partial sums over row ranges (fp32) followed by a fixed-order
+ * reduction - no atomics, bit-reproducible.  x: (rows_x, ca); g: (rows, cb);
+ * gw: (K, ca, cb) in `dtype`, or (K, cb, ca) when out_transposed != 0 (the
+ * deconvolution's weight layout, ocnn/nn/octree_conv.py:287-290). */
+int64_t ocnn_conv_wgrad_workspace_bytes(int64_t rows, int K, int ca, int cb);
+int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
+                    const int32_t* table, int64_t rows, int K, int ca, int cb,
+                    int out_transposed, void* gw, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+
+/* Depth-wise engine, ocnn/nn/octree_dwconv.py:30-118.  w: (K, c).
+ * fwd : out[i][c] = sum_k in[t[i][k]][c] * w[k'][c]   (k' = K-1-k if
+ *       reverse_slots; with a transposed or mirrored table this is also the
+ *       data gradient);
+ * wgrad: gw[k][c] = sum_i x[t[i][k]][c] * g[i][c] (two-pass, deterministic). */
+int ocnn_dwconv_gather(int dtype, const void* in, int64_t rows_in,
+                       const int32_t* table, int64_t rows_out, int K,
+                       const void* w, int channels, int reverse_slots,
+                       const void* bias, void* out, void* stream);
+int64_t ocnn_dwconv_wgrad_workspace_bytes(int64_t rows, int K, int channels);
+int ocnn_dwconv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
+                      const int32_t* table, int64_t rows, int K, int channels,
+                      void* gw, void* workspace, int64_t workspace_bytes,
+                      void* stream);
+
+/* ocnn/nn/octree_pad.py:13-39.  pad: out (n, c) = val except out[q] =
+ * data[children[q]] where children[q] >= 0; depad: out[children[q]] = data[q]. */
+int ocnn_pad(int dtype, const void* data, const int32_t* children, int64_t n,
+             int channels, float val, void* out, void* stream);
+int ocnn_depad(int dtype, const void* data, const int32_t* children, int64_t n,
+               int channels, void* out, void* stream);
+
+/* Column sum (grad_bias = grad.sum(0), ocnn/nn/kernels/
+ * conv_bwd_implicit_gemm_splitk.py:343-345), two-pass deterministic.
+ * workspace: ocnn_colsum_workspace_bytes(rows, channels). */
+int64_t ocnn_colsum_workspace_bytes(int64_t rows, int channels);
+int ocnn_colsum(int dtype, const void* g, int64_t rows, int channels, void* out,
+                void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OCNN_HIP_H_ */

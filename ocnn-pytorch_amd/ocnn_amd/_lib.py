@@ -1,0 +1,110 @@
+"""ctypes binding of libocnn_hip.so (the C ABI declared in include/ocnn_hip.h).
+
+There is no CPU fallback: if the library cannot be loaded the package raises.
+"""
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
+
+import torch
+
+from . import build as _build
+
+_i, _l, _p, _f = c_int, c_int64, c_void_p, c_float
+
+# name -> (restype, argtypes); mirrors include/ocnn_hip.h one to one
+SIGNATURES = {
+    'ocnn_last_error': (c_char_p, []),
+    'ocnn_abi_version': (_i, []),
+    'ocnn_xyz2key': (_i, [_p, _p, _p, _p, _l, _i, _p, _p]),
+    'ocnn_key2xyz': (_i, [_p, _l, _i, _p, _p, _p, _p, _p]),
+    'ocnn_points2key': (_i, [_p, _l, POINTER(_f), _f, _p, _i, _i, _p, _p, _p]),
+    'ocnn_host_encode_key': (_l, [_l, _l, _l, _l, _i]),
+    'ocnn_host_decode_key': (None, [_l, _i, POINTER(_l)]),
+    'ocnn_sort_unique_workspace_bytes': (_l, [_l]),
+    'ocnn_sort_unique': (_i, [_p, _l, _i, _i, _p, _l, _p, _p, _p, _p, _p, _p, _p]),
+    'ocnn_build_level_workspace_bytes': (_l, [_l]),
+    'ocnn_build_level_count': (_i, [_p, _l, _p, _l, _p, _p, _p]),
+    'ocnn_build_level_fill': (_i, [_p, _p, _l, _l, _i, _p, _p, _p, _p]),
+    'ocnn_leaf_average': (_i, [_p, _i, _p, _p, _l, _i, _p, _p]),
+    'ocnn_neigh_full': (_i, [_i, _i, _p, _p, _p]),
+    'ocnn_neigh_from_parent': (_i, [_p, _p, _p, _l, _p, _p, _p]),
+    'ocnn_host_child_slot_lut': (None, [_i, _i, POINTER(_i), POINTER(_i)]),
+    'ocnn_nempty_index': (_i, [_p, _l, _p, _p, _p]),
+    'ocnn_neigh_select': (_i, [_p, _p, _i, _p, POINTER(_i), _i, _l, _p, _p, _p]),
+    'ocnn_table_to_i64': (_i, [_p, _l, _p, _p]),
+    'ocnn_table_to_i32': (_i, [_p, _l, _p, _p]),
+    'ocnn_table_transpose': (_i, [_p, _l, _i, _l, _p, _p]),
+    'ocnn_conv_workspace_bytes': (_l, [_i, _i, _i]),
+    'ocnn_conv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _i, _i, _p, _p, _p, _l, _p]),
+    'ocnn_set_wgrad_transpose_load': (None, [_i]),
+    'ocnn_conv_wgrad_workspace_bytes': (_l, [_l, _i, _i, _i]),
+    'ocnn_conv_wgrad': (_i, [_i, _p, _l, _p, _p, _l, _i, _i, _i, _i, _p, _p, _l, _p]),
+    'ocnn_dwconv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _p, _p, _p]),
+    'ocnn_dwconv_wgrad_workspace_bytes': (_l, [_l, _i, _i]),
+    'ocnn_dwconv_wgrad': (_i, [_i, _p, _l, _p, _p, _l, _i, _i, _p, _p, _l, _p]),
+    'ocnn_pad': (_i, [_i, _p, _p, _l, _i, _f, _p, _p]),
+    'ocnn_depad': (_i, [_i, _p, _p, _l, _i, _p, _p]),
+    'ocnn_colsum_workspace_bytes': (_l, [_l, _i]),
+    'ocnn_colsum': (_i, [_i, _p, _l, _i, _p, _p, _l, _p]),
+}
+
+_lib = None
+
+
+def lib():
+  """Loads the library once.  Builds it first only when no built file exists."""
+  global _lib
+  if _lib is not None:
+    return _lib
+  path = _build.LIB_PATH
+  if not os.path.exists(path):
+    _build.build_library()
+  handle = ctypes.CDLL(path)
+  for name, (res, args) in SIGNATURES.items():
+    fn = getattr(handle, name)      # AttributeError if the symbol is missing
+    fn.restype = res
+    fn.argtypes = args
+  _lib = handle
+  return _lib
+
+
+class OcnnHipError(RuntimeError):
+  pass
+
+
+def check(rc):
+  if rc != 0:
+    raise OcnnHipError('libocnn_hip: {} (code {})'.format(
+        lib().ocnn_last_error().decode('utf-8', 'replace'), rc))
+
+
+DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def dtype_code(t):
+  try:
+    return DTYPE_CODE[t.dtype]
+  except KeyError:
+    raise TypeError('unsupported feature dtype {}; use float32, float16 or bfloat16'.format(t.dtype))
+
+
+def require_gpu(*tensors):
+  """The kernels run on the GPU only; anything else is an error, not a fallback."""
+  for t in tensors:
+    if t is not None and not t.is_cuda:
+      raise RuntimeError('ocnn_amd kernels need tensors on a HIP device, got a tensor on '
+                         '{}'.format(t.device))
+
+
+def ptr(t):
+  return None if t is None else t.data_ptr()
+
+
+def stream():
+  return torch.cuda.current_stream().cuda_stream
+
+
+def workspace(nbytes, device):
+  return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)

@@ -1,0 +1,12 @@
+from .octree_pad import octree_pad, octree_depad
+from .octree_conv import (OctreeConv, OctreeDeconv, OctreeConvBase, octree_conv, octree_deconv,
+                          conv_gather, conv_wgrad, column_sum)
+from .octree_dwconv import OctreeDWConv, octree_dwconv
+from .octree_conv_t import (OctreeConvTriton, OctreeConvT, octree_conv_triton,
+                            convert_conv_triton, conv_fwd_implicit_gemm_splitk,
+                            conv_bwd_implicit_gemm_splitk)
+
+__all__ = ['octree_pad', 'octree_depad', 'OctreeConv', 'OctreeDeconv', 'octree_conv',
+           'octree_deconv', 'OctreeDWConv', 'octree_dwconv', 'OctreeConvTriton', 'OctreeConvT',
+           'octree_conv_triton', 'convert_conv_triton', 'conv_fwd_implicit_gemm_splitk',
+           'conv_bwd_implicit_gemm_splitk']

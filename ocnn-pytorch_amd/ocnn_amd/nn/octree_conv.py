@@ -1,0 +1,274 @@
+"""OctreeConv / OctreeDeconv with the module and functional API of the
+reference (ocnn/nn/octree_conv.py), running on the HIP gather-GEMM and split-K
+weight-gradient kernels.
+
+Engine view.  With T the (rows, K) neighbour table of the layer:
+  forward_gemm  : out[i]  = sum_k data[T[i,k]] @ W[k]            (gather)
+  backward_gemm : gin[j] += sum_{T[i,k]=j} grad[i] @ W[k]^T      (scatter)
+  weight_gemm   : gW[k]   = sum_i data[T[i,k]]^T (x) grad[i]
+The scatter is run as a gather too: through the mirrored slot K-1-k when the
+table is centrally symmetric (stride 1, every kernel but 2x2x2) and through
+the inverse table otherwise, so no atomics are involved anywhere.
+"""
+
+from typing import List
+
+import torch
+import torch.nn
+from torch.autograd import Function
+
+from .. import _lib
+from ..utils import list2str, resize_with_last_val, xavier_uniform_
+from .octree_pad import octree_depad, octree_pad
+
+
+def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None):
+  """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K))."""
+  _lib.require_gpu(data, table, W)
+  L = _lib.lib()
+  data, W, table = data.contiguous(), W.contiguous(), table.contiguous()
+  rows, K = table.shape
+  cin = data.shape[1]
+  assert W.dtype == data.dtype and table.dtype == torch.int32
+  assert W.numel() == K * cin * cout, 'weights do not match the table and channels'
+  if bias is not None:
+    bias = bias.to(data.dtype).contiguous()
+  out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
+  nbytes = L.ocnn_conv_workspace_bytes(K, cin, cout)
+  ws = _lib.workspace(nbytes, data.device)
+  _lib.check(L.ocnn_conv_gather(
+      _lib.dtype_code(data), _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(W),
+      cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
+      ws.numel(), _lib.stream()))
+  return out
+
+
+def conv_wgrad(x, g, table, out_transposed=False):
+  """gW (K, ca, cb) [or (K, cb, ca)] = sum_i x[T[i,k]]^T (x) g[i]."""
+  _lib.require_gpu(x, g, table)
+  L = _lib.lib()
+  x, g, table = x.contiguous(), g.contiguous(), table.contiguous()
+  rows, K = table.shape
+  ca, cb = x.shape[1], g.shape[1]
+  assert g.shape[0] == rows and x.dtype == g.dtype and table.dtype == torch.int32
+  shape = (K, cb, ca) if out_transposed else (K, ca, cb)
+  gw = torch.empty(shape, dtype=x.dtype, device=x.device)
+  ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes(rows, K, ca, cb), x.device)
+  _lib.check(L.ocnn_conv_wgrad(
+      _lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
+      int(out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  return gw
+
+
+def column_sum(g):
+  """g.sum(0) with a fixed reduction order."""
+  _lib.require_gpu(g)
+  L = _lib.lib()
+  g = g.contiguous()
+  out = torch.empty(g.shape[1], dtype=g.dtype, device=g.device)
+  ws = _lib.workspace(L.ocnn_colsum_workspace_bytes(g.shape[0], g.shape[1]), g.device)
+  _lib.check(L.ocnn_colsum(_lib.dtype_code(g), _lib.ptr(g), g.shape[0], g.shape[1],
+                           _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  return out
+
+
+class OctreeConvBase:
+  """Shapes and the three engine passes (ocnn/nn/octree_conv.py:26-202)."""
+
+  def __init__(self, in_channels: int, out_channels: int, kernel_size: List[int] = [3],
+               stride: int = 1, nempty: bool = False, max_buffer: int = int(2e8)):
+    super().__init__()
+    self.in_channels = in_channels
+    self.out_channels = out_channels
+    self.kernel_size = resize_with_last_val(kernel_size)
+    self.kernel = list2str(self.kernel_size)
+    self.stride = stride
+    self.nempty = nempty
+    self.max_buffer = max_buffer      # accepted for compatibility; nothing is buffered
+    self.kdim = self.kernel_size[0] * self.kernel_size[1] * self.kernel_size[2]
+    self.in_conv = in_channels if self.is_conv_layer() else out_channels
+    self.out_conv = out_channels if self.is_conv_layer() else in_channels
+    self.weights_shape = (self.kdim, self.in_conv, self.out_conv)
+
+  def is_conv_layer(self):
+    raise NotImplementedError
+
+  def setup(self, octree, depth: int):
+    """Heights of input/output and the table (ocnn/nn/octree_conv.py:51-100)."""
+    self.in_depth = self.out_depth = self.neigh_depth = depth
+    if self.stride == 2:
+      if self.is_conv_layer():
+        self.out_depth = depth - 1
+      else:
+        self.out_depth = depth + 1
+        self.neigh_depth = depth + 1
+    if self.nempty:
+      in_h = octree.nnum_nempty[self.in_depth]
+      out_h = octree.nnum_nempty[self.out_depth]
+    else:
+      in_h = octree.nnum[self.in_depth]
+      out_h = octree.nnum[self.out_depth]
+      if self.stride == 2:
+        if self.is_conv_layer():
+          out_h = octree.nnum_nempty[self.out_depth]
+        else:
+          in_h = octree.nnum_nempty[self.in_depth]
+    self.in_h, self.out_h = int(in_h), int(out_h)
+    self.in_shape = (self.in_h, self.in_channels)
+    self.out_shape = (self.out_h, self.out_channels)
+    self.octree = octree
+    self.neigh = octree._table(self.neigh_depth, self.kernel, self.stride, self.nempty)
+    # rows on the "fine" side of the table (what its entries index)
+    self.fine_h = self.in_h if self.is_conv_layer() else self.out_h
+    self.symmetric = self.stride == 1 and self.kernel != '222'
+
+  def check_and_init(self, data: torch.Tensor):
+    check = tuple(data.shape) == self.in_shape
+    assert check, ('The shape of input data is wrong: ' +
+                   'expected {}, got {}.'.format(self.in_shape, data.shape))
+
+  def _inverse_table(self):
+    return self.octree._table_t(self.neigh_depth, self.kernel, self.stride, self.nempty,
+                                self.fine_h)
+
+  def forward_gemm(self, data, weights, bias=None):
+    """(fine rows, in_conv) -> (table rows, out_conv)."""
+    return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias)
+
+  def backward_gemm(self, grad, weights, bias=None):
+    """(table rows, out_conv) -> (fine rows, in_conv)."""
+    if self.symmetric:
+      return conv_gather(grad, grad.shape[0], self.neigh, weights, self.in_conv, True, True, bias)
+    return conv_gather(grad, grad.shape[0], self._inverse_table(), weights, self.in_conv, True,
+                       False, bias)
+
+  def weight_gemm(self, data, grad, out_transposed=False):
+    """data: fine rows; grad: table rows -> (K, in_conv, out_conv)."""
+    return conv_wgrad(data, grad, self.neigh, out_transposed)
+
+
+class _OctreeConv(OctreeConvBase):
+  def is_conv_layer(self): return True
+
+
+class _OctreeDeconv(OctreeConvBase):
+  def is_conv_layer(self): return False
+
+
+class OctreeConvFunction(Function):
+  """Autograd wiring of the convolution (ocnn/nn/octree_conv.py:219-254)."""
+
+  @staticmethod
+  def forward(ctx, data, weights, octree, depth: int, in_channels: int, out_channels: int,
+              kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
+              max_buffer: int = int(2e8)):
+    eng = _OctreeConv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
+    eng.setup(octree, depth)
+    eng.check_and_init(data)
+    data = data.contiguous()
+    weights = weights.to(data.dtype).contiguous()
+    out = eng.forward_gemm(data, weights)
+    ctx.save_for_backward(data, weights)
+    ctx.eng = eng
+    return out
+
+  @staticmethod
+  def backward(ctx, grad):
+    data, weights = ctx.saved_tensors
+    eng = ctx.eng
+    grad = grad.contiguous()
+    grad_out = eng.backward_gemm(grad, weights) if ctx.needs_input_grad[0] else None
+    grad_w = eng.weight_gemm(data, grad) if ctx.needs_input_grad[1] else None
+    return (grad_out, grad_w) + (None,) * 8
+
+
+class OctreeDeconvFunction(Function):
+  """Autograd wiring of the deconvolution (ocnn/nn/octree_conv.py:257-292)."""
+
+  @staticmethod
+  def forward(ctx, data, weights, octree, depth: int, in_channels: int, out_channels: int,
+              kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
+              max_buffer: int = int(2e8)):
+    eng = _OctreeDeconv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
+    eng.setup(octree, depth)
+    eng.check_and_init(data)
+    data = data.contiguous()
+    weights = weights.to(data.dtype).contiguous()
+    out = eng.backward_gemm(data, weights)
+    ctx.save_for_backward(data, weights)
+    ctx.eng = eng
+    return out
+
+  @staticmethod
+  def backward(ctx, grad):
+    data, weights = ctx.saved_tensors
+    eng = ctx.eng
+    grad = grad.contiguous()
+    grad_out = eng.forward_gemm(grad, weights) if ctx.needs_input_grad[0] else None
+    # weights are (K, out_channels, in_channels): x = grad (fine side), g = data
+    grad_w = eng.weight_gemm(grad, data) if ctx.needs_input_grad[1] else None
+    return (grad_out, grad_w) + (None,) * 8
+
+
+octree_conv = OctreeConvFunction.apply
+octree_deconv = OctreeDeconvFunction.apply
+
+
+class OctreeConv(OctreeConvBase, torch.nn.Module):
+  """Octree convolution.  Constructor, parameters (`weights` (kdim, Cin, Cout),
+  `bias`) and forward(data, octree, depth) follow ocnn/nn/octree_conv.py:300-431.
+  `method` and `max_buffer` are accepted and ignored: every kernel shape,
+  stride and nempty mode runs on the same HIP engine."""
+
+  def __init__(self, in_channels: int, out_channels: int, kernel_size: List[int] = [3],
+               stride: int = 1, nempty: bool = False, method: str = 'triton',
+               use_bias: bool = False, max_buffer: int = int(2e8)):
+    super().__init__(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
+    self.use_bias = use_bias
+    self.method = self.check_method(method)
+    self.weights = torch.nn.Parameter(torch.Tensor(*self.weights_shape))
+    self.bias = torch.nn.Parameter(torch.Tensor(out_channels)) if use_bias else None
+    self.reset_parameters()
+
+  def check_method(self, method: str):
+    if method not in ('explicit_gemm', 'block_gemm', 'triton', 'hip'):
+      raise ValueError('Unknown method: {}'.format(method))
+    return 'hip'
+
+  def reset_parameters(self):
+    xavier_uniform_(self.weights)
+    if self.use_bias:
+      torch.nn.init.zeros_(self.bias)
+
+  def is_conv_layer(self): return True
+
+  def forward(self, data: torch.Tensor, octree, depth: int):
+    out = octree_conv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
+                      self.kernel_size, self.stride, self.nempty, self.max_buffer)
+    if self.use_bias:
+      out = out + self.bias.to(out.dtype)
+    if self.stride == 2 and not self.nempty:
+      out = octree_pad(out, octree, depth - 1)
+    return out
+
+  def extra_repr(self) -> str:
+    return ('in_channels={}, out_channels={}, kernel_size={}, stride={}, '
+            'nempty={}, bias={}, method={}').format(
+                self.in_channels, self.out_channels, self.kernel_size, self.stride,
+                self.nempty, self.use_bias, self.method)
+
+
+class OctreeDeconv(OctreeConv):
+  """Octree deconvolution (ocnn/nn/octree_conv.py:433-466); weights are
+  (kdim, out_channels, in_channels)."""
+
+  def is_conv_layer(self): return False
+
+  def forward(self, data: torch.Tensor, octree, depth: int):
+    if self.stride == 2 and not self.nempty:
+      data = octree_depad(data, octree, depth)
+    out = octree_deconv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
+                        self.kernel_size, self.stride, self.nempty, self.max_buffer)
+    if self.use_bias:
+      out = out + self.bias.to(out.dtype)
+    return out

@@ -1,0 +1,611 @@
+"""Octree with the contract of the reference's ``ocnn.octree.Octree``
+(ocnn/octree/octree.py), built and searched by HIP kernels.
+
+Layout in device memory, per depth d:
+  keys[d]      int64 (nnum[d],)      ascending Morton keys, batch id at bit 48
+  children[d]  int32 (nnum[d],)      ordinal among the non-empty nodes, or -1
+  neighs[d]    (nnum[d], 27)         row indices of the 3x3x3 window, or -1
+The neighbour tables are kept as int32 (what the convolution kernels read);
+``octree.neighs[d]`` widens one to the reference's int64 on first access.
+nnum / nnum_nempty stay on the host, as in the reference.
+"""
+
+from typing import List, Union
+
+import ctypes
+
+import torch
+import torch.nn.functional as F
+
+from .. import _lib
+from ..utils import cumsum, range_grid, trunc_div
+from .points import Points
+from .shuffled_key import key2xyz, xyz2key
+
+LUT_KERNEL = {
+    '222': [13, 14, 16, 17, 22, 23, 25, 26],
+    '311': [4, 13, 22],
+    '131': [10, 13, 16],
+    '113': [12, 13, 14],
+    '331': [1, 4, 7, 10, 13, 16, 19, 22, 25],
+    '313': [3, 4, 5, 12, 13, 14, 21, 22, 23],
+    '133': [9, 10, 11, 12, 13, 14, 15, 16, 17],
+}
+
+
+class _NeighTables:
+  """List-like holder of the per-depth tables: int32 for the kernels, int64
+  (the public dtype) made on demand and cached."""
+
+  def __init__(self, num):
+    self._t32 = [None] * num
+    self._t64 = [None] * num
+
+  def __len__(self):
+    return len(self._t32)
+
+  def _get(self, i):
+    if self._t64[i] is None and self._t32[i] is not None:
+      t32 = self._t32[i]
+      if t32.is_cuda:
+        out = torch.empty(t32.shape, dtype=torch.long, device=t32.device)
+        _lib.check(_lib.lib().ocnn_table_to_i64(_lib.ptr(t32), t32.numel(), _lib.ptr(out),
+                                                _lib.stream()))
+      else:
+        out = t32.long()
+      self._t64[i] = out
+    return self._t64[i]
+
+  def __getitem__(self, i):
+    if isinstance(i, slice):
+      return [self._get(j) for j in range(*i.indices(len(self)))]
+    return self._get(range(len(self))[i])
+
+  def __setitem__(self, i, value):
+    i = range(len(self))[i]
+    self._t32[i] = self._t64[i] = None
+    if value is None:
+      return
+    if value.dtype == torch.int32:
+      self._t32[i] = value
+    else:
+      self._t64[i] = value.long()
+
+  def __iter__(self):
+    return (self._get(i) for i in range(len(self)))
+
+  def append(self, value):
+    self._t32.append(None)
+    self._t64.append(None)
+    self[len(self) - 1] = value
+
+  def get32(self, i):
+    if self._t32[i] is None and self._t64[i] is not None:
+      t64 = self._t64[i].contiguous()
+      if t64.is_cuda:
+        out = torch.empty(t64.shape, dtype=torch.int32, device=t64.device)
+        _lib.check(_lib.lib().ocnn_table_to_i32(_lib.ptr(t64), t64.numel(), _lib.ptr(out),
+                                                _lib.stream()))
+      else:
+        out = t64.int()
+      self._t32[i] = out
+    return self._t32[i]
+
+  def has(self, i):
+    return self._t32[i] is not None or self._t64[i] is not None
+
+  def moved(self, device, non_blocking=False):
+    out = _NeighTables(len(self))
+    for i in range(len(self)):
+      if self._t32[i] is not None:
+        out._t32[i] = self._t32[i].to(device, non_blocking=non_blocking)
+      if self._t64[i] is not None:
+        out._t64[i] = self._t64[i].to(device, non_blocking=non_blocking)
+    return out
+
+
+class Octree:
+  """Same constructor, attributes and methods as the reference class
+  (ocnn/octree/octree.py:18-106)."""
+
+  def __init__(self, depth: int, full_depth: int = 2, batch_size: int = 1,
+               device: Union[torch.device, str] = 'cpu', **kwargs):
+    self.depth = depth
+    self.full_depth = full_depth
+    self.batch_size = batch_size
+    self.device = device
+    self.reset()
+
+  def reset(self):
+    num = self.depth + 1
+    self.keys = [None] * num
+    self.children = [None] * num
+    self.neighs = _NeighTables(num)
+    self.features = [None] * num
+    self.normals = [None] * num
+    self.points = [None] * num
+    self.nempty_masks = [None] * num
+    self.nempty_indices = [None] * num
+    self.nempty_neighs = [None] * num
+    self._nempty_indices32 = [None] * num
+    self._tables = {}        # (depth, kernel, stride, nempty) -> int32 table
+    self._tables_t = {}      # same key -> inverse table
+
+    self.nnum = torch.zeros(num, dtype=torch.long)
+    self.nnum_nempty = torch.zeros(num, dtype=torch.long)
+    bs = self.batch_size
+    self.batch_nnum = torch.zeros(num, bs, dtype=torch.long)
+    self.batch_nnum_nempty = torch.zeros(num, bs, dtype=torch.long)
+
+    # the reference's public lookup tables (ocnn/octree/octree.py:85-106); the
+    # kernels compute the first two arithmetically
+    dev = self.device
+    grid = range_grid(2, 3, dev).unsqueeze(1) + range_grid(-1, 1, dev)
+    self.lut_parent = (trunc_div(grid, 2) * torch.tensor([9, 3, 1], device=dev)).sum(2)
+    self.lut_child = ((grid % 2) * torch.tensor([4, 2, 1], device=dev)).sum(2)
+    self.lut_kernel = {k: torch.tensor(v, device=dev) for k, v in LUT_KERNEL.items()}
+
+  # ---- cache bookkeeping ---------------------------------------------------
+  def _drop_tables(self, depth, nempty_only=False):
+    for cache in (self._tables, self._tables_t):
+      for key in [k for k in cache if k[0] == depth and (k[3] or not nempty_only)]:
+        del cache[key]
+
+  def _drop_nempty(self, depth):
+    self.nempty_masks[depth] = None
+    self.nempty_indices[depth] = None
+    self.nempty_neighs[depth] = None
+    self._nempty_indices32[depth] = None
+    self._drop_tables(depth, nempty_only=True)
+
+  # ---- simple accessors (ocnn/octree/octree.py:108-145) ---------------------
+  def key(self, depth: int, nempty: bool = False):
+    key = self.keys[depth]
+    return key[self.nempty_index(depth)] if nempty else key
+
+  def xyzb(self, depth: int, nempty: bool = False):
+    return key2xyz(self.key(depth, nempty), depth)
+
+  def batch_id(self, depth: int, nempty: bool = False):
+    batch_id = self.keys[depth] >> 48
+    return batch_id[self.nempty_index(depth)] if nempty else batch_id
+
+  # ---- non-empty bookkeeping (ocnn/octree/octree.py:147-199) ----------------
+  def nempty_mask(self, depth: int, reset: bool = False):
+    if self.nempty_masks[depth] is None or reset:
+      self.nempty_masks[depth] = self.children[depth] >= 0
+    return self.nempty_masks[depth]
+
+  def _make_nempty_index(self, depth):
+    child = self.children[depth]
+    _lib.require_gpu(child)
+    n = int(self.nnum_nempty[depth])
+    i32 = torch.empty(n, dtype=torch.int32, device=child.device)
+    i64 = torch.empty(n, dtype=torch.long, device=child.device)
+    _lib.check(_lib.lib().ocnn_nempty_index(_lib.ptr(child), child.numel(), _lib.ptr(i32),
+                                            _lib.ptr(i64), _lib.stream()))
+    self._nempty_indices32[depth] = i32
+    self.nempty_indices[depth] = i64
+
+  def nempty_index(self, depth: int, reset: bool = False):
+    if self.nempty_indices[depth] is None or reset:
+      self._make_nempty_index(depth)
+    return self.nempty_indices[depth]
+
+  def _nempty_index32(self, depth):
+    if self._nempty_indices32[depth] is None:
+      self._make_nempty_index(depth)
+    return self._nempty_indices32[depth]
+
+  def nempty_neigh(self, depth: int, reset: bool = False):
+    if self.nempty_neighs[depth] is None or reset:
+      if reset:
+        self._drop_tables(depth, nempty_only=True)
+      self.nempty_neighs[depth] = self._widen(self._table(depth, '333', 1, True))
+    return self.nempty_neighs[depth]
+
+  def remap_nempty_neigh(self, neigh: torch.Tensor, depth: int):
+    """In-place remap of valid entries to non-empty ordinals
+    (ocnn/octree/octree.py:188-199)."""
+    valid = neigh >= 0
+    neigh[valid] = self.children[depth][neigh[valid]].long()
+    return neigh
+
+  # ---- build (ocnn/octree/octree.py:201-287) --------------------------------
+  def build_octree(self, point_cloud: Points, bbmin: Union[float, torch.Tensor] = -1.0,
+                   bbmax: Union[float, torch.Tensor] = 1.0):
+    self.device = point_cloud.device
+    assert point_cloud.batch_size == self.batch_size, 'Inconsistent batch_size'
+    pts = point_cloud.points
+    _lib.require_gpu(pts)
+    L = _lib.lib()
+    dev = pts.device
+    depth = self.depth
+
+    # normalisation constants exactly as Points.normalize forms them
+    box = bbmax - bbmin
+    if type(box) is torch.Tensor:
+      box = box.max().item()
+    assert box > 0, 'The bounding box size must be greater than 0.'
+    factor = (2 ** depth) / box
+    if isinstance(bbmin, torch.Tensor):
+      lo = [float(v) for v in bbmin.detach().float().cpu().view(-1).tolist()]
+      lo = lo * 3 if len(lo) == 1 else lo
+    else:
+      lo = [float(bbmin)] * 3
+    h_lo = (ctypes.c_float * 3)(*lo)
+
+    pts = pts.float().contiguous()
+    npt = pts.shape[0]
+    batch, batch_is_float = None, 0
+    if self.batch_size > 1:
+      batch = point_cloud.batch_id.view(-1)
+      if batch.is_floating_point():
+        batch, batch_is_float = batch.float().contiguous(), 1
+      else:
+        batch = batch.long().contiguous()
+    pts_norm = torch.empty_like(pts)
+    key = torch.empty(npt, dtype=torch.long, device=dev)
+    st = _lib.stream()
+    _lib.check(L.ocnn_points2key(_lib.ptr(pts), npt, h_lo, factor, _lib.ptr(batch),
+                                 batch_is_float, depth, _lib.ptr(pts_norm), _lib.ptr(key), st))
+
+    # sorted unique keys + inverse map + counts
+    ws = _lib.workspace(L.ocnn_sort_unique_workspace_bytes(npt), dev)
+    node_key = torch.empty(npt, dtype=torch.long, device=dev)
+    idx = torch.empty(npt, dtype=torch.long, device=dev)
+    counts = torch.empty(npt, dtype=torch.long, device=dev)
+    seg_start = torch.empty(npt + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(npt, dtype=torch.int32, device=dev)
+    n_dev = torch.zeros(1, dtype=torch.long, device=dev)
+    batch_bits = max(0, (self.batch_size - 1).bit_length())
+    _lib.check(L.ocnn_sort_unique(_lib.ptr(key), npt, 3 * depth, batch_bits, _lib.ptr(ws),
+                                  ws.numel(), _lib.ptr(node_key), _lib.ptr(idx),
+                                  _lib.ptr(counts), _lib.ptr(seg_start), _lib.ptr(perm),
+                                  _lib.ptr(n_dev), st))
+    n = int(n_dev.item())
+    nleaf = n
+    node_key = node_key[:n]
+
+    for d in range(self.full_depth + 1):
+      self.octree_grow_full(d, update_neigh=False)
+
+    # sparse levels, finest first
+    for d in range(depth, self.full_depth, -1):
+      n = node_key.numel()
+      ws = _lib.workspace(L.ocnn_build_level_workspace_bytes(n), dev)
+      pidx = torch.empty(n, dtype=torch.int32, device=dev)
+      _lib.check(L.ocnn_build_level_count(_lib.ptr(node_key), n, _lib.ptr(ws), ws.numel(),
+                                          _lib.ptr(pidx), _lib.ptr(n_dev), st))
+      n_parent = int(n_dev.item())
+      keys = torch.empty(8 * n_parent, dtype=torch.long, device=dev)
+      children = torch.empty(8 * n_parent, dtype=torch.int32, device=dev)
+      next_key = torch.empty(n_parent, dtype=torch.long, device=dev)
+      _lib.check(L.ocnn_build_level_fill(_lib.ptr(node_key), _lib.ptr(pidx), n, n_parent,
+                                         int(self.batch_size > 1), _lib.ptr(keys),
+                                         _lib.ptr(children), _lib.ptr(next_key), st))
+      self.keys[d] = keys
+      self.children[d] = children
+      self.nnum[d] = 8 * n_parent
+      self.nnum_nempty[d] = n
+      node_key = next_key
+
+    # children of the deepest full layer
+    d = self.full_depth
+    children = -torch.ones_like(self.children[d])
+    at = node_key if self.batch_size == 1 else \
+        ((node_key >> 48) << (3 * d)) | (node_key & ((1 << 48) - 1))
+    children[at] = torch.arange(node_key.numel(), dtype=torch.int32, device=dev)
+    self.children[d] = children
+    self.nnum_nempty[d] = node_key.numel()
+
+    # per-leaf signals
+    def leaf(src, mode):
+      src = src.float().contiguous()
+      out = torch.empty(nleaf, src.shape[1], dtype=torch.float32, device=dev)
+      _lib.check(L.ocnn_leaf_average(_lib.ptr(src), src.shape[1], _lib.ptr(perm),
+                                     _lib.ptr(seg_start), nleaf, mode, _lib.ptr(out), st))
+      return out
+
+    self.points[depth] = leaf(pts_norm, 0)
+    if point_cloud.normals is not None:
+      self.normals[depth] = leaf(point_cloud.normals, 1)
+    if point_cloud.features is not None:
+      self.features[depth] = leaf(point_cloud.features, 0)
+
+    num = depth + 1
+    self.nempty_masks = [None] * num
+    self.nempty_indices = [None] * num
+    self.nempty_neighs = [None] * num
+    self._nempty_indices32 = [None] * num
+    self._tables, self._tables_t = {}, {}
+    return idx
+
+  def octree_grow_full(self, depth: int, update_neigh: bool = True):
+    """Dense layer (ocnn/octree/octree.py:289-321)."""
+    assert depth <= self.full_depth, 'error'
+    num = 1 << (3 * depth)
+    bs = self.batch_size
+    self.nnum[depth] = num * bs
+    self.nnum_nempty[depth] = num * bs
+    key = torch.arange(num, dtype=torch.long, device=self.device)
+    b = torch.arange(bs, dtype=torch.long, device=self.device)
+    self.keys[depth] = (key.unsqueeze(0) | (b.unsqueeze(1) << 48)).view(-1)
+    self.children[depth] = torch.arange(num * bs, dtype=torch.int32, device=self.device)
+    self._drop_nempty(depth)
+    if update_neigh:
+      self.construct_neigh(depth)
+
+  def octree_split(self, split: torch.Tensor, depth: int):
+    """Sets which nodes of `depth` are split (ocnn/octree/octree.py:323-351)."""
+    empty = split == 0
+    total = cumsum(split, dim=0, exclusive=True)
+    children, nnum_nempty = torch.split(total, [split.shape[0], 1])
+    children[empty] = -1
+    if nnum_nempty == 0:
+      nnum_nempty = 1
+      children[0] = 0
+    self.children[depth] = children.int()
+    self.nnum_nempty[depth] = nnum_nempty
+    self._drop_nempty(depth)
+
+  def octree_grow(self, depth: int, update_neigh: bool = True):
+    """Adds the children layer of the split nodes (ocnn/octree/octree.py:353-402)."""
+    if depth > self.depth:
+      assert depth == self.depth + 1
+      self.depth = depth
+      for lst in (self.keys, self.children, self.features, self.normals, self.points,
+                  self.nempty_masks, self.nempty_indices, self.nempty_neighs,
+                  self._nempty_indices32):
+        lst.append(None)
+      self.neighs.append(None)
+      zero = torch.zeros(1, dtype=torch.long)
+      self.nnum = torch.cat([self.nnum, zero])
+      self.nnum_nempty = torch.cat([self.nnum_nempty, zero])
+      zero = torch.zeros([1, self.batch_size], dtype=torch.long)
+      self.batch_nnum = torch.cat([self.batch_nnum, zero], dim=0)
+      self.batch_nnum_nempty = torch.cat([self.batch_nnum_nempty, zero], dim=0)
+
+    nnum = self.nnum_nempty[depth - 1] * 8
+    self.nnum[depth] = nnum
+    self.nnum_nempty[depth] = nnum
+    key = self.key(depth - 1, nempty=True)
+    batch_id = (key >> 48) << 48
+    key = ((key & ((1 << 48) - 1)) << 3) | batch_id
+    key = key.unsqueeze(1) + torch.arange(8, device=key.device)
+    self.keys[depth] = key.view(-1)
+    self.children[depth] = torch.arange(int(nnum), dtype=torch.int32, device=self.device)
+    self._drop_nempty(depth)
+    if update_neigh:
+      self.construct_neigh(depth)
+
+  # ---- neighbour search (ocnn/octree/octree.py:404-446) ---------------------
+  def construct_neigh(self, depth: int):
+    L = _lib.lib()
+    dev = torch.device(self.device) if isinstance(self.device, str) else self.device
+    if dev.type != 'cuda':
+      raise RuntimeError('ocnn_amd kernels need the octree on a HIP device, it is on '
+                         '{}'.format(dev))
+    st = _lib.stream()
+    if depth <= self.full_depth:
+      rows = self.batch_size << (3 * depth)
+      out = torch.empty(rows, 27, dtype=torch.int32, device=dev)
+      _lib.check(L.ocnn_neigh_full(depth, self.batch_size, None, _lib.ptr(out), st))
+    else:
+      child_p = self.children[depth - 1]
+      neigh_p = self.neighs.get32(depth - 1)
+      assert neigh_p is not None, 'construct_neigh({}) first'.format(depth - 1)
+      n_ne = int(self.nnum_nempty[depth - 1])
+      assert 8 * n_ne == int(self.nnum[depth]), 'octree layers are inconsistent'
+      out = torch.empty(8 * n_ne, 27, dtype=torch.int32, device=dev)
+      _lib.check(L.ocnn_neigh_from_parent(_lib.ptr(child_p), _lib.ptr(neigh_p.contiguous()),
+                                          _lib.ptr(self._nempty_index32(depth - 1)), n_ne, None,
+                                          _lib.ptr(out), st))
+    self.neighs[depth] = out
+    self.nempty_neighs[depth] = None
+    self._drop_tables(depth)
+
+  def construct_all_neigh(self):
+    for depth in range(1, self.depth + 1):
+      self.construct_neigh(depth)
+
+  # ---- search (ocnn/octree/octree.py:448-488) -------------------------------
+  def search_xyzb(self, query: torch.Tensor, depth: int, nempty: bool = False):
+    key = xyz2key(query[:, 0], query[:, 1], query[:, 2], query[:, 3], depth)
+    return self.search_key(key, depth, nempty)
+
+  def search_key(self, query: torch.Tensor, depth: int, nempty: bool = False):
+    key = self.key(depth, nempty)
+    idx = torch.searchsorted(key, query)
+    valid = idx < key.shape[0]
+    found = torch.zeros_like(valid)
+    found[valid] = key[idx[valid]] == query[valid]
+    idx[found.logical_not()] = -1
+    return idx
+
+  # ---- tables for the layers ------------------------------------------------
+  def _table(self, depth, kernel='333', stride=1, nempty=False):
+    """int32 table of get_neigh(depth, kernel, stride, nempty), cached."""
+    if stride not in (1, 2):
+      raise ValueError('Unsupported stride {}'.format(stride))
+    if kernel != '333' and kernel not in LUT_KERNEL:
+      raise ValueError('Unsupported kernel {}'.format(kernel))
+    ck = (depth, kernel, stride, bool(nempty))
+    if ck in self._tables:
+      return self._tables[ck]
+    base = self.neighs.get32(depth)
+    assert base is not None, 'construct_neigh({}) first'.format(depth)
+    if kernel == '333' and stride == 1 and not nempty:
+      self._tables[ck] = base
+      return base
+    _lib.require_gpu(base)
+    cols = LUT_KERNEL.get(kernel)
+    K = 27 if cols is None else len(cols)
+    h_cols = None if cols is None else (ctypes.c_int * K)(*cols)
+    row_index, row_stride, rows = None, 1, base.shape[0]
+    if stride == 2:
+      row_stride, rows = 8, base.shape[0] // 8
+    elif nempty:
+      row_index, rows = self._nempty_index32(depth), int(self.nnum_nempty[depth])
+    children = self.children[depth] if nempty else None
+    out = torch.empty(rows, K, dtype=torch.int32, device=base.device)
+    _lib.check(_lib.lib().ocnn_neigh_select(
+        _lib.ptr(base), _lib.ptr(row_index), row_stride, _lib.ptr(children), h_cols, K, rows,
+        None, _lib.ptr(out), _lib.stream()))
+    self._tables[ck] = out
+    return out
+
+  def _table_t(self, depth, kernel, stride, nempty, rows_in):
+    """Inverse table: row j, slot k -> the row i with table[i][k] == j."""
+    ck = (depth, kernel, stride, bool(nempty))
+    if ck not in self._tables_t:
+      t = self._table(depth, kernel, stride, nempty)
+      out = torch.empty(rows_in, t.shape[1], dtype=torch.int32, device=t.device)
+      _lib.check(_lib.lib().ocnn_table_transpose(_lib.ptr(t), t.shape[0], t.shape[1], rows_in,
+                                                 _lib.ptr(out), _lib.stream()))
+      self._tables_t[ck] = out
+    return self._tables_t[ck]
+
+  @staticmethod
+  def _widen(t32):
+    out = torch.empty(t32.shape, dtype=torch.long, device=t32.device)
+    _lib.check(_lib.lib().ocnn_table_to_i64(_lib.ptr(t32), t32.numel(), _lib.ptr(out),
+                                            _lib.stream()))
+    return out
+
+  def get_neigh(self, depth: int, kernel: str = '333', stride: int = 1, nempty: bool = False):
+    """int64 table (rows, K) with the reference's semantics
+    (ocnn/octree/octree.py:490-523): the cached tensor itself for stride 1 (all
+    nodes, or non-empty nodes with kernel '333'), a fresh tensor otherwise."""
+    if stride not in (1, 2):
+      raise ValueError('Unsupported stride {}'.format(stride))
+    if kernel != '333' and kernel not in LUT_KERNEL:
+      raise ValueError('Unsupported kernel {}'.format(kernel))
+    if kernel == '333' and stride == 1:
+      return self.nempty_neigh(depth) if nempty else self.neighs[depth]
+    return self._widen(self._table(depth, kernel, stride, nempty))
+
+  # ---- input signal (ocnn/octree/octree.py:525-568) -------------------------
+  def get_input_feature(self, feature: str, nempty: bool = False):
+    from ..nn.octree_pad import octree_pad
+    features = []
+    depth = self.depth
+    feature = feature.upper()
+    if 'N' in feature:
+      features.append(self.normals[depth])
+    if 'L' in feature or 'D' in feature:
+      local_points = self.points[depth].frac() - 0.5
+    if 'D' in feature:
+      features.append(torch.sum(local_points * self.normals[depth], dim=1, keepdim=True))
+    if 'L' in feature:
+      features.append(local_points)
+    if 'P' in feature:
+      features.append(self.points[depth] * (2 ** (1 - depth)) - 1.0)
+    if 'F' in feature:
+      features.append(self.features[depth])
+    out = torch.cat(features, dim=1)
+    if not nempty:
+      out = octree_pad(out, self, depth)
+    return out
+
+  def to_points(self, rescale: bool = True):
+    depth = self.depth
+    xyz = self.points[depth]
+    batch_id = self.batch_id(depth, nempty=True)
+    if xyz is None:
+      x, y, z, batch_id = self.xyzb(depth, nempty=True)
+      xyz = torch.stack([x, y, z], dim=1) + 0.5
+    if rescale:
+      xyz = xyz * (2 ** (1 - depth)) - 1.0
+    return Points(xyz, self.normals[depth], self.features[depth], batch_id=batch_id,
+                  batch_size=self.batch_size)
+
+  # ---- device moves, batching (ocnn/octree/octree.py:600-752) ---------------
+  def to(self, device: Union[torch.device, str], non_blocking: bool = False):
+    if isinstance(device, str):
+      device = torch.device(device)
+    if self.device == device:
+      return self
+
+    def mv(prop):
+      return [p.to(device, non_blocking=non_blocking) if isinstance(p, torch.Tensor) else None
+              for p in prop]
+
+    octree = Octree.init_like(self, device)
+    octree.keys = mv(self.keys)
+    octree.children = mv(self.children)
+    octree.neighs = self.neighs.moved(device, non_blocking)
+    octree.features = mv(self.features)
+    octree.normals = mv(self.normals)
+    octree.points = mv(self.points)
+    octree.nnum = self.nnum.clone()
+    octree.nnum_nempty = self.nnum_nempty.clone()
+    octree.batch_nnum = self.batch_nnum.clone()
+    octree.batch_nnum_nempty = self.batch_nnum_nempty.clone()
+    return octree
+
+  def cuda(self, non_blocking: bool = False):
+    return self.to('cuda', non_blocking)
+
+  def cpu(self):
+    return self.to('cpu')
+
+  def merge_octrees(self, octrees: List['Octree']):
+    """Batches single octrees (ocnn/octree/octree.py:653-717)."""
+    bs = len(octrees)
+    self.batch_size = bs
+    for o in octrees[1:]:
+      assert (o.depth == self.depth and o.full_depth == self.full_depth and
+              o.device == self.device), 'The check of merge_octrees failed'
+    batch_nnum = torch.stack([o.nnum for o in octrees], dim=1)
+    batch_nnum_nempty = torch.stack([o.nnum_nempty for o in octrees], dim=1)
+    self.nnum = torch.sum(batch_nnum, dim=1)
+    self.nnum_nempty = torch.sum(batch_nnum_nempty, dim=1)
+    self.batch_nnum = batch_nnum
+    self.batch_nnum_nempty = batch_nnum_nempty
+    offset = cumsum(batch_nnum_nempty, dim=1, exclusive=True)
+
+    num = self.depth + 1
+    self.neighs = _NeighTables(num)
+    self.nempty_masks = [None] * num
+    self.nempty_indices = [None] * num
+    self.nempty_neighs = [None] * num
+    self._nempty_indices32 = [None] * num
+    self._tables, self._tables_t = {}, {}
+    low48 = (1 << 48) - 1
+    for d in range(num):
+      self.keys[d] = torch.cat([(o.keys[d] & low48) | (i << 48)
+                                for i, o in enumerate(octrees)], dim=0)
+      kids = []
+      for i, o in enumerate(octrees):
+        c = o.children[d]
+        kids.append(torch.where(c >= 0, c + int(offset[d, i]), c))
+      self.children[d] = torch.cat(kids, dim=0)
+      if d == self.depth:
+        for name in ('features', 'normals', 'points'):
+          if getattr(octrees[0], name)[d] is not None:
+            getattr(self, name)[d] = torch.cat([getattr(o, name)[d] for o in octrees], dim=0)
+    return self
+
+  @classmethod
+  def init_like(cls, octree: 'Octree', device: Union[torch.device, str, None] = None):
+    device = device if device is not None else octree.device
+    return cls(depth=octree.depth, full_depth=octree.full_depth,
+               batch_size=octree.batch_size, device=device)
+
+  @classmethod
+  def init_octree(cls, depth: int, full_depth: int = 2, batch_size: int = 1,
+                  device: Union[torch.device, str] = 'cpu'):
+    octree = cls(depth, full_depth, batch_size, device)
+    for d in range(full_depth + 1):
+      octree.octree_grow_full(depth=d)
+    return octree
+
+
+def merge_octrees(octrees: List['Octree']):
+  return Octree.init_like(octrees[0]).merge_octrees(octrees)
+
+
+def init_octree(depth: int, full_depth: int = 2, batch_size: int = 1,
+                device: Union[torch.device, str] = 'cpu'):
+  return Octree.init_octree(depth, full_depth, batch_size, device)

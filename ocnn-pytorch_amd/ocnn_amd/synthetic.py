@@ -1,0 +1,113 @@
+"""Seeded synthetic point clouds for benchmarks and tests (CPU float32 tensors).
+
+Every cloud lies strictly inside [-1, 1]^3 and carries analytic unit normals.
+"""
+
+import math
+
+import torch
+
+
+def _gen(seed):
+  g = torch.Generator()
+  g.manual_seed(int(seed))
+  return g
+
+
+def sphere_points(n, g, radius=0.99, center=(0.0, 0.0, 0.0)):
+  d = torch.randn(n, 3, generator=g)
+  d = d / d.norm(dim=1, keepdim=True).clamp_min(1e-12)
+  return d * radius + torch.tensor(center, dtype=torch.float32), d
+
+
+def box_points(n, g, lo, hi):
+  """Uniform on the surface of the axis-aligned box [lo, hi] (area weighted)."""
+  lo = torch.tensor(lo, dtype=torch.float32)
+  hi = torch.tensor(hi, dtype=torch.float32)
+  ext = hi - lo
+  area = torch.stack([ext[1] * ext[2], ext[0] * ext[2], ext[0] * ext[1]]).repeat_interleave(2)
+  face = torch.multinomial(area / area.sum(), n, replacement=True, generator=g)
+  axis, side = face // 2, face % 2
+  p = lo + torch.rand(n, 3, generator=g) * ext
+  rows = torch.arange(n)
+  p[rows, axis] = torch.where(side == 1, hi[axis], lo[axis])
+  nrm = torch.zeros(n, 3)
+  nrm[rows, axis] = side.float() * 2 - 1
+  return p, nrm
+
+
+def plane_points(n, g, normal, offset, half=0.98):
+  """Points of the plane {x : <x, normal> = offset} inside the cube (rejection)."""
+  nvec = torch.tensor(normal, dtype=torch.float32)
+  nvec = nvec / nvec.norm()
+  out = []
+  got = 0
+  while got < n:
+    q = (torch.rand(2 * n, 3, generator=g) * 2 - 1) * half
+    q = q - ((q @ nvec) - offset).unsqueeze(1) * nvec
+    q = q[(q.abs() <= half).all(1)]
+    out.append(q)
+    got += q.shape[0]
+  p = torch.cat(out)[:n]
+  return p, nvec.expand(n, 3).clone()
+
+
+def sphere_cloud(n=20000, seed=1000):
+  """Config 0: points on the unit sphere scaled by 0.99, normals = direction."""
+  return sphere_points(n, _gen(seed))
+
+
+def mixed_cloud(n=100000, seed=1001, n_spheres=3, n_boxes=2):
+  """Configs 1/2: spheres (radius U[0.1,0.5]) and axis-aligned boxes, each
+  fully inside 0.98 * [-1,1]^3, equal share of the points."""
+  g = _gen(seed)
+  parts = n_spheres + n_boxes
+  per = [n // parts + (1 if i < n % parts else 0) for i in range(parts)]
+  pts, nrm = [], []
+  for i in range(n_spheres):
+    r = 0.1 + 0.4 * torch.rand(1, generator=g).item()
+    c = ((torch.rand(3, generator=g) * 2 - 1) * (0.98 - r)).tolist()
+    p, m = sphere_points(per[i], g, r, c)
+    pts.append(p)
+    nrm.append(m)
+  for i in range(n_boxes):
+    a = (torch.rand(3, generator=g) * 2 - 1) * 0.98
+    b = (torch.rand(3, generator=g) * 2 - 1) * 0.98
+    lo, hi = torch.minimum(a, b), torch.maximum(a, b)
+    hi = torch.maximum(hi, lo + 0.05).clamp(max=0.98)
+    p, m = box_points(per[n_spheres + i], g, lo.tolist(), hi.tolist())
+    pts.append(p)
+    nrm.append(m)
+  return torch.cat(pts), torch.cat(nrm)
+
+
+def planes_cloud(n=250000, seed=1003, n_planes=4, n_spheres=3):
+  """Config 3: random planes clipped to the cube plus spheres."""
+  g = _gen(seed)
+  parts = n_planes + n_spheres
+  per = [n // parts + (1 if i < n % parts else 0) for i in range(parts)]
+  pts, nrm = [], []
+  for i in range(n_planes):
+    normal = torch.randn(3, generator=g).tolist()
+    offset = (torch.rand(1, generator=g).item() * 2 - 1) * 0.5
+    p, m = plane_points(per[i], g, normal, offset)
+    pts.append(p)
+    nrm.append(m)
+  for i in range(n_spheres):
+    r = 0.1 + 0.4 * torch.rand(1, generator=g).item()
+    c = ((torch.rand(3, generator=g) * 2 - 1) * (0.98 - r)).tolist()
+    p, m = sphere_points(per[n_planes + i], g, r, c)
+    pts.append(p)
+    nrm.append(m)
+  return torch.cat(pts), torch.cat(nrm)
+
+
+def batch_clouds(maker, batch, seed, **kw):
+  """`batch` clouds -> (points, normals, batch_id as float32 (N,1))."""
+  pts, nrm, bid = [], [], []
+  for b in range(batch):
+    p, m = maker(seed=seed * 100 + b, **kw)
+    pts.append(p)
+    nrm.append(m)
+    bid.append(torch.full((p.shape[0], 1), float(b)))
+  return torch.cat(pts), torch.cat(nrm), torch.cat(bid)

@@ -1,0 +1,113 @@
+"""CPU checks of the shipped package: the C-ABI library loads and exports every
+symbol the header declares, the host-evaluable kernel arithmetic agrees with
+the oracle, and the host-side logic (shapes, errors, no CPU fallback)."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import ocnn_amd
+from ocnn_amd import _lib
+from oracle import octree_ref as R
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+  text = open(os.path.join(ROOT, 'include', 'ocnn_hip.h')).read()
+  text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+  return sorted(set(re.findall(r'\b(ocnn_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+  names = declared_symbols()
+  assert len(names) >= 30
+  handle = ctypes.CDLL(ocnn_amd.build.LIB_PATH)
+  for name in names:
+    assert hasattr(handle, name), name
+  assert sorted(_lib.SIGNATURES) == names          # the binding covers the header exactly
+  assert _lib.lib().ocnn_abi_version() == 1
+
+
+@pytest.mark.parametrize('depth', [1, 4, 8, 9, 13, 16])
+def test_host_key_arithmetic_matches_oracle(depth):
+  L = _lib.lib()
+  rng = np.random.default_rng(depth)
+  xyz = rng.integers(-3, (1 << depth) + 3, size=(300, 3))
+  b = rng.integers(0, 32768, size=300)
+  want = R.xyz2key(xyz[:, 0], xyz[:, 1], xyz[:, 2], b, depth)
+  buf = (ctypes.c_int64 * 4)()
+  for i in range(300):
+    got = L.ocnn_host_encode_key(int(xyz[i, 0]), int(xyz[i, 1]), int(xyz[i, 2]), int(b[i]), depth)
+    assert got == int(want[i])
+    L.ocnn_host_decode_key(got, depth, buf)
+    x, y, z, bb = R.key2xyz(np.array([got]), depth)
+    assert list(buf) == [int(x[0]), int(y[0]), int(z[0]), int(bb[0])]
+
+
+def test_host_child_slot_lut_matches_reference_tables():
+  L = _lib.lib()
+  lut_parent, lut_child = R.neigh_luts()
+  lp, lc = ctypes.c_int(), ctypes.c_int()
+  for j in range(8):
+    for k in range(27):
+      L.ocnn_host_child_slot_lut(j, k, ctypes.byref(lp), ctypes.byref(lc))
+      assert (lp.value, lc.value) == (int(lut_parent[j, k]), int(lut_child[j, k]))
+
+
+def test_octree_public_luts_and_errors():
+  o = ocnn_amd.Octree(depth=5, full_depth=2, batch_size=2)
+  lut_parent, lut_child = R.neigh_luts()
+  assert np.array_equal(o.lut_parent.numpy(), lut_parent)
+  assert np.array_equal(o.lut_child.numpy(), lut_child)
+  for k, v in R.LUT_KERNEL.items():
+    assert o.lut_kernel[k].tolist() == v
+  assert o.nnum.dtype == torch.long and o.nnum.device.type == 'cpu'
+  assert len(o.neighs) == 6 and o.neighs[3] is None
+  with pytest.raises(ValueError):
+    o.get_neigh(3, '123')
+  with pytest.raises(ValueError):
+    o.get_neigh(3, '333', stride=3)
+
+
+def test_no_cpu_fallback():
+  pts = ocnn_amd.Points(torch.rand(10, 3) * 0.5)
+  o = ocnn_amd.Octree(depth=4, full_depth=2)
+  with pytest.raises(RuntimeError):
+    o.build_octree(pts)
+  with pytest.raises(RuntimeError):
+    ocnn_amd.octree.xyz2key(torch.zeros(3), torch.zeros(3), torch.zeros(3), depth=4)
+  with pytest.raises(RuntimeError):
+    o.construct_neigh(1)
+
+
+def test_module_contract():
+  from ocnn_amd.nn import OctreeConv, OctreeDeconv, OctreeDWConv
+  c = OctreeConv(3, 5, [3], stride=1, nempty=True, use_bias=True)
+  assert tuple(c.weights.shape) == (27, 3, 5) and tuple(c.bias.shape) == (5,)
+  assert c.kernel == '333' and c.kernel_size == [3, 3, 3] and c.kdim == 27
+  assert set(c.state_dict()) == {'weights', 'bias'}
+  d = OctreeDeconv(3, 5, [2], stride=2)
+  assert tuple(d.weights.shape) == (8, 5, 3) and d.bias is None
+  w = OctreeDWConv(7, [3, 1, 1])
+  assert tuple(w.weights.shape) == (3, 1, 7) and not hasattr(w, 'bias')
+  bound = (3.0 ** 0.5) * (2.0 / (27 * 3 + 27 * 5)) ** 0.5
+  assert float(c.weights.abs().max()) <= bound
+  with pytest.raises(ValueError):
+    OctreeConv(3, 5, method='nope')
+  assert 'kernel_size=[3, 3, 3]' in repr(c)
+
+
+def test_points_normalize_and_merge():
+  from ocnn_amd.octree import Points, merge_points
+  p = Points(torch.tensor([[-1.0, 0.0, 0.5]]))
+  assert torch.equal(p.normalize(-1.0, 1.0, 64), torch.tensor([[0.0, 32.0, 48.0]]))
+  m = merge_points([Points(torch.zeros(2, 3)), Points(torch.ones(3, 3))])
+  assert m.batch_size == 2 and m.batch_id.view(-1).tolist() == [0, 0, 1, 1, 1]
+  assert m.batch_id.dtype == torch.float32
+  with pytest.raises(AssertionError):
+    Points(torch.zeros(2, 2))

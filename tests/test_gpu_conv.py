@@ -1,0 +1,287 @@
+"""GPU parity of OctreeConv / OctreeDeconv / OctreeDWConv (forward, data
+gradient, weight gradient) through the C ABI against the fp64 oracle.
+
+Tolerances (relative to the largest magnitude of the expected tensor):
+  float32            1e-4
+  float16, bfloat16  2e-2 against the fp64 result on the same (rounded) inputs
+"""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import ocnn_amd
+from ocnn_amd import _lib, synthetic
+from ocnn_amd.nn import (OctreeConv, OctreeConvTriton, OctreeDeconv, OctreeDWConv, octree_conv,
+                         octree_conv_triton, octree_depad, octree_pad)
+from ocnn_amd.octree import Octree, Points, merge_points
+from oracle import conv_ref as C
+from oracle import octree_ref as R
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+
+
+def say(*a):
+  print(*a, flush=True)
+  sys.stdout.flush()
+
+
+def rel_err(got, want):
+  got = got.detach().double().cpu().numpy()
+  scale = max(1e-30, float(np.abs(want).max()))
+  return float(np.abs(got - want).max()) / scale
+
+
+def f64(t):
+  return t.detach().double().cpu().numpy()
+
+
+class Pair:
+  """The same octree on the GPU (HIP path) and in the oracle."""
+
+  def __init__(self, pts, nrm, bid, depth, full_depth, batch):
+    pc = Points(pts.to(DEV), nrm.to(DEV), batch_id=None if bid is None else bid.to(DEV),
+                batch_size=batch)
+    self.gpu = Octree(depth, full_depth, batch_size=batch)
+    self.gpu.build_octree(pc)
+    self.gpu.construct_all_neigh()
+    self.ref, _ = R.build_octree(pts.numpy(), nrm.numpy(),
+                                 batch_id=None if bid is None else bid.numpy(), depth=depth,
+                                 full_depth=full_depth, batch_size=batch)
+    R.construct_all_neigh(self.ref)
+
+
+@pytest.fixture(scope='module')
+def small(ref_data):
+  d4 = np.load(os.path.join(ref_data, 'octree/test_004.npz'))
+  d5 = np.load(os.path.join(ref_data, 'octree/test_005.npz'))
+  pts = torch.from_numpy(np.concatenate([d4['points'], d5['points']]))
+  nrm = torch.from_numpy(np.concatenate([d4['normals'], d5['normals']]))
+  bid = torch.cat([torch.zeros(len(d4['points']), 1), torch.ones(len(d5['points']), 1)])
+  return Pair(pts, nrm, bid, 6, 3, 2)
+
+
+@pytest.fixture(scope='module')
+def medium():
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 3, 11, n=40000)
+  return Pair(pts, nrm, bid, 7, 2, 3)
+
+
+def rows_of(oct_ref, depth, nempty):
+  return int(oct_ref.nnum_nempty[depth] if nempty else oct_ref.nnum[depth])
+
+
+def run_layer(kind, pair, depth, ks, stride, nempty, cin, cout, dtype, seed=0, use_bias=True):
+  """Runs module forward + backward on the GPU and the oracle; returns errors."""
+  g = torch.Generator().manual_seed(seed)
+  K = ks[0] * ks[1] * ks[2]
+  if kind == 'conv':
+    mod = OctreeConv(cin, cout, ks, stride, nempty, use_bias=use_bias)
+    layer = C.conv_layer
+  elif kind == 'deconv':
+    mod = OctreeDeconv(cin, cout, ks, stride, nempty, use_bias=use_bias)
+    layer = C.deconv_layer
+  else:
+    mod = OctreeDWConv(cin, ks, stride, nempty, use_bias=use_bias)
+    layer = C.dwconv_layer
+  with torch.no_grad():
+    mod.weights.copy_(torch.randn(mod.weights.shape, generator=g) / (K * cin) ** 0.5)
+    if use_bias:
+      mod.bias.copy_(torch.randn(mod.bias.shape, generator=g))
+  mod = mod.to(DEV).to(dtype)
+  data = torch.randn(rows_of(pair.ref, depth, nempty), cin, generator=g).to(dtype)
+  x = data.to(DEV).requires_grad_()
+  out = mod(x, pair.gpu, depth)
+  gout = torch.randn(out.shape, generator=g).to(dtype)
+  out.backward(gout.to(DEV))
+  bias = f64(mod.bias) if use_bias else None
+  want = layer(pair.ref, f64(data), f64(mod.weights), depth, ks, stride, nempty, bias=bias,
+               grad=f64(gout))
+  assert tuple(out.shape) == want[0].shape
+  errs = {'out': rel_err(out, want[0]), 'gdata': rel_err(x.grad, want[1]),
+          'gw': rel_err(mod.weights.grad, want[2])}
+  if use_bias:
+    errs['gb'] = rel_err(mod.bias.grad, want[3])
+  assert out.dtype == dtype and x.grad.dtype == dtype and mod.weights.grad.dtype == dtype
+  return errs
+
+
+GRID = [(k, s, ne) for k in ['333', '222', '311', '131', '113', '331', '313', '133']
+        for s in (1, 2) for ne in (False, True)]
+
+
+@pytest.mark.parametrize('kind', ['conv', 'deconv', 'dwconv'])
+def test_fp32_grid(small, kind):
+  """Every kernel shape x stride x nempty, fp32 (plain kernels, odd channels)."""
+  for kern, stride, ne in GRID:
+    ks = [int(c) for c in kern]
+    depth = 4 if kind == 'deconv' else 5
+    say('fp32', kind, kern, 'stride', stride, 'nempty', ne)
+    errs = run_layer(kind, small, depth, ks, stride, ne, 5, 7, torch.float32)
+    assert max(errs.values()) < TOL[torch.float32], (kind, kern, stride, ne, errs)
+
+
+MFMA_SHAPES = [(32, 32), (64, 64), (64, 128), (128, 64), (32, 48), (96, 16)]
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('tr', [1, 0])
+def test_mfma_conv_333(small, medium, dtype, tr):
+  """3x3x3 stride-1 conv on the MFMA kernels, several channel shapes, both
+  nempty modes, both ways of reading the weight-gradient tiles."""
+  _lib.lib().ocnn_set_wgrad_transpose_load(tr)
+  try:
+    for cin, cout in MFMA_SHAPES:
+      for pair, depth in ((small, 6), (medium, 7), (medium, 5)):
+        for ne in (False, True):
+          say('mfma conv', dtype, 'tr', tr, cin, cout, 'depth', depth, 'nempty', ne)
+          errs = run_layer('conv', pair, depth, [3], 1, ne, cin, cout, dtype)
+          assert max(errs.values()) < TOL[dtype], (cin, cout, depth, ne, errs)
+  finally:
+    _lib.lib().ocnn_set_wgrad_transpose_load(1)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_mfma_stride2_deconv_dw(medium, dtype):
+  """The child/parent paths: 2x2x2 stride-2 conv and deconv, 3x3x3 stride-2,
+  and the depth-wise kernel, in 16-bit types."""
+  for ne in (False, True):
+    say('mfma s2 conv 64->128', dtype, ne)
+    errs = run_layer('conv', medium, 7, [2], 2, ne, 64, 128, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
+    say('mfma s2 deconv 128->64', dtype, ne)
+    errs = run_layer('deconv', medium, 6, [2], 2, ne, 128, 64, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
+    say('mfma s2 conv 333 32->32', dtype, ne)
+    errs = run_layer('conv', medium, 7, [3], 2, ne, 32, 32, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
+    say('mfma s1 deconv 333 32->64', dtype, ne)
+    errs = run_layer('deconv', medium, 6, [3], 1, ne, 32, 64, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
+    say('dwconv 128', dtype, ne)
+    errs = run_layer('dwconv', medium, 6, [3], 1, ne, 128, 128, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
+    errs = run_layer('dwconv', medium, 7, [2], 2, ne, 24, 24, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
+
+
+def test_fp32_larger(medium):
+  say('fp32 32->32 at depth 6 (the CPU-runnable reference case shape)')
+  errs = run_layer('conv', medium, 6, [3], 1, False, 32, 32, torch.float32)
+  assert max(errs.values()) < TOL[torch.float32], errs
+  errs = run_layer('conv', medium, 6, [3], 1, True, 32, 32, torch.float32)
+  assert max(errs.values()) < TOL[torch.float32], errs
+
+
+def test_mixed_precision_and_no_bias(small):
+  say('fp32 parameters with fp16 data (weights cast inside, grads cast back)')
+  conv = OctreeConv(32, 32, [3], 1, nempty=True, use_bias=False).to(DEV)
+  data = torch.randn(rows_of(small.ref, 6, True), 32, generator=torch.Generator().manual_seed(1))
+  x = data.half().to(DEV).requires_grad_()
+  out = conv(x, small.gpu, 6)
+  assert out.dtype == torch.float16
+  out.sum().backward()
+  assert conv.weights.grad.dtype == torch.float32 and x.grad.dtype == torch.float16
+  want = C.conv_layer(small.ref, f64(data.half()), f64(conv.weights.half()), 6, [3], 1, True)
+  assert rel_err(out, want) < 2e-2
+
+
+def test_table_level_api(small):
+  say('octree_conv_triton(data, weight(Co,V,Ci), bias, neigh) parity with the module')
+  g = torch.Generator().manual_seed(5)
+  cin, cout, depth = 32, 64, 6
+  neigh = small.gpu.get_neigh(depth, '333', 1, False)            # int64, as the reference passes
+  w = (torch.randn(27, cin, cout, generator=g) / 30).half().to(DEV).requires_grad_()
+  b = torch.randn(cout, generator=g).half().to(DEV).requires_grad_()
+  x = torch.randn(neigh.shape[0], cin, generator=g).half().to(DEV).requires_grad_()
+  out = octree_conv_triton(x, w.permute(2, 0, 1), b, neigh)
+  gout = torch.randn(out.shape, generator=g).half().to(DEV)
+  out.backward(gout)
+  want = C.conv_layer(small.ref, f64(x), f64(w), depth, [3], 1, False, bias=f64(b), grad=f64(gout))
+  assert rel_err(out, want[0]) < 2e-2 and rel_err(x.grad, want[1]) < 2e-2
+  assert rel_err(w.grad, want[2]) < 2e-2 and rel_err(b.grad, want[3]) < 2e-2
+  mod = OctreeConvTriton(cin, cout, [3], 1, use_bias=True).to(DEV).half()
+  with torch.no_grad():
+    mod.weights.copy_(w)
+    mod.bias.copy_(b)
+  assert rel_err(mod(x.detach(), small.gpu, depth), want[0]) < 2e-2
+
+
+def test_pad_depad(small):
+  say('octree_pad / octree_depad')
+  d = 5
+  x = torch.randn(int(small.ref.nnum_nempty[d]), 6).to(DEV).requires_grad_()
+  p = octree_pad(x, small.gpu, d, val=1.5)
+  assert np.array_equal(f64(p), C.octree_pad(f64(x), small.ref, d, 1.5))
+  assert torch.equal(octree_depad(p, small.gpu, d), x.detach())
+  p.sum().backward()
+  assert torch.equal(x.grad, torch.ones_like(x))
+  for dt in (torch.float16, torch.bfloat16):
+    y = torch.randn(int(small.ref.nnum[d]), 9).to(dt).to(DEV)
+    assert np.array_equal(f64(octree_depad(y, small.gpu, d)), C.octree_depad(f64(y), small.ref, d))
+
+
+def test_errors(small):
+  say('error behaviour')
+  conv = OctreeConv(4, 4).to(DEV)
+  with pytest.raises(AssertionError):
+    conv(torch.zeros(3, 4, device=DEV), small.gpu, 5)
+  with pytest.raises(RuntimeError):
+    conv(torch.zeros(int(small.ref.nnum[5]), 4), small.gpu, 5)        # CPU tensor: no fallback
+  with pytest.raises(TypeError):
+    conv.double()(torch.zeros(int(small.ref.nnum[5]), 4, device=DEV, dtype=torch.double),
+                  small.gpu, 5)
+  with pytest.raises(ValueError):
+    OctreeConv(4, 4, [5]).to(DEV)(torch.zeros(int(small.ref.nnum[5]), 4, device=DEV), small.gpu, 5)
+
+
+def test_weight_gradient_is_bit_reproducible(medium):
+  say('two runs of the split-K weight gradient give identical bits')
+  g = torch.Generator().manual_seed(9)
+  t = medium.gpu._table(7, '333', 1, False)
+  x = torch.randn(t.shape[0], 64, generator=g).bfloat16().to(DEV)
+  gr = torch.randn(t.shape[0], 64, generator=g).bfloat16().to(DEV)
+  a = ocnn_amd.nn.conv_wgrad(x, gr, t)
+  b = ocnn_amd.nn.conv_wgrad(x, gr, t)
+  assert torch.equal(a, b)
+
+
+def test_benchmark_shape_properties():
+  """Depth 8, batch 8, 64->64, fp16 and bf16 at the benchmark size: adjoint and
+  bilinear identities (size independent), plus a sampled oracle comparison."""
+  say('benchmark-size properties: build')
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 8, 1001, n=100000)
+  pc = Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=8)
+  o = Octree(8, 2, batch_size=8)
+  o.build_octree(pc)
+  o.construct_all_neigh()
+  rows = int(o.nnum[8])
+  g = torch.Generator().manual_seed(2)
+  for dtype in (torch.float16, torch.bfloat16):
+    say('benchmark-size properties:', dtype, rows, 'rows')
+    conv = OctreeConv(64, 64, [3], 1).to(DEV).to(dtype)
+    x = torch.randn(rows, 64, generator=g).to(dtype).to(DEV).requires_grad_()
+    out = conv(x, o, 8)
+    gout = torch.randn(rows, 64, generator=g).to(dtype).to(DEV)
+    out.backward(gout)
+    lhs = (out.double() * gout.double()).sum().item()
+    rhs_x = (x.detach().double() * x.grad.double()).sum().item()
+    rhs_w = (conv.weights.detach().double() * conv.weights.grad.double()).sum().item()
+    scale = (out.double().norm() * gout.double().norm()).item()
+    assert abs(lhs - rhs_x) / scale < 2e-3, (lhs, rhs_x, scale)
+    assert abs(lhs - rhs_w) / scale < 2e-3, (lhs, rhs_w, scale)
+    # sampled rows against the definition, from the GPU table itself
+    t = o._table(8, '333', 1, False)
+    sel = torch.randint(0, rows, (512,), generator=g)
+    tt = t[sel.to(DEV)].cpu().numpy()
+    xd, wd = f64(x), f64(conv.weights)
+    want = np.zeros((512, 64))
+    for k in range(27):
+      v = tt[:, k] >= 0
+      want[v] += xd[tt[v, k]] @ wd[k]
+    assert rel_err(out[sel.to(DEV)], want) < TOL[dtype]

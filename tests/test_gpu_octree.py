@@ -1,0 +1,316 @@
+"""GPU parity of the octree build and neighbour search: the HIP path (through the
+C ABI) against the reference's data files and the numpy oracle, bit exact."""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import ocnn_amd
+from ocnn_amd import synthetic
+from ocnn_amd.octree import Octree, Points, key2xyz, merge_octrees, merge_points, xyz2key
+from oracle import octree_ref as R
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def say(*a):
+  print(*a, flush=True)
+  sys.stdout.flush()
+
+
+def np_(t):
+  return t.detach().cpu().numpy()
+
+
+def fixture_points(ref_data, i):
+  d = np.load(os.path.join(ref_data, 'octree/test_%03d.npz' % i))
+  pc = Points(torch.from_numpy(d['points']).to(DEV), torch.from_numpy(d['normals']).to(DEV))
+  return pc, d
+
+
+def fixture_octree(ref_data, i):
+  pc, d = fixture_points(ref_data, i)
+  o = Octree(int(d['depth']), int(d['full_depth']))
+  idx = o.build_octree(pc)
+  return o, idx, d
+
+
+def check_against(o, d):
+  assert np.array_equal(o.nnum.numpy(), d['nnum'])
+  assert np.array_equal(o.nnum_nempty.numpy(), d['nnum_nempty'])
+  key = np_(torch.cat(o.keys))
+  child = np_(torch.cat(o.children))
+  assert key.dtype == np.int64 and child.dtype == np.int32
+  assert np.array_equal(key, d['key'])
+  assert np.array_equal(child, d['child'])
+  assert np.allclose(np_(o.normals[o.depth]), d['feature'][:, :3])
+
+
+def test_keys_gpu_vs_oracle():
+  say('keys: random 16-bit coordinates')
+  g = torch.Generator().manual_seed(0)
+  for depth in (3, 8, 9, 16):
+    xyz = torch.randint(-2, (1 << depth) + 2, (5000, 3), generator=g)
+    b = torch.randint(0, 32768, (5000,), generator=g)
+    key = xyz2key(xyz[:, 0].to(DEV), xyz[:, 1].to(DEV), xyz[:, 2].to(DEV), b.to(DEV), depth)
+    want = R.xyz2key(xyz[:, 0].numpy(), xyz[:, 1].numpy(), xyz[:, 2].numpy(), b.numpy(), depth)
+    assert np.array_equal(np_(key), want)
+    x, y, z, bb = key2xyz(key, depth)
+    wx, wy, wz, wb = R.key2xyz(want, depth)
+    assert np.array_equal(np_(x), wx) and np.array_equal(np_(y), wy)
+    assert np.array_equal(np_(z), wz) and np.array_equal(np_(bb), wb)
+  # float inputs truncate toward zero; scalar batch; no batch
+  f = torch.tensor([0.9, 1.1, -0.5, 3.99], device=DEV)
+  assert np.array_equal(np_(xyz2key(f, f, f, 3, 4)),
+                        R.xyz2key(np_(f), np_(f), np_(f), np.full(4, 3), 4))
+  assert np.array_equal(np_(xyz2key(f, f, f, depth=4)), R.xyz2key(np_(f), np_(f), np_(f), None, 4))
+  # empty input
+  e = torch.zeros(0, device=DEV)
+  assert xyz2key(e, e, e, depth=4).numel() == 0
+
+
+def test_three_point_known_answer():
+  say('build: 3-point literal case')
+  pts = torch.tensor([[-1, -1, -1], [0, 0, -1], [0.0625, 0.0625, -1]], dtype=torch.float32)
+  nrm = torch.tensor([[1, 0, 0], [-1, 0, 0], [0, 1, 0]], dtype=torch.float32)
+  fea = torch.tensor([[1, -1], [2, -2], [3, -3]], dtype=torch.float32)
+  o = Octree(depth=5, full_depth=1, device=DEV)
+  idx = o.build_octree(Points(pts.to(DEV), nrm.to(DEV), fea.to(DEV)))
+  assert o.nnum.tolist() == [1, 8, 16, 16, 16, 16]
+  assert o.nnum_nempty.tolist() == [1, 2, 2, 2, 2, 3]
+  tails = {2: 48, 3: 384, 4: 3072, 5: 24576}
+  for d in range(2, 6):
+    assert np_(o.keys[d]).tolist() == list(range(8)) + list(range(tails[d], tails[d] + 8))
+  assert np_(o.children[1]).tolist() == [0, -1, -1, -1, -1, -1, 1, -1]
+  assert np_(o.children[5]).tolist() == [0] + [-1] * 7 + [1] + [-1] * 5 + [2, -1]
+  assert [np_(o.nempty_index(d)).tolist() for d in range(6)] == \
+      [[0], [0, 6], [0, 8], [0, 8], [0, 8], [0, 8, 14]]
+  assert torch.equal(o.normals[5].cpu(), nrm) and torch.equal(o.features[5].cpu(), fea)
+  assert np_(idx).tolist() == [0, 1, 2]
+  for d in range(6):
+    assert torch.equal(o.nempty_mask(d), o.children[d] >= 0)
+
+
+@pytest.mark.parametrize('i', [1, 2, 3, 4, 5])
+def test_build_against_reference_fixture(ref_data, i):
+  say('build: reference fixture', i)
+  o, idx, d = fixture_octree(ref_data, i)
+  check_against(o, d)
+  want, widx = R.build_octree(d['points'], d['normals'], depth=int(d['depth']),
+                              full_depth=int(d['full_depth']))
+  assert np.array_equal(np_(idx), widx)
+  assert np.array_equal(np_(o.points[o.depth]), want.points[o.depth])     # same sum order
+  assert np.allclose(np_(o.normals[o.depth]), want.normals[o.depth], atol=1e-6)
+
+
+def batched_points(ref_data):
+  p4, _ = fixture_points(ref_data, 4)
+  p5, _ = fixture_points(ref_data, 5)
+  return merge_points([p4, p5])
+
+
+def test_batched_build_against_reference_fixture(ref_data):
+  say('build: batch of two, reference fixture')
+  d = np.load(os.path.join(ref_data, 'batch_45.npz'))
+  o = Octree(int(d['depth']), int(d['full_depth']), batch_size=2)
+  o.build_octree(batched_points(ref_data))
+  check_against(o, d)
+  o.construct_all_neigh()
+  neigh = torch.cat(o.neighs[1:], dim=0)
+  assert neigh.dtype == torch.long
+  assert np.array_equal(np_(neigh), d['neigh'])
+
+
+def merged_octree(ref_data):
+  o4, _, _ = fixture_octree(ref_data, 4)
+  o5, _, _ = fixture_octree(ref_data, 5)
+  o = merge_octrees([o4, o5])
+  o.construct_all_neigh()
+  return o
+
+
+def test_merge_and_neigh_against_reference_fixture(ref_data):
+  say('neigh: merged octrees, reference fixture')
+  d = np.load(os.path.join(ref_data, 'batch_45.npz'))
+  o = merged_octree(ref_data)
+  check_against(o, d)
+  assert np.array_equal(np_(torch.cat(o.neighs[1:], dim=0)), d['neigh'])
+  assert o.batch_nnum.sum(1).tolist() == o.nnum.tolist()
+  # moving to the host keeps every table
+  c = o.to('cpu')
+  assert np.array_equal(torch.cat(c.neighs[1:], dim=0).numpy(), d['neigh'])
+  assert np.array_equal(torch.cat(c.keys).numpy(), d['key'])
+
+
+def test_neigh_branches_agree(ref_data):
+  say('neigh: full-layer branch == parent branch at depth 3')
+  o = merged_octree(ref_data)
+  full = o.neighs[3].clone()
+  o.full_depth = 2
+  o.construct_neigh(3)
+  assert torch.equal(full, o.neighs[3])
+
+
+def oracle_batch(ref_data):
+  d4 = np.load(os.path.join(ref_data, 'octree/test_004.npz'))
+  d5 = np.load(os.path.join(ref_data, 'octree/test_005.npz'))
+  pts = np.concatenate([d4['points'], d5['points']])
+  nrm = np.concatenate([d4['normals'], d5['normals']])
+  bid = np.concatenate([np.zeros(len(d4['points'])), np.ones(len(d5['points']))])
+  o, _ = R.build_octree(pts, nrm, batch_id=bid, depth=6, full_depth=3, batch_size=2)
+  R.construct_all_neigh(o)
+  return o
+
+
+KERNELS = ['333', '222', '311', '131', '113', '331', '313', '133']
+
+
+def test_get_neigh_grid_vs_oracle(ref_data):
+  say('get_neigh: 8 kernels x 2 strides x nempty, depths 3..6')
+  o = merged_octree(ref_data)
+  w = oracle_batch(ref_data)
+  for d in (3, 4, 5, 6):
+    for kern in KERNELS:
+      for stride in (1, 2):
+        for ne in (False, True):
+          got = o.get_neigh(d, kern, stride, ne)
+          assert got.dtype == torch.long
+          assert np.array_equal(np_(got), w.get_neigh(d, kern, stride, ne)), (d, kern, stride, ne)
+          t32 = o._table(d, kern, stride, ne)
+          assert t32.dtype == torch.int32 and np.array_equal(np_(t32), np_(got))
+    assert np.array_equal(np_(o.nempty_index(d)), w.nempty_index(d))
+    assert np.array_equal(np_(o.nempty_neigh(d)), w.nempty_neigh(d))
+  assert o.get_neigh(5) is o.get_neigh(5)                 # the cached tensor itself
+  assert o.get_neigh(5, '222', 2) is not o.get_neigh(5, '222', 2)
+  with pytest.raises(ValueError):
+    o.get_neigh(5, '223')
+  with pytest.raises(ValueError):
+    o.get_neigh(5, '333', 4)
+
+
+def test_inverse_table_vs_oracle(ref_data):
+  say('inverse tables')
+  o = merged_octree(ref_data)
+  w = oracle_batch(ref_data)
+  d = 5
+  for kern, stride, ne in [('333', 2, True), ('333', 2, False), ('222', 2, True),
+                           ('222', 1, False), ('313', 2, True)]:
+    rows_in = int(w.nnum_nempty[d] if ne else w.nnum[d])
+    got = o._table_t(d, kern, stride, ne, rows_in)
+    want = R.transpose_table(w.get_neigh(d, kern, stride, ne), rows_in)
+    assert np.array_equal(np_(got), want), (kern, stride, ne)
+
+
+def test_search_key_fixture(ref_data):
+  say('search_key: reference fixture')
+  d = np.load(os.path.join(ref_data, 'search_key.npz'))
+  o = merged_octree(ref_data)
+  xyzb = torch.from_numpy(d['xyzb']).to(DEV)
+  key = xyz2key(xyzb[:, 0], xyzb[:, 1], xyzb[:, 2], xyzb[:, 3], 5)
+  assert np.array_equal(np_(o.search_key(key, 5, False)), d['idx'])
+  assert np.array_equal(np_(o.search_key(key, 5, True)), d['idx_ne'])
+  assert np.array_equal(np_(o.search_xyzb(xyzb, 5, False)), d['idx'])
+  assert np.array_equal(np_(o.search_xyzb(xyzb, 5, True)), d['idx_ne'])
+
+
+def test_octree_grow_split(ref_data):
+  say('grow/split: regrow from the split masks')
+  d = np.load(os.path.join(ref_data, 'batch_45.npz'))
+  gt = merged_octree(ref_data)
+  depth, full_depth = 6, 3
+  o = Octree(depth, full_depth, batch_size=2, device=DEV)
+  for dd in range(full_depth + 1):
+    o.octree_grow_full(depth=dd)
+  for dd in range(full_depth, depth + 1):
+    o.octree_split((gt.children[dd] >= 0).long(), dd)
+    if dd < depth:
+      o.octree_grow(dd + 1)
+  o.normals[depth] = gt.normals[depth]
+  check_against(o, d)
+  assert np.array_equal(np_(torch.cat(o.neighs[1:], dim=0)), d['neigh'])
+
+
+def test_out_of_range_points_wrap():
+  say('build: points outside [-1,1) wrap like the reference')
+  pts = np.array([[1.0, 0.5, -0.25], [-1.01, 0.0, 0.0], [0.3, 1.2, -1.0], [0.999, -0.999, 0.1]],
+                 np.float32)
+  nrm = np.tile(np.array([[0, 0, 1]], np.float32), (4, 1))
+  o = Octree(6, 2)
+  idx = o.build_octree(Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV)))
+  w, widx = R.build_octree(pts, nrm, depth=6, full_depth=2)
+  assert np.array_equal(np_(torch.cat(o.keys)), np.concatenate(w.keys))
+  assert np.array_equal(np_(torch.cat(o.children)), np.concatenate(w.children))
+  assert np.array_equal(np_(idx), widx)
+
+
+def test_bbox_arguments(ref_data):
+  say('build: tensor bbmin/bbmax')
+  d = np.load(os.path.join(ref_data, 'octree/test_002.npz'))
+  lo = np.array([-1.1, -1.0, -1.2], np.float32)
+  hi = np.array([1.0, 1.3, 1.0], np.float32)
+  o = Octree(6, 2)
+  o.build_octree(Points(torch.from_numpy(d['points']).to(DEV), torch.from_numpy(d['normals']).to(DEV)),
+                 bbmin=torch.from_numpy(lo).to(DEV), bbmax=torch.from_numpy(hi).to(DEV))
+  w, _ = R.build_octree(d['points'], d['normals'], depth=6, full_depth=2, bbmin=lo, bbmax=hi)
+  assert np.array_equal(np_(torch.cat(o.keys)), np.concatenate(w.keys))
+  assert np.array_equal(np_(torch.cat(o.children)), np.concatenate(w.children))
+
+
+def test_larger_synthetic_batch_vs_oracle():
+  say('build+neigh: 4 clouds x 30k points, depth 7, vs oracle')
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 4, 7, n=30000)
+  fea = torch.randn(pts.shape[0], 5, generator=torch.Generator().manual_seed(3))
+  pc = Points(pts.to(DEV), nrm.to(DEV), fea.to(DEV), batch_id=bid.to(DEV), batch_size=4)
+  o = Octree(7, 2, batch_size=4)
+  idx = o.build_octree(pc)
+  o.construct_all_neigh()
+  w, widx = R.build_octree(pts.numpy(), nrm.numpy(), fea.numpy(), bid.numpy(), 7, 2, 4)
+  R.construct_all_neigh(w)
+  assert np.array_equal(o.nnum.numpy(), w.nnum) and np.array_equal(o.nnum_nempty.numpy(), w.nnum_nempty)
+  for d in range(8):
+    assert np.array_equal(np_(o.keys[d]), w.keys[d]), d
+    assert np.array_equal(np_(o.children[d]), w.children[d]), d
+    if d:
+      assert np.array_equal(np_(o.neighs[d]), w.neighs[d]), d
+  assert np.array_equal(np_(idx), widx)
+  assert np.array_equal(np_(o.points[7]), w.points[7])
+  assert np.array_equal(np_(o.features[7]), w.features[7])
+  assert np.allclose(np_(o.normals[7]), w.normals[7], atol=1e-6)
+  for kern, stride, ne in [('333', 1, True), ('222', 2, False), ('222', 2, True), ('333', 2, True)]:
+    assert np.array_equal(np_(o._table(7, kern, stride, ne)), w.get_neigh(7, kern, stride, ne))
+
+
+def test_full_size_invariants():
+  say('build+neigh at the benchmark size: 8 x 100k points, depth 8 (properties only)')
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 8, 1001, n=100000)
+  pc = Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=8)
+  o = Octree(8, 2, batch_size=8)
+  idx = o.build_octree(pc)
+  o.construct_all_neigh()
+  assert int(idx.max()) + 1 == int(o.nnum_nempty[8])
+  for d in range(3, 9):
+    k = o.keys[d]
+    assert bool((k[1:] > k[:-1]).all())                               # sorted, unique
+    assert int(o.nnum[d]) == 8 * int(o.nnum_nempty[d - 1])
+    c = o.children[d]
+    assert torch.equal(c[c >= 0].long(), torch.arange(int(o.nnum_nempty[d]), device=DEV))
+    t = o._table(d, '333', 1, False).long()
+    n = t.shape[0]
+    assert torch.equal(t[:, 13], torch.arange(n, device=DEV))          # centre slot = itself
+    rows, slots = torch.nonzero(t >= 0, as_tuple=True)
+    assert torch.equal(t[t[rows, slots], 26 - slots], rows)            # central symmetry
+    # parent of every node holds it as a child: keys agree
+    assert torch.equal(o.keys[d] >> 3 & ((1 << 45) - 1),
+                       (o.keys[d - 1][o.nempty_index(d - 1)] & ((1 << 48) - 1)).repeat_interleave(8))
+    t2 = o._table(d, '222', 2, False).long()
+    assert torch.equal(t2, (torch.arange(n // 8, device=DEV) * 8).unsqueeze(1) +
+                       torch.arange(8, device=DEV))
+  # leaf of every point: its key is the leaf key
+  leaf_key = o.keys[8][o.nempty_index(8)]
+  p = (pts.to(DEV) + 1.0) * 128.0
+  key = xyz2key(p[:, 0], p[:, 1], p[:, 2], bid.to(DEV).view(-1), 8)
+  assert torch.equal(leaf_key[idx], key)
