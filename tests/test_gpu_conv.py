@@ -79,6 +79,7 @@ def rows_of(oct_ref, depth, nempty):
 def run_layer(kind, pair, depth, ks, stride, nempty, cin, cout, dtype, seed=0, use_bias=True):
   """Runs module forward + backward on the GPU and the oracle; returns errors."""
   g = torch.Generator().manual_seed(seed)
+  ks = (list(ks) + [ks[-1]] * 3)[:3]
   K = ks[0] * ks[1] * ks[2]
   if kind == 'conv':
     mod = OctreeConv(cin, cout, ks, stride, nempty, use_bias=use_bias)
