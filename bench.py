@@ -37,6 +37,11 @@ def parse():
   ap.add_argument('--channels', type=int, default=64)
   ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
   ap.add_argument('--cpu-rows', type=int, default=262144)
+  ap.add_argument('--only', default='all', choices=['all', 'fwd', 'bwd_data', 'wgrad'],
+                  help='run a single pass per step (for counter collection); the JSON line is '
+                       'then not a benchmark result')
+  ap.add_argument('--calib', action='store_true',
+                  help='also run one 1 GiB device copy, to scale FETCH_SIZE / WRITE_SIZE')
   return ap.parse_args()
 
 
@@ -164,11 +169,29 @@ def main():
   t_gather = KernelTimer(torch, conv_mod, 'conv_gather')
   t_wgrad = KernelTimer(torch, conv_mod, 'conv_wgrad')
 
+  eng = conv_mod._OctreeConv(C, C, [3], 1, nempty)
+  eng.setup(octree, depth)
+  w_cast = conv.weights.detach()
+
   def step():
-    x.grad = None
-    conv.weights.grad = None
-    out = conv(x, octree, depth)
-    out.backward(gout)
+    if args.only == 'fwd':
+      eng.forward_gemm(x.detach(), w_cast)
+    elif args.only == 'bwd_data':
+      eng.backward_gemm(gout, w_cast)
+    elif args.only == 'wgrad':
+      eng.weight_gemm(x.detach(), gout)
+    else:
+      x.grad = None
+      conv.weights.grad = None
+      out = conv(x, octree, depth)
+      out.backward(gout)
+
+  if args.calib:
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
   for _ in range(args.warmup):
     step()
@@ -182,8 +205,8 @@ def main():
   ms = dt * 1e3 / args.steps
 
   flops_step = 6.0 * nnz * C * C
-  gather_ms = t_gather.mean_ms()
-  wgrad_ms = t_wgrad.mean_ms()
+  gather_ms = t_gather.mean_ms() or float('nan')
+  wgrad_ms = t_wgrad.mean_ms() or float('nan')
   flops_launch = 2.0 * nnz * C * C
   achieved = flops_launch / (gather_ms * 1e-3) / 1e12
   es = 2                                               # bytes per feature element
@@ -241,6 +264,8 @@ def main():
           'nnum_nempty': octree.nnum_nempty.tolist(),
       },
   }
+  if args.only != 'all':
+    result['note'] = 'single-pass run (--only {}): not a benchmark result'.format(args.only)
   if not args.no_cpu:
     result['cpu_baseline'] = cpu_baseline(torch, table, x.shape[0], C, C, args.cpu_rows)
   print(json.dumps(result))

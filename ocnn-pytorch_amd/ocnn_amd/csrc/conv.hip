@@ -365,6 +365,15 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(
     for (int n = 0; n < NB; ++n) acc[q][n] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   u32x4 greg, xreg[KG];
+  int32_t idxn[KG];
+  // table entries are fetched one step ahead of the rows they address, so the
+  // row loads of the next step never wait on an index load
+  auto load_idx = [&](int64_t r0) {
+    int64_t row = r0 + lrow;
+    bool ok = loader && row < r_end;
+#pragma unroll
+    for (int q = 0; q < KG; ++q) idxn[q] = (ok && k0 + q < K) ? table[row * K + k0 + q] : -1;
+  };
   auto issue = [&](int64_t r0) {
     int64_t row = r0 + lrow;
     bool ok = loader && row < r_end;
@@ -373,13 +382,17 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(
     greg = __builtin_amdgcn_raw_buffer_load_b128(rs_g, goff, 0, 0);
 #pragma unroll
     for (int q = 0; q < KG; ++q) {
-      int32_t idx = (ok && k0 + q < K) ? table[row * K + k0 + q] : -1;
+      int32_t idx = idxn[q];
       uint32_t off = idx >= 0 ? (uint32_t)idx * xrow_bytes + a_off : 0xffffffffu - 64u;
       xreg[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, off, 0, 0);
     }
   };
 
-  if (r_begin < r_end) issue(r_begin);
+  if (r_begin < r_end) {
+    load_idx(r_begin);
+    issue(r_begin);
+    load_idx(r_begin + 32);
+  }
   for (int64_t r0 = r_begin; r0 < r_end; r0 += 32) {
     if (loader) {
       *(u32x4*)(&s_g[lrow * PITCH + lchunk * 8]) = greg;
@@ -387,7 +400,10 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(
       for (int q = 0; q < KG; ++q) *(u32x4*)(&s_x[q][lrow * PITCH + lchunk * 8]) = xreg[q];
     }
     __syncthreads();
-    if (r0 + 32 < r_end) issue(r0 + 32);
+    if (r0 + 32 < r_end) {
+      issue(r0 + 32);
+      load_idx(r0 + 64);
+    }
     u32x4 bf[NB];
 #pragma unroll
     for (int n = 0; n < NB; ++n) bf[n] = read_frag_t<T, USE_TR>(s_g, PITCH, (b_t0 + n) * 16, lane);
@@ -512,6 +528,8 @@ static int run_gather_plain(const void* in, int64_t rows_in, const int32_t* tabl
   return check_launch("conv_gather_plain");
 }
 
+constexpr int kWgradSlots = 3;   // kernel slots accumulated by one workgroup
+
 struct WgradPlan {
   bool mfma;
   int TILE;
@@ -529,7 +547,7 @@ static WgradPlan plan_wgrad(int dtype, int64_t rows_x, int64_t rows, int K, int 
     p.TILE = (ca % 64 == 0 && cb % 64 == 0) ? 64 : 32;
   }
   int64_t cols;   // workgroups per split
-  if (p.mfma) cols = (int64_t)cdiv(K, 9) * (ca / p.TILE) * (cb / p.TILE);
+  if (p.mfma) cols = (int64_t)cdiv(K, kWgradSlots) * (ca / p.TILE) * (cb / p.TILE);
   else cols = (int64_t)K * cdiv((int64_t)ca * cb, 256);
   int64_t want = cdiv(2048, cols);
   int64_t min_rows = p.mfma ? 512 : 64;
@@ -605,7 +623,7 @@ static int run_wgrad(int dtype, const void* x, int64_t rows_x, const void* g, co
   float* partial = (float*)ws;
   if constexpr (!std::is_same<T, float>::value) {
     if (p.mfma && rows > 0) {
-      constexpr int KG = 9;
+      constexpr int KG = kWgradSlots;
       dim3 grid(p.splits, (unsigned)(cdiv(K, KG) * (ca / p.TILE)), (unsigned)(cb / p.TILE));
       uint32_t xb = (uint32_t)(rows_x * ca * sizeof(T)), gb = (uint32_t)(rows * cb * sizeof(T));
 #define OCNN_WGRAD_CASE(tile_, tr_)                                                             \
