@@ -165,6 +165,32 @@ int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
                      int reverse_slots, const void* bias, void* out,
                      void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Tile plan of a table: for every tile of ocnn_tile_plan_rows() consecutive
+ * table rows, the ascending list of distinct rows the tile reads, and for every
+ * table entry its position in that list (0xffff for -1).  Lets a kernel bring
+ * each distinct row into LDS once per tile instead of once per (row, slot).
+ *   count: ucount[tile] = number of distinct rows        (tiles = ceil(rows / R))
+ *   fill : uptr (tiles + 1) = exclusive prefix sum of ucount, made by the caller;
+ *          urows[uptr[tile] + u] = u-th distinct row; loc (rows, K) uint16.
+ * No counterpart in the reference: its kernels gather per (row, slot)
+ * (ocnn/nn/kernels/conv_fwd_implicit_gemm.py:57-72). */
+int ocnn_tile_plan_rows(void);
+int ocnn_tile_plan_count(const int32_t* table, int64_t rows, int K, int32_t* ucount,
+                         void* stream);
+int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
+                        int32_t* urows, uint16_t* loc, void* stream);
+
+/* ocnn_conv_gather over a tile plan (same arguments otherwise, same result).
+ * Supported for f16 / bf16 with cin and cout multiples of 64 and an input
+ * smaller than 4 GiB; ocnn_conv_gather_planned_supported() tells. */
+int ocnn_conv_gather_planned_supported(int dtype, int64_t rows_in, int cin, int cout);
+int ocnn_conv_gather_planned(int dtype, const void* in, int64_t rows_in,
+                             const uint16_t* loc, const int32_t* uptr,
+                             const int32_t* urows, int64_t rows_out, int K,
+                             const void* w, int cin, int cout, int w_transposed,
+                             int reverse_slots, const void* bias, void* out,
+                             void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Selects how the MFMA weight-gradient kernel reads its LDS tiles: 1 (default)
  * = transposing LDS loads, 0 = 16-bit loads.  Same results either way. */
 void ocnn_set_wgrad_transpose_load(int on);

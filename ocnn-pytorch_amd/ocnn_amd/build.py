@@ -18,6 +18,8 @@ SOURCES = {
     'build.hip': ['-ffp-contract=off'],
     'neigh.hip': [],
     'conv.hip': [],
+    'conv_staged.hip': [],
+    'plan.hip': [],
     'misc.hip': [],
 }
 

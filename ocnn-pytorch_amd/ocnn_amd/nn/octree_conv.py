@@ -22,8 +22,9 @@ from ..utils import list2str, resize_with_last_val, xavier_uniform_
 from .octree_pad import octree_depad, octree_pad
 
 
-def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None):
-  """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K))."""
+def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None):
+  """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K)).  With a
+  tile plan of the same table (and a supported shape) the staged kernel runs."""
   _lib.require_gpu(data, table, W)
   L = _lib.lib()
   data, W, table = data.contiguous(), W.contiguous(), table.contiguous()
@@ -36,8 +37,15 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None):
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
   nbytes = L.ocnn_conv_workspace_bytes(K, cin, cout)
   ws = _lib.workspace(nbytes, data.device)
+  code = _lib.dtype_code(data)
+  if plan is not None and L.ocnn_conv_gather_planned_supported(code, rows_in, cin, cout):
+    _lib.check(L.ocnn_conv_gather_planned(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
+        _lib.ptr(plan.urows), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
+        _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return out
   _lib.check(L.ocnn_conv_gather(
-      _lib.dtype_code(data), _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(W),
+      code, _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(W),
       cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
       ws.numel(), _lib.stream()))
   return out
@@ -131,16 +139,29 @@ class OctreeConvBase:
     return self.octree._table_t(self.neigh_depth, self.kernel, self.stride, self.nempty,
                                 self.fine_h)
 
+  def _plan(self, data, cin, cout, inverse=False):
+    """Tile plan for the staged kernel, when the shape can use it."""
+    if not _lib.lib().ocnn_conv_gather_planned_supported(
+        _lib.DTYPE_CODE.get(data.dtype, -1), data.shape[0], cin, cout):
+      return None
+    return self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse,
+                             self.fine_h)
+
   def forward_gemm(self, data, weights, bias=None):
     """(fine rows, in_conv) -> (table rows, out_conv)."""
-    return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias)
+    plan = self._plan(data, self.in_conv, self.out_conv)
+    return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias,
+                       plan)
 
   def backward_gemm(self, grad, weights, bias=None):
     """(table rows, out_conv) -> (fine rows, in_conv)."""
     if self.symmetric:
-      return conv_gather(grad, grad.shape[0], self.neigh, weights, self.in_conv, True, True, bias)
+      plan = self._plan(grad, self.out_conv, self.in_conv)
+      return conv_gather(grad, grad.shape[0], self.neigh, weights, self.in_conv, True, True, bias,
+                         plan)
+    plan = self._plan(grad, self.out_conv, self.in_conv, inverse=True)
     return conv_gather(grad, grad.shape[0], self._inverse_table(), weights, self.in_conv, True,
-                       False, bias)
+                       False, bias, plan)
 
   def weight_gemm(self, data, grad, out_transposed=False):
     """data: fine rows; grad: table rows -> (K, in_conv, out_conv)."""

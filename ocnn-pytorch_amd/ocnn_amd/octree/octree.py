@@ -104,6 +104,31 @@ class _NeighTables:
     return out
 
 
+class TilePlan:
+  """Per-tile distinct-row lists of a table (see ocnn_tile_plan_* in the C ABI)."""
+
+  def __init__(self, table: torch.Tensor):
+    _lib.require_gpu(table)
+    L = _lib.lib()
+    table = table.contiguous()
+    rows, K = table.shape
+    tile_rows = L.ocnn_tile_plan_rows()
+    tiles = (rows + tile_rows - 1) // tile_rows
+    dev = table.device
+    st = _lib.stream()
+    ucount = torch.zeros(tiles, dtype=torch.int32, device=dev)
+    _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(ucount), st))
+    uptr = torch.zeros(tiles + 1, dtype=torch.int32, device=dev)
+    uptr[1:] = torch.cumsum(ucount, 0)
+    total = int(uptr[-1].item()) if tiles > 0 else 0
+    self.uptr = uptr
+    self.urows = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
+    self.loc = torch.empty((rows, K), dtype=torch.int16, device=dev)     # uint16 payload
+    _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(uptr),
+                                     _lib.ptr(self.urows), _lib.ptr(self.loc), st))
+    self.rows, self.K, self.total = rows, K, total
+
+
 class Octree:
   """Same constructor, attributes and methods as the reference class
   (ocnn/octree/octree.py:18-106)."""
@@ -130,6 +155,7 @@ class Octree:
     self._nempty_indices32 = [None] * num
     self._tables = {}        # (depth, kernel, stride, nempty) -> int32 table
     self._tables_t = {}      # same key -> inverse table
+    self._plans = {}         # (key, inverse) -> TilePlan
 
     self.nnum = torch.zeros(num, dtype=torch.long)
     self.nnum_nempty = torch.zeros(num, dtype=torch.long)
@@ -150,6 +176,8 @@ class Octree:
     for cache in (self._tables, self._tables_t):
       for key in [k for k in cache if k[0] == depth and (k[3] or not nempty_only)]:
         del cache[key]
+    for key in [k for k in self._plans if k[0][0] == depth and (k[0][3] or not nempty_only)]:
+      del self._plans[key]
 
   def _drop_nempty(self, depth):
     self.nempty_masks[depth] = None
@@ -318,7 +346,7 @@ class Octree:
     self.nempty_indices = [None] * num
     self.nempty_neighs = [None] * num
     self._nempty_indices32 = [None] * num
-    self._tables, self._tables_t = {}, {}
+    self._tables, self._tables_t, self._plans = {}, {}, {}
     return idx
 
   def octree_grow_full(self, depth: int, update_neigh: bool = True):
@@ -466,6 +494,15 @@ class Octree:
       self._tables_t[ck] = out
     return self._tables_t[ck]
 
+  def _plan(self, depth, kernel, stride, nempty, inverse=False, rows_in=None):
+    """Tile plan of the table (or of its inverse), cached with the table."""
+    ck = ((depth, kernel, stride, bool(nempty)), bool(inverse))
+    if ck not in self._plans:
+      t = (self._table_t(depth, kernel, stride, nempty, rows_in) if inverse
+           else self._table(depth, kernel, stride, nempty))
+      self._plans[ck] = TilePlan(t)
+    return self._plans[ck]
+
   @staticmethod
   def _widen(t32):
     out = torch.empty(t32.shape, dtype=torch.long, device=t32.device)
@@ -571,7 +608,7 @@ class Octree:
     self.nempty_indices = [None] * num
     self.nempty_neighs = [None] * num
     self._nempty_indices32 = [None] * num
-    self._tables, self._tables_t = {}, {}
+    self._tables, self._tables_t, self._plans = {}, {}, {}
     low48 = (1 << 48) - 1
     for d in range(num):
       self.keys[d] = torch.cat([(o.keys[d] & low48) | (i << 48)

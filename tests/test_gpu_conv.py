@@ -286,3 +286,53 @@ def test_benchmark_shape_properties():
       v = tt[:, k] >= 0
       want[v] += xd[tt[v, k]] @ wd[k]
     assert rel_err(out[sel.to(DEV)], want) < TOL[dtype]
+
+
+def test_tile_plan_reconstructs_table(medium):
+  say('tile plan: distinct-row lists and positions reproduce the table')
+  from ocnn_amd.octree.octree import TilePlan
+  for kern, stride, ne in [('333', 1, False), ('333', 1, True), ('222', 2, False)]:
+    t = medium.gpu._table(7, kern, stride, ne)
+    plan = TilePlan(t)
+    tab = t.cpu().numpy()
+    loc = plan.loc.cpu().numpy().view(np.uint16)
+    uptr = plan.uptr.cpu().numpy()
+    urows = plan.urows.cpu().numpy()
+    R = _lib.lib().ocnn_tile_plan_rows()
+    assert uptr[0] == 0 and uptr[-1] == plan.total
+    for tile in range(0, (tab.shape[0] + R - 1) // R, 7):
+      blk = tab[tile * R:(tile + 1) * R]
+      u = urows[uptr[tile]:uptr[tile + 1]]
+      assert np.array_equal(u, np.unique(blk[blk >= 0])), tile
+      lb = loc[tile * R:(tile + 1) * R]
+      assert np.array_equal(lb == 0xffff, blk < 0)
+      assert np.array_equal(u[lb[blk >= 0]], blk[blk >= 0])
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_staged_kernel_many_passes(dtype):
+  """A table with no locality: tiles need far more distinct rows than fit in
+  LDS at once, so the staged kernel takes several passes per tile."""
+  say('staged gather-GEMM on a random table (multi-pass)', dtype)
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(21)
+  rows_in, rows, K, cin, cout = 6000, 300, 27, 128, 64
+  table = torch.randint(0, rows_in, (rows, K), generator=g, dtype=torch.int32)
+  table[torch.rand(rows, K, generator=g) < 0.3] = -1
+  x = torch.randn(rows_in, cin, generator=g).to(dtype)
+  w = (torch.randn(K, cin, cout, generator=g) / 40).to(dtype)
+  b = torch.randn(cout, generator=g).to(dtype)
+  tg = table.to(DEV)
+  plan = TilePlan(tg)
+  assert int((plan.uptr[1:] - plan.uptr[:-1]).max()) > 320
+  got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), cout, False, False, b.to(DEV), plan)
+  want = C.forward_gemm(f64(x), f64(w), table.numpy().astype(np.int64)) + f64(b)
+  assert rel_err(got, want) < TOL[dtype]
+  old = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), cout, False, False, b.to(DEV))
+  assert rel_err(old, want) < TOL[dtype]
+  # transposed + mirrored weights through the same plan
+  wt = (torch.randn(K, cout, cin, generator=g) / 40).to(dtype)
+  got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, wt.to(DEV), cout, True, True, None, plan)
+  want = C.forward_gemm(f64(x), np.ascontiguousarray(f64(wt)[::-1].transpose(0, 2, 1)),
+                        table.numpy().astype(np.int64))
+  assert rel_err(got, want) < TOL[dtype]
