@@ -191,6 +191,19 @@ int ocnn_conv_gather_planned(int dtype, const void* in, int64_t rows_in,
                              int reverse_slots, const void* bias, void* out,
                              void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ocnn_conv_gather for 64 -> 64 channels with register-resident weights: one
+ * persistent workgroup per CU keeps all K x 64 x 64 weights in VGPRs and walks
+ * its tiles of the plan.  plan_max_distinct = largest number of distinct rows
+ * of any tile (max of ucount); the kernel needs it <= 512.  plan_total = number
+ * of entries of urows (uptr[tiles]).  Same result as ocnn_conv_gather. */
+int ocnn_conv_gather_rw_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
+                                  int plan_max_distinct);
+int ocnn_conv_gather_rw(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,
+                        const int32_t* uptr, const int32_t* urows, int plan_max_distinct,
+                        int64_t plan_total, int64_t rows_out, int K, const void* w, int cin, int cout,
+                        int w_transposed, int reverse_slots, const void* bias, void* out,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Selects how the MFMA weight-gradient kernel reads its LDS tiles: 1 (default)
  * = transposing LDS loads, 0 = 16-bit loads.  Same results either way. */
 void ocnn_set_wgrad_transpose_load(int on);

@@ -19,6 +19,7 @@ SOURCES = {
     'neigh.hip': [],
     'conv.hip': [],
     'conv_staged.hip': [],
+    'conv_rw.hip': [],
     'plan.hip': [],
     'misc.hip': [],
 }

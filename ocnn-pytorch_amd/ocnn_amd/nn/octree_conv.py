@@ -38,6 +38,12 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   nbytes = L.ocnn_conv_workspace_bytes(K, cin, cout)
   ws = _lib.workspace(nbytes, data.device)
   code = _lib.dtype_code(data)
+  if plan is not None and L.ocnn_conv_gather_rw_supported(code, rows_in, K, cin, cout, plan.umax):
+    _lib.check(L.ocnn_conv_gather_rw(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
+        _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
+        int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return out
   if plan is not None and L.ocnn_conv_gather_planned_supported(code, rows_in, cin, cout):
     _lib.check(L.ocnn_conv_gather_planned(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),

@@ -120,13 +120,14 @@ class TilePlan:
     _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(ucount), st))
     uptr = torch.zeros(tiles + 1, dtype=torch.int32, device=dev)
     uptr[1:] = torch.cumsum(ucount, 0)
-    total = int(uptr[-1].item()) if tiles > 0 else 0
+    total, umax = (int(v) for v in torch.stack([uptr[-1], ucount.max()]).tolist()) \
+        if tiles > 0 else (0, 0)
     self.uptr = uptr
     self.urows = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
     self.loc = torch.empty((rows, K), dtype=torch.int16, device=dev)     # uint16 payload
     _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(uptr),
                                      _lib.ptr(self.urows), _lib.ptr(self.loc), st))
-    self.rows, self.K, self.total = rows, K, total
+    self.rows, self.K, self.total, self.umax = rows, K, total, umax
 
 
 class Octree:
