@@ -167,11 +167,13 @@ int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
 
 /* Tile plan of a table: for every tile of ocnn_tile_plan_rows() consecutive
  * table rows, the ascending list of distinct rows the tile reads, and for every
- * table entry its position in that list (0xffff for -1).  Lets a kernel bring
+ * table entry its position in that list plus one (0 for -1).  Lets a kernel bring
  * each distinct row into LDS once per tile instead of once per (row, slot).
  *   count: ucount[tile] = number of distinct rows        (tiles = ceil(rows / R))
  *   fill : uptr (tiles + 1) = exclusive prefix sum of ucount, made by the caller;
- *          urows[uptr[tile] + u] = u-th distinct row; loc (rows, K) uint16.
+ *          urows[uptr[tile] + u] = u-th distinct row; loc (tiles, K, R) uint16:
+ *          loc[tile][k][r] = 1 + position of table[tile * R + r][k], or 0 for -1 and
+ *          for the rows of the last tile past the table.
  * No counterpart in the reference: its kernels gather per (row, slot)
  * (ocnn/nn/kernels/conv_fwd_implicit_gemm.py:57-72). */
 int ocnn_tile_plan_rows(void);
@@ -220,6 +222,20 @@ int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
                     const int32_t* table, int64_t rows, int K, int ca, int cb,
                     int out_transposed, void* gw, void* workspace,
                     int64_t workspace_bytes, void* stream);
+
+/* ocnn_conv_wgrad over a tile plan of the same table, for ca = cb = 64 (same
+ * reference lines, same result up to the fp32 summation order, which is fixed).
+ * Per tile the distinct x rows and the g rows are staged once in LDS; persistent
+ * workgroups keep the sums of all K slots in accumulator registers over a range
+ * of tiles.  plan_max_distinct must be <= 416; ..._supported() tells. */
+int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
+                                      int cb, int plan_max_distinct);
+int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K);
+int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const void* g,
+                            const uint16_t* loc, const int32_t* uptr, const int32_t* urows,
+                            int plan_max_distinct, int64_t plan_total, int64_t rows, int K,
+                            int ca, int cb, int out_transposed, void* gw, void* workspace,
+                            int64_t workspace_bytes, void* stream);
 
 /* Depth-wise engine, ocnn/nn/octree_dwconv.py:30-118.  w: (K, c).
  * fwd : out[i][c] = sum_k in[t[i][k]][c] * w[k'][c]   (k' = K-1-k if

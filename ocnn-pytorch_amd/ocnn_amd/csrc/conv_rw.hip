@@ -17,22 +17,6 @@
 
 namespace ocnn {
 
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-
-template <typename T> struct Mma32;
-template <> struct Mma32<bf16> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma32<f16> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-};
-
 constexpr int kRwRows = 128;   // rows per tile (the plan's tile size)
 constexpr int kRwCap = 512;    // staged rows; plans with a larger tile use another kernel
 
@@ -59,8 +43,6 @@ __global__ void pack_weights_rw_kernel(const T* __restrict__ w, T* __restrict__ 
   int kk = reverse ? K - 1 - k : k;
   out[e] = transposed ? w[((int64_t)kk * 64 + co) * 64 + chan] : w[((int64_t)kk * 64 + chan) * 64 + co];
 }
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 template <typename T, int UPW>
 __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
@@ -96,7 +78,6 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
         wreg[u][s][tM] = v;
       }
   }
-  if (tid < 8) *(u32x4*)(&s_rows[kRwCap * 64 + tid * 8]) = u32x4{0u, 0u, 0u, 0u};   // the zero row
 
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
   const __amdgpu_buffer_rsrc_t rs_loc = make_rsrc(loc, loc_bytes);
@@ -112,14 +93,16 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
   // asynchronous staging of one tile: its U distinct rows (ids in s_u[ubuf]) -> s_rows, its
   // table positions -> s_loc[buf]
   auto stage = [&](int64_t tile, int U, int ubuf, int buf) {
-    const int ngrp = (U + 7) >> 3;
+    // LDS row p (p >= 1) holds the (p - 1)-th distinct row; row 0 is the zero row that the
+    // empty table entries (position 0) read: its lanes load from an out-of-range offset
+    const int ngrp = (U + 8) >> 3;
     // four groups of 8 rows per round: the four row ids are read first, then the loads go out
     for (int g0 = wave; g0 < ngrp; g0 += 16) {
       int32_t g[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         int u = (g0 + 4 * i) * 8 + (lane >> 3);
-        g[i] = u < U ? s_u[ubuf][u] : -1;
+        g[i] = (u >= 1 && u <= U) ? s_u[ubuf][u - 1] : -1;
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -133,7 +116,7 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
         }
       }
     }
-    // kRwRows * K positions (2 B each), 1 KiB per wave instruction; past the end reads 0
+    // kRwRows * K positions (2 B each, [slot][row]), 1 KiB per wave instruction
     const uint32_t lbase = (uint32_t)(tile * kRwRows * K * 2);
     const int nchunk = (kRwRows * K * 2 + 1023) >> 10;
     for (int c = wave; c < nchunk; c += 4)
@@ -188,13 +171,13 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
         int gid = min(u * 4 + wave, 2 * K - 1);
         int k = gid >> 1;
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) l[nt] = lc[(rbase + 32 * nt) * K + k];
+        for (int nt = 0; nt < 2; ++nt) l[nt] = lc[k * kRwRows + rbase + 32 * nt];
       };
       // LDS addresses of the two 16-byte pieces a lane reads of its neighbour row
       auto addr = [&](int u, uint32_t lv, const T*& p0, const T*& p1) {
         int gid = min(u * 4 + wave, 2 * K - 1);
         int half = gid & 1;
-        uint32_t l = lv >= (uint32_t)kRwCap ? (uint32_t)kRwCap : lv;       // empty -> zero row
+        const uint32_t l = lv;                                            // 0 = empty = the zero row
         uint32_t swz = (l >> 1) & 7;
         p0 = &s_rows[l * 64 + (((uint32_t)(4 * half + q) ^ swz) * 8)];
         p1 = &s_rows[l * 64 + (((uint32_t)(4 * half + 2 + q) ^ swz) * 8)];
@@ -368,7 +351,7 @@ static void launch_rw(const void* in, int64_t rows_in, const uint16_t* loc, cons
   int64_t per = cdiv(tiles, wgs);
   wgs = cdiv(tiles, per);
   hipLaunchKernelGGL((conv_gather_rw_kernel<T, UPW>), dim3((unsigned)wgs), dim3(256), 0, st,
-                     (const T*)in, (uint32_t)(rows_in * 128), loc, (uint32_t)(rows_out * K * 2), uptr,
+                     (const T*)in, (uint32_t)(rows_in * 128), loc, (uint32_t)(tiles * kRwRows * K * 2), uptr,
                      urows, urows_bytes, (const T*)ws, (const T*)bias, (T*)out, rows_out, K, tiles, per, g_rw_dbg);
 }
 

@@ -73,11 +73,10 @@ __global__ __launch_bounds__(256) void conv_gather_staged_kernel(
   const int ncb = cin >> 6;
   const uint32_t row_bytes = (uint32_t)cin * 2u;
 
-  // table positions of the tile -> LDS; rows past the end read "empty"
+  // table positions of the tile ([slot][row], padded to whole tiles by the plan) -> LDS
   {
     const int64_t base = row0 * K;
-    const int64_t lim = rows_out * (int64_t)K;
-    for (int e = tid; e < kRT * K; e += 256) s_loc[e] = (base + e < lim) ? loc[base + e] : 0xffff;
+    for (int e = tid; e < kRT * K; e += 256) s_loc[e] = loc[base + e];
   }
   if (tid < 8) *(u32x4*)(&s_rows[kUCAP * 64 + tid * 8]) = u32x4{0u, 0u, 0u, 0u};   // the zero row
 
@@ -140,7 +139,7 @@ __global__ __launch_bounds__(256) void conv_gather_staged_kernel(
         for (int t = 0; t < 4; ++t) a[t] = *(const u32x4*)(wsrc + t * 512);
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
-          uint32_t local = (uint32_t)s_loc[(64 * rh + 16 * n + r16) * K + k] - (uint32_t)p0;
+          uint32_t local = (uint32_t)s_loc[k * kRT + 64 * rh + 16 * n + r16] - 1u - (uint32_t)p0;   // 0 = empty
           if (local >= (uint32_t)kUCAP) local = kUCAP;                  // empty or other pass: zero row
           uint32_t pos = (uint32_t)(4 * h + g) ^ ((local >> 1) & 7);
           b[n] = *(const u32x4*)(&s_rows[local * 64 + pos * 8]);

@@ -43,6 +43,26 @@ template <> struct Mma<f16> {
   }
 };
 
+// v_mfma_f32_32x32x16_{f16,bf16}: A (32 x 16): lane l holds A[l % 32][8 * (l / 32) + j];
+// B (16 x 32): lane l holds B[8 * (l / 32) + j][l % 32];
+// D (32 x 32): lane l, register r holds D[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32].
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+template <typename T> struct Mma32;
+template <> struct Mma32<bf16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma32<f16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
 template <typename T> __device__ __forceinline__ unsigned pack2(float a, float b) {
   typedef __attribute__((ext_vector_type(2))) T v2;
   v2 v = {(T)a, (T)b};

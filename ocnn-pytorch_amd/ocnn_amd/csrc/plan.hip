@@ -9,7 +9,8 @@ constexpr int kPlanRows = 128;          // table rows per tile
 constexpr int kPlanMaxEntries = 4096;   // >= kPlanRows * 27, power of two
 
 // mode 0: ucount[tile] = number of distinct valid entries
-// mode 1: urows[uptr[tile] + u] = u-th distinct row; loc[row][k] = u or 0xffff
+// mode 1: urows[uptr[tile] + u] = u-th distinct row; loc[tile][k][row in tile] = u + 1, or
+//         0 for an empty entry (also for the rows of the last tile that lie past the table)
 __global__ __launch_bounds__(256) void tile_plan_kernel(
     const int32_t* __restrict__ table, int64_t rows, int K, int npad, int mode,
     int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, int32_t* __restrict__ urows,
@@ -70,18 +71,17 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
   const int32_t ub = uptr[tile];
   for (int u = tid; u < total; u += 256) urows[ub + u] = s_uq[u];
   for (int e = tid; e < n; e += 256) {
-    if (e0 + e >= lim) break;
-    int32_t v = table[e0 + e];
-    uint16_t r = 0xffff;
+    int32_t v = e0 + e < lim ? table[e0 + e] : -1;
+    uint16_t r = 0;
     if (v >= 0) {
       int lo = 0, hi = total - 1;
       while (lo < hi) {
         int mid = (lo + hi) >> 1;
         if (s_uq[mid] < v) lo = mid + 1; else hi = mid;
       }
-      r = (uint16_t)lo;
+      r = (uint16_t)(lo + 1);
     }
-    loc[e0 + e] = r;
+    loc[e0 + (int64_t)(e % K) * kPlanRows + e / K] = r;
   }
 }
 

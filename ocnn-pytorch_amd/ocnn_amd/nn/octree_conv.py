@@ -57,8 +57,9 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   return out
 
 
-def conv_wgrad(x, g, table, out_transposed=False):
-  """gW (K, ca, cb) [or (K, cb, ca)] = sum_i x[T[i,k]]^T (x) g[i]."""
+def conv_wgrad(x, g, table, out_transposed=False, plan=None):
+  """gW (K, ca, cb) [or (K, cb, ca)] = sum_i x[T[i,k]]^T (x) g[i].  With a tile
+  plan of the same table (and a supported shape) the staged kernel runs."""
   _lib.require_gpu(x, g, table)
   L = _lib.lib()
   x, g, table = x.contiguous(), g.contiguous(), table.contiguous()
@@ -67,6 +68,15 @@ def conv_wgrad(x, g, table, out_transposed=False):
   assert g.shape[0] == rows and x.dtype == g.dtype and table.dtype == torch.int32
   shape = (K, cb, ca) if out_transposed else (K, ca, cb)
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
+  code = _lib.DTYPE_CODE.get(x.dtype, -1)
+  if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
+                                                              plan.umax):
+    ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K), x.device)
+    _lib.check(L.ocnn_conv_wgrad_planned(
+        code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
+        _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, ca, cb, int(out_transposed),
+        _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return gw
   ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes(rows, K, ca, cb), x.device)
   _lib.check(L.ocnn_conv_wgrad(
       _lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
@@ -171,7 +181,8 @@ class OctreeConvBase:
 
   def weight_gemm(self, data, grad, out_transposed=False):
     """data: fine rows; grad: table rows -> (K, in_conv, out_conv)."""
-    return conv_wgrad(data, grad, self.neigh, out_transposed)
+    plan = self._plan(data, self.in_conv, self.out_conv)
+    return conv_wgrad(data, grad, self.neigh, out_transposed, plan)
 
 
 class _OctreeConv(OctreeConvBase):

@@ -124,7 +124,8 @@ class TilePlan:
         if tiles > 0 else (0, 0)
     self.uptr = uptr
     self.urows = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
-    self.loc = torch.empty((rows, K), dtype=torch.int16, device=dev)     # uint16 payload
+    # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"
+    self.loc = torch.empty((tiles, K, tile_rows), dtype=torch.int16, device=dev)
     _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(uptr),
                                      _lib.ptr(self.urows), _lib.ptr(self.loc), st))
     self.rows, self.K, self.total, self.umax = rows, K, total, umax

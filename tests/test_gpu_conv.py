@@ -304,9 +304,10 @@ def test_tile_plan_reconstructs_table(medium):
       blk = tab[tile * R:(tile + 1) * R]
       u = urows[uptr[tile]:uptr[tile + 1]]
       assert np.array_equal(u, np.unique(blk[blk >= 0])), tile
-      lb = loc[tile * R:(tile + 1) * R]
-      assert np.array_equal(lb == 0xffff, blk < 0)
-      assert np.array_equal(u[lb[blk >= 0]], blk[blk >= 0])
+      lb = loc[tile].T[:blk.shape[0]]                      # (slot, row) -> (row, slot)
+      assert (loc[tile].T[blk.shape[0]:] == 0).all()       # rows past the table: empty
+      assert np.array_equal(lb == 0, blk < 0)              # 0 = empty, else position + 1
+      assert np.array_equal(u[lb[blk >= 0] - 1], blk[blk >= 0])
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
@@ -336,3 +337,97 @@ def test_staged_kernel_many_passes(dtype):
   want = C.forward_gemm(f64(x), np.ascontiguousarray(f64(wt)[::-1].transpose(0, 2, 1)),
                         table.numpy().astype(np.int64))
   assert rel_err(got, want) < TOL[dtype]
+
+
+def _local_table(rows, rows_in, K, g, spread=40, empty=0.3):
+  """A table with the locality of an octree neighbourhood: entry (r, k) points near
+  r * rows_in / rows, so a 128-row tile touches a few hundred distinct rows."""
+  base = (torch.arange(rows, dtype=torch.float64) * (rows_in / max(rows, 1))).long()[:, None]
+  off = torch.randint(-spread, spread + 1, (rows, K), generator=g)
+  t = (base + off).clamp_(0, rows_in - 1).to(torch.int32)
+  t[torch.rand(rows, K, generator=g) < empty] = -1
+  return t
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('K', [27, 9, 8, 3])
+def test_planned_64x64_kernels(dtype, K):
+  """The persistent 64 -> 64 kernels (gather-GEMM with register-resident weights,
+  weight gradient on the tile plan) for every slot count they are built for, on
+  tables whose row count is not a multiple of the tile, against the oracle and
+  against the plan-free kernels."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(100 + K)
+  for rows, rows_in in [(1000, 1000), (4133, 2300), (130, 150), (128 * 300 + 1, 128 * 300 + 1)]:
+    say('planned kernels', dtype, 'K', K, 'rows', rows, 'rows_in', rows_in)
+    table = _local_table(rows, rows_in, K, g)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+    assert L.ocnn_conv_gather_rw_supported(code, rows_in, K, 64, 64, plan.umax)
+    assert L.ocnn_conv_wgrad_planned_supported(code, rows_in, rows, K, 64, 64, plan.umax)
+    x = torch.randn(rows_in, 64, generator=g).to(dtype)
+    w = (torch.randn(K, 64, 64, generator=g) / (K * 64) ** 0.5).to(dtype)
+    b = torch.randn(64, generator=g).to(dtype)
+    gr = torch.randn(rows, 64, generator=g).to(dtype)
+    t64 = table.numpy().astype(np.int64)
+    # gather-GEMM, with bias
+    got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), 64, False, False, b.to(DEV), plan)
+    want = C.forward_gemm(f64(x), f64(w), t64) + f64(b)
+    assert rel_err(got, want) < TOL[dtype]
+    # transposed, mirrored weights (the data gradient of a symmetric table)
+    got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), 64, True, True, None, plan)
+    want = C.forward_gemm(f64(x), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
+    assert rel_err(got, want) < TOL[dtype]
+    # weight gradient, both output layouts; same bits on a second run
+    gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+    want = C.weight_gemm(f64(x), f64(gr), t64)
+    assert rel_err(gw, want) < TOL[dtype]
+    assert rel_err(ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg), want) < TOL[dtype]
+    gwt = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, True, plan)
+    assert torch.equal(gwt, gw.transpose(1, 2).contiguous())
+    assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
+
+
+def test_planned_kernels_non_finite_rows():
+  """Rows past the end of the table and empty entries must not pick up values of
+  staged rows: NaN / Inf rows that no valid entry refers to stay out of the result."""
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(77)
+  rows, rows_in, K = 200, 260, 27
+  table = _local_table(rows, rows_in - 4, K, g)            # the last 4 input rows are never referenced
+  x = torch.randn(rows_in, 64, generator=g).half()
+  x[-4:] = float('nan')
+  x[0] = float('inf')
+  table[table == 0] = -1                                    # nor is row 0
+  gr = torch.randn(rows, 64, generator=g).half()
+  w = (torch.randn(K, 64, 64, generator=g) / 40).half()
+  tg = table.to(DEV)
+  plan = TilePlan(tg)
+  out = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), 64, False, False, None, plan)
+  gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+  assert torch.isfinite(out).all() and torch.isfinite(gw).all()
+
+
+def test_planned_kernels_fall_back_on_large_tiles():
+  """A tile with more distinct rows than the persistent kernels stage: the entry points
+  report it and the Python layer takes the other kernels (same results)."""
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(5)
+  rows, rows_in, K = 500, 50000, 27
+  table = torch.randint(0, rows_in, (rows, K), generator=g, dtype=torch.int32)
+  tg = table.to(DEV)
+  plan = TilePlan(tg)
+  assert plan.umax > 512
+  L = _lib.lib()
+  assert not L.ocnn_conv_gather_rw_supported(1, rows_in, K, 64, 64, plan.umax)
+  assert not L.ocnn_conv_wgrad_planned_supported(1, rows_in, rows, K, 64, 64, plan.umax)
+  x = torch.randn(rows_in, 64, generator=g).half()
+  gr = torch.randn(rows, 64, generator=g).half()
+  w = (torch.randn(K, 64, 64, generator=g) / 40).half()
+  t64 = table.numpy().astype(np.int64)
+  out = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), 64, False, False, None, plan)
+  assert rel_err(out, C.forward_gemm(f64(x), f64(w), t64)) < 2e-2
+  gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+  assert rel_err(gw, C.weight_gemm(f64(x), f64(gr), t64)) < 2e-2
