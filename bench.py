@@ -22,6 +22,10 @@ for p in (ROOT, os.path.join(ROOT, 'ocnn-pytorch_amd')):
 
 PEAK_MFMA_16BIT_TFLOPS = 2500.0     # MI355X dense bf16 / fp16
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the gather-GEMM kernel at the default workload (fp16, depth 8,
+# batch 8), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy; None for
+# any other workload.  The summary under profiles/ gives the counter readings.
+TRAFFIC_GATHER_DEFAULT = int((205800 * 2.0 + 235700 * 1.0) * 1024)
 
 
 def parse():
@@ -213,6 +217,8 @@ def main():
   bytes_gather = es * (rows * C + rows * C + 27 * C * C) + 4 * rows * 27
   bytes_wgrad = es * (rows * C + rows * C) + 4 * rows * 27 + 4 * 27 * C * C
 
+  default_workload = (args.depth, args.batch, args.points, C, nempty) == (8, 8, 100000, 64, False)
+  TRAFFIC_GATHER_BYTES = TRAFFIC_GATHER_DEFAULT if default_workload else None
   result = {
       'metric': 'OctreeConv 3x3x3 64->64 fwd+bwd at depth 8 (batch 8): effective TFLOP/s '
                 'over non-empty neighbours',
@@ -235,14 +241,14 @@ def main():
           'rows': rows, 'nnz': nnz, 'valid_per_row': nnz / rows,
       },
       'roofline': {
-          'kernel': 'conv_gather_mfma_kernel (forward and data gradient; mean of both launches, '
+          'kernel': 'conv_gather_rw_kernel (forward and data gradient; mean of both launches, '
                     'each bracketed with its weight-pack pre-pass)',
           'bound': 'mfma',
           'achieved': achieved,
           'peak': PEAK_MFMA_16BIT_TFLOPS,
           'unit': 'TFLOP/s',
           'frac': achieved / PEAK_MFMA_16BIT_TFLOPS,
-          'traffic': None,
+          'traffic': TRAFFIC_GATHER_BYTES,
           'launches': t_gather.count(),
           'avg_launch_ms': gather_ms,
           'algorithmic_flops_per_launch': flops_launch,
@@ -254,6 +260,8 @@ def main():
           'conv_wgrad_ms': wgrad_ms,
           'conv_wgrad_tflops': flops_launch / (wgrad_ms * 1e-3) / 1e12,
           'conv_wgrad_algorithmic_bytes': bytes_wgrad,
+          'sustained_mfma_note': 'v_mfma_f32_32x32x16_f16 alone sustains 1.67 PFLOP/s on this part with '
+                                 'random operands (2.38 with constant ones): clocks drop under load',
           'fraction_of_mfma_peak_whole_step': flops_step / (ms * 1e-3) / 1e12 / PEAK_MFMA_16BIT_TFLOPS,
       },
       'octree': {
