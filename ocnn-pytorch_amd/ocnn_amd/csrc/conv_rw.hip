@@ -11,9 +11,14 @@
 // units (v_mfma_f32_32x32x16, M = 64 output channels, N = 128 rows), and the four
 // partial sums are added through LDS in wave order (deterministic).
 #include <algorithm>
+#include <type_traits>
 
 #include "common.hpp"
 #include "mma.hpp"
+
+#ifndef OCNN_RW_EXP
+#define OCNN_RW_EXP 0   // timing experiments: bit 0 no partial-sum writes, 1 no barriers, 2 no reads/adds, 3 no stores
+#endif
 
 namespace ocnn {
 
@@ -54,9 +59,11 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
   __shared__ __attribute__((aligned(16))) T s_rows[(kRwCap + 1) * 64];
   // table positions, double buffered; filled 1 KiB per wave instruction, hence the rounding
   __shared__ __attribute__((aligned(16))) uint16_t s_loc[2][(kRwRows * 27 * 2 + 1023) / 1024 * 512];
-  __shared__ f32x4 s_red[4 * 3 * 4 * 64];                                  // 48 KiB
+  __shared__ f32x4 s_red[4 * 4 * 4 * 64];                                  // 64 KiB: [writer][combination][quarter][lane]
+  __shared__ __attribute__((aligned(16))) float s_bias[64];
   __shared__ __attribute__((aligned(16))) int32_t s_u[2][kRwCap + 64];     // row lists, 2 tiles ahead
 
+  constexpr int KK = UPW == 14 ? 27 : UPW == 5 ? 9 : UPW == 4 ? 8 : 3;   // slots (= K)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // wave-uniform: lives in an SGPR
   const int q = lane >> 5, r32 = lane & 31;
@@ -143,181 +150,187 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
 #else
   constexpr bool timing = false;
 #endif
-  long long t_main = 0, t_epi = 0, t_wait = 0, t_mark = 0, t_e0 = 0, t_e1 = 0, t_e2 = 0, t_e3 = 0;
+  long long t_main = 0, t_stage = 0, t_wait = 0, t_mark = 0;
+
+  // bias as fp32 in LDS (zeros without one); a lane finishes the 16 output channels
+  // 32 (wave % 2) + 16 q .. of a row
+  if (tid < 64) s_bias[tid] = bias ? to_f32(bias[tid]) : 0.f;
+  const f32x4* bias4 = (const f32x4*)(&s_bias[32 * (wave & 1) + 16 * q]);
+
+  // Two accumulator sets: while a 64-row half is being multiplied into one, the partial sums
+  // of the half before it (the other set) are exchanged through LDS and stored, a piece per
+  // step of the main loop, in the shadow of the MFMAs.
+  f32x16 acc[2][2][2];
+
+  // ---- the cross-wave sum of one half, cut into pieces for the steps of a main loop ----
+  // Wave w finishes (row tile w / 2, M tile w % 2).  Pieces 0..15 write all four
+  // combinations to s_red (also the own one: the code is then the same for every wave and
+  // free of branches, which cost a wave far more than an LDS round trip), piece 19 is
+  // the barrier after them, 20..23 read the four partial sums of the own combination,
+  // 21..24 add them in wave order, 23 and 25 store.
+  f32x4 red[4], rb;        // partial sums and bias of a quarter (read at piece j, used at j + 1)
+  unsigned pk[4];
+  auto exch_piece = [&](auto SETC, int j, int64_t row0, bool drain) {     // row0: first row of that half
+    constexpr int S = decltype(SETC)::value;
+    if (j < 16) {
+      const int c = j >> 2, r4 = j & 3;                       // combination c = 2 nt + tM
+      if (!(OCNN_RW_EXP & 1))
+        s_red[((wave * 4 + c) * 4 + r4) * 64 + lane] =
+            f32x4{acc[S][c >> 1][c & 1][4 * r4], acc[S][c >> 1][c & 1][4 * r4 + 1],
+                  acc[S][c >> 1][c & 1][4 * r4 + 2], acc[S][c >> 1][c & 1][4 * r4 + 3]};
+    } else if (j == 19) {
+      // With 28 steps a wave has by now consumed LDS reads that it issued after its last
+      // write, so the writes are done (LDS operations of a wave complete in order); in the
+      // shorter loops, and without a main loop around, it waits for them.
+      if (OCNN_RW_EXP & 2) {}
+      else if (drain) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_barrier" ::: "memory");
+    } else if (j >= 20 && j <= 25) {
+      if (j == 23 || j == 25) {                               // channels 0-7 after quarter 1, 8-15 after 3
+        const int64_t row = row0 + 32 * (wave >> 1) + r32;
+        if (row < rows_out && !(OCNN_RW_EXP & 8))
+          *(u32x4*)(out + row * 64 + 32 * (wave & 1) + 16 * q + (j == 23 ? 0 : 8)) =
+              u32x4{pk[0], pk[1], pk[2], pk[3]};
+      }
+      if (j >= 21 && j <= 24 && !(OCNN_RW_EXP & 4)) {         // add quarter j - 21 in wave order, pack
+        const int r4 = j - 21;
+        const f32x4 sum = ((red[0] + red[1]) + red[2]) + red[3];
+        pk[2 * (r4 & 1)] = pack2<T>(sum[0] + rb[0], sum[1] + rb[1]);
+        pk[2 * (r4 & 1) + 1] = pack2<T>(sum[2] + rb[2], sum[3] + rb[3]);
+      }
+      if (j <= 23 && !(OCNN_RW_EXP & 4)) {                    // read the partial sums of quarter j - 20
+        const int r4 = j - 20;
+#pragma unroll
+        for (int src = 0; src < 4; ++src) red[src] = s_red[((src * 4 + wave) * 4 + r4) * 64 + lane];
+        rb = bias4[r4];
+      }
+    }
+  };
+
+  // ---- one 64-row half: main loop into acc[S], exchange of the previous half (acc[1 - S]) ----
+  // (prev_row0 past the last row: nothing is stored, as for the first half of a range)
+  auto half_body = [&](auto SETC, const uint16_t* lc, int64_t prev_row0) {
+    constexpr int S = decltype(SETC)::value;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int tM = 0; tM < 2; ++tM)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[S][nt][tM][r] = 0.f;
+
+    // The main loop is a flat sequence of steps (unit u, row tile nt).  The B operand of
+    // a step (lane: row r32 of the row tile, k group q -> 2 x 16 B of its neighbour row)
+    // is fetched from LDS three steps ahead of its four MFMAs; the table positions of a
+    // unit are read three units ahead.  Units past 2K have zero weights.
+    // unit u of wave w is (slot 2u + w / 2, input-channel half w % 2): one base address per
+    // half, immediate offsets per unit
+    const uint16_t* lcw = lc + (wave >> 1) * kRwRows + 64 * S + r32;
+    auto read_loc = [&](int u, uint32_t (&l)[2]) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        uint32_t v = lcw[2 * u * kRwRows + 32 * nt];
+        if (4 * u + 3 >= 2 * KK) v = (4 * u + wave < 2 * KK) ? v : 0u;   // a unit past the last slot: zero row
+        l[nt] = v;
+      }
+    };
+    // LDS addresses of the two 16-byte pieces a lane reads of its neighbour row
+    const uint32_t c0 = (uint32_t)(4 * (wave & 1) + q);
+    auto addr = [&](int u, uint32_t l, const T*& p0, const T*& p1) {   // l = 0: empty = the zero row
+      (void)u;
+      if (OCNN_RW_EXP & 64) {            // timing experiment: one VALU per look-up
+        p0 = &s_rows[(l << 3) + c0 * 8];
+        p1 = p0 + 16;
+        return;
+      }
+      const uint32_t swz = (l >> 1) & 7;
+      p0 = &s_rows[l * 64 + ((c0 ^ swz) * 8)];
+      p1 = &s_rows[l * 64 + (((c0 + 2) ^ swz) * 8)];
+    };
+
+    constexpr int STEPS = UPW * 2;
+    uint32_t lcur[2], lnxt[2] = {0u, 0u};
+    u32x4 ring[3][2];
+    const T *pa, *pb;
+    read_loc(0, lcur);
+    if (UPW > 1) read_loc(1, lnxt);
+    addr(0, lcur[0], pa, pb);
+    ring[0][0] = *(const u32x4*)pa;
+    ring[0][1] = *(const u32x4*)pb;
+    addr(0, lcur[1], pa, pb);
+    ring[1][0] = *(const u32x4*)pa;
+    ring[1][1] = *(const u32x4*)pb;
+    __builtin_amdgcn_sched_barrier(0);
+    // Every step issues its four MFMAs with the LDS traffic of step j + 2 placed between
+    // them, so that the address arithmetic and the reads issue while an MFMA executes.
+    // The exchange pieces are spread over the steps whatever their number.
+    constexpr int EPS = (26 + STEPS - 1) / STEPS;           // exchange pieces per step
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+      const int u = j >> 1, nt = j & 1;
+      const bool pre = j + 2 < STEPS;
+      const int nt2 = nt;                                    // step j + 2: unit u + 1, same row tile
+      acc[S][nt][0] = Mma32<T>::run(wreg[u][0][0], ring[j % 3][0], acc[S][nt][0]);
+      if (pre) addr(u + 1, lnxt[nt2], pa, pb);
+      acc[S][nt][1] = Mma32<T>::run(wreg[u][0][1], ring[j % 3][0], acc[S][nt][1]);
+      if (pre) ring[(j + 2) % 3][0] = *(const u32x4*)pa;
+      acc[S][nt][0] = Mma32<T>::run(wreg[u][1][0], ring[j % 3][1], acc[S][nt][0]);
+      if (pre) ring[(j + 2) % 3][1] = *(const u32x4*)pb;
+      if (nt == 1) {
+        // the next unit becomes current; read the positions of the one two units on
+        lcur[0] = lnxt[0];
+        lcur[1] = lnxt[1];
+        if (u + 2 < UPW) read_loc(u + 2, lnxt);
+      }
+      acc[S][nt][1] = Mma32<T>::run(wreg[u][1][1], ring[j % 3][1], acc[S][nt][1]);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = j * EPS; e < (j + 1) * EPS && e < 26; ++e)
+        exch_piece(std::integral_constant<int, 1 - S>{}, e, prev_row0, UPW != 14);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // s_red may be written again (next half) once every owner has used what it read
+    if (!(OCNN_RW_EXP & 2)) asm volatile("s_barrier" ::: "memory");
+  };
+
   for (int64_t tile = t_begin; tile < t_end; ++tile) {
     const int cur = (int)(tile - t_begin) & 1;
     const uint16_t* lc = s_loc[cur];
     // list boundary three tiles ahead (scalar load, used after the main loop)
     const int32_t p_nx3 = uptr[min(tile + 3, tiles)];
-
-    // the tile is processed as two halves of 64 rows, so that the accumulators take 64
-    // registers and the weights have room next to them
-    for (int half_t = 0; half_t < 2; ++half_t) {
-      if (timing) t_mark = clock64();
-      f32x16 acc[2][2];
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int tM = 0; tM < 2; ++tM)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[nt][tM][r] = 0.f;
-
-      // The main loop is a flat sequence of steps (unit u, row tile nt).  The B operand of
-      // a step (lane: row r32 of the row tile, k group q -> 2 x 16 B of its neighbour row)
-      // is fetched from LDS three steps ahead of its four MFMAs; the table positions of a
-      // unit are read three units ahead.  Units past 2K have zero weights.
-      const int rbase = 64 * half_t + r32;
-      auto read_loc = [&](int u, uint32_t (&l)[2]) {
-        int gid = min(u * 4 + wave, 2 * K - 1);
-        int k = gid >> 1;
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) l[nt] = lc[k * kRwRows + rbase + 32 * nt];
-      };
-      // LDS addresses of the two 16-byte pieces a lane reads of its neighbour row
-      auto addr = [&](int u, uint32_t lv, const T*& p0, const T*& p1) {
-        int gid = min(u * 4 + wave, 2 * K - 1);
-        int half = gid & 1;
-        const uint32_t l = lv;                                            // 0 = empty = the zero row
-        uint32_t swz = (l >> 1) & 7;
-        p0 = &s_rows[l * 64 + (((uint32_t)(4 * half + q) ^ swz) * 8)];
-        p1 = &s_rows[l * 64 + (((uint32_t)(4 * half + 2 + q) ^ swz) * 8)];
-      };
-
-      constexpr int STEPS = UPW * 2;
-      uint32_t lcur[2], lnxt[2], lnx2[2] = {0u, 0u};
-      u32x4 ring[4][2];
-      const T *pa, *pb;
-      read_loc(0, lcur);
-      if (UPW > 1) read_loc(1, lnxt);
-      if (UPW > 2) read_loc(2, lnx2);
-      addr(0, lcur[0], pa, pb);
-      ring[0][0] = *(const u32x4*)pa;
-      ring[0][1] = *(const u32x4*)pb;
-      addr(0, lcur[1], pa, pb);
-      ring[1][0] = *(const u32x4*)pa;
-      ring[1][1] = *(const u32x4*)pb;
-      if (UPW > 1) {
-        addr(1, lnxt[0], pa, pb);
-        ring[2][0] = *(const u32x4*)pa;
-        ring[2][1] = *(const u32x4*)pb;
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // Every step issues its four MFMAs with the LDS traffic of step j + 3 placed between
-      // them, so that the address arithmetic and the reads issue while an MFMA executes.
-#pragma unroll
-      for (int j = 0; j < STEPS; ++j) {
-        const int u = j >> 1, nt = j & 1;
-        const bool pre = j + 3 < STEPS;
-        const int u3 = (j + 3) >> 1, nt3 = (j + 3) & 1;
-        acc[nt][0] = Mma32<T>::run(wreg[u][0][0], ring[j & 3][0], acc[nt][0]);
-        if (pre) addr(u3, u3 == u + 1 ? lnxt[nt3] : lnx2[nt3], pa, pb);
-        acc[nt][1] = Mma32<T>::run(wreg[u][0][1], ring[j & 3][0], acc[nt][1]);
-        if (pre) ring[(j + 3) & 3][0] = *(const u32x4*)pa;
-        acc[nt][0] = Mma32<T>::run(wreg[u][1][0], ring[j & 3][1], acc[nt][0]);
-        if (pre) ring[(j + 3) & 3][1] = *(const u32x4*)pb;
-        if (nt == 1) {
-          // the next unit becomes current; read the positions of the one three units on
-          lcur[0] = lnxt[0];
-          lcur[1] = lnxt[1];
-          lnxt[0] = lnx2[0];
-          lnxt[1] = lnx2[1];
-          if (u + 3 < UPW) read_loc(u + 3, lnx2);
-        }
-        acc[nt][1] = Mma32<T>::run(wreg[u][1][1], ring[j & 3][1], acc[nt][1]);
-        // 1 MFMA, then some VALU / LDS work in its shadow, four times
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (timing) { long long t = clock64(); t_main += t - t_mark; t_mark = t; }
-
-      // ---- cross-wave sum: wave w finishes (row tile w / 2, M tile w % 2) of this half ----
-      __syncthreads();           // s_red is free; after the second half also s_rows / s_loc[cur]
-      long long tq = 0;
-      if (timing) { tq = clock64(); t_e0 += tq - t_mark; }
-      if (half_t == 1) {
-        if (tile + 1 < t_end) {
-          stage(tile + 1, p_nx2 - p_nxt, cur ^ 1, cur ^ 1);      // ids came in one tile ago
-          if (tile + 2 < t_end) stage_list(p_nx2, cur);          // s_u[cur] was consumed a tile ago
-        }
-        p_nxt = p_nx2;
-        p_nx2 = p_nx3;
-      }
-      if (timing) { long long t = clock64(); t_e1 += t - tq; tq = t; }
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int tM = 0; tM < 2; ++tM) {
-          const int owner = nt * 2 + tM;
-          if (owner != wave) {
-            const int d3 = owner < wave ? owner : owner - 1;
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4)
-              s_red[((wave * 3 + d3) * 4 + r4) * 64 + lane] =
-                  f32x4{acc[nt][tM][4 * r4], acc[nt][tM][4 * r4 + 1], acc[nt][tM][4 * r4 + 2],
-                        acc[nt][tM][4 * r4 + 3]};
-          }
-        }
-      if (timing) { long long t = clock64(); t_e2 += t - tq; tq = t; }
-      __syncthreads();
-      if (timing) { long long t = clock64(); t_e3 += t - tq; tq = t; }
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int tM = 0; tM < 2; ++tM) {
-          const int owner = nt * 2 + tM;
-          if (owner == wave) {
-            const int64_t row = tile * kRwRows + 64 * half_t + 32 * nt + r32;
-            const int co0 = 32 * tM + 16 * q;
-            unsigned pk[8];
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-              f32x4 sum = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-              for (int src = 0; src < 4; ++src) {          // wave order: deterministic
-                f32x4 v;
-                if (src == owner) {
-                  v = f32x4{acc[nt][tM][4 * r4], acc[nt][tM][4 * r4 + 1], acc[nt][tM][4 * r4 + 2],
-                            acc[nt][tM][4 * r4 + 3]};
-                } else {
-                  const int d3 = owner < src ? owner : owner - 1;
-                  v = s_red[((src * 3 + d3) * 4 + r4) * 64 + lane];
-                }
-                sum = src == 0 ? v : sum + v;
-              }
-              float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
-              if (bias) {
-                b0 = to_f32(bias[co0 + 4 * r4]);
-                b1 = to_f32(bias[co0 + 4 * r4 + 1]);
-                b2 = to_f32(bias[co0 + 4 * r4 + 2]);
-                b3 = to_f32(bias[co0 + 4 * r4 + 3]);
-              }
-              pk[2 * r4] = pack2<T>(sum[0] + b0, sum[1] + b1);
-              pk[2 * r4 + 1] = pack2<T>(sum[2] + b2, sum[3] + b3);
-            }
-            if (row < rows_out) {
-              T* dst = out + row * 64 + co0;
-              *(u32x4*)(dst) = u32x4{pk[0], pk[1], pk[2], pk[3]};
-              *(u32x4*)(dst + 8) = u32x4{pk[4], pk[5], pk[6], pk[7]};
-            }
-          }
-        }
-      if (timing) { long long t = clock64(); t_epi += t - t_mark; t_mark = t; }
+    if (timing) t_mark = clock64();
+    half_body(std::integral_constant<int, 0>{}, lc, tile > t_begin ? (tile - 1) * kRwRows + 64 : rows_out);
+    half_body(std::integral_constant<int, 1>{}, lc, tile * kRwRows);
+    if (timing) { long long t = clock64(); t_main += t - t_mark; t_mark = t; }
+    // every wave is past its last read of s_rows / s_loc[cur] (the barrier closing the half)
+    if (tile + 1 < t_end) {
+      stage(tile + 1, p_nx2 - p_nxt, cur ^ 1, cur ^ 1);      // ids came in one tile ago
+      if (tile + 2 < t_end) stage_list(p_nx2, cur);          // s_u[cur] was consumed a tile ago
     }
+    p_nxt = p_nx2;
+    p_nx2 = p_nx3;
+    if (timing) { long long t = clock64(); t_stage += t - t_mark; t_mark = t; }
     __builtin_amdgcn_s_waitcnt(0);            // the next tile has landed (own loads)
     __syncthreads();                          // ... everyone's
     if (timing) { long long t = clock64(); t_wait += t - t_mark; t_mark = t; }
   }
+  // the last half of the range: its exchange has no main loop to hide under
+#pragma unroll
+  for (int e = 0; e < 26; ++e) {
+    exch_piece(std::integral_constant<int, 1>{}, e, (t_end - 1) * kRwRows + 64, true);
+    __builtin_amdgcn_sched_barrier(0);
+  }
   if (timing && lane == 0) {
     long long* d = dbg + ((int64_t)blockIdx.x * 4 + wave) * 8;
-    d[0] = t_main; d[1] = t_epi; d[2] = t_wait; d[3] = t_end - t_begin;
-    d[4] = t_e0; d[5] = t_e1; d[6] = t_e2; d[7] = t_e3;
+    d[0] = t_main; d[1] = t_stage; d[2] = t_wait; d[3] = t_end - t_begin;
+    d[4] = 0; d[5] = 0; d[6] = 0; d[7] = 0;
   }
 }
 
