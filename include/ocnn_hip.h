@@ -196,7 +196,7 @@ int ocnn_conv_gather_planned(int dtype, const void* in, int64_t rows_in,
 /* ocnn_conv_gather for 64 -> 64 channels with register-resident weights: one
  * persistent workgroup per CU keeps all K x 64 x 64 weights in VGPRs and walks
  * its tiles of the plan.  plan_max_distinct = largest number of distinct rows
- * of any tile (max of ucount); the kernel needs it <= 512.  plan_total = number
+ * of any tile (max of ucount); the kernel needs it <= 416.  plan_total = number
  * of entries of urows (uptr[tiles]).  Same result as ocnn_conv_gather. */
 int ocnn_conv_gather_rw_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                   int plan_max_distinct);

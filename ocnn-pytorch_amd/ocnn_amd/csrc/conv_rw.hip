@@ -23,7 +23,7 @@
 namespace ocnn {
 
 constexpr int kRwRows = 128;   // rows per tile (the plan's tile size)
-constexpr int kRwCap = 512;    // staged rows; plans with a larger tile use another kernel
+constexpr int kRwCap = 416;    // staged rows; plans with a larger tile use another kernel
 
 // Packed weights: [gid = 2 * slot + half][k-step s][M tile tM][lane][8].
 // v_mfma_f32_32x32x16 A operand: lane l holds A[l % 32][8 * (l / 32) + j];
@@ -49,6 +49,18 @@ __global__ void pack_weights_rw_kernel(const T* __restrict__ w, T* __restrict__ 
   out[e] = transposed ? w[((int64_t)kk * 64 + co) * 64 + chan] : w[((int64_t)kk * 64 + chan) * 64 + co];
 }
 
+// What the staging pieces of a tile need (plain types: the arguments of the global->LDS
+// load builtin must not be type-dependent expressions).
+struct RwStage {
+  uint32_t loc_off;     // byte offset of the tile's table positions
+  uint32_t list_off;    // per lane: byte offset of its part of the list of the tile after, or out of range
+  int groups;           // 8-row groups of LDS rows the tile fills (row 0 = zero row included)
+  const int32_t* su;    // list of the tile's distinct rows (LDS), entry -1 readable and -1
+  int32_t* su_out;      // where the next list goes (LDS)
+  char* rows;           // destination buffers (LDS)
+  char* locs;
+};
+
 template <typename T, int UPW>
 __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const uint16_t* __restrict__ loc,
@@ -56,12 +68,19 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
     uint32_t urows_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
     T* __restrict__ out, int64_t rows_out, int K, int64_t tiles, int64_t tiles_per_wg,
     long long* dbg) {
-  __shared__ __attribute__((aligned(16))) T s_rows[(kRwCap + 1) * 64];
-  // table positions, double buffered; filled 1 KiB per wave instruction, hence the rounding
-  __shared__ __attribute__((aligned(16))) uint16_t s_loc[2][(kRwRows * 27 * 2 + 1023) / 1024 * 512];
-  __shared__ f32x4 s_red[4 * 4 * 4 * 64];                                  // 64 KiB: [writer][combination][quarter][lane]
+  constexpr int kLocElems = (kRwRows * 27 * 2 + 1023) / 1024 * 512;   // whole KiB: filled 1 KiB per instruction
+  // Everything a tile needs is double buffered, one array per buffer so that the compiler
+  // can tell the buffer being filled from the one being read.
+  constexpr int kRowsAlloc = (kRwCap + 8) / 8 * 8;               // rows 0..kRwCap, whole 8-row groups
+  __shared__ __attribute__((aligned(16))) T s_rows0[kRowsAlloc * 64];
+  __shared__ __attribute__((aligned(16))) T s_rows1[kRowsAlloc * 64];
+  __shared__ __attribute__((aligned(16))) uint16_t s_loc0[kLocElems];
+  __shared__ __attribute__((aligned(16))) uint16_t s_loc1[kLocElems];
+  // lists of distinct rows from entry 4 on; entry 3 stays -1 ("the row before the first")
+  __shared__ __attribute__((aligned(16))) int32_t s_u0[4 + 512];
+  __shared__ __attribute__((aligned(16))) int32_t s_u1[4 + 512];
+  __shared__ f32x4 s_red[4 * 4 * 2 * 64];      // 32 KiB: [writer][combination][quarter of a round][lane]
   __shared__ __attribute__((aligned(16))) float s_bias[64];
-  __shared__ __attribute__((aligned(16))) int32_t s_u[2][kRwCap + 64];     // row lists, 2 tiles ahead
 
   constexpr int KK = UPW == 14 ? 27 : UPW == 5 ? 9 : UPW == 4 ? 8 : 3;   // slots (= K)
   const int tid = threadIdx.x, lane = tid & 63;
@@ -85,77 +104,68 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
         wreg[u][s][tM] = v;
       }
   }
+  // bias as fp32 in LDS (zeros without one); a lane finishes the 16 output channels
+  // 32 (wave % 2) + 16 q .. of a row
+  if (tid < 64) s_bias[tid] = bias ? to_f32(bias[tid]) : 0.f;
+  if (tid == 0) s_u0[3] = s_u1[3] = -1;
+  const f32x4* bias4 = (const f32x4*)(&s_bias[32 * (wave & 1) + 16 * q]);
 
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
   const __amdgpu_buffer_rsrc_t rs_loc = make_rsrc(loc, loc_bytes);
   const __amdgpu_buffer_rsrc_t rs_u = make_rsrc(urows, urows_bytes);
+  const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(uptr, (uint32_t)(tiles + 1) * 4u);
 
-  // asynchronous load of a tile's list of distinct rows (first entry `first`) -> s_u[buf]
-  auto stage_list = [&](int32_t first, int buf) {
-    if (wave < 2)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_u, (lds_ptr_t)(&s_u[buf][wave * 256]), 16,
-                                               (uint32_t)first * 4u + (uint32_t)wave * 1024u + lane * 16u,
-                                               0, 0, 0);
+  // ---- staging of one tile, cut into per-wave pieces (one 1 KiB load instruction each) ----
+  //   piece 0, 1      table positions (chunks wave, wave + 4)
+  //   piece 2         the list of distinct rows of the tile after (waves 0 and 1)
+  //   piece 3 + i     LDS rows 8 (wave + 4 i) .. + 7: row p >= 1 holds the (p - 1)-th distinct
+  //                   row, row 0 is the zero row that empty table entries (position 0) read;
+  //                   it comes from an out-of-range offset (list entry -1 = -1)
+  // A lane's 16-byte chunk c of row p lands at chunk c ^ ((p >> 1) & 7) (bank swizzle); with
+  // p = 8 (wave + 4 i) + lane / 8 that is a per-lane constant.
+  constexpr int kRowPieces = (kRwCap + 1 + 31) / 32;            // per wave
+  constexpr int kPieces = 3 + kRowPieces;
+  const uint32_t st_c = (uint32_t)(((lane & 7) ^ (((lane >> 4) + 4 * wave) & 7)) * 16);
+  const int st_p = 8 * wave + (lane >> 3);                      // LDS row of row piece 0; piece i: + 32 i
+  auto make_stage = [&](int64_t tile, int U, int32_t list_first, int32_t list_len, const int32_t* su,
+                        int32_t* su_out, T* rows, uint16_t* locs) {
+    RwStage st;
+    const int64_t tc = min(tile, tiles - 1);                    // past the range: any valid tile
+    st.loc_off = (uint32_t)(tc * kRwRows * KK * 2);
+    const int e = wave * 256 + lane * 4;                        // the four list entries this lane brings in
+    st.list_off = e < list_len ? (uint32_t)(list_first + e) * 4u : 0xffffff00u;
+    st.groups = (U + 8) >> 3;
+    st.su = su; st.su_out = su_out; st.rows = (char*)rows; st.locs = (char*)locs;
+    return st;
   };
-  // asynchronous staging of one tile: its U distinct rows (ids in s_u[ubuf]) -> s_rows, its
-  // table positions -> s_loc[buf]
-  auto stage = [&](int64_t tile, int U, int ubuf, int buf) {
-    // LDS row p (p >= 1) holds the (p - 1)-th distinct row; row 0 is the zero row that the
-    // empty table entries (position 0) read: its lanes load from an out-of-range offset
-    const int ngrp = (U + 8) >> 3;
-    // four groups of 8 rows per round: the four row ids are read first, then the loads go out
-    for (int g0 = wave; g0 < ngrp; g0 += 16) {
-      int32_t g[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int u = (g0 + 4 * i) * 8 + (lane >> 3);
-        g[i] = (u >= 1 && u <= U) ? s_u[ubuf][u - 1] : -1;
+  auto stage_id = [&](int t, const RwStage& st) -> int32_t {    // the list entry a lane needs for piece t
+    return t >= 3 ? st.su[st_p + 32 * (t - 3) - 1] : 0;
+  };
+  auto stage_piece = [&](int t, const RwStage& st, int32_t id) {
+    if (t < 2) {
+      constexpr int nchunk = (kRwRows * KK * 2 + 1023) >> 10;
+      if (4 * t < nchunk) {
+        const int c = min(wave + 4 * t, nchunk - 1);            // a spare wave repeats the last chunk
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_loc, (lds_ptr_t)(st.locs + c * 1024), 16,
+                                                 st.loc_off + (uint32_t)c * 1024u + lane * 16u, 0, 0, 0);
       }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int grp = g0 + 4 * i;
-        if (grp < ngrp) {
-          int u = grp * 8 + (lane >> 3);
-          uint32_t chunk = (uint32_t)((lane & 7) ^ ((u >> 1) & 7));      // bank swizzle
-          uint32_t off = g[i] < 0 ? 0xffffff00u : (uint32_t)g[i] * 128u + chunk * 16u;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(&s_rows[grp * 8 * 64]), 16, off, 0,
-                                                   0, 0);
-        }
-      }
+    } else if (t == 2) {
+      if (wave < 2)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_u, (lds_ptr_t)(st.su_out + wave * 256), 16, st.list_off,
+                                                 0, 0, 0);
+    } else {
+      if (wave + 4 * (t - 3) < st.groups)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(st.rows + (wave + 4 * (t - 3)) * 1024), 16,
+                                                 ((uint32_t)id << 7) | st_c, 0, 0, 0);
     }
-    // kRwRows * K positions (2 B each, [slot][row]), 1 KiB per wave instruction
-    const uint32_t lbase = (uint32_t)(tile * kRwRows * K * 2);
-    const int nchunk = (kRwRows * K * 2 + 1023) >> 10;
-    for (int c = wave; c < nchunk; c += 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_loc, (lds_ptr_t)(&s_loc[buf][c * 512]), 16,
-                                               lbase + (uint32_t)c * 1024u + lane * 16u, 0, 0, 0);
   };
-
-  // prologue: list of the first tile, then its rows and the list of the second tile
-  int32_t p_nxt = uptr[t_begin + 1];
-  int32_t p_nx2 = uptr[min(t_begin + 2, tiles)];
-  {
-    int32_t p_cur = uptr[t_begin];
-    stage_list(p_cur, 0);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    stage(t_begin, p_nxt - p_cur, 0, 0);
-    stage_list(p_nxt, 1);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-  }
 
 #ifdef OCNN_RW_TIMING
   const bool timing = dbg != nullptr;
 #else
   constexpr bool timing = false;
 #endif
-  long long t_main = 0, t_stage = 0, t_wait = 0, t_mark = 0;
-
-  // bias as fp32 in LDS (zeros without one); a lane finishes the 16 output channels
-  // 32 (wave % 2) + 16 q .. of a row
-  if (tid < 64) s_bias[tid] = bias ? to_f32(bias[tid]) : 0.f;
-  const f32x4* bias4 = (const f32x4*)(&s_bias[32 * (wave & 1) + 16 * q]);
+  long long t_main = 0, t_wait = 0, t_mark = 0;
 
   // Two accumulator sets: while a 64-row half is being multiplied into one, the partial sums
   // of the half before it (the other set) are exchanged through LDS and stored, a piece per
@@ -163,53 +173,61 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
   f32x16 acc[2][2][2];
 
   // ---- the cross-wave sum of one half, cut into pieces for the steps of a main loop ----
-  // Wave w finishes (row tile w / 2, M tile w % 2).  Pieces 0..15 write all four
-  // combinations to s_red (also the own one: the code is then the same for every wave and
-  // free of branches, which cost a wave far more than an LDS round trip), piece 19 is
-  // the barrier after them, 20..23 read the four partial sums of the own combination,
-  // 21..24 add them in wave order, 23 and 25 store.
-  f32x4 red[4], rb;        // partial sums and bias of a quarter (read at piece j, used at j + 1)
+  // Wave w finishes (row tile w / 2, M tile w % 2).  Two rounds of two register quarters:
+  // every wave writes all four combinations to s_red (also its own: the code is then the
+  // same for every wave and free of branches, which cost a wave far more than an LDS round
+  // trip), barrier, the owner reads the four partial sums, adds them in wave order, stores.
+  f32x4 red[4], rb;        // partial sums and bias of a quarter (read at one piece, used at the next)
   unsigned pk[4];
-  auto exch_piece = [&](auto SETC, int j, int64_t row0, bool drain) {     // row0: first row of that half
+  auto exch_piece = [&](auto SETC, int e, int64_t row0, bool drain) {     // row0: first row of that half
     constexpr int S = decltype(SETC)::value;
-    if (j < 16) {
-      const int c = j >> 2, r4 = j & 3;                       // combination c = 2 nt + tM
-      if (!(OCNN_RW_EXP & 1))
-        s_red[((wave * 4 + c) * 4 + r4) * 64 + lane] =
-            f32x4{acc[S][c >> 1][c & 1][4 * r4], acc[S][c >> 1][c & 1][4 * r4 + 1],
-                  acc[S][c >> 1][c & 1][4 * r4 + 2], acc[S][c >> 1][c & 1][4 * r4 + 3]};
-    } else if (j == 19) {
-      // With 28 steps a wave has by now consumed LDS reads that it issued after its last
-      // write, so the writes are done (LDS operations of a wave complete in order); in the
-      // shorter loops, and without a main loop around, it waits for them.
-      if (OCNN_RW_EXP & 2) {}
-      else if (drain) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    const int rnd = e >= 13 ? 1 : 0, f = e - 13 * rnd;       // round, piece of the round
+    auto barrier = [&]() {
+      // With 28 steps a wave has consumed, before a barrier piece, LDS reads that it issued
+      // after its last write or read of s_red (LDS operations of a wave complete in order);
+      // in the shorter loops, and without a main loop around, it waits.
+      if (drain) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       else asm volatile("s_barrier" ::: "memory");
-    } else if (j >= 20 && j <= 25) {
-      if (j == 23 || j == 25) {                               // channels 0-7 after quarter 1, 8-15 after 3
-        const int64_t row = row0 + 32 * (wave >> 1) + r32;
-        if (row < rows_out && !(OCNN_RW_EXP & 8))
-          *(u32x4*)(out + row * 64 + 32 * (wave & 1) + 16 * q + (j == 23 ? 0 : 8)) =
-              u32x4{pk[0], pk[1], pk[2], pk[3]};
-      }
-      if (j >= 21 && j <= 24 && !(OCNN_RW_EXP & 4)) {         // add quarter j - 21 in wave order, pack
-        const int r4 = j - 21;
-        const f32x4 sum = ((red[0] + red[1]) + red[2]) + red[3];
-        pk[2 * (r4 & 1)] = pack2<T>(sum[0] + rb[0], sum[1] + rb[1]);
-        pk[2 * (r4 & 1) + 1] = pack2<T>(sum[2] + rb[2], sum[3] + rb[3]);
-      }
-      if (j <= 23 && !(OCNN_RW_EXP & 4)) {                    // read the partial sums of quarter j - 20
-        const int r4 = j - 20;
+    };
+    if (e >= 26) return;
+    if (f < 4) {                                              // two writes: combination f, both quarters
 #pragma unroll
-        for (int src = 0; src < 4; ++src) red[src] = s_red[((src * 4 + wave) * 4 + r4) * 64 + lane];
-        rb = bias4[r4];
+      for (int h = 0; h < 2; ++h) {
+        const int r4 = 2 * rnd + h;
+        s_red[((wave * 4 + f) * 2 + h) * 64 + lane] =
+            f32x4{acc[S][f >> 1][f & 1][4 * r4], acc[S][f >> 1][f & 1][4 * r4 + 1],
+                  acc[S][f >> 1][f & 1][4 * r4 + 2], acc[S][f >> 1][f & 1][4 * r4 + 3]};
       }
+    } else if (f == 7) {
+      barrier();                                              // the partial sums are in place
+    } else if (f >= 8 && f <= 11) {
+      if (f == 9 || f == 10) {                                // add the quarter read one piece ago
+        const int h = f - 9;
+        const f32x4 sum = ((red[0] + red[1]) + red[2]) + red[3];
+        pk[2 * h] = pack2<T>(sum[0] + rb[0], sum[1] + rb[1]);
+        pk[2 * h + 1] = pack2<T>(sum[2] + rb[2], sum[3] + rb[3]);
+      }
+      if (f == 8 || f == 9) {                                 // read quarter f - 8 of the round
+        const int h = f - 8;
+#pragma unroll
+        for (int src = 0; src < 4; ++src) red[src] = s_red[((src * 4 + wave) * 2 + h) * 64 + lane];
+        rb = bias4[2 * rnd + h];
+      }
+      if (f == 11) {                                          // 8 channels = 16 bytes per lane
+        const int64_t row = row0 + 32 * (wave >> 1) + r32;
+        if (row < rows_out)
+          *(u32x4*)(out + row * 64 + 32 * (wave & 1) + 16 * q + 8 * rnd) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+      }
+    } else if (f == 12) {
+      barrier();                                              // the round has been read: s_red is free again
     }
   };
 
-  // ---- one 64-row half: main loop into acc[S], exchange of the previous half (acc[1 - S]) ----
-  // (prev_row0 past the last row: nothing is stored, as for the first half of a range)
-  auto half_body = [&](auto SETC, const uint16_t* lc, int64_t prev_row0) {
+  // ---- one 64-row half out of the buffers (rows, lc): main loop into acc[S], exchange of the
+  // half before it (acc[1 - S]; prev_row0 past the last row: nothing is stored), staging
+  // pieces t0, t0 + 1, .. of the next tile every other step (t0 < 0: none)
+  auto half_body = [&](auto SETC, const T* rows, const uint16_t* lc, int64_t prev_row0, int t0, int tn,
+                       const RwStage& st) {
     constexpr int S = decltype(SETC)::value;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
@@ -218,10 +236,6 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[S][nt][tM][r] = 0.f;
 
-    // The main loop is a flat sequence of steps (unit u, row tile nt).  The B operand of
-    // a step (lane: row r32 of the row tile, k group q -> 2 x 16 B of its neighbour row)
-    // is fetched from LDS three steps ahead of its four MFMAs; the table positions of a
-    // unit are read three units ahead.  Units past 2K have zero weights.
     // unit u of wave w is (slot 2u + w / 2, input-channel half w % 2): one base address per
     // half, immediate offsets per unit
     const uint16_t* lcw = lc + (wave >> 1) * kRwRows + 64 * S + r32;
@@ -235,42 +249,38 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
     };
     // LDS addresses of the two 16-byte pieces a lane reads of its neighbour row
     const uint32_t c0 = (uint32_t)(4 * (wave & 1) + q);
-    auto addr = [&](int u, uint32_t l, const T*& p0, const T*& p1) {   // l = 0: empty = the zero row
-      (void)u;
-      if (OCNN_RW_EXP & 64) {            // timing experiment: one VALU per look-up
-        p0 = &s_rows[(l << 3) + c0 * 8];
-        p1 = p0 + 16;
-        return;
-      }
+    auto addr = [&](uint32_t l, const T*& p0, const T*& p1) {   // l = 0: empty = the zero row
       const uint32_t swz = (l >> 1) & 7;
-      p0 = &s_rows[l * 64 + ((c0 ^ swz) * 8)];
-      p1 = &s_rows[l * 64 + (((c0 + 2) ^ swz) * 8)];
+      p0 = &rows[l * 64 + ((c0 ^ swz) * 8)];
+      p1 = &rows[l * 64 + (((c0 + 2) ^ swz) * 8)];
     };
 
+    // The main loop is a flat sequence of steps (unit u, row tile nt).  The B operand of
+    // a step (lane: row r32 of the row tile, k group q -> 2 x 16 B of its neighbour row)
+    // is fetched from LDS two steps ahead of its four MFMAs; the table positions of a
+    // unit are read two units ahead.  Units past 2K have zero weights.
     constexpr int STEPS = UPW * 2;
     uint32_t lcur[2], lnxt[2] = {0u, 0u};
     u32x4 ring[3][2];
     const T *pa, *pb;
     read_loc(0, lcur);
     if (UPW > 1) read_loc(1, lnxt);
-    addr(0, lcur[0], pa, pb);
+    addr(lcur[0], pa, pb);
     ring[0][0] = *(const u32x4*)pa;
     ring[0][1] = *(const u32x4*)pb;
-    addr(0, lcur[1], pa, pb);
+    addr(lcur[1], pa, pb);
     ring[1][0] = *(const u32x4*)pa;
     ring[1][1] = *(const u32x4*)pb;
     __builtin_amdgcn_sched_barrier(0);
-    // Every step issues its four MFMAs with the LDS traffic of step j + 2 placed between
-    // them, so that the address arithmetic and the reads issue while an MFMA executes.
-    // The exchange pieces are spread over the steps whatever their number.
     constexpr int EPS = (26 + STEPS - 1) / STEPS;           // exchange pieces per step
+    constexpr int SPS = STEPS >= 28 ? 1 : (kPieces + STEPS - 1) / STEPS + 1;   // staging pieces per step slot
+    int32_t id_next = 0;
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
       const int u = j >> 1, nt = j & 1;
       const bool pre = j + 2 < STEPS;
-      const int nt2 = nt;                                    // step j + 2: unit u + 1, same row tile
       acc[S][nt][0] = Mma32<T>::run(wreg[u][0][0], ring[j % 3][0], acc[S][nt][0]);
-      if (pre) addr(u + 1, lnxt[nt2], pa, pb);
+      if (pre) addr(lnxt[nt], pa, pb);                       // step j + 2: unit u + 1, same row tile
       acc[S][nt][1] = Mma32<T>::run(wreg[u][0][1], ring[j % 3][0], acc[S][nt][1]);
       if (pre) ring[(j + 2) % 3][0] = *(const u32x4*)pa;
       acc[S][nt][0] = Mma32<T>::run(wreg[u][1][0], ring[j % 3][1], acc[S][nt][0]);
@@ -294,32 +304,72 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
 #pragma unroll
       for (int e = j * EPS; e < (j + 1) * EPS && e < 26; ++e)
         exch_piece(std::integral_constant<int, 1 - S>{}, e, prev_row0, UPW != 14);
+      // staging: the list entry is read on an even step, its load goes out on the odd one after
+      if (t0 >= 0) {
+        if (STEPS >= 28) {
+          const int t = t0 + (j >> 1);
+          if (t < tn) {
+            if ((j & 1) == 0) id_next = stage_id(t, st);
+            else stage_piece(t, st, id_next);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < SPS; ++i) {
+            const int t = t0 + j * SPS + i;
+            if (t < tn) stage_piece(t, st, stage_id(t, st));
+          }
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    // s_red may be written again (next half) once every owner has used what it read
-    if (!(OCNN_RW_EXP & 2)) asm volatile("s_barrier" ::: "memory");
   };
 
-  for (int64_t tile = t_begin; tile < t_end; ++tile) {
-    const int cur = (int)(tile - t_begin) & 1;
-    const uint16_t* lc = s_loc[cur];
-    // list boundary three tiles ahead (scalar load, used after the main loop)
-    const int32_t p_nx3 = uptr[min(tile + 3, tiles)];
-    if (timing) t_mark = clock64();
-    half_body(std::integral_constant<int, 0>{}, lc, tile > t_begin ? (tile - 1) * kRwRows + 64 : rows_out);
-    half_body(std::integral_constant<int, 1>{}, lc, tile * kRwRows);
-    if (timing) { long long t = clock64(); t_main += t - t_mark; t_mark = t; }
-    // every wave is past its last read of s_rows / s_loc[cur] (the barrier closing the half)
-    if (tile + 1 < t_end) {
-      stage(tile + 1, p_nx2 - p_nxt, cur ^ 1, cur ^ 1);      // ids came in one tile ago
-      if (tile + 2 < t_end) stage_list(p_nx2, cur);          // s_u[cur] was consumed a tile ago
-    }
+  // ---- prologue: first list, first tile, second list ----
+  int32_t p_nxt = uptr[t_begin + 1];
+  int32_t p_nx2 = uptr[min(t_begin + 2, tiles)];
+  int32_t p_nx3 = uptr[min(t_begin + 3, tiles)];
+  {
+    const int32_t p_cur = uptr[t_begin];
+    RwStage st = make_stage(t_begin, 0, p_cur, p_nxt - p_cur, s_u0 + 4, s_u0 + 4, s_rows0, s_loc0);
+    stage_piece(2, st, 0);                                   // list of the first tile -> s_u0
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    st = make_stage(t_begin, p_nxt - p_cur, p_nxt, p_nx2 - p_nxt, s_u0 + 4, s_u1 + 4, s_rows0, s_loc0);
+#pragma unroll
+    for (int t = 0; t < kPieces; ++t) stage_piece(t, st, stage_id(t, st));     // also: list of the second tile
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+  }
+
+  // one tile out of buffer B; the next tile is staged into buffer 1 - B meanwhile
+  constexpr int kHalfSteps = UPW;                            // staging slots in a half (one per two steps)
+  auto tile_body = [&](auto BC, int64_t tile) {
+    constexpr int B = decltype(BC)::value;
+    const T* rows = B ? s_rows1 : s_rows0;
+    const uint16_t* lc = B ? s_loc1 : s_loc0;
+    // next tile -> the other buffers (its list is in the other s_u); list of the tile after
+    // it -> this tile's s_u, which has been used up
+    const RwStage st = make_stage(tile + 1, p_nx2 - p_nxt, p_nx2, p_nx3 - p_nx2, B ? s_u0 + 4 : s_u1 + 4,
+                                  B ? s_u1 + 4 : s_u0 + 4, B ? s_rows0 : s_rows1, B ? s_loc0 : s_loc1);
+    // list boundary four tiles ahead, as a vector load: a scalar load would share its counter
+    // with the LDS reads and force them to drain where it is used
+    const uint32_t p_raw = __builtin_amdgcn_raw_buffer_load_b32(rs_p, (uint32_t)min(tile + 4, tiles) * 4u, 0, 0);
     p_nxt = p_nx2;
     p_nx2 = p_nx3;
-    if (timing) { long long t = clock64(); t_stage += t - t_mark; t_mark = t; }
-    __builtin_amdgcn_s_waitcnt(0);            // the next tile has landed (own loads)
-    __syncthreads();                          // ... everyone's
+    if (timing) t_mark = clock64();
+    half_body(std::integral_constant<int, 0>{}, rows, lc, tile > t_begin ? (tile - 1) * kRwRows + 64 : rows_out,
+              0, kPieces, st);
+    half_body(std::integral_constant<int, 1>{}, rows, lc, tile * kRwRows, (UPW >= 14 ? kHalfSteps : kPieces), kPieces, st);
+    if (timing) { long long t = clock64(); t_main += t - t_mark; t_mark = t; }
+    // the next tile has landed (own loads, then everyone's); every wave is past its last read
+    // of this tile's buffers and of s_red
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    p_nx3 = __builtin_amdgcn_readfirstlane((int32_t)p_raw);
     if (timing) { long long t = clock64(); t_wait += t - t_mark; t_mark = t; }
+  };
+  for (int64_t tile = t_begin; tile < t_end; tile += 2) {
+    tile_body(std::integral_constant<int, 0>{}, tile);
+    if (tile + 1 < t_end) tile_body(std::integral_constant<int, 1>{}, tile + 1);
   }
   // the last half of the range: its exchange has no main loop to hide under
 #pragma unroll
@@ -329,7 +379,7 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
   }
   if (timing && lane == 0) {
     long long* d = dbg + ((int64_t)blockIdx.x * 4 + wave) * 8;
-    d[0] = t_main; d[1] = t_stage; d[2] = t_wait; d[3] = t_end - t_begin;
+    d[0] = t_main; d[1] = 0; d[2] = t_wait; d[3] = t_end - t_begin;
     d[4] = 0; d[5] = 0; d[6] = 0; d[7] = 0;
   }
 }
