@@ -1,0 +1,127 @@
+"""Per-layer timings of the other layer configurations of the hot path on one
+MI355X (the headline number is bench.py's; these lines are supporting data).
+
+  config 2: depth-8 batch of 8 (100k points each), bf16: OctreeConv 2x2x2 stride 2
+            64->128 (depth 8->7), OctreeDeconv 2x2x2 stride 2 128->64 (7->8),
+            OctreeDWConv 3x3x3 on 128 channels at depth 7; also the 3x3x3 64->64 layer
+            with nempty=True.
+  config 3: batch of 4, depth 9, 250k points each (planes + spheres), bf16:
+            OctreeConv 3x3x3 32->32 at depth 9 and 256->256 at depth 6; build_octree and
+            construct_all_neigh on the 1M points.
+
+Every layer runs forward + backward through the module (autograd included); one JSON
+line per layer: ms per fwd+bwd, effective TFLOP/s over non-empty neighbours, and the
+rate at the algorithmic byte count as a fraction of 8 TB/s.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, 'ocnn-pytorch_amd')):
+  if p not in sys.path:
+    sys.path.insert(0, p)
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--steps', type=int, default=30)
+  ap.add_argument('--warmup', type=int, default=5)
+  ap.add_argument('--configs', default='2,3')
+  args = ap.parse_args()
+  import torch
+  from ocnn_amd import synthetic
+  from ocnn_amd.nn import OctreeConv, OctreeDeconv, OctreeDWConv
+  from ocnn_amd.octree import Octree, Points
+  assert torch.cuda.is_available(), 'bench_layers.py needs a GPU'
+  dev = 'cuda:0'
+  torch.cuda.set_device(0)
+
+  def build(cloud, batch, seed, n, depth):
+    pts, nrm, bid = synthetic.batch_clouds(cloud, batch, seed, n=n)
+    pc = Points(pts.to(dev), nrm.to(dev), batch_id=bid.to(dev), batch_size=batch)
+    times = []
+    for _ in range(3):
+      o = Octree(depth, 2, batch_size=batch)
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      o.build_octree(pc)
+      torch.cuda.synchronize()
+      t1 = time.perf_counter()
+      o.construct_all_neigh()
+      torch.cuda.synchronize()
+      times.append((t1 - t0, time.perf_counter() - t1))
+    return o, min(t[0] for t in times) * 1e3, min(t[1] for t in times) * 1e3, int(pts.shape[0])
+
+  def run(tag, mod, octree, depth, rows_in, cin, cout, table, dtype, dw=False):
+    g = torch.Generator().manual_seed(7)
+    mod = mod.to(dev).to(dtype)
+    x = torch.randn(rows_in, cin, generator=g).to(dtype).to(dev).requires_grad_()
+    out = mod(x, octree, depth)
+    gout = torch.randn(out.shape, generator=g).to(dtype).to(dev)
+
+    def step():
+      x.grad = None
+      mod.weights.grad = None
+      mod(x, octree, depth).backward(gout)
+
+    for _ in range(args.warmup):
+      step()
+    torch.cuda.synchronize()
+    s = torch.cuda.Event(enable_timing=True)
+    e = torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(args.steps):
+      step()
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / args.steps
+    rows, K = table.shape
+    nnz = int((table >= 0).sum())
+    flops = 6.0 * nnz * (cin if dw else cin * cout)
+    es = 2
+    if dw:
+      bytes_ = 3 * (es * (rows_in * cin + rows * cin + K * cin) + 4 * rows * K)
+    else:
+      bytes_ = 3 * (es * (rows_in * cin + rows * cout) + 4 * rows * K) + 2 * es * K * cin * cout + 4 * K * cin * cout
+    print(json.dumps({
+        'layer': tag, 'dtype': str(dtype).replace('torch.', ''), 'rows_in': rows_in, 'rows_table': rows,
+        'K': K, 'nnz': nnz, 'ms_fwd_bwd': ms, 'eff_tflops': flops / ms / 1e9,
+        'frac_mfma_peak': flops / ms / 1e9 / 2500.0,
+        'algorithmic_bytes': bytes_, 'frac_hbm_peak_at_algorithmic_bytes': bytes_ / ms / 1e6 / 8000.0,
+    }), flush=True)
+
+  bf = torch.bfloat16
+  if '2' in args.configs.split(','):
+    o, b_ms, n_ms, npts = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
+    print(json.dumps({'octree': 'config 2 (batch 8, depth 8)', 'points': npts, 'build_octree_ms': b_ms,
+                      'construct_all_neigh_ms': n_ms, 'nnum': o.nnum.tolist(),
+                      'nnum_nempty': o.nnum_nempty.tolist()}), flush=True)
+    nn8, ne8, nn7, ne7 = int(o.nnum[8]), int(o.nnum_nempty[8]), int(o.nnum[7]), int(o.nnum_nempty[7])
+    run('conv 2x2x2 s2 64->128 d8->7', OctreeConv(64, 128, [2], 2), o, 8, nn8, 64, 128,
+        o._table(8, '222', 2, False), bf)
+    run('deconv 2x2x2 s2 128->64 d7->8', OctreeDeconv(128, 64, [2], 2), o, 7, nn7, 128, 64,
+        o._table(8, '222', 2, False), bf)
+    run('dwconv 3x3x3 128 d7', OctreeDWConv(128, [3], 1), o, 7, nn7, 128, 128,
+        o._table(7, '333', 1, False), bf, dw=True)
+    run('conv 3x3x3 s1 64->64 d8 nempty', OctreeConv(64, 64, [3], 1, nempty=True), o, 8, ne8, 64, 64,
+        o._table(8, '333', 1, True), bf)
+    run('conv 3x3x3 s1 64->64 d8', OctreeConv(64, 64, [3], 1), o, 8, nn8, 64, 64,
+        o._table(8, '333', 1, False), bf)
+    del o
+  if '3' in args.configs.split(','):
+    o, b_ms, n_ms, npts = build(synthetic.planes_cloud, 4, 1003, 250000, 9)
+    print(json.dumps({'octree': 'config 3 (batch 4, depth 9)', 'points': npts, 'build_octree_ms': b_ms,
+                      'construct_all_neigh_ms': n_ms, 'nnum': o.nnum.tolist(),
+                      'nnum_nempty': o.nnum_nempty.tolist()}), flush=True)
+    run('conv 3x3x3 s1 32->32 d9', OctreeConv(32, 32, [3], 1), o, 9, int(o.nnum[9]), 32, 32,
+        o._table(9, '333', 1, False), bf)
+    run('conv 3x3x3 s1 256->256 d6', OctreeConv(256, 256, [3], 1), o, 6, int(o.nnum[6]), 256, 256,
+        o._table(6, '333', 1, False), bf)
+
+
+if __name__ == '__main__':
+  main()

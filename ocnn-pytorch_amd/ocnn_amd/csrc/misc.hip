@@ -3,6 +3,7 @@
 #include <algorithm>
 
 #include "common.hpp"
+#include "mma.hpp"
 #include "reduce.hpp"
 
 namespace ocnn {
@@ -66,6 +67,176 @@ __global__ __launch_bounds__(256) void dw_wgrad_kernel(
       partial[((int64_t)split * K + k) * C + c] =
           ((s_acc[0][cl] + s_acc[1][cl]) + s_acc[2][cl]) + s_acc[3][cl];
   }
+}
+
+// ---- depth-wise kernels with all KK slots per thread -------------------------------
+// A thread owns 4 consecutive channels; C / 4 lanes cover a row and 256 / (C / 4) rows
+// are in flight per workgroup.  The table rows of 64 rows are brought into LDS with
+// coalesced loads; the feature rows are read with raw buffer loads whose offset is
+// out of range for an empty entry (reads zero, no branch).  KK is a template parameter
+// so that the slot loop has no branches at all.
+constexpr int kDwChunk = 64;
+
+template <typename T> struct DwVec;     // 4 channels
+template <> struct DwVec<float> {
+  static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, uint32_t off, float (&v)[4]) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    const f32x4 f = __builtin_bit_cast(f32x4, t);     // (a bit cast of one element t[i] reads element 0)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = f[i];
+  }
+};
+template <> struct DwVec<f16> {
+  static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, uint32_t off, float (&v)[4]) {
+    u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    typedef __attribute__((ext_vector_type(4))) _Float16 h4;
+    h4 h = __builtin_bit_cast(h4, t);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (float)h[i];
+  }
+};
+template <> struct DwVec<bf16> {
+  static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, uint32_t off, float (&v)[4]) {
+    u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    v[0] = __builtin_bit_cast(float, t[0] << 16);
+    v[1] = __builtin_bit_cast(float, t[0] & 0xffff0000u);
+    v[2] = __builtin_bit_cast(float, t[1] << 16);
+    v[3] = __builtin_bit_cast(float, t[1] & 0xffff0000u);
+  }
+};
+
+template <typename T, int KK>
+__global__ __launch_bounds__(256) void dw_gather_rows_kernel(
+    const T* __restrict__ in, uint32_t in_bytes, const int32_t* __restrict__ table, int64_t rows_out,
+    const T* __restrict__ w, int C, int reverse, const T* __restrict__ bias, T* __restrict__ out,
+    uint32_t out_bytes, int64_t rows_per_wg) {
+  __shared__ int32_t s_tab[kDwChunk * KK];
+  const int tid = threadIdx.x;
+  const int lpr = C >> 2, rp = 256 / lpr;
+  const int cl = tid % lpr, rl = tid / lpr;
+  const uint32_t coff = (uint32_t)cl * 4u * (uint32_t)sizeof(T);
+  const uint32_t row_bytes = (uint32_t)C * (uint32_t)sizeof(T);
+  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
+  const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(w, (uint32_t)(KK * C) * (uint32_t)sizeof(T));
+  float wr[KK][4], b4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < KK; ++k) DwVec<T>::load(rs_w, (uint32_t)(reverse ? KK - 1 - k : k) * row_bytes + coff, wr[k]);
+  if (bias) {
+    const __amdgpu_buffer_rsrc_t rs_b = make_rsrc(bias, row_bytes);
+    DwVec<T>::load(rs_b, coff, b4);
+  }
+  const int64_t r_begin = (int64_t)blockIdx.x * rows_per_wg;
+  const int64_t r_end = min(rows_out, r_begin + rows_per_wg);
+  for (int64_t r0 = r_begin; r0 < r_end; r0 += kDwChunk) {
+    const int nrows = (int)min<int64_t>(kDwChunk, r_end - r0);
+    __syncthreads();
+    for (int e = tid; e < nrows * KK; e += 256) s_tab[e] = table[r0 * KK + e];
+    __syncthreads();
+    for (int rr = rl; rr < nrows; rr += rp) {
+      float acc[4] = {b4[0], b4[1], b4[2], b4[3]};
+      float xv[KK][4];
+#pragma unroll
+      for (int k = 0; k < KK; ++k) {
+        const int32_t idx = s_tab[rr * KK + k];
+        DwVec<T>::load(rs_in, idx < 0 ? 0xffffff00u : (uint32_t)idx * row_bytes + coff, xv[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < KK; ++k)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[v] += xv[k][v] * wr[k][v];
+      T* dst = out + (r0 + rr) * C + cl * 4;
+      if constexpr (sizeof(T) == 4) {
+        *(f32x4*)dst = f32x4{acc[0], acc[1], acc[2], acc[3]};
+      } else {
+        *(u32x2*)dst = u32x2{pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
+      }
+    }
+  }
+}
+
+// partial[wg][k][c] = sum over the rows of workgroup wg
+template <typename T, int KK>
+__global__ __launch_bounds__(256) void dw_wgrad_rows_kernel(
+    const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes,
+    const int32_t* __restrict__ table, int64_t rows, int C, int64_t rows_per_wg,
+    float* __restrict__ partial) {
+  __shared__ int32_t s_tab[kDwChunk * KK];
+  __shared__ float s_red[256 * 4];
+  const int tid = threadIdx.x;
+  const int lpr = C >> 2, rp = 256 / lpr;
+  const int cl = tid % lpr, rl = tid / lpr;
+  const uint32_t coff = (uint32_t)cl * 4u * (uint32_t)sizeof(T);
+  const uint32_t row_bytes = (uint32_t)C * (uint32_t)sizeof(T);
+  const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, x_bytes);
+  const __amdgpu_buffer_rsrc_t rs_g = make_rsrc(g, g_bytes);
+  float acc[KK][4];
+#pragma unroll
+  for (int k = 0; k < KK; ++k)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc[k][v] = 0.f;
+  const int64_t r_begin = (int64_t)blockIdx.x * rows_per_wg;
+  const int64_t r_end = min(rows, r_begin + rows_per_wg);
+  for (int64_t r0 = r_begin; r0 < r_end; r0 += kDwChunk) {
+    const int nrows = (int)min<int64_t>(kDwChunk, r_end - r0);
+    __syncthreads();
+    for (int e = tid; e < nrows * KK; e += 256) s_tab[e] = table[r0 * KK + e];
+    __syncthreads();
+    for (int rr = rl; rr < nrows; rr += rp) {
+      float gv[4], xv[KK][4];
+      DwVec<T>::load(rs_g, (uint32_t)(r0 + rr) * row_bytes + coff, gv);
+#pragma unroll
+      for (int k = 0; k < KK; ++k) {
+        const int32_t idx = s_tab[rr * KK + k];
+        DwVec<T>::load(rs_x, idx < 0 ? 0xffffff00u : (uint32_t)idx * row_bytes + coff, xv[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < KK; ++k)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[k][v] += xv[k][v] * gv[v];
+    }
+  }
+  // the row lanes of the workgroup, added in lane order
+  float* dst = partial + (int64_t)blockIdx.x * KK * C;
+#pragma unroll
+  for (int k = 0; k < KK; ++k) {
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < 4; ++v) s_red[(rl * lpr + cl) * 4 + v] = acc[k][v];
+    __syncthreads();
+    if (tid < C) {
+      float sum = 0.f;
+      for (int r = 0; r < rp; ++r) sum += s_red[(r * lpr + (tid >> 2)) * 4 + (tid & 3)];
+      dst[k * C + tid] = sum;
+    }
+  }
+}
+
+// shapes the all-slots kernels take: C / 4 lanes per row must tile a 256-thread workgroup
+static bool dw_rows_ok(int K, int C, int64_t rows_in, int es) {
+  if (K != 27 && K != 9 && K != 8 && K != 3) return false;
+  if (C < 4 || C > 1024 || (C & (C - 1)) != 0) return false;
+  return (int64_t)rows_in * C * es < 0xfff00000ll;
+}
+
+// 16 bytes per thread: `chunks` 16-byte pieces per row
+__global__ void pad16_kernel(const u32x4* __restrict__ data, const int32_t* __restrict__ children,
+                             int64_t n, int chunks, u32x4 fill, u32x4* __restrict__ out) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * chunks) return;
+  int64_t q = t / chunks;
+  int c = (int)(t % chunks);
+  int32_t ch = children[q];
+  out[t] = ch >= 0 ? data[(int64_t)ch * chunks + c] : fill;
+}
+
+__global__ void depad16_kernel(const u32x4* __restrict__ data, const int32_t* __restrict__ children,
+                               int64_t n, int chunks, u32x4* __restrict__ out) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * chunks) return;
+  int64_t q = t / chunks;
+  int c = (int)(t % chunks);
+  int32_t ch = children[q];
+  if (ch >= 0) out[(int64_t)ch * chunks + c] = data[t];
 }
 
 template <typename T>
@@ -142,6 +313,23 @@ extern "C" int ocnn_dwconv_gather(int dtype, const void* in, int64_t rows_in,
   if (rows_out <= 0) return OCNN_OK;
   hipStream_t st = (hipStream_t)stream;
   const int C = channels;
+  if (dw_rows_ok(K, C, std::max(rows_in, rows_out), dtype_size(dtype))) {
+    const int64_t wgs = std::min<int64_t>(cdiv(rows_out, kDwChunk), 2048);
+    const int64_t per = align_up(cdiv(rows_out, wgs), kDwChunk);
+    const unsigned grid = (unsigned)cdiv(rows_out, per);
+#define OCNN_DW_GATHER(KK_)                                                                          \
+  OCNN_DISPATCH_DTYPE(dtype, {                                                                       \
+    hipLaunchKernelGGL((dw_gather_rows_kernel<T, KK_>), dim3(grid), dim3(256), 0, st, (const T*)in,  \
+                       (uint32_t)(rows_in * C * sizeof(T)), table, rows_out, (const T*)w, C,         \
+                       reverse_slots, (const T*)bias, (T*)out, (uint32_t)(rows_out * C * sizeof(T)), per); \
+  })
+    if (K == 27) OCNN_DW_GATHER(27);
+    else if (K == 9) OCNN_DW_GATHER(9);
+    else if (K == 8) OCNN_DW_GATHER(8);
+    else OCNN_DW_GATHER(3);
+#undef OCNN_DW_GATHER
+    return check_launch("dwconv_gather");
+  }
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     if (C % VEC == 0) {
@@ -175,6 +363,27 @@ extern "C" int ocnn_dwconv_wgrad(int dtype, const void* x, int64_t rows_x, const
     set_error("dwconv_wgrad: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
+  if (rows > 0 && dw_rows_ok(K, channels, std::max(rows_x, rows), dtype_size(dtype))) {
+    const int C = channels;
+    const int64_t wgs = std::min<int64_t>(cdiv(rows, kDwChunk), 512);
+    const int64_t per = align_up(cdiv(rows, wgs), kDwChunk);
+    const int used = (int)cdiv(rows, per);
+    float* part = (float*)workspace;
+#define OCNN_DW_WGRAD(KK_)                                                                         \
+  OCNN_DISPATCH_DTYPE(dtype, {                                                                     \
+    hipLaunchKernelGGL((dw_wgrad_rows_kernel<T, KK_>), dim3(used), dim3(256), 0, st, (const T*)x,  \
+                       (uint32_t)(rows_x * C * sizeof(T)), (const T*)g,                            \
+                       (uint32_t)(rows * C * sizeof(T)), table, rows, C, per, part);               \
+    hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3(cdiv((int64_t)K * C, 256)), dim3(256), 0, st,  \
+                       part, used, K, 1, C, 0, (T*)gw);                                            \
+  })
+    if (K == 27) OCNN_DW_WGRAD(27);
+    else if (K == 9) OCNN_DW_WGRAD(9);
+    else if (K == 8) OCNN_DW_WGRAD(8);
+    else OCNN_DW_WGRAD(3);
+#undef OCNN_DW_WGRAD
+    return check_launch("dwconv_wgrad");
+  }
   float* partial = (float*)workspace;
   OCNN_DISPATCH_DTYPE(dtype, {
     if (rows > 0)
@@ -191,6 +400,24 @@ extern "C" int ocnn_pad(int dtype, const void* data, const int32_t* children, in
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1, "pad: bad arguments");
   if (n <= 0) return OCNN_OK;
   hipStream_t st = (hipStream_t)stream;
+  const int64_t row_bytes = (int64_t)channels * dtype_size(dtype);
+  if (row_bytes % 16 == 0 && ((uintptr_t)data % 16 == 0) && ((uintptr_t)out % 16 == 0)) {
+    const int chunks = (int)(row_bytes / 16);
+    u32x4 fill;
+    if (dtype == OCNN_F32) {
+      const unsigned b = __builtin_bit_cast(unsigned, val);
+      fill = u32x4{b, b, b, b};
+    } else {
+      unsigned short h;
+      if (dtype == OCNN_F16) { f16 v = (f16)val; h = __builtin_bit_cast(unsigned short, v); }
+      else { bf16 v = (bf16)val; h = __builtin_bit_cast(unsigned short, v); }
+      const unsigned b = (unsigned)h | ((unsigned)h << 16);
+      fill = u32x4{b, b, b, b};
+    }
+    hipLaunchKernelGGL(pad16_kernel, dim3(cdiv(n * chunks, 256)), dim3(256), 0, st, (const u32x4*)data,
+                       children, n, chunks, fill, (u32x4*)out);
+    return check_launch("pad");
+  }
   OCNN_DISPATCH_DTYPE(dtype, {
     hipLaunchKernelGGL(pad_kernel<T>, dim3(cdiv(n * channels, 256)), dim3(256), 0, st,
                        (const T*)data, children, n, channels, val, (T*)out);
@@ -203,6 +430,13 @@ extern "C" int ocnn_depad(int dtype, const void* data, const int32_t* children, 
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1, "depad: bad arguments");
   if (n <= 0) return OCNN_OK;
   hipStream_t st = (hipStream_t)stream;
+  const int64_t row_bytes = (int64_t)channels * dtype_size(dtype);
+  if (row_bytes % 16 == 0 && ((uintptr_t)data % 16 == 0) && ((uintptr_t)out % 16 == 0)) {
+    const int chunks = (int)(row_bytes / 16);
+    hipLaunchKernelGGL(depad16_kernel, dim3(cdiv(n * chunks, 256)), dim3(256), 0, st, (const u32x4*)data,
+                       children, n, chunks, (u32x4*)out);
+    return check_launch("depad");
+  }
   OCNN_DISPATCH_DTYPE(dtype, {
     hipLaunchKernelGGL(depad_kernel<T>, dim3(cdiv(n * channels, 256)), dim3(256), 0, st,
                        (const T*)data, children, n, channels, (T*)out);

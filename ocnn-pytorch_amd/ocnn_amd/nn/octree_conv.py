@@ -44,7 +44,8 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
         int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return out
-  if plan is not None and L.ocnn_conv_gather_planned_supported(code, rows_in, cin, cout):
+  if plan is not None and plan.reuse >= 2.0 and L.ocnn_conv_gather_planned_supported(
+      code, rows_in, cin, cout):
     _lib.check(L.ocnn_conv_gather_planned(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
@@ -145,6 +146,11 @@ class OctreeConvBase:
     # rows on the "fine" side of the table (what its entries index)
     self.fine_h = self.in_h if self.is_conv_layer() else self.out_h
     self.symmetric = self.stride == 1 and self.kernel != '222'
+    # 2x2x2 stride 2 over all nodes: row p of the table is exactly the 8 children 8p .. 8p+7
+    # (children of a non-empty node are numbered consecutively, ocnn/octree/octree.py:235-259),
+    # so the layer is a dense GEMM on the (P, 8 * C) view of the fine side: no gather at all
+    self.dense_children = (self.kernel == '222' and self.stride == 2 and not self.nempty and
+                           self.fine_h == 8 * self.neigh.shape[0])
 
   def check_and_init(self, data: torch.Tensor):
     check = tuple(data.shape) == self.in_shape
@@ -163,14 +169,35 @@ class OctreeConvBase:
     return self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse,
                              self.fine_h)
 
+  def _identity(self, rows, device):
+    """(rows, 1) table [0, 1, ..]: the one-slot 'gather' of the dense form."""
+    cache = self.octree.__dict__.setdefault('_identity_tables', {})
+    key = (rows, str(device))
+    if key not in cache:
+      cache[key] = torch.arange(rows, dtype=torch.int32, device=device).view(rows, 1)
+    return cache[key]
+
   def forward_gemm(self, data, weights, bias=None):
     """(fine rows, in_conv) -> (table rows, out_conv)."""
+    if self.dense_children:
+      P = self.neigh.shape[0]
+      return conv_gather(data.view(P, 8 * self.in_conv), P, self._identity(P, data.device),
+                         weights.view(1, 8 * self.in_conv, self.out_conv), self.out_conv, False,
+                         False, bias, None)
     plan = self._plan(data, self.in_conv, self.out_conv)
     return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias,
                        plan)
 
   def backward_gemm(self, grad, weights, bias=None):
     """(table rows, out_conv) -> (fine rows, in_conv)."""
+    if self.dense_children:
+      # gin.view(P, 8 * in_conv) = grad @ W'^T with W' = weights.view(8 * in_conv, out_conv)
+      P = self.neigh.shape[0]
+      b8 = None if bias is None else bias.repeat(8)
+      out = conv_gather(grad, P, self._identity(P, grad.device),
+                        weights.view(1, 8 * self.in_conv, self.out_conv), 8 * self.in_conv, True,
+                        False, b8, None)
+      return out.view(8 * P, self.in_conv)
     if self.symmetric:
       plan = self._plan(grad, self.out_conv, self.in_conv)
       return conv_gather(grad, grad.shape[0], self.neigh, weights, self.in_conv, True, True, bias,
@@ -181,6 +208,11 @@ class OctreeConvBase:
 
   def weight_gemm(self, data, grad, out_transposed=False):
     """data: fine rows; grad: table rows -> (K, in_conv, out_conv)."""
+    if self.dense_children:
+      P = self.neigh.shape[0]
+      gw = conv_wgrad(data.view(P, 8 * self.in_conv), grad, self._identity(P, data.device), False,
+                      None).view(8, self.in_conv, self.out_conv)
+      return gw.transpose(1, 2).contiguous() if out_transposed else gw
     plan = self._plan(data, self.in_conv, self.out_conv)
     return conv_wgrad(data, grad, self.neigh, out_transposed, plan)
 

@@ -120,8 +120,10 @@ class TilePlan:
     _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(ucount), st))
     uptr = torch.zeros(tiles + 1, dtype=torch.int32, device=dev)
     uptr[1:] = torch.cumsum(ucount, 0)
-    total, umax = (int(v) for v in torch.stack([uptr[-1], ucount.max()]).tolist()) \
-        if tiles > 0 else (0, 0)
+    total, umax, nnz = (int(v) for v in torch.stack(
+        [uptr[-1], ucount.max(), (table >= 0).sum().int()]).tolist()) if tiles > 0 else (0, 0, 0)
+    # how often a staged row is used by its tile: near 1 there is nothing to gain from staging
+    self.reuse = nnz / max(total, 1)
     self.uptr = uptr
     self.urows = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
     # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"

@@ -326,6 +326,7 @@ def test_staged_kernel_many_passes(dtype):
   tg = table.to(DEV)
   plan = TilePlan(tg)
   assert int((plan.uptr[1:] - plan.uptr[:-1]).max()) > 320
+  plan.reuse = 10.0          # a random table has no reuse; make the layer above take the staged kernel anyway
   got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), cout, False, False, b.to(DEV), plan)
   want = C.forward_gemm(f64(x), f64(w), table.numpy().astype(np.int64)) + f64(b)
   assert rel_err(got, want) < TOL[dtype]
@@ -431,3 +432,26 @@ def test_planned_kernels_fall_back_on_large_tiles():
   assert rel_err(out, C.forward_gemm(f64(x), f64(w), t64)) < 2e-2
   gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
   assert rel_err(gw, C.weight_gemm(f64(x), f64(gr), t64)) < 2e-2
+
+
+def test_dwconv_all_slot_kernels(medium):
+  """Depth-wise kernels that keep all slots of a row in one thread (power-of-two channel
+  counts), every slot count, fp32 and 16-bit, against the oracle."""
+  for dtype in (torch.float32, torch.float16, torch.bfloat16):
+    for ks, stride, ne, C, depth in [([3], 1, False, 32, 6), ([3], 1, True, 64, 7), ([2], 2, False, 16, 7),
+                                     ([2], 2, True, 8, 6), ([3, 1, 3], 1, False, 128, 5),
+                                     ([1, 1, 3], 1, True, 4, 6)]:
+      say('dwconv', dtype, ks, stride, ne, C, depth)
+      errs = run_layer('dwconv', medium, depth, ks, stride, ne, C, C, dtype)
+      assert max(errs.values()) < TOL[dtype], (dtype, ks, stride, ne, C, errs)
+
+
+def test_pad_depad_wide_rows(small):
+  """16-byte-per-thread pad / depad (row size a multiple of 16 bytes)."""
+  d = 5
+  for dt, ch in ((torch.float32, 8), (torch.float16, 64), (torch.bfloat16, 24)):
+    x = torch.randn(int(small.ref.nnum_nempty[d]), ch).to(dt).to(DEV)
+    p = octree_pad(x, small.gpu, d, val=-2.5)
+    assert np.array_equal(f64(p), C.octree_pad(f64(x), small.ref, d, -2.5))
+    y = torch.randn(int(small.ref.nnum[d]), ch).to(dt).to(DEV)
+    assert np.array_equal(f64(octree_depad(y, small.gpu, d)), C.octree_depad(f64(y), small.ref, d))
