@@ -7,47 +7,69 @@ namespace ocnn {
 
 constexpr int kPlanRows = 128;          // table rows per tile
 constexpr int kPlanMaxEntries = 4096;   // >= kPlanRows * 27, power of two
+constexpr int kPlanHash = 8192;         // open-addressing slots (load <= 42 %)
+constexpr int kPlanRankMax = 1024;      // up to here the distinct rows are ordered by counting
+
+__device__ __forceinline__ int plan_hash(int32_t v) {
+  return (int)(((uint32_t)v * 2654435761u) >> 19);      // 13 bits
+}
 
 // mode 0: ucount[tile] = number of distinct valid entries
 // mode 1: urows[uptr[tile] + u] = u-th distinct row; loc[tile][k][row in tile] = u + 1, or
 //         0 for an empty entry (also for the rows of the last tile that lie past the table)
+//
+// The distinct rows are found with a hash set in LDS (a tile of an octree table has a few
+// hundred distinct rows among its 3456 entries), ordered by counting (no barriers) or, for
+// tables without locality, by a bitonic sort; positions come back out of the hash set.
 __global__ __launch_bounds__(256) void tile_plan_kernel(
-    const int32_t* __restrict__ table, int64_t rows, int K, int npad, int mode,
+    const int32_t* __restrict__ table, int64_t rows, int K, int mode,
     int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, int32_t* __restrict__ urows,
     uint16_t* __restrict__ loc) {
-  __shared__ int32_t s_key[kPlanMaxEntries];
-  __shared__ int32_t s_uq[kPlanMaxEntries];
+  __shared__ int32_t s_key[kPlanHash];
+  __shared__ uint16_t s_val[kPlanHash];
+  __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];
   __shared__ int32_t s_scan[256];
+  __shared__ int32_t s_tab[kPlanRows * 27];
   const int tid = threadIdx.x;
   const int64_t tile = blockIdx.x;
   const int64_t e0 = tile * kPlanRows * K;
   const int64_t lim = rows * (int64_t)K;
   const int n = kPlanRows * K;
-  for (int e = tid; e < npad; e += 256) {
-    int32_t v = (e < n && e0 + e < lim) ? table[e0 + e] : -1;
-    s_key[e] = v < 0 ? 0x7fffffff : v;
+  // the tile's entries -> LDS: all loads in flight at once, then used twice
+  constexpr int kPer = (kPlanRows * 27 + 255) / 256;      // entries per thread, at most
+  int32_t ent[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int e = tid + 256 * i;
+    ent[i] = (e < n && e0 + e < lim) ? table[e0 + e] : -1;
   }
+  for (int i = tid; i < kPlanHash; i += 256) s_key[i] = -1;
+#pragma unroll
+  for (int i = 0; i < kPer; ++i)
+    if (tid + 256 * i < n) s_tab[tid + 256 * i] = ent[i];
   __syncthreads();
-  // bitonic sort, ascending
-  for (int k = 2; k <= npad; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int t = tid; t < (npad >> 1); t += 256) {
-        int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-        int p = i | j;
-        int32_t a = s_key[i], b = s_key[p];
-        bool up = (i & k) == 0;
-        if ((a > b) == up) { s_key[i] = b; s_key[p] = a; }
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int32_t v = ent[i];
+    if (v >= 0) {
+      int h = plan_hash(v);
+      while (true) {
+        const int32_t old = atomicCAS(&s_key[h], -1, v);
+        if (old == -1 || old == v) break;
+        h = (h + 1) & (kPlanHash - 1);
       }
-      __syncthreads();
     }
   }
-  // distinct values: head flags, block scan over per-thread counts
-  const int per = npad / 256;           // npad is a multiple of 256
-  const int b0 = tid * per;
+  __syncthreads();
+  // occupied slots: per-thread counts (slots tid, tid + 256, ..: the order of the distinct
+  // rows does not matter before they are ranked), block scan
+  constexpr int per = kPlanHash / 256;
+  int32_t held[per];
   int cnt = 0;
-  for (int e = b0; e < b0 + per; ++e) {
-    int32_t v = s_key[e];
-    cnt += (v != 0x7fffffff && (e == 0 || s_key[e - 1] != v)) ? 1 : 0;
+#pragma unroll
+  for (int i = 0; i < per; ++i) {
+    held[i] = s_key[tid + 256 * i];
+    cnt += held[i] >= 0 ? 1 : 0;
   }
   s_scan[tid] = cnt;
   __syncthreads();
@@ -63,25 +85,89 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
     return;
   }
   int pos = s_scan[tid] - cnt;
-  for (int e = b0; e < b0 + per; ++e) {
-    int32_t v = s_key[e];
-    if (v != 0x7fffffff && (e == 0 || s_key[e - 1] != v)) s_uq[pos++] = v;
-  }
+#pragma unroll
+  for (int i = 0; i < per; ++i)
+    if (held[i] >= 0) s_uq[pos++] = held[i];
   __syncthreads();
   const int32_t ub = uptr[tile];
-  for (int u = tid; u < total; u += 256) urows[ub + u] = s_uq[u];
-  for (int e = tid; e < n; e += 256) {
-    int32_t v = e0 + e < lim ? table[e0 + e] : -1;
-    uint16_t r = 0;
-    if (v >= 0) {
-      int lo = 0, hi = total - 1;
-      while (lo < hi) {
-        int mid = (lo + hi) >> 1;
-        if (s_uq[mid] < v) lo = mid + 1; else hi = mid;
+  auto slot_of = [&](int32_t v) {
+    int h = plan_hash(v);
+    while (s_key[h] != v) h = (h + 1) & (kPlanHash - 1);
+    return h;
+  };
+  if (total <= kPlanRankMax) {
+    // rank of a value = number of smaller distinct values
+    const int tpad = (total + 15) & ~15;                  // whole groups of 16; the padding ranks last
+    for (int e = total + tid; e < tpad; e += 256) s_uq[e] = 0x7fffffff;
+    __syncthreads();
+    typedef __attribute__((ext_vector_type(4))) int i32x4;
+    for (int j = tid; j < total; j += 256) {
+      const int32_t v = s_uq[j];
+      int r = 0;
+      for (int i = 0; i < tpad; i += 16) {                // 4 x 16-byte broadcast reads in flight
+        i32x4 q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) q[u] = *(const i32x4*)(&s_uq[i + 4 * u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          r += (q[u][0] < v ? 1 : 0) + (q[u][1] < v ? 1 : 0) + (q[u][2] < v ? 1 : 0) + (q[u][3] < v ? 1 : 0);
       }
-      r = (uint16_t)(lo + 1);
+      s_val[slot_of(v)] = (uint16_t)(r + 1);
+      urows[ub + r] = v;
     }
-    loc[e0 + (int64_t)(e % K) * kPlanRows + e / K] = r;
+  } else {
+    int npad = kPlanRankMax * 2;
+    while (npad < total) npad <<= 1;
+    for (int e = total + tid; e < npad; e += 256) s_uq[e] = 0x7fffffff;
+    __syncthreads();
+    for (int k = 2; k <= npad; k <<= 1) {          // bitonic sort, ascending
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        for (int t = tid; t < (npad >> 1); t += 256) {
+          int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+          int p = i | j;
+          int32_t a = s_uq[i], b = s_uq[p];
+          bool up = (i & k) == 0;
+          if ((a > b) == up) { s_uq[i] = b; s_uq[p] = a; }
+        }
+        __syncthreads();
+      }
+    }
+    for (int j = tid; j < total; j += 256) {
+      const int32_t v = s_uq[j];
+      s_val[slot_of(v)] = (uint16_t)(j + 1);
+      urows[ub + j] = v;
+    }
+  }
+  __syncthreads();
+  // positions, written in the order they are stored ([slot][row]: coalesced); the first
+  // probes of all entries of a thread are in flight together
+  int32_t vv[kPer], kk[kPer];
+  int hh[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int o = tid + 256 * i;
+    vv[i] = o < n ? s_tab[(o % kPlanRows) * K + o / kPlanRows] : -1;
+  }
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    hh[i] = plan_hash(vv[i] < 0 ? 0 : vv[i]);
+    kk[i] = s_key[hh[i]];
+  }
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    if (vv[i] >= 0)
+      while (kk[i] != vv[i]) {
+        hh[i] = (hh[i] + 1) & (kPlanHash - 1);
+        kk[i] = s_key[hh[i]];
+      }
+  }
+  uint16_t pp[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) pp[i] = s_val[hh[i]];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int o = tid + 256 * i;
+    if (o < n) loc[e0 + o] = vv[i] >= 0 ? pp[i] : (uint16_t)0;
   }
 }
 
@@ -95,11 +181,9 @@ static int plan_launch(const int32_t* table, int64_t rows, int K, int mode, int3
                        const int32_t* uptr, int32_t* urows, uint16_t* loc, void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows >= 0 && rows < (1ll << 31), "tile_plan: bad shape");
   if (rows == 0) return OCNN_OK;
-  int npad = 256;
-  while (npad < kPlanRows * K) npad <<= 1;
   int64_t tiles = cdiv(rows, kPlanRows);
   hipLaunchKernelGGL(tile_plan_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream,
-                     table, rows, K, npad, mode, ucount, uptr, urows, loc);
+                     table, rows, K, mode, ucount, uptr, urows, loc);
   return check_launch("tile_plan");
 }
 
