@@ -159,6 +159,11 @@ int ocnn_table_transpose(const int32_t* table, int64_t rows, int K,
  * bias may be NULL.  Rows of `in` are addressed by table values only.
  * workspace: ocnn_conv_workspace_bytes(K, cin, cout) bytes (packed weights). */
 int64_t ocnn_conv_workspace_bytes(int K, int cin, int cout);
+/* Workspace of ocnn_conv_gather including, for fp32 with cin % 32 == 0 and cout % 16 == 0,
+ * the room to run on the bf16 MFMA kernel as three bf16 pieces ([hi | hi | lo] input channels
+ * against [hi; lo; hi] weights, fp32 accumulation and output, about 1e-5 relative).  With
+ * only ocnn_conv_workspace_bytes() of room fp32 runs on the plain kernel. */
+int64_t ocnn_conv_gather_workspace_bytes(int dtype, int64_t rows_in, int K, int cin, int cout);
 int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
                      const int32_t* table, int64_t rows_out, int K,
                      const void* w, int cin, int cout, int w_transposed,
@@ -218,6 +223,11 @@ void ocnn_set_wgrad_transpose_load(int on);
  * gw: (K, ca, cb) in `dtype`, or (K, cb, ca) when out_transposed != 0 (the
  * deconvolution's weight layout, ocnn/nn/octree_conv.py:287-290). */
 int64_t ocnn_conv_wgrad_workspace_bytes(int64_t rows, int K, int ca, int cb);
+/* The same with the room an fp32 layer needs to run on the MFMA kernels as three bf16
+ * pieces (hi/lo split of both operands, about 1e-5 relative; without that room fp32 runs on
+ * the plain kernel). */
+int64_t ocnn_conv_wgrad_workspace_bytes_for(int dtype, int64_t rows_x, int64_t rows, int K,
+                                            int ca, int cb);
 int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
                     const int32_t* table, int64_t rows, int K, int ca, int cb,
                     int out_transposed, void* gw, void* workspace,

@@ -37,6 +37,7 @@ SIGNATURES = {
     'ocnn_table_to_i32': (_i, [_p, _l, _p, _p]),
     'ocnn_table_transpose': (_i, [_p, _l, _i, _l, _p, _p]),
     'ocnn_conv_workspace_bytes': (_l, [_i, _i, _i]),
+    'ocnn_conv_gather_workspace_bytes': (_l, [_i, _l, _i, _i, _i]),
     'ocnn_conv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _i, _i, _p, _p, _p, _l, _p]),
     'ocnn_tile_plan_rows': (_i, []),
     'ocnn_tile_plan_count': (_i, [_p, _l, _i, _p, _p]),
@@ -49,6 +50,7 @@ SIGNATURES = {
                                  _p, _l, _p]),
     'ocnn_set_wgrad_transpose_load': (None, [_i]),
     'ocnn_conv_wgrad_workspace_bytes': (_l, [_l, _i, _i, _i]),
+    'ocnn_conv_wgrad_workspace_bytes_for': (_l, [_i, _l, _l, _i, _i, _i]),
     'ocnn_conv_wgrad': (_i, [_i, _p, _l, _p, _p, _l, _i, _i, _i, _i, _p, _p, _l, _p]),
     'ocnn_conv_wgrad_planned_supported': (_i, [_i, _l, _l, _i, _i, _i, _i]),
     'ocnn_conv_wgrad_planned_workspace_bytes': (_l, [_i]),

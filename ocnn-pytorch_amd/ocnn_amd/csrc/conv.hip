@@ -50,10 +50,11 @@ __global__ void pack_weights_kernel(const T* __restrict__ w, T* __restrict__ out
 // One workgroup (4 waves) owns 4*NT*16 output rows and 16*MT output channels.
 // Output rows are the N dimension of the MFMA, output channels the M dimension,
 // so that a lane ends up with 4*MT consecutive channels of one row.
-template <typename T, int CB, int MT, int NT>
+// O is the output (and bias) type: T, or float when the operands are bf16 pieces of fp32 data.
+template <typename T, typename O, int CB, int MT, int NT>
 __global__ __launch_bounds__(256) void conv_gather_mfma_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const int32_t* __restrict__ table,
-    const T* __restrict__ wpk, const T* __restrict__ bias, T* __restrict__ out,
+    const T* __restrict__ wpk, const O* __restrict__ bias, O* __restrict__ out,
     int64_t rows_out, int K, int cin, int cout, int64_t tiles, int64_t tiles_per_xcd) {
   constexpr int KS = CB / 32;
   constexpr int ROWS = 4 * NT * 16;
@@ -166,21 +167,84 @@ __global__ __launch_bounds__(256) void conv_gather_mfma_kernel(
   for (int n = 0; n < NT; ++n) {
     int64_t row = row0 + lrow + n * 16;
     if (row >= rows_out) continue;
-    unsigned pk[2 * MT];
+    O* dst = out + row * cout + co0;
+    if constexpr (std::is_same<O, float>::value) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      pk[2 * t + 0] = pack2<T>(acc[t][n][0] + bv[4 * t + 0], acc[t][n][1] + bv[4 * t + 1]);
-      pk[2 * t + 1] = pack2<T>(acc[t][n][2] + bv[4 * t + 2], acc[t][n][3] + bv[4 * t + 3]);
-    }
-    T* dst = out + row * cout + co0;
-    if constexpr (MT >= 2) {
-#pragma unroll
-      for (int c = 0; c < 2 * MT; c += 4)
-        *(u32x4*)(dst + 2 * c) = u32x4{pk[c], pk[c + 1], pk[c + 2], pk[c + 3]};
+      for (int t = 0; t < MT; ++t)
+        *(f32x4*)(dst + 4 * t) = f32x4{acc[t][n][0] + bv[4 * t + 0], acc[t][n][1] + bv[4 * t + 1],
+                                       acc[t][n][2] + bv[4 * t + 2], acc[t][n][3] + bv[4 * t + 3]};
     } else {
-      *(u32x2*)(dst) = u32x2{pk[0], pk[1]};
+      unsigned pk[2 * MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        pk[2 * t + 0] = pack2<T>(acc[t][n][0] + bv[4 * t + 0], acc[t][n][1] + bv[4 * t + 1]);
+        pk[2 * t + 1] = pack2<T>(acc[t][n][2] + bv[4 * t + 2], acc[t][n][3] + bv[4 * t + 3]);
+      }
+      if constexpr (MT >= 2) {
+#pragma unroll
+        for (int c = 0; c < 2 * MT; c += 4)
+          *(u32x4*)(dst + 2 * c) = u32x4{pk[c], pk[c + 1], pk[c + 2], pk[c + 3]};
+      } else {
+        *(u32x2*)(dst) = u32x2{pk[0], pk[1]};
+      }
     }
   }
+}
+
+// fp32 data as three bf16 pieces: x = hi + lo (+ 2^-17 |x|), and
+// x * w = hi_x hi_w + hi_x lo_w + lo_x hi_w (+ 3 * 2^-18 |x w|), so a bf16 MFMA over the
+// input channels [hi | hi | lo] against the weights [hi; lo; hi] accumulates, in fp32,
+// the fp32 product to about 1e-5 relative.
+__global__ void split3_rows_kernel(const float* __restrict__ x, int64_t n, int cin,
+                                   bf16* __restrict__ out) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n * cin) return;
+  int64_t r = e / cin;
+  int c = (int)(e % cin);
+  float v = x[e];
+  bf16 hi = (bf16)v;
+  bf16 lo = (bf16)(v - (float)hi);
+  bf16* o = out + r * 3 * cin;
+  o[c] = hi;
+  o[cin + c] = hi;
+  o[2 * cin + c] = lo;
+}
+
+// (K, cin, cout) -> (K, 3 cin, cout) rows [hi; lo; hi]; stored transposed (K, cout, cin) ->
+// (K, cout, 3 cin) columns [hi | lo | hi]
+__global__ void split3_weights_kernel(const float* __restrict__ w, int K, int cin, int cout,
+                                      int transposed, bf16* __restrict__ out) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (int64_t)K * cin * cout) return;
+  float v = w[e];
+  bf16 hi = (bf16)v;
+  bf16 lo = (bf16)(v - (float)hi);
+  if (transposed) {
+    int ci = (int)(e % cin);
+    int64_t kc = e / cin;                        // k * cout + co
+    bf16* o = out + kc * 3 * cin;
+    o[ci] = hi;
+    o[cin + ci] = lo;
+    o[2 * cin + ci] = hi;
+  } else {
+    int co = (int)(e % cout);
+    int ci = (int)((e / cout) % cin);
+    int64_t k = e / ((int64_t)cin * cout);
+    bf16* o = out + k * 3 * cin * cout + co;
+    o[(int64_t)ci * cout] = hi;
+    o[(int64_t)(cin + ci) * cout] = lo;
+    o[(int64_t)(2 * cin + ci) * cout] = hi;
+  }
+}
+
+__global__ void split2_kernel(const float* __restrict__ x, int64_t n, bf16* __restrict__ hi,
+                              bf16* __restrict__ lo) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n) return;
+  float v = x[e];
+  bf16 h = (bf16)v;
+  hi[e] = h;
+  lo[e] = (bf16)(v - (float)h);
 }
 
 // --------------------------------------------------------------------------
@@ -427,7 +491,7 @@ static GatherPlan plan_gather(int dtype, int64_t rows_in, int64_t rows_out, int 
   return p;
 }
 
-template <typename T, int CB, int MT, int NT>
+template <typename T, typename O, int CB, int MT, int NT>
 static void launch_gather(const GatherPlan&, const void* in, int64_t rows_in, const int32_t* table,
                           int64_t rows_out, int K, int cin, int cout, const void* wpk,
                           const void* bias, void* out, hipStream_t st) {
@@ -435,12 +499,12 @@ static void launch_gather(const GatherPlan&, const void* in, int64_t rows_in, co
   int64_t tiles = cdiv(rows_out, ROWS);
   int64_t per_xcd = cdiv(tiles, 8);
   dim3 grid((unsigned)(per_xcd * 8), (unsigned)(cout / (16 * MT)));
-  hipLaunchKernelGGL((conv_gather_mfma_kernel<T, CB, MT, NT>), grid, dim3(256), 0, st,
+  hipLaunchKernelGGL((conv_gather_mfma_kernel<T, O, CB, MT, NT>), grid, dim3(256), 0, st,
                      (const T*)in, (uint32_t)(rows_in * cin * sizeof(T)), table, (const T*)wpk,
-                     (const T*)bias, (T*)out, rows_out, K, cin, cout, tiles, per_xcd);
+                     (const O*)bias, (O*)out, rows_out, K, cin, cout, tiles, per_xcd);
 }
 
-template <typename T>
+template <typename T, typename O = T>
 static int run_gather_mfma(const GatherPlan& p, const void* in, int64_t rows_in,
                            const int32_t* table, int64_t rows_out, int K, const void* w, int cin,
                            int cout, int w_transposed, int reverse, const void* bias, void* out,
@@ -450,7 +514,7 @@ static int run_gather_mfma(const GatherPlan& p, const void* in, int64_t rows_in,
                      (const T*)w, (T*)ws, K, cin, cout, p.CB, p.MT, w_transposed, reverse);
 #define OCNN_GATHER_CASE(cb_, mt_, nt_)                                                        \
   if (p.CB == cb_ && p.MT == mt_ && p.NT == nt_) {                                             \
-    launch_gather<T, cb_, mt_, nt_>(p, in, rows_in, table, rows_out, K, cin, cout, ws, bias,   \
+    launch_gather<T, O, cb_, mt_, nt_>(p, in, rows_in, table, rows_out, K, cin, cout, ws, bias,   \
                                     out, st);                                                  \
     return check_launch("conv_gather_mfma");                                                   \
   }
@@ -517,6 +581,21 @@ extern "C" int64_t ocnn_conv_workspace_bytes(int K, int cin, int cout) {
   return align_up((int64_t)K * cin * cout * 4, 256);
 }
 
+// room for the bf16 pieces of an fp32 layer: packed weights, split weights, split rows;
+// 0 when the shape cannot take that path
+static int64_t f32_gather_workspace(int64_t rows_in, int K, int cin, int cout) {
+  if (cin % 32 != 0 || cout % 16 != 0) return 0;
+  if ((int64_t)rows_in * 3 * cin * 2 > 0xfffff000ll - (int64_t)3 * cin * 2) return 0;
+  return 2 * align_up((int64_t)K * 3 * cin * cout * 2, 256) + align_up(rows_in * 3 * cin * 2, 256);
+}
+
+extern "C" int64_t ocnn_conv_gather_workspace_bytes(int dtype, int64_t rows_in, int K, int cin,
+                                                    int cout) {
+  int64_t base = ocnn_conv_workspace_bytes(K, cin, cout);
+  if (dtype == OCNN_F32) base = std::max(base, f32_gather_workspace(rows_in, K, cin, cout));
+  return base;
+}
+
 extern "C" int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in, const int32_t* table,
                                 int64_t rows_out, int K, const void* w, int cin, int cout,
                                 int w_transposed, int reverse_slots, const void* bias, void* out,
@@ -540,9 +619,26 @@ extern "C" int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in, cons
     return run_gather_mfma<bf16>(p, in, rows_in, table, rows_out, K, w, cin, cout, w_transposed,
                                  reverse_slots, bias, out, workspace, st);
   }
-  if (dtype == OCNN_F32)
+  if (dtype == OCNN_F32) {
+    // bf16 pieces on the MFMA kernel when the shape allows and the caller brought the room
+    // (ocnn_conv_gather_workspace_bytes); else the plain kernel
+    const int64_t need = f32_gather_workspace(rows_in, K, cin, cout);
+    GatherPlan p3 = plan_gather(OCNN_BF16, rows_in, rows_out, 3 * cin, cout);
+    if (p3.mfma && need > 0 && workspace_bytes >= need && rows_in > 0) {
+      const int64_t wbytes = align_up((int64_t)K * 3 * cin * cout * 2, 256);
+      bf16* wpk = (bf16*)workspace;
+      bf16* wsp = (bf16*)((char*)workspace + wbytes);
+      bf16* xs = (bf16*)((char*)workspace + 2 * wbytes);
+      hipLaunchKernelGGL(split3_rows_kernel, dim3((unsigned)cdiv(rows_in * cin, 256)), dim3(256), 0, st,
+                         (const float*)in, rows_in, cin, xs);
+      hipLaunchKernelGGL(split3_weights_kernel, dim3((unsigned)cdiv((int64_t)K * cin * cout, 256)),
+                         dim3(256), 0, st, (const float*)w, K, cin, cout, w_transposed, wsp);
+      return run_gather_mfma<bf16, float>(p3, xs, rows_in, table, rows_out, K, wsp, 3 * cin, cout,
+                                          w_transposed, reverse_slots, bias, out, wpk, st);
+    }
     return run_gather_plain<float>(in, rows_in, table, rows_out, K, w, cin, cout, w_transposed,
                                    reverse_slots, bias, out, st);
+  }
   if (dtype == OCNN_F16)
     return run_gather_plain<f16>(in, rows_in, table, rows_out, K, w, cin, cout, w_transposed,
                                  reverse_slots, bias, out, st);
@@ -594,6 +690,57 @@ static int run_wgrad(int dtype, const void* x, int64_t rows_x, const void* g, co
   return check_launch("conv_wgrad");
 }
 
+// fp32 weight gradient through bf16 pieces: three passes of the MFMA kernel
+// (hi_x hi_g, hi_x lo_g, lo_x hi_g) into three sets of partial sums, one reduction
+static int64_t f32_wgrad_workspace(int64_t rows_x, int64_t rows, int K, int ca, int cb) {
+  if (ca % 32 != 0 || cb % 32 != 0) return 0;
+  if ((int64_t)rows_x * ca * 2 >= 0xffff0000ll || (int64_t)rows * cb * 2 >= 0xffff0000ll) return 0;
+  WgradPlan p = plan_wgrad(OCNN_BF16, rows_x, rows, K, ca, cb);
+  return 2 * align_up(rows_x * ca * 2, 256) + 2 * align_up(rows * cb * 2, 256) +
+         align_up((int64_t)3 * p.splits * K * ca * cb * 4, 256);
+}
+
+static int run_wgrad_f32_split(const void* x, int64_t rows_x, const void* g, const int32_t* table,
+                               int64_t rows, int K, int ca, int cb, int out_transposed, void* gw,
+                               void* ws, hipStream_t st) {
+  WgradPlan p = plan_wgrad(OCNN_BF16, rows_x, rows, K, ca, cb);
+  const int64_t xb = align_up(rows_x * ca * 2, 256), gb = align_up(rows * cb * 2, 256);
+  bf16* xh = (bf16*)ws;
+  bf16* xl = (bf16*)((char*)ws + xb);
+  bf16* gh = (bf16*)((char*)ws + 2 * xb);
+  bf16* gl = (bf16*)((char*)ws + 2 * xb + gb);
+  float* partial = (float*)((char*)ws + 2 * xb + 2 * gb);
+  hipLaunchKernelGGL(split2_kernel, dim3((unsigned)cdiv(rows_x * ca, 256)), dim3(256), 0, st,
+                     (const float*)x, rows_x * ca, xh, xl);
+  hipLaunchKernelGGL(split2_kernel, dim3((unsigned)cdiv(rows * cb, 256)), dim3(256), 0, st,
+                     (const float*)g, rows * cb, gh, gl);
+  constexpr int KG = kWgradSlots;
+  dim3 grid(p.splits, (unsigned)(cdiv(K, KG) * (ca / p.TILE)), (unsigned)(cb / p.TILE));
+  const uint32_t xbytes = (uint32_t)(rows_x * ca * 2), gbytes = (uint32_t)(rows * cb * 2);
+  const int64_t pstride = (int64_t)p.splits * K * ca * cb;
+  const bf16* xs[3] = {xh, xh, xl};
+  const bf16* gs[3] = {gh, gl, gh};
+  for (int i = 0; i < 3; ++i) {
+    if (p.TILE == 64)
+      hipLaunchKernelGGL((conv_wgrad_mfma_kernel<bf16, 64, KG, true>), grid, dim3(256), 0, st, xs[i], xbytes,
+                         gs[i], gbytes, table, rows, K, ca, cb, p.rows_per_split, partial + i * pstride);
+    else
+      hipLaunchKernelGGL((conv_wgrad_mfma_kernel<bf16, 32, KG, true>), grid, dim3(256), 0, st, xs[i], xbytes,
+                         gs[i], gbytes, table, rows, K, ca, cb, p.rows_per_split, partial + i * pstride);
+  }
+  int64_t per = (int64_t)K * ca * cb;
+  hipLaunchKernelGGL(wgrad_reduce_kernel<float>, dim3(cdiv(per, 256)), dim3(256), 0, st, partial,
+                     3 * p.splits, K, ca, cb, out_transposed, (float*)gw);
+  return check_launch("conv_wgrad (bf16 pieces)");
+}
+
+extern "C" int64_t ocnn_conv_wgrad_workspace_bytes_for(int dtype, int64_t rows_x, int64_t rows, int K,
+                                                       int ca, int cb) {
+  int64_t base = ocnn_conv_wgrad_workspace_bytes(rows, K, ca, cb);
+  if (dtype == OCNN_F32) base = std::max(base, f32_wgrad_workspace(rows_x, rows, K, ca, cb));
+  return base;
+}
+
 extern "C" int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
                                const int32_t* table, int64_t rows, int K, int ca, int cb,
                                int out_transposed, void* gw, void* workspace,
@@ -603,9 +750,13 @@ extern "C" int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const v
   OCNN_REQUIRE(rows >= 0 && rows < (1ll << 31) && rows_x >= 0 && rows_x < (1ll << 31),
                "conv_wgrad: rows out of range");
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == OCNN_F32)
+  if (dtype == OCNN_F32) {
+    const int64_t need = f32_wgrad_workspace(rows_x, rows, K, ca, cb);
+    if (need > 0 && workspace_bytes >= need && rows > 0 && rows_x > 0)
+      return run_wgrad_f32_split(x, rows_x, g, table, rows, K, ca, cb, out_transposed, gw, workspace, st);
     return run_wgrad<float>(dtype, x, rows_x, g, table, rows, K, ca, cb, out_transposed, gw,
                             workspace, workspace_bytes, st);
+  }
   if (dtype == OCNN_F16)
     return run_wgrad<f16>(dtype, x, rows_x, g, table, rows, K, ca, cb, out_transposed, gw,
                           workspace, workspace_bytes, st);

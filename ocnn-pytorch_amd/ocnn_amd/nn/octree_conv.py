@@ -35,9 +35,9 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   if bias is not None:
     bias = bias.to(data.dtype).contiguous()
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
-  nbytes = L.ocnn_conv_workspace_bytes(K, cin, cout)
-  ws = _lib.workspace(nbytes, data.device)
   code = _lib.dtype_code(data)
+  nbytes = L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout)
+  ws = _lib.workspace(nbytes, data.device)
   if plan is not None and L.ocnn_conv_gather_rw_supported(code, rows_in, K, cin, cout, plan.umax):
     _lib.check(L.ocnn_conv_gather_rw(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
@@ -78,7 +78,8 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None):
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, ca, cb, int(out_transposed),
         _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw
-  ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes(rows, K, ca, cb), x.device)
+  ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes_for(_lib.dtype_code(x), x.shape[0], rows, K,
+                                                            ca, cb), x.device)
   _lib.check(L.ocnn_conv_wgrad(
       _lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
       int(out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))

@@ -177,6 +177,15 @@ def test_fp32_larger(medium):
   assert max(errs.values()) < TOL[torch.float32], errs
   errs = run_layer('conv', medium, 6, [3], 1, True, 32, 32, torch.float32)
   assert max(errs.values()) < TOL[torch.float32], errs
+  # fp32 on the MFMA kernels as bf16 pieces: every layer kind and table form, still 1e-4
+  for kind, depth, ks, stride, ne, cin, cout in [
+      ('conv', 7, [3], 1, False, 64, 64), ('conv', 7, [2], 2, False, 64, 128),
+      ('conv', 7, [2], 2, True, 32, 64), ('deconv', 6, [2], 2, False, 128, 64),
+      ('deconv', 6, [3], 1, True, 32, 32), ('conv', 6, [3], 2, False, 32, 48),
+      ('conv', 6, [3, 1, 3], 1, False, 64, 32)]:
+    say('fp32 via bf16 pieces', kind, depth, ks, stride, ne, cin, cout)
+    errs = run_layer(kind, medium, depth, ks, stride, ne, cin, cout, torch.float32)
+    assert max(errs.values()) < TOL[torch.float32], (kind, ks, stride, ne, cin, cout, errs)
 
 
 def test_mixed_precision_and_no_bias(small):
