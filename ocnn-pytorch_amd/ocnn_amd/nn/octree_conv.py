@@ -14,12 +14,16 @@ the inverse table otherwise, so no atomics are involved anywhere.
 from typing import List
 
 import torch
+import torch.nn.functional as F
 import torch.nn
 from torch.autograd import Function
 
 from .. import _lib
 from ..utils import list2str, resize_with_last_val, xavier_uniform_
 from .octree_pad import octree_depad, octree_pad
+
+
+PAD_MIN_ROWS = 16384     # from this many table rows on, odd channel counts are zero-padded
 
 
 def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None):
@@ -34,6 +38,15 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   assert W.numel() == K * cin * cout, 'weights do not match the table and channels'
   if bias is not None:
     bias = bias.to(data.dtype).contiguous()
+  # channel counts the MFMA kernels do not take (cin % 32, cout % 16) are padded with zeros
+  # when the layer is large enough for that to beat the plain kernel
+  if rows >= PAD_MIN_ROWS and (cin % 32 or cout % 16) and data.dtype in _lib.DTYPE_CODE:
+    cin_p, cout_p = -(-cin // 32) * 32, -(-cout // 16) * 16
+    Wk = W.view(K, cout, cin) if transposed else W.view(K, cin, cout)
+    pad_w = (0, cin_p - cin, 0, cout_p - cout) if transposed else (0, cout_p - cout, 0, cin_p - cin)
+    out = conv_gather(F.pad(data, (0, cin_p - cin)), rows_in, table, F.pad(Wk, pad_w), cout_p,
+                      transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), None)
+    return out[:, :cout].contiguous()
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
   code = _lib.dtype_code(data)
   nbytes = L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout)
@@ -67,6 +80,10 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None):
   rows, K = table.shape
   ca, cb = x.shape[1], g.shape[1]
   assert g.shape[0] == rows and x.dtype == g.dtype and table.dtype == torch.int32
+  if rows >= PAD_MIN_ROWS and (ca % 32 or cb % 32) and x.dtype in _lib.DTYPE_CODE:
+    ca_p, cb_p = -(-ca // 32) * 32, -(-cb // 32) * 32
+    gw = conv_wgrad(F.pad(x, (0, ca_p - ca)), F.pad(g, (0, cb_p - cb)), table, out_transposed, None)
+    return (gw[:, :cb, :ca] if out_transposed else gw[:, :ca, :cb]).contiguous()
   shape = (K, cb, ca) if out_transposed else (K, ca, cb)
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
   code = _lib.DTYPE_CODE.get(x.dtype, -1)

@@ -464,3 +464,18 @@ def test_pad_depad_wide_rows(small):
     assert np.array_equal(f64(p), C.octree_pad(f64(x), small.ref, d, -2.5))
     y = torch.randn(int(small.ref.nnum[d]), ch).to(dt).to(DEV)
     assert np.array_equal(f64(octree_depad(y, small.gpu, d)), C.octree_depad(f64(y), small.ref, d))
+
+
+def test_odd_channels_on_large_layers(medium):
+  """Channel counts the MFMA kernels do not take are zero-padded once the layer is large
+  (first and last layers of a network: 4 -> 32, 32 -> 10 ...)."""
+  conv_mod = sys.modules['ocnn_amd.nn.octree_conv']
+  assert rows_of(medium.ref, 7, False) >= conv_mod.PAD_MIN_ROWS
+  for dtype in (torch.float32, torch.bfloat16):
+    for kind, ks, stride, ne, cin, cout in [('conv', [3], 1, False, 4, 32), ('conv', [3], 1, False, 32, 10),
+                                            ('conv', [2], 2, False, 5, 7), ('deconv', [2], 2, False, 12, 6),
+                                            ('conv', [3], 1, True, 3, 3)]:
+      depth = 6 if kind == 'deconv' else 7
+      say('padded channels', dtype, kind, ks, stride, ne, cin, cout)
+      errs = run_layer(kind, medium, depth, ks, stride, ne, cin, cout, dtype)
+      assert max(errs.values()) < TOL[dtype], (dtype, kind, ks, stride, ne, cin, cout, errs)
