@@ -685,8 +685,8 @@ static int run_wgrad(int dtype, const void* x, int64_t rows_x, const void* g, co
                        (const T*)g, table, rows, K, ca, cb, p.rows_per_split, partial);
   }
   int64_t per = (int64_t)K * ca * cb;
-  hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3(cdiv(per, 256)), dim3(256), 0, st, partial,
-                     p.splits, K, ca, cb, out_transposed, (T*)gw);
+  (void)per;
+  launch_wgrad_reduce<T>(partial, p.splits, K, ca, cb, out_transposed, (T*)gw, st);
   return check_launch("conv_wgrad");
 }
 
@@ -729,8 +729,8 @@ static int run_wgrad_f32_split(const void* x, int64_t rows_x, const void* g, con
                          gs[i], gbytes, table, rows, K, ca, cb, p.rows_per_split, partial + i * pstride);
   }
   int64_t per = (int64_t)K * ca * cb;
-  hipLaunchKernelGGL(wgrad_reduce_kernel<float>, dim3(cdiv(per, 256)), dim3(256), 0, st, partial,
-                     3 * p.splits, K, ca, cb, out_transposed, (float*)gw);
+  (void)per;
+  launch_wgrad_reduce<float>(partial, 3 * p.splits, K, ca, cb, out_transposed, (float*)gw, st);
   return check_launch("conv_wgrad (bf16 pieces)");
 }
 

@@ -436,8 +436,7 @@ static int run_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* 
     else if (K == 8) launch_wp<T, 8, 2, 0, 1>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st);
     else launch_wp<T, 3, 1, 0, 1>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st);
   }
-  hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3(cdiv((int64_t)K * 4096, 256)), dim3(256), 0, st, partial,
-                     rows > 0 ? used : 0, K, 64, 64, out_transposed, (T*)gw);
+  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, 64, 64, out_transposed, (T*)gw, st);
   return check_launch("conv_wgrad_planned");
 }
 
