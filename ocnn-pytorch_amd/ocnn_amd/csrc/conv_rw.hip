@@ -257,20 +257,26 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
 
     // The main loop is a flat sequence of steps (unit u, row tile nt).  The B operand of
     // a step (lane: row r32 of the row tile, k group q -> 2 x 16 B of its neighbour row)
-    // is fetched from LDS two steps ahead of its four MFMAs; the table positions of a
-    // unit are read two units ahead.  Units past 2K have zero weights.
+    // is fetched from LDS three steps ahead of its four MFMAs; the table positions of a
+    // unit are read three units ahead.  Units past 2K have zero weights.
     constexpr int STEPS = UPW * 2;
-    uint32_t lcur[2], lnxt[2] = {0u, 0u};
-    u32x4 ring[3][2];
+    uint32_t lcur[2], lnxt[2] = {0u, 0u}, lnx2[2] = {0u, 0u};
+    u32x4 ring[4][2];
     const T *pa, *pb;
     read_loc(0, lcur);
     if (UPW > 1) read_loc(1, lnxt);
+    if (UPW > 2) read_loc(2, lnx2);
     addr(lcur[0], pa, pb);
     ring[0][0] = *(const u32x4*)pa;
     ring[0][1] = *(const u32x4*)pb;
     addr(lcur[1], pa, pb);
     ring[1][0] = *(const u32x4*)pa;
     ring[1][1] = *(const u32x4*)pb;
+    if (UPW > 1) {
+      addr(lnxt[0], pa, pb);
+      ring[2][0] = *(const u32x4*)pa;
+      ring[2][1] = *(const u32x4*)pb;
+    }
     __builtin_amdgcn_sched_barrier(0);
     constexpr int EPS = (26 + STEPS - 1) / STEPS;           // exchange pieces per step
     constexpr int SPS = STEPS >= 28 ? 1 : (kPieces + STEPS - 1) / STEPS + 1;   // staging pieces per step slot
@@ -278,20 +284,23 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
       const int u = j >> 1, nt = j & 1;
-      const bool pre = j + 2 < STEPS;
-      acc[S][nt][0] = Mma32<T>::run(wreg[u][0][0], ring[j % 3][0], acc[S][nt][0]);
-      if (pre) addr(lnxt[nt], pa, pb);                       // step j + 2: unit u + 1, same row tile
-      acc[S][nt][1] = Mma32<T>::run(wreg[u][0][1], ring[j % 3][0], acc[S][nt][1]);
-      if (pre) ring[(j + 2) % 3][0] = *(const u32x4*)pa;
-      acc[S][nt][0] = Mma32<T>::run(wreg[u][1][0], ring[j % 3][1], acc[S][nt][0]);
-      if (pre) ring[(j + 2) % 3][1] = *(const u32x4*)pb;
+      const bool pre = j + 3 < STEPS;
+      const int u3 = (j + 3) >> 1, nt3 = (j + 3) & 1;
+      acc[S][nt][0] = Mma32<T>::run(wreg[u][0][0], ring[j & 3][0], acc[S][nt][0]);
+      if (pre) addr(u3 == u + 1 ? lnxt[nt3] : lnx2[nt3], pa, pb);      // step j + 3
+      acc[S][nt][1] = Mma32<T>::run(wreg[u][0][1], ring[j & 3][0], acc[S][nt][1]);
+      if (pre) ring[(j + 3) & 3][0] = *(const u32x4*)pa;
+      acc[S][nt][0] = Mma32<T>::run(wreg[u][1][0], ring[j & 3][1], acc[S][nt][0]);
+      if (pre) ring[(j + 3) & 3][1] = *(const u32x4*)pb;
       if (nt == 1) {
-        // the next unit becomes current; read the positions of the one two units on
+        // the next unit becomes current; read the positions of the one three units on
         lcur[0] = lnxt[0];
         lcur[1] = lnxt[1];
-        if (u + 2 < UPW) read_loc(u + 2, lnxt);
+        lnxt[0] = lnx2[0];
+        lnxt[1] = lnx2[1];
+        if (u + 3 < UPW) read_loc(u + 3, lnx2);
       }
-      acc[S][nt][1] = Mma32<T>::run(wreg[u][1][1], ring[j % 3][1], acc[S][nt][1]);
+      acc[S][nt][1] = Mma32<T>::run(wreg[u][1][1], ring[j & 3][1], acc[S][nt][1]);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
