@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the gather-GEMM kernel at the default workload (fp16, depth 8,
 # batch 8), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy; None for
 # any other workload.  The summary under profiles/ gives the counter readings.
-TRAFFIC_GATHER_DEFAULT = int((205800 * 2.0 + 235700 * 1.0) * 1024)
+TRAFFIC_GATHER_DEFAULT = int((209100 * 2.0 + 235970 * 1.0) * 1024)
 
 
 def parse():
