@@ -198,8 +198,9 @@ int ocnn_conv_gather_planned(int dtype, const void* in, int64_t rows_in,
                              int reverse_slots, const void* bias, void* out,
                              void* workspace, int64_t workspace_bytes, void* stream);
 
-/* ocnn_conv_gather for 64 -> 64 channels with register-resident weights: one
- * persistent workgroup per CU keeps all K x 64 x 64 weights in VGPRs and walks
+/* ocnn_conv_gather for 64 -> 64 and 32 -> 32 channels with register-resident
+ * weights: one persistent workgroup per CU keeps all K x C x C weights in VGPRs
+ * (split over its four waves at C = 64, whole in every wave at C = 32) and walks
  * its tiles of the plan.  plan_max_distinct = largest number of distinct rows
  * of any tile (max of ucount); the kernel needs it <= 416.  plan_total = number
  * of entries of urows (uptr[tiles]).  Same result as ocnn_conv_gather. */

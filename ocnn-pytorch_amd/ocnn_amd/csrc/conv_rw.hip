@@ -393,6 +393,197 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// 32 -> 32 channels: the weights of all K slots (27 x 32 x 32 x 2 B = 54 KiB) fit the registers
+// of ONE wave, so every wave keeps all of them and finishes its own 32 rows of a tile alone:
+// no split over the slots, no cross-wave sum.  A row is 64 bytes; per slot a lane reads two
+// 16-byte pieces of its neighbour row (the two k steps of 16 input channels) and issues two
+// v_mfma_f32_32x32x16.  LDS reads and MFMAs take the same number of clocks at their peaks
+// (64 flop per input byte at 32 output channels), so this shape is LDS-bound by nature.
+// ---------------------------------------------------------------------------------------
+
+// packed weights: [slot][k step s][lane][8]; input channel = 16 s + 8 (lane / 32) + j,
+// output channel = perm(lane % 32) as above (a lane ends with 16 consecutive output channels)
+template <typename T>
+__global__ void pack_weights_rw32_kernel(const T* __restrict__ w, T* __restrict__ out, int K,
+                                         int transposed, int reverse) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (int64_t)K * 1024) return;
+  int j = (int)(e & 7);
+  int lane = (int)((e >> 3) & 63);
+  int s = (int)((e >> 9) & 1);
+  int k = (int)(e >> 10);
+  int q = lane >> 5, m = lane & 31;
+  int chan = 16 * s + 8 * q + j;
+  int co = 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
+  int kk = reverse ? K - 1 - k : k;
+  out[e] = transposed ? w[((int64_t)kk * 32 + co) * 32 + chan] : w[((int64_t)kk * 32 + chan) * 32 + co];
+}
+
+template <typename T, int KK>
+__global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
+    const T* __restrict__ in, uint32_t in_bytes, const uint16_t* __restrict__ loc,
+    uint32_t loc_bytes, const int32_t* __restrict__ uptr, const int32_t* __restrict__ urows,
+    uint32_t urows_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
+    T* __restrict__ out, int64_t rows_out, int64_t tiles, int64_t tiles_per_wg) {
+  constexpr int kLocElems = (kRwRows * 27 * 2 + 1023) / 1024 * 512;
+  constexpr int kRowsAlloc = (kRwCap + 16) / 16 * 16;            // rows 0..kRwCap, whole 16-row groups
+  __shared__ __attribute__((aligned(16))) T s_rows0[kRowsAlloc * 32];
+  __shared__ __attribute__((aligned(16))) T s_rows1[kRowsAlloc * 32];
+  __shared__ __attribute__((aligned(16))) uint16_t s_loc0[kLocElems];
+  __shared__ __attribute__((aligned(16))) uint16_t s_loc1[kLocElems];
+  __shared__ __attribute__((aligned(16))) int32_t s_u0[4 + 512];
+  __shared__ __attribute__((aligned(16))) int32_t s_u1[4 + 512];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int q = lane >> 5, r32 = lane & 31;
+  const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_wg;
+  const int64_t t_end = min(tiles, t_begin + tiles_per_wg);
+  if (t_begin >= t_end) return;
+
+  u32x4 wreg[KK][2];
+#pragma unroll
+  for (int k = 0; k < KK; ++k)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) wreg[k][s] = *(const u32x4*)(wpk + ((int64_t)(k * 2 + s) * 64 + lane) * 8);
+  float bq[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) bq[i] = bias ? to_f32(bias[16 * q + i]) : 0.f;
+  if (tid == 0) s_u0[3] = s_u1[3] = -1;
+
+  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
+  const __amdgpu_buffer_rsrc_t rs_loc = make_rsrc(loc, loc_bytes);
+  const __amdgpu_buffer_rsrc_t rs_u = make_rsrc(urows, urows_bytes);
+  const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(uptr, (uint32_t)(tiles + 1) * 4u);
+
+  // staging pieces per wave: 0, 1 table positions; 2 list of the tile after; 3 + i LDS rows
+  // 16 (wave + 4 i) .. + 15 (row p >= 1 = distinct row p - 1, row 0 = zero row).  The 16-byte
+  // chunk c of row p lands at chunk c ^ ((p >> 2) & 3), a per-lane constant here.
+  constexpr int kRowPieces = (kRwCap + 1 + 63) / 64;
+  constexpr int kPieces = 3 + kRowPieces;
+  const uint32_t st_c = (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+  const int st_p = 16 * wave + (lane >> 2);
+  auto make_stage = [&](int64_t tile, int U, int32_t list_first, int32_t list_len, const int32_t* su,
+                        int32_t* su_out, T* rows, uint16_t* locs) {
+    RwStage st;
+    const int64_t tc = min(tile, tiles - 1);
+    st.loc_off = (uint32_t)(tc * kRwRows * KK * 2);
+    const int e = wave * 256 + lane * 4;
+    st.list_off = e < list_len ? (uint32_t)(list_first + e) * 4u : 0xffffff00u;
+    st.groups = (U + 16) >> 4;
+    st.su = su; st.su_out = su_out; st.rows = (char*)rows; st.locs = (char*)locs;
+    return st;
+  };
+  auto stage_id = [&](int t, const RwStage& st) -> int32_t {
+    return t >= 3 ? st.su[st_p + 64 * (t - 3) - 1] : 0;
+  };
+  auto stage_piece = [&](int t, const RwStage& st, int32_t id) {
+    if (t < 2) {
+      constexpr int nchunk = (kRwRows * KK * 2 + 1023) >> 10;
+      if (4 * t < nchunk) {
+        const int c = min(wave + 4 * t, nchunk - 1);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_loc, (lds_ptr_t)(st.locs + c * 1024), 16,
+                                                 st.loc_off + (uint32_t)c * 1024u + lane * 16u, 0, 0, 0);
+      }
+    } else if (t == 2) {
+      if (wave < 2)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_u, (lds_ptr_t)(st.su_out + wave * 256), 16, st.list_off,
+                                                 0, 0, 0);
+    } else {
+      if (wave + 4 * (t - 3) < st.groups)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(st.rows + (wave + 4 * (t - 3)) * 1024), 16,
+                                                 ((uint32_t)id << 6) | st_c, 0, 0, 0);
+    }
+  };
+
+  int32_t p_nxt = uptr[t_begin + 1];
+  int32_t p_nx2 = uptr[min(t_begin + 2, tiles)];
+  int32_t p_nx3 = uptr[min(t_begin + 3, tiles)];
+  {
+    const int32_t p_cur = uptr[t_begin];
+    RwStage st = make_stage(t_begin, 0, p_cur, p_nxt - p_cur, s_u0 + 4, s_u0 + 4, s_rows0, s_loc0);
+    stage_piece(2, st, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    st = make_stage(t_begin, p_nxt - p_cur, p_nxt, p_nx2 - p_nxt, s_u0 + 4, s_u1 + 4, s_rows0, s_loc0);
+#pragma unroll
+    for (int t = 0; t < kPieces; ++t) stage_piece(t, st, stage_id(t, st));
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+  }
+
+  constexpr int PD = 8;      // table positions are read PD slots ahead of their MFMAs ...
+  constexpr int BD = 4;      // ... and the neighbour rows BD slots ahead
+  auto tile_body = [&](auto BC, int64_t tile) {
+    constexpr int B = decltype(BC)::value;
+    const T* rows = B ? s_rows1 : s_rows0;
+    const uint16_t* lc = B ? s_loc1 : s_loc0;
+    const RwStage st = make_stage(tile + 1, p_nx2 - p_nxt, p_nx2, p_nx3 - p_nx2, B ? s_u0 + 4 : s_u1 + 4,
+                                  B ? s_u1 + 4 : s_u0 + 4, B ? s_rows0 : s_rows1, B ? s_loc0 : s_loc1);
+    const uint32_t p_raw = __builtin_amdgcn_raw_buffer_load_b32(rs_p, (uint32_t)min(tile + 4, tiles) * 4u, 0, 0);
+    p_nxt = p_nx2;
+    p_nx2 = p_nx3;
+
+    const uint16_t* lcw = lc + 32 * wave + r32;                 // this lane's row, slot k at + 128 k
+    uint32_t pos[PD];
+    u32x4 ring[PD][2];
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    auto issue_b = [&](int k) {                                  // the two 16-byte pieces of slot k
+      const uint32_t l = pos[k % PD];
+      const uint32_t swz = (l >> 2) & 3;
+      ring[k % PD][0] = *(const u32x4*)(&rows[l * 32 + (((uint32_t)q ^ swz) * 8)]);
+      ring[k % PD][1] = *(const u32x4*)(&rows[l * 32 + (((uint32_t)(2 + q) ^ swz) * 8)]);
+    };
+#pragma unroll
+    for (int k = 0; k < PD && k < KK; ++k) pos[k] = lcw[kRwRows * k];
+#pragma unroll
+    for (int k = 0; k < BD && k < KK; ++k) issue_b(k);
+    __builtin_amdgcn_sched_barrier(0);
+    int32_t id_next = 0;
+#pragma unroll
+    for (int k = 0; k < KK; ++k) {
+      acc = Mma32<T>::run(wreg[k][0], ring[k % PD][0], acc);
+      if (k + BD < KK) issue_b(k + BD);
+      acc = Mma32<T>::run(wreg[k][1], ring[k % PD][1], acc);
+      if (k + PD < KK) pos[k % PD] = lcw[kRwRows * (k + PD)];
+      __builtin_amdgcn_sched_barrier(0);
+      // staging of the next tile: list entry on an even slot, its load on the odd one after
+      {
+        const int t = k >> 1;
+        if (t < kPieces) {
+          if ((k & 1) == 0) id_next = stage_id(t, st);
+          else stage_piece(t, st, id_next);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (KK < 2 * kPieces) {                                      // few slots: the rest of the pieces
+#pragma unroll
+      for (int t = KK / 2; t < kPieces; ++t) stage_piece(t, st, stage_id(t, st));
+    }
+    // bias, pack, two 16-byte stores: 16 consecutive output channels of one row per lane
+    const int64_t row = tile * kRwRows + 32 * wave + r32;
+    if (row < rows_out) {
+      unsigned pk[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pk[i] = pack2<T>(acc[2 * i] + bq[2 * i], acc[2 * i + 1] + bq[2 * i + 1]);
+      T* dst = out + row * 32 + 16 * q;
+      *(u32x4*)(dst) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+      *(u32x4*)(dst + 8) = u32x4{pk[4], pk[5], pk[6], pk[7]};
+    }
+    // the next tile has landed; every wave is past its last read of this tile's buffers
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    p_nx3 = __builtin_amdgcn_readfirstlane((int32_t)p_raw);
+  };
+  for (int64_t tile = t_begin; tile < t_end; tile += 2) {
+    tile_body(std::integral_constant<int, 0>{}, tile);
+    if (tile + 1 < t_end) tile_body(std::integral_constant<int, 1>{}, tile + 1);
+  }
+}
+
 }  // namespace ocnn
 
 using namespace ocnn;
@@ -407,10 +598,10 @@ extern "C" void ocnn_debug_set_rw_timing(long long* p) { g_rw_dbg = p; }
 extern "C" int ocnn_conv_gather_rw_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                              int plan_max_distinct) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (cin != 64 || cout != 64) return 0;
+  if (!((cin == 64 && cout == 64) || (cin == 32 && cout == 32))) return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
   if (plan_max_distinct > kRwCap) return 0;
-  if ((int64_t)rows_in * 128 > 0xfff00000ll) return 0;
+  if ((int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -427,10 +618,23 @@ static void launch_rw(const void* in, int64_t rows_in, const uint16_t* loc, cons
                      urows, urows_bytes, (const T*)ws, (const T*)bias, (T*)out, rows_out, K, tiles, per, g_rw_dbg);
 }
 
+template <typename T, int KK>
+static void launch_rw32(const void* in, int64_t rows_in, const uint16_t* loc, const int32_t* uptr,
+                        const int32_t* urows, uint32_t urows_bytes, int64_t rows_out, const void* ws,
+                        const void* bias, void* out, int n_cu, hipStream_t st) {
+  int64_t tiles = cdiv(rows_out, kRwRows);
+  int64_t wgs = std::min<int64_t>(tiles, n_cu);
+  int64_t per = cdiv(tiles, wgs);
+  wgs = cdiv(tiles, per);
+  hipLaunchKernelGGL((conv_gather_rw32_kernel<T, KK>), dim3((unsigned)wgs), dim3(256), 0, st, (const T*)in,
+                     (uint32_t)(rows_in * 64), loc, (uint32_t)(tiles * kRwRows * KK * 2), uptr, urows,
+                     urows_bytes, (const T*)ws, (const T*)bias, (T*)out, rows_out, tiles, per);
+}
+
 template <typename T>
 static int run_rw(const void* in, int64_t rows_in, const uint16_t* loc, const int32_t* uptr,
-                  const int32_t* urows, int64_t plan_total, int64_t rows_out, int K, const void* w, int w_transposed,
-                  int reverse, const void* bias, void* out, void* ws, hipStream_t st) {
+                  const int32_t* urows, int64_t plan_total, int64_t rows_out, int K, int cin, const void* w,
+                  int w_transposed, int reverse, const void* bias, void* out, void* ws, hipStream_t st) {
   static int n_cu = 0;
   if (n_cu == 0) {
     int dev = 0;
@@ -442,6 +646,15 @@ static int run_rw(const void* in, int64_t rows_in, const uint16_t* loc, const in
     n_cu = prop.multiProcessorCount;
   }
   const uint32_t ub = (uint32_t)(plan_total * 4);
+  if (cin == 32) {
+    hipLaunchKernelGGL(pack_weights_rw32_kernel<T>, dim3(cdiv((int64_t)K * 1024, 256)), dim3(256), 0, st,
+                       (const T*)w, (T*)ws, K, w_transposed, reverse);
+    if (K == 27) launch_rw32<T, 27>(in, rows_in, loc, uptr, urows, ub, rows_out, ws, bias, out, n_cu, st);
+    else if (K == 9) launch_rw32<T, 9>(in, rows_in, loc, uptr, urows, ub, rows_out, ws, bias, out, n_cu, st);
+    else if (K == 8) launch_rw32<T, 8>(in, rows_in, loc, uptr, urows, ub, rows_out, ws, bias, out, n_cu, st);
+    else launch_rw32<T, 3>(in, rows_in, loc, uptr, urows, ub, rows_out, ws, bias, out, n_cu, st);
+    return check_launch("conv_gather_rw32");
+  }
   hipLaunchKernelGGL(pack_weights_rw_kernel<T>, dim3(cdiv((int64_t)K * 4096, 256)), dim3(256), 0, st,
                      (const T*)w, (T*)ws, K, w_transposed, reverse);
   if (K == 27) launch_rw<T, 14>(in, rows_in, loc, uptr, urows, ub, rows_out, K, ws, bias, out, n_cu, st);
@@ -463,14 +676,14 @@ extern "C" int ocnn_conv_gather_rw(int dtype, const void* in, int64_t rows_in, c
                    plan_total >= 0 && plan_total < (1ll << 29),
                "conv_gather_rw: rows out of range");
   if (rows_out == 0) return OCNN_OK;
-  if (workspace_bytes < (int64_t)K * 8192) {
+  if (workspace_bytes < (int64_t)K * cin * cout * 2) {
     set_error("conv_gather_rw: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
-    return run_rw<f16>(in, rows_in, loc, uptr, urows, plan_total, rows_out, K, w, w_transposed, reverse_slots,
+    return run_rw<f16>(in, rows_in, loc, uptr, urows, plan_total, rows_out, K, cin, w, w_transposed, reverse_slots,
                        bias, out, workspace, st);
-  return run_rw<bf16>(in, rows_in, loc, uptr, urows, plan_total, rows_out, K, w, w_transposed, reverse_slots, bias,
+  return run_rw<bf16>(in, rows_in, loc, uptr, urows, plan_total, rows_out, K, cin, w, w_transposed, reverse_slots, bias,
                       out, workspace, st);
 }

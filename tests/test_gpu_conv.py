@@ -361,7 +361,8 @@ def _local_table(rows, rows_in, K, g, spread=40, empty=0.3):
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('K', [27, 9, 8, 3])
-def test_planned_64x64_kernels(dtype, K):
+@pytest.mark.parametrize('ch', [64, 32])
+def test_planned_64x64_kernels(dtype, K, ch):
   """The persistent 64 -> 64 kernels (gather-GEMM with register-resident weights,
   weight gradient on the tile plan) for every slot count they are built for, on
   tables whose row count is not a multiple of the tile, against the oracle and
@@ -375,19 +376,20 @@ def test_planned_64x64_kernels(dtype, K):
     tg = table.to(DEV)
     plan = TilePlan(tg)
     code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
-    assert L.ocnn_conv_gather_rw_supported(code, rows_in, K, 64, 64, plan.umax)
-    assert L.ocnn_conv_wgrad_planned_supported(code, rows_in, rows, K, 64, 64, plan.umax)
-    x = torch.randn(rows_in, 64, generator=g).to(dtype)
-    w = (torch.randn(K, 64, 64, generator=g) / (K * 64) ** 0.5).to(dtype)
-    b = torch.randn(64, generator=g).to(dtype)
-    gr = torch.randn(rows, 64, generator=g).to(dtype)
+    assert L.ocnn_conv_gather_rw_supported(code, rows_in, K, ch, ch, plan.umax)
+    if ch == 64:
+      assert L.ocnn_conv_wgrad_planned_supported(code, rows_in, rows, K, 64, 64, plan.umax)
+    x = torch.randn(rows_in, ch, generator=g).to(dtype)
+    w = (torch.randn(K, ch, ch, generator=g) / (K * ch) ** 0.5).to(dtype)
+    b = torch.randn(ch, generator=g).to(dtype)
+    gr = torch.randn(rows, ch, generator=g).to(dtype)
     t64 = table.numpy().astype(np.int64)
     # gather-GEMM, with bias
-    got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), 64, False, False, b.to(DEV), plan)
+    got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), ch, False, False, b.to(DEV), plan)
     want = C.forward_gemm(f64(x), f64(w), t64) + f64(b)
     assert rel_err(got, want) < TOL[dtype]
     # transposed, mirrored weights (the data gradient of a symmetric table)
-    got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), 64, True, True, None, plan)
+    got = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), ch, True, True, None, plan)
     want = C.forward_gemm(f64(x), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
     assert rel_err(got, want) < TOL[dtype]
     # weight gradient, both output layouts; same bits on a second run
