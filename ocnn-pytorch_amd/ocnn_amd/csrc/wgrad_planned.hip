@@ -1,4 +1,4 @@
-// Weight gradient for 64 x 64 channels on the tile plan of the neighbour table.
+// Weight gradient for 64 x 64 and 32 x 32 channels on the tile plan of the neighbour table.
 //
 //   dW[k][a][b] = sum over table rows r of  x[table[r][k]][a] * g[r][b]
 //
@@ -26,7 +26,7 @@
 namespace ocnn {
 
 constexpr int kWpRows = 128;   // rows per tile (the plan's tile size)
-constexpr int kWpCap = 416;    // staged distinct rows per tile
+constexpr int kWpCap = 415;    // staged distinct rows per tile: with the zero row, 26 groups of 16
 constexpr int kWpLoc = (kWpRows * 27 * 2 + 1023) / 1024 * 512;   // u16 per buffer, whole KiB
 constexpr int kWpXHalf = (kWpCap + 1) * 32;   // elements of one channel half of the x rows (+ zero row)
 constexpr int kWpGHalf = kWpRows * 32;
@@ -50,35 +50,41 @@ struct WpStage {
   char* sl;
 };
 
-// NFULL slots per wave with both x-channel halves, NHALF (0/1) slot shared by two
-// waves (one x-channel half each); GROUPS workgroups split the K slots.
+// C = 64 or 32 channels on both sides.  NFULL slots per wave with all x channels, NHALF
+// (0/1, C = 64 only) slot shared by two waves (one x-channel half each); GROUPS workgroups
+// split the K slots.
 //
 // LDS layout: the two 32-channel halves of the staged rows live in separate arrays
 // of 64-byte rows.  A transposing read of a 16-lane group touches 4 rows x 32 B, a
 // half wave 4 rows x 64 B; at a 64-byte pitch four consecutive positions cover all
 // 64 banks, and the second half is the first plus a constant.
-template <typename T, int KK, int NFULL, int NHALF, int GROUPS>
+template <typename T, int C, int KK, int NFULL, int NHALF, int GROUPS>
 __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes,
     const uint16_t* __restrict__ loc, uint32_t loc_bytes, const int32_t* __restrict__ uptr,
     const int32_t* __restrict__ urows, uint32_t urows_bytes, int64_t tiles,
     int64_t tiles_per_split, int nsplit, float* __restrict__ partial, long long* dbg) {
-  constexpr int NU = 2 * NFULL + NHALF;       // 32 x 64 accumulator units per wave
+  constexpr int H = C / 32;                   // 32-channel halves of a row
+  constexpr int NU = H * NFULL + NHALF;       // 32 x C accumulator units per wave
   constexpr int NS = NFULL + NHALF;           // distinct slots per wave
   constexpr int SPG = 4 * NFULL + 2 * NHALF;  // slots per group
   constexpr int NL = 2 * NS;                  // table look-ups per lane and step
-  constexpr int NM = 2 * NU;                  // MFMAs per step
+  constexpr int NM = H * NU;                  // MFMAs per step
   constexpr int XH = kWpXHalf * 2, GH = kWpGHalf * 2;   // byte offsets of the second halves
-  constexpr int PF0 = (NM - NL) < 4 ? (NM - NL) : 4;   // MFMAs between the position reads and their use
+  // C = 64: MFMAs between the position reads and their use
+  constexpr int PF0 = H == 1 ? 1 : ((NM - NL) < 4 ? (NM - NL) : 4);
   constexpr int IP = (NL + 4 + PF0 - 1) / PF0;
-  static_assert(NU <= 7 && PF0 >= 1, "unit layout");
+  // C = 32: positions and g with the first MFMA, the x reads XP per MFMA from MFMA XS on
+  constexpr int XS = NM > 2 ? 2 : NM - 1;
+  constexpr int XP = (NL + (NM - XS) - 1) / (NM - XS);
+  static_assert((H == 1 || H == 2) && NU <= 7 && PF0 >= 1 && (H == 2 || NHALF == 0), "unit layout");
 
   // one array per buffer, so that the compiler can tell the buffer being filled
   // from the one being read
-  __shared__ __attribute__((aligned(16))) T s_x0[2 * kWpXHalf];
-  __shared__ __attribute__((aligned(16))) T s_x1[2 * kWpXHalf];
-  __shared__ __attribute__((aligned(16))) T s_g0[2 * kWpGHalf];
-  __shared__ __attribute__((aligned(16))) T s_g1[2 * kWpGHalf];
+  __shared__ __attribute__((aligned(16))) T s_x0[H * kWpXHalf];
+  __shared__ __attribute__((aligned(16))) T s_x1[H * kWpXHalf];
+  __shared__ __attribute__((aligned(16))) T s_g0[H * kWpGHalf];
+  __shared__ __attribute__((aligned(16))) T s_g1[H * kWpGHalf];
   __shared__ __attribute__((aligned(16))) uint16_t s_loc0[kWpLoc];
   __shared__ __attribute__((aligned(16))) uint16_t s_loc1[kWpLoc];
   // lists of distinct rows, from entry 4 on; entry 3 stays -1 ("the row before the first")
@@ -109,6 +115,14 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   const uint32_t byte0 = 32u * (gq & 1) + 8u * (i16 & 3);
   const uint32_t lbF = (uint32_t)(slotF_rd * kWpRows + 8 * q + rs) * 2u;   // [slot][row] positions, 2 B each
   const uint32_t lbH = (uint32_t)(slotH_rd * kWpRows + 8 * q + rs) * 2u;
+  // C = 32: a wave's slots can end inside its group of NFULL (K = 27: slots 21..27), so
+  // every slot clamps on its own
+  uint32_t lbS[H == 1 ? NFULL : 1];
+  if constexpr (H == 1) {
+#pragma unroll
+    for (int sl = 0; sl < NFULL; ++sl)
+      lbS[sl] = (uint32_t)(min(slotF + sl, KK - 1) * kWpRows + 8 * q + rs) * 2u;
+  }
   uint32_t gad[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) gad[h] = (uint32_t)(8 * q + 4 * h + rs) * 64u + byte0;
@@ -122,24 +136,30 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(uptr, (uint32_t)(tiles + 1) * 4u);
 
   // ---- staging of one tile, cut into per-wave pieces `t` (one load instruction each, 1 KiB):
-  //   t = 0..3   g rows: 16 rows of one channel half
-  //   t = 4, 5   table positions
-  //   t = 6..18  x rows: 16 distinct rows (ids in su) of one channel half
-  //   t = 19     the list of distinct rows of the tile after (waves 0 and 1)
+  //   NG pieces  g rows: 16 rows of one channel half
+  //   2 pieces   table positions
+  //   NX pieces  x rows: 16 distinct rows (ids in su) of one channel half
+  //   1 piece    the list of distinct rows of the tile after (waves 0 and 1)
+  // (C = 64: 4 + 2 + 13 + 1, a wave takes one half of every second 16-row group;
+  //  C = 32: 2 + 2 + 7 + 1, a wave takes every fourth group.)
   // The pieces are branch-free: whatever lies past the end of a list, of the table or of
   // the tile range is an out-of-range offset (loads zeros) or row 0.  A wave has one
   // instruction stream for the MFMAs and everything else, so each instruction saved here
   // is MFMA issue time won.
-  constexpr int kPieces = 20;
-  const uint32_t st_xc = (uint32_t)(wave & 1) * 64u + (uint32_t)(lane & 3) * 16u;   // byte within a row
-  const int st_pos = (wave >> 1) * 16 + (lane >> 2);       // position / row of piece 0; piece j: + 32 j
-  const uint32_t st_gc = (uint32_t)st_pos * 128u + st_xc;
-  const int st_half = wave & 1, st_g16 = wave >> 1;
+  constexpr int NG = 2 * H, GST = 4 / H;                   // g pieces; 16-row groups between a wave's pieces
+  constexpr int NX = ((kWpCap + 16) / 16 + GST - 1) / GST;
+  constexpr int tL = NG, tX = NG + 2, tU = NG + 2 + NX, kPieces = tU + 1;
+  static_assert(kPieces <= 20 && (kWpCap + 1) % 16 == 0, "five steps of four pieces stage a tile");
+  constexpr int RSH = 5 + H;                               // log2 of the bytes of a row in memory
+  const int st_half = H == 2 ? (wave & 1) : 0, st_g16 = H == 2 ? (wave >> 1) : wave;
+  const uint32_t st_xc = (uint32_t)st_half * 64u + (uint32_t)(lane & 3) * 16u;   // byte within a row
+  const int st_pos = st_g16 * 16 + (lane >> 2);            // position / row of piece 0; piece j: + 16 GST j
+  const uint32_t st_gc = ((uint32_t)st_pos << RSH) + st_xc;
   auto make_stage = [&](int64_t tile, int U, int32_t list_first, int32_t list_len, const int32_t* su,
                         int32_t* su_out, T* sx, T* sg, uint16_t* sl) {
     WpStage st;
     const int64_t tc = min(tile, tiles - 1);              // past the range: any valid tile
-    st.g_off = (uint32_t)(tc * kWpRows) * 128u;
+    st.g_off = (uint32_t)(tc * kWpRows) << RSH;
     st.loc_off = (uint32_t)(tc * kWpRows * KK * 2);
     const int e = wave * 256 + lane * 4;                   // the four list entries this lane brings in
     st.list_off = e < list_len ? (uint32_t)(list_first + e) * 4u : 0xffffff00u;
@@ -148,36 +168,36 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     return st;
   };
   auto stage_id = [&](int t, const WpStage& st) -> int32_t {     // row id a lane needs for piece t
-    return (t >= 6 && t <= 18) ? st.su[st_pos + 32 * (t - 6) - 1] : 0;   // position p holds list entry p - 1
+    return (t >= tX && t < tU) ? st.su[st_pos + 16 * GST * (t - tX) - 1] : 0;   // position p holds list entry p - 1
   };
   auto stage_piece = [&](int t, const WpStage& st, int32_t id) {
-    if (t < 4) {
+    if (t < NG) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rs_g, (lds_ptr_t)(st.sg + (st_half * kWpGHalf + (st_g16 + 2 * t) * 512) * 2), 16,
-          st.g_off + st_gc + (uint32_t)(t * 4096), 0, 0, 0);
-    } else if (t < 6) {
+          rs_g, (lds_ptr_t)(st.sg + (st_half * kWpGHalf + (st_g16 + GST * t) * 512) * 2), 16,
+          st.g_off + st_gc + (uint32_t)(t * 4096), 0, 0, 0);      // 16 GST rows further: 4 KiB either way
+    } else if (t < tX) {
       constexpr int nchunk = (kWpRows * KK * 2 + 1023) >> 10;
-      if (4 * (t - 4) < nchunk) {
-        const int c = min(wave + 4 * (t - 4), nchunk - 1);     // a spare wave repeats the last chunk
+      if (4 * (t - tL) < nchunk) {
+        const int c = min(wave + 4 * (t - tL), nchunk - 1);     // a spare wave repeats the last chunk
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_loc, (lds_ptr_t)(st.sl + c * 1024), 16,
                                                  st.loc_off + (uint32_t)c * 1024u + lane * 16u, 0, 0, 0);
       }
-    } else if (t < 19) {
-      if ((st_g16 + 2 * (t - 6)) < st.groups)
+    } else if (t < tU) {
+      if ((st_g16 + GST * (t - tX)) < st.groups)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rs_x, (lds_ptr_t)(st.sx + (st_half * kWpXHalf + (st_g16 + 2 * (t - 6)) * 512) * 2), 16,
-          ((uint32_t)id << 7) | st_xc, 0, 0, 0);
+          rs_x, (lds_ptr_t)(st.sx + (st_half * kWpXHalf + (st_g16 + GST * (t - tX)) * 512) * 2), 16,
+          ((uint32_t)id << RSH) | st_xc, 0, 0, 0);
     } else if (wave < 2) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_u, (lds_ptr_t)(st.su_out + wave * 256), 16, st.list_off, 0,
                                                0, 0);
     }
   };
 
-  f32x16 acc[NU][2];
+  f32x16 acc[NU][H];
 #pragma unroll
   for (int u = 0; u < NU; ++u)
 #pragma unroll
-    for (int bh = 0; bh < 2; ++bh)
+    for (int bh = 0; bh < H; ++bh)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[u][bh][r] = 0.f;
 
@@ -187,7 +207,9 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   // ---- the pieces of one step's operand fetch ----
   auto pf_loc = [&](int j, const char* lcs, int sn) {       // j = 2 * slot + h
     const int sl = j >> 1, h = j & 1;
-    const uint32_t off = (sl < NFULL ? lbF + (uint32_t)(sl * kWpRows * 2) : lbH) + (uint32_t)(sn * 32 + h * 8);
+    uint32_t off;
+    if constexpr (H == 1) off = lbS[sl] + (uint32_t)(sn * 32 + h * 8);
+    else off = (sl < NFULL ? lbF + (uint32_t)(sl * kWpRows * 2) : lbH) + (uint32_t)(sn * 32 + h * 8);
     pv[j] = *(const uint16_t*)(lcs + off);
   };
   auto pf_g = [&](int j, const char* gs, int sn, WpOps& on) {   // j = 2 * bh + h
@@ -198,14 +220,14 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     const int sl = j >> 1, h = j & 1;
     const uint32_t ad = (pv[j] << 6) + byte0;                 // position 0 is the zero row
     if (sl < NFULL) {
-      on.a[2 * sl][h] = Mma<T>::read_tr((const T*)(xs + ad));
-      on.a[2 * sl + 1][h] = Mma<T>::read_tr((const T*)(xs + ad + (uint32_t)XH));
+      on.a[H * sl][h] = Mma<T>::read_tr((const T*)(xs + ad));
+      if constexpr (H == 2) on.a[2 * sl + 1][h] = Mma<T>::read_tr((const T*)(xs + ad + (uint32_t)XH));
     } else {
-      on.a[2 * NFULL][h] = Mma<T>::read_tr((const T*)(xs + ad + ahH));
+      on.a[H * NFULL][h] = Mma<T>::read_tr((const T*)(xs + ad + ahH));
     }
   };
   auto mm = [&](int m, const WpOps& oc) {
-    const int u = m >> 1, bh = m & 1;
+    const int u = m / H, bh = m % H;
     const u32x4 av = u32x4{oc.a[u][0][0], oc.a[u][0][1], oc.a[u][1][0], oc.a[u][1][1]};
     const u32x4 bv = u32x4{oc.b[bh][0][0], oc.b[bh][0][1], oc.b[bh][1][0], oc.b[bh][1][1]};
     acc[u][bh] = Mma32<T>::run(av, bv, acc[u][bh]);
@@ -226,14 +248,27 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
       mm(m, oc);
       // operand fetch of the next step: table positions and g first, then the x reads
       // that depend on the positions, PF0 MFMAs later
-      if (m < PF0) {
+      if constexpr (H == 2) {
+        if (m < PF0) {
 #pragma unroll
-        for (int t = m * IP; t < (m + 1) * IP && t < NL + 4; ++t) {
-          if (t < NL) { if (!(OCNN_WP_EXP & 8)) pf_loc(t, lcs, sn); }
-          else if (!(OCNN_WP_EXP & 4)) pf_g(t - NL, gs, sn, on);
+          for (int t = m * IP; t < (m + 1) * IP && t < NL + 4; ++t) {
+            if (t < NL) { if (!(OCNN_WP_EXP & 8)) pf_loc(t, lcs, sn); }
+            else if (!(OCNN_WP_EXP & 4)) pf_g(t - NL, gs, sn, on);
+          }
+        } else if (m - PF0 < NL) {
+          if (!(OCNN_WP_EXP & 2)) pf_x(m - PF0, xs, on);
         }
-      } else if (m - PF0 < NL) {
-        if (!(OCNN_WP_EXP & 2)) pf_x(m - PF0, xs, on);
+      } else {
+        if (m == 0) {
+#pragma unroll
+          for (int t = 0; t < NL; ++t) pf_loc(t, lcs, sn);
+#pragma unroll
+          for (int t = 0; t < 2; ++t) pf_g(t, gs, sn, on);
+        }
+        if (m >= XS) {
+#pragma unroll
+          for (int t = (m - XS) * XP; t < (m - XS + 1) * XP && t < NL; ++t) pf_x(t, xs, on);
+        }
       }
       if (!(OCNN_WP_EXP & 1) && t0 >= 0) {
         if (m == 0) {
@@ -266,7 +301,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
 #pragma unroll
     for (int t = 0; t < NL; ++t) pf_loc(t, lcs, 0);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) pf_g(t, gs, 0, on);
+    for (int t = 0; t < 2 * H; ++t) pf_g(t, gs, 0, on);
 #pragma unroll
     for (int t = 0; t < NL; ++t) pf_x(t, xs, on);
   };
@@ -278,7 +313,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   {
     const int32_t p_cur = uptr[t_begin];
     WpStage st = make_stage(t_begin, 0, p_cur, p_nxt - p_cur, s_u0 + 4, s_u0 + 4, s_x0, s_g0, s_loc0);
-    stage_piece(19, st, 0);                                // list of the first tile -> s_u0
+    stage_piece(tU, st, 0);                                // list of the first tile -> s_u0
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     st = make_stage(t_begin, p_nxt - p_cur, p_nxt, p_nx2 - p_nxt, s_u0 + 4, s_u1 + 4, s_x0, s_g0, s_loc0);
@@ -287,7 +322,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
 #if OCNN_WP_EXP & 1
     st.sx = (char*)s_x1; st.sg = (char*)s_g1; st.sl = (char*)s_loc1;
 #pragma unroll
-    for (int t = 0; t < 19; ++t) stage_piece(t, st, stage_id(t, st));   // timing experiment: both buffers filled
+    for (int t = 0; t < tU; ++t) stage_piece(t, st, stage_id(t, st));   // timing experiment: both buffers filled
 #endif
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
@@ -346,16 +381,16 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   const int b32 = lane & 31;
 #pragma unroll
   for (int u = 0; u < NU; ++u) {
-    const int slot = u < 2 * NFULL ? slotF + (u >> 1) : slotH;
-    const int ah = u < 2 * NFULL ? (u & 1) : (wave & 1);
+    const int slot = u < H * NFULL ? slotF + u / H : slotH;
+    const int ah = u < H * NFULL ? u % H : (wave & 1);
     if (slot >= KK) continue;
-    float* dst = partial + ((int64_t)split * KK + slot) * 4096;
+    float* dst = partial + ((int64_t)split * KK + slot) * (C * C);
 #pragma unroll
-    for (int bh = 0; bh < 2; ++bh)
+    for (int bh = 0; bh < H; ++bh)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int a = 32 * ah + 8 * (r >> 2) + 4 * q + (r & 3);
-        dst[a * 64 + 32 * bh + b32] = acc[u][bh][r];
+        dst[a * C + 32 * bh + b32] = acc[u][bh][r];
       }
   }
 }
@@ -370,8 +405,8 @@ static long long* g_wp_dbg = nullptr;
 extern "C" void ocnn_debug_set_wp_timing(long long* p) { g_wp_dbg = p; }
 #endif
 
-static int wp_splits(int K, int n_cu) {
-  const int groups = K == 27 ? 2 : 1;
+static int wp_splits(int K, int c, int n_cu) {
+  const int groups = (K == 27 && c == 64) ? 2 : 1;
   int s = std::max(8, n_cu / groups / 8 * 8);      // a multiple of 8: ranges are dealt to the XCDs
   return std::min(s, 256);
 }
@@ -390,10 +425,10 @@ static int wp_cu_count() {
 extern "C" int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
                                                  int cb, int plan_max_distinct) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (ca != 64 || cb != 64) return 0;
+  if (ca != cb || (ca != 64 && ca != 32)) return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
   if (plan_max_distinct > kWpCap) return 0;
-  if ((int64_t)rows_x * 128 > 0xfff00000ll || ((int64_t)rows + kWpRows) * 128 > 0xfff00000ll) return 0;
+  if ((int64_t)rows_x * ca * 2 > 0xfff00000ll || ((int64_t)rows + kWpRows) * ca * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -401,42 +436,52 @@ extern "C" int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K) {
   return align_up((int64_t)256 * K * 4096 * 4, 256);
 }
 
-template <typename T, int KK, int NFULL, int NHALF, int GROUPS>
+template <typename T, int C, int KK, int NFULL, int NHALF, int GROUPS>
 static void launch_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* loc, const int32_t* uptr,
                       const int32_t* urows, int64_t plan_total, int64_t rows, int nsplit, int64_t per,
                       float* partial, hipStream_t st) {
   const int64_t tiles = cdiv(rows, kWpRows);
-  hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, KK, NFULL, NHALF, GROUPS>), dim3(nsplit * GROUPS),
-                     dim3(256), 0, st, (const T*)x, (uint32_t)(rows_x * 128), (const T*)g,
-                     (uint32_t)(rows * 128), loc, (uint32_t)(tiles * kWpRows * KK * 2), uptr, urows,
+  hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS>), dim3(nsplit * GROUPS),
+                     dim3(256), 0, st, (const T*)x, (uint32_t)(rows_x * C * 2), (const T*)g,
+                     (uint32_t)(rows * C * 2), loc, (uint32_t)(tiles * kWpRows * KK * 2), uptr, urows,
                      (uint32_t)(plan_total * 4), tiles, per, nsplit, partial, g_wp_dbg);
 }
 
 template <typename T>
 static int run_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* loc, const int32_t* uptr,
-                  const int32_t* urows, int64_t plan_total, int64_t rows, int K, int out_transposed,
+                  const int32_t* urows, int64_t plan_total, int64_t rows, int K, int c, int out_transposed,
                   void* gw, void* ws, int64_t ws_bytes, hipStream_t st) {
   const int n_cu = wp_cu_count();
   if (n_cu <= 0) {
     set_error("conv_wgrad_planned: cannot query the device");
     return OCNN_ERR_HIP;
   }
-  const int nsplit = wp_splits(K, n_cu);
+  const int nsplit = wp_splits(K, c, n_cu);
   const int64_t tiles = cdiv(rows, kWpRows);
   const int64_t per = std::max<int64_t>(1, cdiv(tiles, nsplit));
   const int used = (int)cdiv(tiles, per);                 // ranges that hold tiles
-  if (ws_bytes < (int64_t)used * K * 4096 * 4) {
+  if (ws_bytes < (int64_t)used * K * c * c * 4) {
     set_error("conv_wgrad_planned: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
   float* partial = (float*)ws;
   if (rows > 0) {
-    if (K == 27) launch_wp<T, 27, 3, 1, 2>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st);
-    else if (K == 9) launch_wp<T, 9, 2, 1, 1>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st);
-    else if (K == 8) launch_wp<T, 8, 2, 0, 1>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st);
-    else launch_wp<T, 3, 1, 0, 1>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st);
+#define OCNN_WP_LAUNCH(CC, KK, NF, NH, GR) \
+  launch_wp<T, CC, KK, NF, NH, GR>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st)
+    if (c == 64) {
+      if (K == 27) OCNN_WP_LAUNCH(64, 27, 3, 1, 2);
+      else if (K == 9) OCNN_WP_LAUNCH(64, 9, 2, 1, 1);
+      else if (K == 8) OCNN_WP_LAUNCH(64, 8, 2, 0, 1);
+      else OCNN_WP_LAUNCH(64, 3, 1, 0, 1);
+    } else {
+      if (K == 27) OCNN_WP_LAUNCH(32, 27, 7, 0, 1);
+      else if (K == 9) OCNN_WP_LAUNCH(32, 9, 3, 0, 1);
+      else if (K == 8) OCNN_WP_LAUNCH(32, 8, 2, 0, 1);
+      else OCNN_WP_LAUNCH(32, 3, 1, 0, 1);
+    }
+#undef OCNN_WP_LAUNCH
   }
-  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, 64, 64, out_transposed, (T*)gw, st);
+  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, c, c, out_transposed, (T*)gw, st);
   return check_launch("conv_wgrad_planned");
 }
 
@@ -452,8 +497,8 @@ extern "C" int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x,
                "conv_wgrad_planned: rows out of range");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
-    return run_wp<f16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, out_transposed, gw, workspace,
+    return run_wp<f16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, out_transposed, gw, workspace,
                        workspace_bytes, st);
-  return run_wp<bf16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, out_transposed, gw, workspace,
+  return run_wp<bf16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, out_transposed, gw, workspace,
                       workspace_bytes, st);
 }

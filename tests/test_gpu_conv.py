@@ -363,7 +363,7 @@ def _local_table(rows, rows_in, K, g, spread=40, empty=0.3):
 @pytest.mark.parametrize('K', [27, 9, 8, 3])
 @pytest.mark.parametrize('ch', [64, 32])
 def test_planned_64x64_kernels(dtype, K, ch):
-  """The persistent 64 -> 64 kernels (gather-GEMM with register-resident weights,
+  """The persistent 64 -> 64 and 32 -> 32 kernels (gather-GEMM with register-resident weights,
   weight gradient on the tile plan) for every slot count they are built for, on
   tables whose row count is not a multiple of the tile, against the oracle and
   against the plan-free kernels."""
@@ -377,8 +377,7 @@ def test_planned_64x64_kernels(dtype, K, ch):
     plan = TilePlan(tg)
     code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
     assert L.ocnn_conv_gather_rw_supported(code, rows_in, K, ch, ch, plan.umax)
-    if ch == 64:
-      assert L.ocnn_conv_wgrad_planned_supported(code, rows_in, rows, K, 64, 64, plan.umax)
+    assert L.ocnn_conv_wgrad_planned_supported(code, rows_in, rows, K, ch, ch, plan.umax)
     x = torch.randn(rows_in, ch, generator=g).to(dtype)
     w = (torch.randn(K, ch, ch, generator=g) / (K * ch) ** 0.5).to(dtype)
     b = torch.randn(ch, generator=g).to(dtype)
@@ -400,6 +399,38 @@ def test_planned_64x64_kernels(dtype, K, ch):
     gwt = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, True, plan)
     assert torch.equal(gwt, gw.transpose(1, 2).contiguous())
     assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
+
+
+@pytest.mark.parametrize('ch', [64, 32])
+def test_planned_kernels_at_the_staging_limit(ch):
+  """Tiles with exactly as many distinct rows as the persistent kernels stage (the last
+  staged position is in use), and one more (the weight gradient then takes another kernel)."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(9)
+  rows, K = 300, 27
+  for distinct in (415, 416, 417):
+    rows_in = 3 * distinct + 7
+    table = torch.full((rows, K), -1, dtype=torch.int32)
+    for t0 in range(0, rows, 128):                     # tile t draws from its own `distinct` rows
+      n = min(128, rows - t0)
+      pool = (torch.randperm(distinct, generator=g) + (t0 // 128) * distinct).to(torch.int32)
+      e = pool[torch.randint(0, distinct, (n * K,), generator=g)]
+      e[:distinct] = pool                              # every one of them at least once
+      table[t0:t0 + n] = e[torch.randperm(n * K, generator=g)].reshape(n, K)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    assert plan.umax == distinct
+    say('staging limit', ch, distinct, 'gather', L.ocnn_conv_gather_rw_supported(1, rows_in, K, ch, ch, plan.umax),
+        'wgrad', L.ocnn_conv_wgrad_planned_supported(1, rows_in, rows, K, ch, ch, plan.umax))
+    x = torch.randn(rows_in, ch, generator=g).half()
+    gr = torch.randn(rows, ch, generator=g).half()
+    w = (torch.randn(K, ch, ch, generator=g) / 30).half()
+    t64 = table.numpy().astype(np.int64)
+    out = ocnn_amd.nn.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), ch, False, False, None, plan)
+    assert rel_err(out, C.forward_gemm(f64(x), f64(w), t64)) < 2e-2
+    gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+    assert rel_err(gw, C.weight_gemm(f64(x), f64(gr), t64)) < 2e-2
 
 
 def test_planned_kernels_non_finite_rows():
