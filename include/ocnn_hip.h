@@ -234,14 +234,15 @@ int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
                     int out_transposed, void* gw, void* workspace,
                     int64_t workspace_bytes, void* stream);
 
-/* ocnn_conv_wgrad over a tile plan of the same table, for ca = cb = 64 or 32 (same
+/* ocnn_conv_wgrad over a tile plan of the same table, for ca = cb = 32 and for ca, cb
+ * multiples of 64 up to 1024, summed in 64 x 64 blocks of channel pairs (same
  * reference lines, same result up to the fp32 summation order, which is fixed).
  * Per tile the distinct x rows and the g rows are staged once in LDS; persistent
  * workgroups keep the sums of all K slots in accumulator registers over a range
  * of tiles.  plan_max_distinct must be <= 415; ..._supported() tells. */
 int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
                                       int cb, int plan_max_distinct);
-int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K);
+int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K, int ca, int cb);
 int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const void* g,
                             const uint16_t* loc, const int32_t* uptr, const int32_t* urows,
                             int plan_max_distinct, int64_t plan_total, int64_t rows, int K,

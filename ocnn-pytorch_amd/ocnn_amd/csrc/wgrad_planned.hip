@@ -1,4 +1,5 @@
-// Weight gradient for 64 x 64 and 32 x 32 channels on the tile plan of the neighbour table.
+// Weight gradient for 32 x 32 channels and for multiples of 64 channels (in 64 x 64 blocks)
+// on the tile plan of the neighbour table.
 //
 //   dW[k][a][b] = sum over table rows r of  x[table[r][k]][a] * g[r][b]
 //
@@ -50,20 +51,21 @@ struct WpStage {
   char* sl;
 };
 
-// C = 64 or 32 channels on both sides.  NFULL slots per wave with all x channels, NHALF
-// (0/1, C = 64 only) slot shared by two waves (one x-channel half each); GROUPS workgroups
-// split the K slots.
+// A workgroup sums a C x C block (C = 64 or 32) of the channel pairs; blockIdx.y picks
+// the block when the layer has more channels (BLK; C = 64).  NFULL slots per wave with all
+// C x channels, NHALF (0/1, C = 64 only) slot shared by two waves (one x-channel half each);
+// GROUPS workgroups split the K slots.
 //
 // LDS layout: the two 32-channel halves of the staged rows live in separate arrays
 // of 64-byte rows.  A transposing read of a 16-lane group touches 4 rows x 32 B, a
 // half wave 4 rows x 64 B; at a 64-byte pitch four consecutive positions cover all
 // 64 banks, and the second half is the first plus a constant.
-template <typename T, int C, int KK, int NFULL, int NHALF, int GROUPS>
+template <typename T, int C, int KK, int NFULL, int NHALF, int GROUPS, bool BLK>
 __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes,
     const uint16_t* __restrict__ loc, uint32_t loc_bytes, const int32_t* __restrict__ uptr,
     const int32_t* __restrict__ urows, uint32_t urows_bytes, int64_t tiles,
-    int64_t tiles_per_split, int nsplit, float* __restrict__ partial, long long* dbg) {
+    int64_t tiles_per_split, int nsplit, int ca, int cb, float* __restrict__ partial, long long* dbg) {
   constexpr int H = C / 32;                   // 32-channel halves of a row
   constexpr int NU = H * NFULL + NHALF;       // 32 x C accumulator units per wave
   constexpr int NS = NFULL + NHALF;           // distinct slots per wave
@@ -150,16 +152,22 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   constexpr int NX = ((kWpCap + 16) / 16 + GST - 1) / GST;
   constexpr int tL = NG, tX = NG + 2, tU = NG + 2 + NX, kPieces = tU + 1;
   static_assert(kPieces <= 20 && (kWpCap + 1) % 16 == 0, "five steps of four pieces stage a tile");
-  constexpr int RSH = 5 + H;                               // log2 of the bytes of a row in memory
+  constexpr int RSH = 5 + H;                               // log2 of the bytes of a C-channel row
+  // a block of a wider layer: rows of ca (cb) channels, this block's 64 start at xb (gb)
+  const int nbb = BLK ? cb / C : 1;
+  const int blk_a = BLK ? (int)blockIdx.y / nbb : 0, blk_b = BLK ? (int)blockIdx.y % nbb : 0;
+  const uint32_t x_pitch = BLK ? (uint32_t)ca * 2u : (1u << RSH), g_pitch = BLK ? (uint32_t)cb * 2u : (1u << RSH);
+  const uint32_t xb = (uint32_t)blk_a << RSH, gb = (uint32_t)blk_b << RSH;
   const int st_half = H == 2 ? (wave & 1) : 0, st_g16 = H == 2 ? (wave >> 1) : wave;
   const uint32_t st_xc = (uint32_t)st_half * 64u + (uint32_t)(lane & 3) * 16u;   // byte within a row
   const int st_pos = st_g16 * 16 + (lane >> 2);            // position / row of piece 0; piece j: + 16 GST j
-  const uint32_t st_gc = ((uint32_t)st_pos << RSH) + st_xc;
+  const uint32_t st_gc = (BLK ? (uint32_t)st_pos * g_pitch + gb : ((uint32_t)st_pos << RSH)) + st_xc;
+  const uint32_t st_gstep = BLK ? 16u * GST * g_pitch : 4096u;   // 16 GST rows further
   auto make_stage = [&](int64_t tile, int U, int32_t list_first, int32_t list_len, const int32_t* su,
                         int32_t* su_out, T* sx, T* sg, uint16_t* sl) {
     WpStage st;
     const int64_t tc = min(tile, tiles - 1);              // past the range: any valid tile
-    st.g_off = (uint32_t)(tc * kWpRows) << RSH;
+    st.g_off = BLK ? (uint32_t)(tc * kWpRows) * g_pitch : (uint32_t)(tc * kWpRows) << RSH;
     st.loc_off = (uint32_t)(tc * kWpRows * KK * 2);
     const int e = wave * 256 + lane * 4;                   // the four list entries this lane brings in
     st.list_off = e < list_len ? (uint32_t)(list_first + e) * 4u : 0xffffff00u;
@@ -174,7 +182,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     if (t < NG) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rs_g, (lds_ptr_t)(st.sg + (st_half * kWpGHalf + (st_g16 + GST * t) * 512) * 2), 16,
-          st.g_off + st_gc + (uint32_t)(t * 4096), 0, 0, 0);      // 16 GST rows further: 4 KiB either way
+          st.g_off + st_gc + (uint32_t)t * st_gstep, 0, 0, 0);
     } else if (t < tX) {
       constexpr int nchunk = (kWpRows * KK * 2 + 1023) >> 10;
       if (4 * (t - tL) < nchunk) {
@@ -186,7 +194,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
       if ((st_g16 + GST * (t - tX)) < st.groups)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rs_x, (lds_ptr_t)(st.sx + (st_half * kWpXHalf + (st_g16 + GST * (t - tX)) * 512) * 2), 16,
-          ((uint32_t)id << RSH) | st_xc, 0, 0, 0);
+          BLK ? (uint32_t)id * x_pitch + (xb + st_xc) : (((uint32_t)id << RSH) | st_xc), 0, 0, 0);
     } else if (wave < 2) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_u, (lds_ptr_t)(st.su_out + wave * 256), 16, st.list_off, 0,
                                                0, 0);
@@ -384,13 +392,15 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     const int slot = u < H * NFULL ? slotF + u / H : slotH;
     const int ah = u < H * NFULL ? u % H : (wave & 1);
     if (slot >= KK) continue;
-    float* dst = partial + ((int64_t)split * KK + slot) * (C * C);
+    const int ldb = BLK ? cb : C;
+    float* dst = BLK ? partial + (((int64_t)split * KK + slot) * ca + blk_a * C) * cb + blk_b * C
+                     : partial + ((int64_t)split * KK + slot) * (C * C);
 #pragma unroll
     for (int bh = 0; bh < H; ++bh)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int a = 32 * ah + 8 * (r >> 2) + 4 * q + (r & 3);
-        dst[a * C + 32 * bh + b32] = acc[u][bh][r];
+        dst[a * ldb + 32 * bh + b32] = acc[u][bh][r];
       }
   }
 }
@@ -405,9 +415,10 @@ static long long* g_wp_dbg = nullptr;
 extern "C" void ocnn_debug_set_wp_timing(long long* p) { g_wp_dbg = p; }
 #endif
 
-static int wp_splits(int K, int c, int n_cu) {
-  const int groups = (K == 27 && c == 64) ? 2 : 1;
-  int s = std::max(8, n_cu / groups / 8 * 8);      // a multiple of 8: ranges are dealt to the XCDs
+static int wp_splits(int K, int ca, int cb, int n_cu) {
+  const int groups = (K == 27 && ca >= 64) ? 2 : 1;
+  const int blocks = ca >= 64 ? (ca / 64) * (cb / 64) : 1;
+  int s = std::max(8, n_cu / (groups * blocks) / 8 * 8);      // a multiple of 8: ranges are dealt to the XCDs
   return std::min(s, 256);
 }
 
@@ -425,50 +436,59 @@ static int wp_cu_count() {
 extern "C" int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
                                                  int cb, int plan_max_distinct) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (ca != cb || (ca != 64 && ca != 32)) return 0;
+  if (!(ca == 32 && cb == 32) && !(ca >= 64 && cb >= 64 && ca % 64 == 0 && cb % 64 == 0 && ca <= 1024 && cb <= 1024))
+    return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
   if (plan_max_distinct > kWpCap) return 0;
-  if ((int64_t)rows_x * ca * 2 > 0xfff00000ll || ((int64_t)rows + kWpRows) * ca * 2 > 0xfff00000ll) return 0;
+  if ((int64_t)rows_x * ca * 2 > 0xfff00000ll || ((int64_t)rows + kWpRows) * cb * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
-extern "C" int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K) {
-  return align_up((int64_t)256 * K * 4096 * 4, 256);
+extern "C" int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K, int ca, int cb) {
+  const int n_cu = wp_cu_count();
+  const int64_t splits = n_cu > 0 ? wp_splits(K, ca, cb, n_cu) : 256;
+  return align_up(splits * K * ca * cb * 4, 256);
 }
 
 template <typename T, int C, int KK, int NFULL, int NHALF, int GROUPS>
 static void launch_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* loc, const int32_t* uptr,
-                      const int32_t* urows, int64_t plan_total, int64_t rows, int nsplit, int64_t per,
-                      float* partial, hipStream_t st) {
+                      const int32_t* urows, int64_t plan_total, int64_t rows, int ca, int cb, int nsplit,
+                      int64_t per, float* partial, hipStream_t st) {
   const int64_t tiles = cdiv(rows, kWpRows);
-  hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS>), dim3(nsplit * GROUPS),
-                     dim3(256), 0, st, (const T*)x, (uint32_t)(rows_x * C * 2), (const T*)g,
-                     (uint32_t)(rows * C * 2), loc, (uint32_t)(tiles * kWpRows * KK * 2), uptr, urows,
-                     (uint32_t)(plan_total * 4), tiles, per, nsplit, partial, g_wp_dbg);
+  const uint32_t xb = (uint32_t)(rows_x * ca * 2), gb = (uint32_t)(rows * cb * 2);
+  const uint32_t lb = (uint32_t)(tiles * kWpRows * KK * 2), ub = (uint32_t)(plan_total * 4);
+  if (ca == C && cb == C)
+    hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS, false>), dim3(nsplit * GROUPS),
+                       dim3(256), 0, st, (const T*)x, xb, (const T*)g, gb, loc, lb, uptr, urows, ub, tiles, per,
+                       nsplit, ca, cb, partial, g_wp_dbg);
+  else if constexpr (C == 64)
+    hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS, true>),
+                       dim3(nsplit * GROUPS, (ca / C) * (cb / C)), dim3(256), 0, st, (const T*)x, xb, (const T*)g,
+                       gb, loc, lb, uptr, urows, ub, tiles, per, nsplit, ca, cb, partial, g_wp_dbg);
 }
 
 template <typename T>
 static int run_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* loc, const int32_t* uptr,
-                  const int32_t* urows, int64_t plan_total, int64_t rows, int K, int c, int out_transposed,
-                  void* gw, void* ws, int64_t ws_bytes, hipStream_t st) {
+                  const int32_t* urows, int64_t plan_total, int64_t rows, int K, int ca, int cb,
+                  int out_transposed, void* gw, void* ws, int64_t ws_bytes, hipStream_t st) {
   const int n_cu = wp_cu_count();
   if (n_cu <= 0) {
     set_error("conv_wgrad_planned: cannot query the device");
     return OCNN_ERR_HIP;
   }
-  const int nsplit = wp_splits(K, c, n_cu);
+  const int nsplit = wp_splits(K, ca, cb, n_cu);
   const int64_t tiles = cdiv(rows, kWpRows);
   const int64_t per = std::max<int64_t>(1, cdiv(tiles, nsplit));
   const int used = (int)cdiv(tiles, per);                 // ranges that hold tiles
-  if (ws_bytes < (int64_t)used * K * c * c * 4) {
+  if (ws_bytes < (int64_t)used * K * ca * cb * 4) {
     set_error("conv_wgrad_planned: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
   float* partial = (float*)ws;
   if (rows > 0) {
 #define OCNN_WP_LAUNCH(CC, KK, NF, NH, GR) \
-  launch_wp<T, CC, KK, NF, NH, GR>(x, rows_x, g, loc, uptr, urows, plan_total, rows, nsplit, per, partial, st)
-    if (c == 64) {
+  launch_wp<T, CC, KK, NF, NH, GR>(x, rows_x, g, loc, uptr, urows, plan_total, rows, ca, cb, nsplit, per, partial, st)
+    if (ca >= 64) {
       if (K == 27) OCNN_WP_LAUNCH(64, 27, 3, 1, 2);
       else if (K == 9) OCNN_WP_LAUNCH(64, 9, 2, 1, 1);
       else if (K == 8) OCNN_WP_LAUNCH(64, 8, 2, 0, 1);
@@ -481,7 +501,7 @@ static int run_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* 
     }
 #undef OCNN_WP_LAUNCH
   }
-  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, c, c, out_transposed, (T*)gw, st);
+  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, ca, cb, out_transposed, (T*)gw, st);
   return check_launch("conv_wgrad_planned");
 }
 
@@ -497,8 +517,8 @@ extern "C" int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x,
                "conv_wgrad_planned: rows out of range");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
-    return run_wp<f16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, out_transposed, gw, workspace,
+    return run_wp<f16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, cb, out_transposed, gw, workspace,
                        workspace_bytes, st);
-  return run_wp<bf16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, out_transposed, gw, workspace,
+  return run_wp<bf16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, cb, out_transposed, gw, workspace,
                       workspace_bytes, st);
 }

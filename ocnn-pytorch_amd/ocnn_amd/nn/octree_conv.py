@@ -89,7 +89,7 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None):
   code = _lib.DTYPE_CODE.get(x.dtype, -1)
   if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
                                                               plan.umax):
-    ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K), x.device)
+    ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K, ca, cb), x.device)
     _lib.check(L.ocnn_conv_wgrad_planned(
         code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, ca, cb, int(out_transposed),

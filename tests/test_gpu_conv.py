@@ -401,6 +401,31 @@ def test_planned_64x64_kernels(dtype, K, ch):
     assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('K,ca,cb', [(27, 128, 128), (27, 64, 192), (9, 256, 64), (8, 128, 64), (3, 192, 128)])
+def test_planned_wgrad_channel_blocks(dtype, K, ca, cb):
+  """Weight gradient of layers with more than 64 channels: the planned kernel sums one
+  64 x 64 block of channel pairs per workgroup."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(K + ca)
+  for rows, rows_in in [(1000, 1000), (128 * 70 + 5, 5000)]:
+    say('wgrad blocks', dtype, K, ca, cb, rows, rows_in)
+    table = _local_table(rows, rows_in, K, g)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+    assert L.ocnn_conv_wgrad_planned_supported(code, rows_in, rows, K, ca, cb, plan.umax)
+    x = torch.randn(rows_in, ca, generator=g).to(dtype)
+    gr = torch.randn(rows, cb, generator=g).to(dtype)
+    want = C.weight_gemm(f64(x), f64(gr), table.numpy().astype(np.int64))
+    gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+    assert rel_err(gw, want) < TOL[dtype]
+    gwt = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, True, plan)
+    assert torch.equal(gwt, gw.transpose(1, 2).contiguous())
+    assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
+
+
 @pytest.mark.parametrize('ch', [64, 32])
 def test_planned_kernels_at_the_staging_limit(ch):
   """Tiles with exactly as many distinct rows as the persistent kernels stage (the last
