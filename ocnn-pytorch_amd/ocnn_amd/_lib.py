@@ -48,6 +48,9 @@ SIGNATURES = {
     'ocnn_conv_gather_rw_supported': (_i, [_i, _l, _i, _i, _i, _i]),
     'ocnn_conv_gather_rw': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                  _p, _l, _p]),
+    'ocnn_conv_gather_wide_supported': (_i, [_i, _l, _i, _i, _i, _i]),
+    'ocnn_conv_gather_wide': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
+                                   _p, _l, _p]),
     'ocnn_set_wgrad_transpose_load': (None, [_i]),
     'ocnn_conv_wgrad_workspace_bytes': (_l, [_l, _i, _i, _i]),
     'ocnn_conv_wgrad_workspace_bytes_for': (_l, [_i, _l, _l, _i, _i, _i]),

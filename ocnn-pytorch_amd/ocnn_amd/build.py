@@ -20,6 +20,7 @@ SOURCES = {
     'conv.hip': [],
     'conv_staged.hip': [],
     'conv_rw.hip': [],
+    'conv_wide.hip': [],
     'wgrad_planned.hip': [],
     'plan.hip': [],
     'misc.hip': [],

@@ -24,6 +24,7 @@ from .octree_pad import octree_depad, octree_pad
 
 
 PAD_MIN_ROWS = 16384     # from this many table rows on, odd channel counts are zero-padded
+USE_WIDE = True          # the wide-layer gather kernel (switch for comparisons)
 
 
 def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None):
@@ -53,6 +54,13 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   ws = _lib.workspace(nbytes, data.device)
   if plan is not None and L.ocnn_conv_gather_rw_supported(code, rows_in, K, cin, cout, plan.umax):
     _lib.check(L.ocnn_conv_gather_rw(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
+        _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
+        int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return out
+  if plan is not None and plan.reuse >= 2.0 and USE_WIDE and L.ocnn_conv_gather_wide_supported(
+      code, rows_in, K, cin, cout, plan.umax):
+    _lib.check(L.ocnn_conv_gather_wide(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
         int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))

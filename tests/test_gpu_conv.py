@@ -401,6 +401,51 @@ def test_planned_64x64_kernels(dtype, K, ch):
     assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
 
 
+def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
+  """ocnn_conv_gather_wide through the C ABI (the Python layer picks it only for plans with
+  enough reuse)."""
+  L = _lib.lib()
+  rows, K = table.shape
+  cin = x.shape[1]
+  code = _lib.dtype_code(x)
+  assert L.ocnn_conv_gather_wide_supported(code, rows_in, K, cin, cout, plan.umax)
+  out = torch.empty((rows, cout), dtype=x.dtype, device=x.device)
+  ws = torch.empty(K * cin * cout * 2, dtype=torch.uint8, device=x.device)
+  _lib.check(L.ocnn_conv_gather_wide(
+      code, _lib.ptr(x), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax,
+      plan.total, rows, K, _lib.ptr(w), cin, cout, int(transposed), int(reverse), _lib.ptr(bias),
+      _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  return out
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('K,cin,cout', [(27, 128, 128), (27, 64, 256), (9, 192, 128), (8, 128, 384), (3, 256, 256),
+                                        (1, 64, 128)])
+def test_wide_gather_kernel(dtype, K, cin, cout):
+  """Gather-GEMM for wide layers (weights streamed into registers, rows staged 64 input
+  channels at a time), both output-channel widths per workgroup, with bias, and the
+  transposed + mirrored form, against the oracle."""
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(7 * K + cin)
+  for rows, rows_in in [(1000, 1000), (130, 150), (128 * 40 + 1, 3000)]:
+    say('wide gather', dtype, K, cin, cout, rows, rows_in)
+    table = _local_table(rows, rows_in, K, g)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    t64 = table.numpy().astype(np.int64)
+    x = torch.randn(rows_in, cin, generator=g).to(dtype)
+    w = (torch.randn(K, cin, cout, generator=g) / (K * cin) ** 0.5).to(dtype)
+    b = torch.randn(cout, generator=g).to(dtype)
+    got = _gather_wide(x.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV))
+    want = C.forward_gemm(f64(x), f64(w), t64) + f64(b)
+    assert rel_err(got, want) < TOL[dtype]
+    if cin % 128 == 0:                                   # the data gradient: cout -> cin
+      gr = torch.randn(rows_in, cout, generator=g).to(dtype)
+      got = _gather_wide(gr.to(DEV), rows_in, tg, plan, w.to(DEV), cin, True, True, None)
+      want = C.forward_gemm(f64(gr), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
+      assert rel_err(got, want) < TOL[dtype]
+
+
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('K,ca,cb', [(27, 128, 128), (27, 64, 192), (9, 256, 64), (8, 128, 64), (3, 192, 128)])
 def test_planned_wgrad_channel_blocks(dtype, K, ca, cb):
