@@ -277,6 +277,26 @@ int ocnn_dwconv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
                       void* gw, void* workspace, int64_t workspace_bytes,
                       void* stream);
 
+/* The depth-wise engine over the tile plan of the table (same reference lines, same
+ * results up to the fp32 summation order, which is fixed): the distinct rows of a tile
+ * are staged once in LDS, 64 channels at a time.  f16 / bf16, channels a multiple of 64,
+ * plan_max_distinct <= 416; the weight gradient for K in {27, 9, 8, 3}. */
+int ocnn_dwconv_gather_planned_supported(int dtype, int64_t rows_in, int K, int channels,
+                                         int plan_max_distinct);
+int ocnn_dwconv_gather_planned(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,
+                               const int32_t* uptr, const int32_t* urows, int plan_max_distinct,
+                               int64_t plan_total, int64_t rows_out, int K, const void* w,
+                               int channels, int reverse_slots, const void* bias, void* out,
+                               void* stream);
+int ocnn_dwconv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K,
+                                        int channels, int plan_max_distinct);
+int64_t ocnn_dwconv_wgrad_planned_workspace_bytes(int K, int channels);
+int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const void* g,
+                              const uint16_t* loc, const int32_t* uptr, const int32_t* urows,
+                              int plan_max_distinct, int64_t plan_total, int64_t rows, int K,
+                              int channels, void* gw, void* workspace, int64_t workspace_bytes,
+                              void* stream);
+
 /* ocnn/nn/octree_pad.py:13-39.  pad: out (n, c) = val except out[q] =
  * data[children[q]] where children[q] >= 0; depad: out[children[q]] = data[q]. */
 int ocnn_pad(int dtype, const void* data, const int32_t* children, int64_t n,

@@ -60,6 +60,11 @@ SIGNATURES = {
     'ocnn_conv_wgrad_planned': (_i, [_i, _p, _l, _p, _p, _p, _p, _i, _l, _l, _i, _i, _i, _i, _p, _p,
                                      _l, _p]),
     'ocnn_dwconv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _p, _p, _p]),
+    'ocnn_dwconv_gather_planned_supported': (_i, [_i, _l, _i, _i, _i]),
+    'ocnn_dwconv_gather_planned': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _p, _p, _p]),
+    'ocnn_dwconv_wgrad_planned_supported': (_i, [_i, _l, _l, _i, _i, _i]),
+    'ocnn_dwconv_wgrad_planned_workspace_bytes': (_l, [_i, _i]),
+    'ocnn_dwconv_wgrad_planned': (_i, [_i, _p, _l, _p, _p, _p, _p, _i, _l, _l, _i, _i, _p, _p, _l, _p]),
     'ocnn_dwconv_wgrad_workspace_bytes': (_l, [_l, _i, _i]),
     'ocnn_dwconv_wgrad': (_i, [_i, _p, _l, _p, _p, _l, _i, _i, _p, _p, _l, _p]),
     'ocnn_pad': (_i, [_i, _p, _p, _l, _i, _f, _p, _p]),

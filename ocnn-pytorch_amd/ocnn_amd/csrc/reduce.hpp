@@ -23,11 +23,13 @@ __global__ void wgrad_reduce_kernel(const float* __restrict__ partial, int split
   out[o] = from_f32<T>(acc);
 }
 
-// The same for per % 4 == 0 and untransposed output: 16 bytes per thread and eight loads
+// The same for cb % 4 == 0: 16 bytes per thread and eight loads
 // in flight; the additions stay in split order, so the result has the same bits.
+// With ca > 0 the output is (K, cb, ca): the four sums of a thread (consecutive b) go to
+// four rows of the transposed block.
 template <typename T>
 __global__ void wgrad_reduce4_kernel(const float* __restrict__ partial, int splits, int64_t per,
-                                     T* __restrict__ out) {
+                                     T* __restrict__ out, int ca, int cb) {
   typedef __attribute__((ext_vector_type(4))) float v4;
   int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (e >= per) return;
@@ -41,8 +43,16 @@ __global__ void wgrad_reduce4_kernel(const float* __restrict__ partial, int spli
     for (int i = 0; i < 8; ++i) acc += v[i];
   }
   for (; s < splits; ++s) acc += *(const v4*)(partial + (int64_t)s * per + e);
+  if (ca > 0) {
+    const int b = (int)(e % cb);
+    const int a = (int)((e / cb) % ca);
+    const int64_t k = e / ((int64_t)ca * cb);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) out[e + i] = from_f32<T>(acc[i]);
+    for (int i = 0; i < 4; ++i) out[(k * cb + b + i) * ca + a] = from_f32<T>(acc[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[e + i] = from_f32<T>(acc[i]);
+  }
 }
 
 // launches the reduction that fits
@@ -50,9 +60,9 @@ template <typename T>
 inline void launch_wgrad_reduce(const float* partial, int splits, int K, int ca, int cb,
                                 int out_transposed, T* out, hipStream_t st) {
   const int64_t per = (int64_t)K * ca * cb;
-  if (!out_transposed && per % 4 == 0 && ((uintptr_t)partial % 16) == 0) {
+  if (cb % 4 == 0 && ((uintptr_t)partial % 16) == 0) {
     hipLaunchKernelGGL(wgrad_reduce4_kernel<T>, dim3((unsigned)cdiv(per / 4, 64)), dim3(64), 0, st, partial,
-                       splits, per, out);
+                       splits, per, out, out_transposed ? ca : 0, cb);
   } else {
     hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3((unsigned)cdiv(per, 256)), dim3(256), 0, st, partial,
                        splits, K, ca, cb, out_transposed, out);

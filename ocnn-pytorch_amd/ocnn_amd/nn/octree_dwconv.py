@@ -12,21 +12,33 @@ from .octree_conv import OctreeConvBase
 from .octree_pad import octree_pad
 
 
-def dw_gather(data, rows_in, table, w, reverse, bias=None):
-  """out[i,c] = sum_k data[T[i,k],c] * w[k',c]."""
+def dw_gather(data, rows_in, table, w, reverse, bias=None, plan=None):
+  """out[i,c] = sum_k data[T[i,k],c] * w[k',c].  With a tile plan of the same table (and a
+  supported shape) the kernel that stages a tile's rows in LDS runs."""
   _lib.require_gpu(data, table, w)
+  L = _lib.lib()
   data, w, table = data.contiguous(), w.contiguous(), table.contiguous()
   rows, K = table.shape
   C = data.shape[1]
   assert w.numel() == K * C and w.dtype == data.dtype and table.dtype == torch.int32
+  if bias is not None:
+    bias = bias.to(data.dtype).contiguous()
   out = torch.empty((rows, C), dtype=data.dtype, device=data.device)
-  _lib.check(_lib.lib().ocnn_dwconv_gather(
+  code = _lib.DTYPE_CODE.get(data.dtype, -1)
+  if plan is not None and plan.reuse >= 2.0 and L.ocnn_dwconv_gather_planned_supported(
+      code, rows_in, K, C, plan.umax):
+    _lib.check(L.ocnn_dwconv_gather_planned(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
+        plan.umax, plan.total, rows, K, _lib.ptr(w), C, int(reverse), _lib.ptr(bias), _lib.ptr(out),
+        _lib.stream()))
+    return out
+  _lib.check(L.ocnn_dwconv_gather(
       _lib.dtype_code(data), _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(w), C,
       int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.stream()))
   return out
 
 
-def dw_wgrad(x, g, table):
+def dw_wgrad(x, g, table, plan=None):
   """gw[k,0,c] = sum_i x[T[i,k],c] * g[i,c]."""
   _lib.require_gpu(x, g, table)
   L = _lib.lib()
@@ -35,6 +47,15 @@ def dw_wgrad(x, g, table):
   C = x.shape[1]
   assert g.shape == (rows, C) and x.dtype == g.dtype
   gw = torch.empty((K, 1, C), dtype=x.dtype, device=x.device)
+  code = _lib.DTYPE_CODE.get(x.dtype, -1)
+  if plan is not None and plan.reuse >= 2.0 and L.ocnn_dwconv_wgrad_planned_supported(
+      code, x.shape[0], rows, K, C, plan.umax):
+    ws = _lib.workspace(L.ocnn_dwconv_wgrad_planned_workspace_bytes(K, C), x.device)
+    _lib.check(L.ocnn_dwconv_wgrad_planned(
+        code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
+        _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, C, _lib.ptr(gw), _lib.ptr(ws), ws.numel(),
+        _lib.stream()))
+    return gw
   ws = _lib.workspace(L.ocnn_dwconv_wgrad_workspace_bytes(rows, K, C), x.device)
   _lib.check(L.ocnn_dwconv_wgrad(_lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g),
                                  _lib.ptr(table), rows, K, C, _lib.ptr(gw), _lib.ptr(ws),
@@ -52,16 +73,26 @@ class OctreeDWConvBase(OctreeConvBase):
 
   def is_conv_layer(self): return True
 
+  def _dw_plan(self, data, inverse=False):
+    """Tile plan of the table, when the staged depth-wise kernels take the shape."""
+    code = _lib.DTYPE_CODE.get(data.dtype, -1)
+    if not _lib.lib().ocnn_dwconv_gather_planned_supported(code, data.shape[0], self.kdim,
+                                                           data.shape[1], 0):
+      return None
+    return self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse,
+                             self.fine_h)
+
   def forward_gemm(self, data, weights, bias=None):
-    return dw_gather(data, self.fine_h, self.neigh, weights, False, bias)
+    return dw_gather(data, self.fine_h, self.neigh, weights, False, bias, self._dw_plan(data))
 
   def backward_gemm(self, grad, weights, bias=None):
     if self.symmetric:
-      return dw_gather(grad, grad.shape[0], self.neigh, weights, True, bias)
-    return dw_gather(grad, grad.shape[0], self._inverse_table(), weights, False, bias)
+      return dw_gather(grad, grad.shape[0], self.neigh, weights, True, bias, self._dw_plan(grad))
+    return dw_gather(grad, grad.shape[0], self._inverse_table(), weights, False, bias,
+                     self._dw_plan(grad, inverse=True))
 
   def weight_gemm(self, data, grad, out_transposed=False):
-    return dw_wgrad(data, grad, self.neigh)
+    return dw_wgrad(data, grad, self.neigh, self._dw_plan(data))
 
 
 class OctreeDWConvFunction(Function):

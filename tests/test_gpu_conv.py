@@ -546,6 +546,39 @@ def test_planned_kernels_fall_back_on_large_tiles():
   assert rel_err(gw, C.weight_gemm(f64(x), f64(gr), t64)) < 2e-2
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('K,ch', [(27, 64), (27, 192), (9, 128), (8, 64), (3, 128), (5, 64)])
+def test_dwconv_planned_kernels(dtype, K, ch):
+  """Depth-wise kernels on the tile plan (rows staged in LDS): gather with bias, with mirrored
+  slots, and the weight gradient (the slot counts it is built for), against the oracle."""
+  from ocnn_amd.nn.octree_dwconv import dw_gather, dw_wgrad
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(11 * K + ch)
+  code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+  for rows, rows_in in [(1000, 1000), (130, 150), (128 * 50 + 7, 4000)]:
+    say('dwconv planned', dtype, K, ch, rows, rows_in)
+    table = _local_table(rows, rows_in, K, g)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    plan.reuse = 10.0                                    # take the staged kernels whatever the table's reuse
+    t64 = table.numpy().astype(np.int64)
+    assert L.ocnn_dwconv_gather_planned_supported(code, rows_in, K, ch, plan.umax)
+    x = torch.randn(rows_in, ch, generator=g).to(dtype)
+    w = torch.randn(K, 1, ch, generator=g).to(dtype)
+    b = torch.randn(ch, generator=g).to(dtype)
+    gr = torch.randn(rows, ch, generator=g).to(dtype)
+    got = dw_gather(x.to(DEV), rows_in, tg, w.to(DEV), False, b.to(DEV), plan)
+    assert rel_err(got, C.dw_forward(f64(x), f64(w), t64) + f64(b)) < TOL[dtype]
+    got = dw_gather(x.to(DEV), rows_in, tg, w.to(DEV), True, None, plan)
+    assert rel_err(got, C.dw_forward(f64(x), f64(w)[::-1], t64)) < TOL[dtype]
+    if K in (27, 9, 8, 3):
+      assert L.ocnn_dwconv_wgrad_planned_supported(code, rows_in, rows, K, ch, plan.umax)
+    gw = dw_wgrad(x.to(DEV), gr.to(DEV), tg, plan)
+    assert rel_err(gw, C.dw_weight(f64(x), f64(gr), t64)) < TOL[dtype]
+    assert torch.equal(gw, dw_wgrad(x.to(DEV), gr.to(DEV), tg, plan))
+
+
 def test_dwconv_all_slot_kernels(medium):
   """Depth-wise kernels that keep all slots of a row in one thread (power-of-two channel
   counts), every slot count, fp32 and 16-bit, against the oracle."""
