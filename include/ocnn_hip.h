@@ -225,6 +225,16 @@ int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint
                           int w_transposed, int reverse_slots, const void* bias, void* out,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* out (rows, cout) = in (rows, cin) W (+ bias): ocnn_conv_gather with the one-slot identity
+ * table, the form that the 2x2x2 stride-2 layers over all nodes take on the (parents, 8 C)
+ * view of the children (ocnn/nn/octree_conv.py:115-168 with neigh[p] = 8p .. 8p+7).
+ * w: (cin, cout), or (cout, cin) with w_transposed.  f16 / bf16, cin % 64 == 0 (<= 1024),
+ * cout % 128 == 0; workspace cin * cout * 2 bytes. */
+int ocnn_conv_dense_supported(int dtype, int64_t rows, int cin, int cout);
+int ocnn_conv_dense(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
+                    int w_transposed, const void* bias, void* out, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+
 /* Selects how the MFMA weight-gradient kernel reads its LDS tiles: 1 (default)
  * = transposing LDS loads, 0 = 16-bit loads.  Same results either way. */
 void ocnn_set_wgrad_transpose_load(int on);

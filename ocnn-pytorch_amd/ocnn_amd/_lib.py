@@ -51,6 +51,8 @@ SIGNATURES = {
     'ocnn_conv_gather_wide_supported': (_i, [_i, _l, _i, _i, _i, _i]),
     'ocnn_conv_gather_wide': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                    _p, _l, _p]),
+    'ocnn_conv_dense_supported': (_i, [_i, _l, _i, _i]),
+    'ocnn_conv_dense': (_i, [_i, _p, _l, _p, _i, _i, _i, _p, _p, _p, _l, _p]),
     'ocnn_set_wgrad_transpose_load': (None, [_i]),
     'ocnn_conv_wgrad_workspace_bytes': (_l, [_l, _i, _i, _i]),
     'ocnn_conv_wgrad_workspace_bytes_for': (_l, [_i, _l, _l, _i, _i, _i]),

@@ -188,6 +188,117 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Dense rows (one slot, row i reads row i): out = in W (+ bias), the form a 2x2x2 stride-2
+// layer over all nodes takes on the (parents, 8 C) view of its children.  HBM-bound: a
+// workgroup brings its 32 RB rows in whole (all input channels, one burst of global->LDS
+// loads), then multiplies as above; two workgroups per CU overlap one's loads with the
+// other's MFMAs.  Weights: the packed layout above with K = 1.
+// ---------------------------------------------------------------------------------------
+template <typename T, int RB, int MB>
+__global__ __launch_bounds__(256, 2) void conv_dense_kernel(
+    const T* __restrict__ in, uint32_t in_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
+    T* __restrict__ out, int64_t rows, int cin, int cout) {
+  constexpr int RT = 32 * RB;
+  extern __shared__ __attribute__((aligned(16))) char s_dyn[];     // [chunk][RT rows][128 B]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int q = lane >> 5, r32 = lane & 31;
+  const int ncc = cin >> 6;
+  const int cg0 = ((int)blockIdx.y * 4 + wave) * MB;
+  const int64_t row0 = (int64_t)blockIdx.x * RT;
+  const uint32_t pitch = (uint32_t)cin * 2u;
+
+  // ---- all rows of the tile -> LDS; rows past the end read zeros (out of range) ----
+  {
+    const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
+    const int rl = lane >> 3;                                       // row within a piece of 8
+    const int pieces = ncc * (RT / 8);
+    for (int i = wave; i < pieces; i += 4) {
+      const int cc = i / (RT / 8), g = i - cc * (RT / 8);
+      const uint32_t swz = (uint32_t)((4 * g + (lane >> 4)) & 7);
+      const uint32_t src = (uint32_t)(row0 + 8 * g + rl) * pitch + (uint32_t)cc * 128u +
+                           (((uint32_t)(lane & 7) ^ swz) << 4);
+      wd_dma16(rs_in, s_dyn + (cc * RT + 8 * g) * 128, src);
+    }
+  }
+
+  f32x16 acc[RB][MB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rb][mb][r] = 0.f;
+
+  // A: weights of k-step t = 4 cc + s, fetched D = R - 1 k-steps ahead into a ring of R (64
+  // registers whatever MB): a k-step is only RB MB MFMAs long, an L2 round trip is many of them
+  constexpr int R = 16 / MB, D = R - 1;
+  const int nsub = 4 * ncc;
+  const T* wbase = wpk + (int64_t)cg0 * 2048 + lane * 8;
+  const int64_t kstride = (int64_t)(cout >> 5) * 2048;       // elements between consecutive chunks
+  u32x4 A[R][MB];
+  auto load_a = [&](int t, u32x4 (&a)[MB]) {
+    const int tc = min(t, nsub - 1);
+    const T* p = wbase + (int64_t)(tc >> 2) * kstride + (tc & 3) * 512;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) a[mb] = *(const u32x4*)(p + mb * 2048);
+  };
+  uint32_t pvb[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const uint32_t l = (uint32_t)(32 * rb + r32);
+    pvb[rb] = (l << 7) | (((l << 3) & 0x70u) ^ ((uint32_t)q << 4));
+  }
+  u32x4 Bb[2][RB];
+  auto read_b = [&](int t, u32x4 (&b)[RB]) {
+    const int tc = min(t, nsub - 1);
+    const char* base = s_dyn + (tc >> 2) * (RT * 128);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) b[rb] = *(const u32x4*)(base + (pvb[rb] ^ ((uint32_t)(tc & 3) << 5)));
+  };
+
+#pragma unroll
+  for (int t = 0; t < D; ++t) load_a(t, A[t]);               // (the rows are still in flight)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  read_b(0, Bb[0]);
+  for (int t0 = 0; t0 < nsub; t0 += R) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int t = t0 + j;
+      if (t < nsub) {
+        load_a(t + D, A[(j + D) % R]);
+        read_b(t + 1, Bb[(j + 1) & 1]);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[j][mb], Bb[j & 1][rb], acc[rb][mb]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int co = 32 * (cg0 + mb) + 16 * q;
+    float bv[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bv[r] = bias ? to_f32(bias[co + r]) : 0.f;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int64_t row = row0 + 32 * rb + r32;
+      if (row >= rows) continue;
+      unsigned pk[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) pk[r] = pack2<T>(acc[rb][mb][2 * r] + bv[2 * r], acc[rb][mb][2 * r + 1] + bv[2 * r + 1]);
+      T* dst = out + row * cout + co;
+      *(u32x4*)(dst) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+      *(u32x4*)(dst + 8) = u32x4{pk[4], pk[5], pk[6], pk[7]};
+    }
+  }
+}
+
 }  // namespace ocnn
 
 using namespace ocnn;
@@ -243,4 +354,68 @@ extern "C" int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in,
                          bias, out, workspace, st);
   return run_wide<bf16>(in, rows_in, loc, uptr, urows, rows_out, K, cin, cout, w, w_transposed, reverse_slots,
                         bias, out, workspace, st);
+}
+
+// ---- dense rows ----
+struct DensePlan { int rb, mb; };
+static DensePlan dense_plan(int cin, int cout) {
+  DensePlan p;
+  const int cap = std::max(1, 32768 / cin / 32);             // 32-row blocks whose rows fit 64 KiB of LDS
+  if (cout % 512 == 0) { p.mb = 4; p.rb = std::min(2, cap); }
+  else if (cout % 256 == 0) { p.mb = 2; p.rb = std::min(4, cap); }
+  else { p.mb = 1; p.rb = std::min(4, cap); }
+  if (p.rb == 3) p.rb = 2;
+  return p;
+}
+
+extern "C" int ocnn_conv_dense_supported(int dtype, int64_t rows, int cin, int cout) {
+  if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
+  if (cin < 64 || cin % 64 != 0 || cin > 1024 || cout < 128 || cout % 128 != 0 || cout > 4096) return 0;
+  if (((int64_t)rows + 128) * cin * 2 > 0xfff00000ll) return 0;
+  return 1;
+}
+
+template <typename T, int RB, int MB>
+static void launch_dense(const void* in, int64_t rows, int cin, int cout, const void* ws, const void* bias,
+                         void* out, hipStream_t st) {
+  const size_t lds = (size_t)32 * RB * cin * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)conv_dense_kernel<T, RB, MB>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((conv_dense_kernel<T, RB, MB>), dim3((unsigned)cdiv(rows, 32 * RB), (unsigned)(cout / (128 * MB))),
+                     dim3(256), lds, st, (const T*)in, (uint32_t)(rows * cin * 2), (const T*)ws, (const T*)bias,
+                     (T*)out, rows, cin, cout);
+}
+
+template <typename T>
+static int run_dense(const void* in, int64_t rows, const void* w, int cin, int cout, int w_transposed,
+                     const void* bias, void* out, void* ws, hipStream_t st) {
+  const int64_t total = (int64_t)cin * cout;
+  hipLaunchKernelGGL(pack_weights_wide_kernel<T>, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, st,
+                     (const T*)w, (T*)ws, 1, cin, cout, w_transposed, 0);
+  const DensePlan p = dense_plan(cin, cout);
+#define OCNN_DENSE_CASE(RB_, MB_) \
+  if (p.rb == RB_ && p.mb == MB_) { launch_dense<T, RB_, MB_>(in, rows, cin, cout, ws, bias, out, st); return check_launch("conv_dense"); }
+  OCNN_DENSE_CASE(4, 1) OCNN_DENSE_CASE(2, 1) OCNN_DENSE_CASE(1, 1)
+  OCNN_DENSE_CASE(4, 2) OCNN_DENSE_CASE(2, 2) OCNN_DENSE_CASE(1, 2)
+  OCNN_DENSE_CASE(2, 4) OCNN_DENSE_CASE(1, 4)
+#undef OCNN_DENSE_CASE
+  set_error("conv_dense: no kernel for rb=%d mb=%d", p.rb, p.mb);
+  return OCNN_ERR_ARG;
+}
+
+extern "C" int ocnn_conv_dense(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
+                               int w_transposed, const void* bias, void* out, void* workspace,
+                               int64_t workspace_bytes, void* stream) {
+  OCNN_REQUIRE(ocnn_conv_dense_supported(dtype, rows, cin, cout), "conv_dense: shape not supported");
+  if (rows <= 0) return OCNN_OK;
+  if (workspace_bytes < (int64_t)cin * cout * 2) {
+    set_error("conv_dense: workspace too small");
+    return OCNN_ERR_WORKSPACE;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == OCNN_F16) return run_dense<f16>(in, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+  return run_dense<bf16>(in, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
 }

@@ -27,9 +27,10 @@ PAD_MIN_ROWS = 16384     # from this many table rows on, odd channel counts are 
 USE_WIDE = True          # the wide-layer gather kernel (switch for comparisons)
 
 
-def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None):
+def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False):
   """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K)).  With a
-  tile plan of the same table (and a supported shape) the staged kernel runs."""
+  tile plan of the same table (and a supported shape) the staged kernel runs.
+  dense: the table is the one-slot identity (row i reads row i)."""
   _lib.require_gpu(data, table, W)
   L = _lib.lib()
   data, W, table = data.contiguous(), W.contiguous(), table.contiguous()
@@ -52,6 +53,13 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   code = _lib.dtype_code(data)
   nbytes = L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout)
   ws = _lib.workspace(nbytes, data.device)
+  # (many input channels into few output channels: the row tile that fits LDS is small and
+  # the weights are streamed once per tile; the plan-free kernel is no slower there)
+  if (dense and K == 1 and rows == rows_in and not (cin >= 512 and cout < 256) and
+      L.ocnn_conv_dense_supported(code, rows, cin, cout)):
+    _lib.check(L.ocnn_conv_dense(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed),
+                                 _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return out
   if plan is not None and L.ocnn_conv_gather_rw_supported(code, rows_in, K, cin, cout, plan.umax):
     _lib.check(L.ocnn_conv_gather_rw(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
@@ -210,7 +218,7 @@ class OctreeConvBase:
       P = self.neigh.shape[0]
       return conv_gather(data.view(P, 8 * self.in_conv), P, self._identity(P, data.device),
                          weights.view(1, 8 * self.in_conv, self.out_conv), self.out_conv, False,
-                         False, bias, None)
+                         False, bias, None, dense=True)
     plan = self._plan(data, self.in_conv, self.out_conv)
     return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias,
                        plan)
@@ -223,7 +231,7 @@ class OctreeConvBase:
       b8 = None if bias is None else bias.repeat(8)
       out = conv_gather(grad, P, self._identity(P, grad.device),
                         weights.view(1, 8 * self.in_conv, self.out_conv), 8 * self.in_conv, True,
-                        False, b8, None)
+                        False, b8, None, dense=True)
       return out.view(8 * P, self.in_conv)
     if self.symmetric:
       plan = self._plan(grad, self.out_conv, self.in_conv)

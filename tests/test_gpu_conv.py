@@ -401,6 +401,31 @@ def test_planned_64x64_kernels(dtype, K, ch):
     assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('cin,cout', [(64, 128), (128, 512), (512, 128), (256, 256), (1024, 384), (192, 1024)])
+def test_dense_rows_kernel(dtype, cin, cout):
+  """out = in W + bias on the kernel for one-slot identity tables (every row-block and
+  output-channel tiling it is built with), both weight layouts, ragged row counts."""
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(cin + cout)
+  code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+  for rows in (1, 130, 4133):
+    say('dense rows', dtype, cin, cout, rows)
+    assert L.ocnn_conv_dense_supported(code, rows, cin, cout)
+    x = torch.randn(rows, cin, generator=g).to(dtype)
+    w = (torch.randn(cin, cout, generator=g) / cin ** 0.5).to(dtype)
+    b = torch.randn(cout, generator=g).to(dtype)
+    want = f64(x) @ f64(w) + f64(b)
+    for transposed in (0, 1):
+      wd = (w.t().contiguous() if transposed else w).to(DEV)
+      out = torch.empty((rows, cout), dtype=dtype, device=DEV)
+      ws = torch.empty(cin * cout * 2, dtype=torch.uint8, device=DEV)
+      xd, bd = x.to(DEV), b.to(DEV)
+      _lib.check(L.ocnn_conv_dense(code, _lib.ptr(xd), rows, _lib.ptr(wd), cin, cout, transposed, _lib.ptr(bd),
+                                   _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+      assert rel_err(out, want) < TOL[dtype]
+
+
 def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
   """ocnn_conv_gather_wide through the C ABI (the Python layer picks it only for plans with
   enough reuse)."""
