@@ -235,6 +235,20 @@ int ocnn_conv_dense(int dtype, const void* in, int64_t rows, const void* w, int 
                     int w_transposed, const void* bias, void* out, void* workspace,
                     int64_t workspace_bytes, void* stream);
 
+/* The same GEMM, and its weight gradient gw (ca, cb) [or (cb, ca)] = x^T g, with what is
+ * reused kept in registers by persistent workgroups (weights, resp. the fp32 sums), so that
+ * each tensor crosses L2 once: cin in {64, 128, 256, 512}, cout % 128 == 0; weight gradient
+ * for ca % 512 == 0 and cb % 128 == 0, both % 256 == 0, or ca % 128 == 0 and cb % 512 == 0. */
+int ocnn_conv_dense_rw_supported(int dtype, int64_t rows, int cin, int cout);
+int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
+                       int w_transposed, const void* bias, void* out, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+int ocnn_conv_dense_wgrad_rw_supported(int dtype, int64_t rows, int ca, int cb);
+int64_t ocnn_conv_dense_wgrad_rw_workspace_bytes(int ca, int cb);
+int ocnn_conv_dense_wgrad_rw(int dtype, const void* x, const void* g, int64_t rows, int ca, int cb,
+                             int out_transposed, void* gw, void* workspace,
+                             int64_t workspace_bytes, void* stream);
+
 /* Selects how the MFMA weight-gradient kernel reads its LDS tiles: 1 (default)
  * = transposing LDS loads, 0 = 16-bit loads.  Same results either way. */
 void ocnn_set_wgrad_transpose_load(int on);

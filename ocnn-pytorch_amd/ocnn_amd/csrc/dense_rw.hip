@@ -1,0 +1,467 @@
+// Dense rows (one-slot identity table) with everything that is reused kept in registers:
+// the form a 2x2x2 stride-2 layer over all nodes takes on the (parents, 8 C) view of its
+// children.  These GEMMs are HBM-bound (about 100 flop per byte), so each tensor must cross
+// L2 -> CU once:
+//   * out = in W (+ bias): persistent workgroups keep their slice of W in VGPRs (wave w: all
+//     input channels x its 32 MB output channels) and stream 64-row tiles through a ring of
+//     two to four buffers in LDS;
+//   * dW = in^T g: persistent workgroups keep a 512 x 128 (or 256 x 256, 128 x 512) block of
+//     fp32 sums in accumulator registers (256 per lane) and stream 32-row tiles of both
+//     operands through a ring of three LDS buffers; per-range sums go to the split reduction
+//     (fixed order, no atomics).
+#include <algorithm>
+#include <type_traits>
+
+#include "common.hpp"
+#include "mma.hpp"
+#include "reduce.hpp"
+
+namespace ocnn {
+
+// (Not in the kernel templates: the arguments of the global->LDS load builtin must not be
+// type-dependent expressions.)
+static __device__ __forceinline__ void dr_dma16(__amdgpu_buffer_rsrc_t rs, char* dst, uint32_t off) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)dst, 16, off, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------------
+// out = in W.  Packed weights: [64-channel chunk cc][32 output channels cg][k-step s][lane][8]
+// (the output channels of a block permuted so that the two lanes of a row hold adjacent
+// 16-byte pieces).  LDS: [chunk][row][128 B],
+// 16-byte chunk c of row r at c ^ ((r >> 1) & 7).
+// ---------------------------------------------------------------------------------------
+template <typename T, int NKS, int MB>
+__global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
+    const T* __restrict__ in, uint32_t in_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
+    T* __restrict__ out, int64_t rows, int cout, int64_t tiles, int64_t tiles_per_wg) {
+  constexpr int RB = 2, RT = 32 * RB, NCC = NKS / 4, CIN = 16 * NKS;
+  constexpr int BUF = NCC * RT * 128;
+  constexpr int NBUF = NCC >= 8 ? 2 : 4;                           // tiles resident in LDS
+  extern __shared__ __attribute__((aligned(16))) char s_dyn[];     // NBUF buffers
+  __shared__ __attribute__((aligned(16))) float s_bias[128 * MB];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int q = lane >> 5, r32 = lane & 31;
+  const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_wg;
+  const int64_t t_end = min(tiles, t_begin + tiles_per_wg);
+  if (t_begin >= t_end) return;
+  const int ncg = cout >> 5;
+  const int cg0 = ((int)blockIdx.y * 4 + wave) * MB;
+
+  // ---- this wave's weights -> registers, once ----
+  u32x4 wreg[NKS][MB];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      wreg[ks][mb] = *(const u32x4*)(wpk + ((int64_t)(((ks >> 2) * ncg + cg0 + mb) * 4 + (ks & 3)) * 64 + lane) * 8);
+
+  const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
+  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(out, (uint32_t)(rows * cout * 2));
+  const int rl = lane >> 3;
+  auto stage = [&](int64_t tile, char* buf) {
+    const uint32_t row0 = (uint32_t)min(tile, tiles) * RT;        // past the table: out of range, zeros
+#pragma unroll
+    for (int j = 0; j < NCC * 2; ++j) {                           // NCC * 8 pieces of 1 KiB, 4 waves
+      const int i = wave + 4 * j;
+      const int cc = i >> 3, g = i & 7;
+      const uint32_t swz = (uint32_t)((4 * g + (lane >> 4)) & 7);
+      dr_dma16(rs_in, buf + (cc * RT + 8 * g) * 128,
+               (row0 + 8 * g + rl) * (uint32_t)(CIN * 2) + (uint32_t)cc * 128u + (((uint32_t)(lane & 7) ^ swz) << 4));
+    }
+  };
+  // B operand of k-step ks, row block rb: 16 bytes of row 32 rb + r32
+  uint32_t pvs[RB][4];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint32_t l = (uint32_t)(32 * rb + r32);
+      pvs[rb][s] = (l << 7) | ((((l << 3) & 0x70u) ^ ((uint32_t)q << 4)) ^ ((uint32_t)s << 5));
+    }
+
+  // ---- ring of NBUF tiles: tile i is multiplied while i + 1 .. i + NBUF - 1 are in flight ----
+  // Vector memory operations complete in issue order, so "tile i + 1 has landed" is a count of
+  // the operations issued after its loads: per tile P loads and NST stores, always exactly
+  // (tiles past the range load zeros or rows of another range; rows past the end are stored
+  // out of range and dropped).  NST dropped stores per prologue tile make the count right from
+  // the first tile on.
+  constexpr int P = NCC * 2, NST = RB * MB * 2;
+  constexpr int kWait = (NBUF - 2) * P + (NBUF - 1) * NST;
+  static_assert(kWait <= 63, "vmcnt is a 6-bit counter");
+#pragma unroll
+  for (int v = 0; v < NBUF - 1; ++v) {
+    stage(t_begin + v, s_dyn + v * BUF);
+#pragma unroll
+    for (int j = 0; j < NST; ++j)
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rs_out, 0xfffffff0u, 0, 0);
+  }
+  for (int i = tid; i < 128 * MB; i += 256)
+    s_bias[i] = bias ? to_f32(bias[(int)blockIdx.y * 128 * MB + i]) : 0.f;
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWait) : "memory");
+  __syncthreads();
+
+  int slot = 0;
+  for (int64_t tile = t_begin; tile < t_end; ++tile) {
+    const char* cur = s_dyn + slot * BUF;
+    {
+      const int sn = slot == 0 ? NBUF - 1 : slot - 1;              // the buffer of the tile before
+      stage(tile + NBUF - 1, s_dyn + sn * BUF);
+    }
+    f32x16 acc[RB][MB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rb][mb][r] = 0.f;
+    constexpr int PD = 3;                                         // k-steps a read runs ahead
+    u32x4 Bb[4][RB];
+    auto read_b = [&](int ks, u32x4 (&b)[RB]) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) b[rb] = *(const u32x4*)(cur + (ks >> 2) * (RT * 128) + pvs[rb][ks & 3]);
+    };
+#pragma unroll
+    for (int ks = 0; ks < PD && ks < NKS; ++ks) read_b(ks, Bb[ks & 3]);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (ks + PD < NKS) read_b(ks + PD, Bb[(ks + PD) & 3]);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(wreg[ks][mb], Bb[ks & 3][rb], acc[rb][mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // a lane holds the output channels 8 q .. 8 q + 7 and 16 + 8 q .. of a row per M tile: the
+    // two lanes of a row write 32 contiguous bytes per store
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int cl = 32 * (wave * MB + mb) + 8 * q;               // channel within the workgroup's block
+      const f32x4* b4 = (const f32x4*)(&s_bias[cl]);
+      const f32x4 bv[4] = {b4[0], b4[1], b4[4], b4[5]};
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const uint32_t off = ((uint32_t)(tile * RT + 32 * rb + r32) * (uint32_t)cout +
+                              (uint32_t)((int)blockIdx.y * 128 * MB + cl)) * 2u;
+        unsigned pk[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          pk[r] = pack2<T>(acc[rb][mb][2 * r] + bv[r >> 1][(2 * r) & 3], acc[rb][mb][2 * r + 1] + bv[r >> 1][(2 * r + 1) & 3]);
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{pk[0], pk[1], pk[2], pk[3]}, rs_out, off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{pk[4], pk[5], pk[6], pk[7]}, rs_out, off + 32u, 0, 0);
+      }
+    }
+    // the next tile has landed; every wave is done with this one
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWait) : "memory");
+    __syncthreads();
+    slot = slot == NBUF - 1 ? 0 : slot + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
+}
+
+// ---------------------------------------------------------------------------------------
+// dW = x^T g.  A workgroup sums a block of 128 WA x 512 / WA channel pairs (WA = 4, 2, 1
+// waves along the x channels); a wave 128 x 128 of it (4 x 4 accumulators of 32 x 32).
+// LDS per 32-row tile: [64-channel group][row][128 B], x groups first; the 64-byte halves
+// of the rows 2, 3 (mod 4) are swapped, so that the four rows of a transposing read fall
+// on different banks.  Both operands are read with ds_read_b64_tr_b16.
+// ---------------------------------------------------------------------------------------
+template <typename T, int WA>
+__global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
+    const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes, int ca, int cb,
+    int64_t tiles, int64_t tiles_per_split, float* __restrict__ partial) {
+  constexpr int WB = 4 / WA;
+  constexpr int GA = 2 * WA, GB = 2 * WB, NG = GA + GB;            // 64-channel groups of a tile
+  constexpr int RT = 32, TILE = NG * RT * 128;                     // 40 KiB (32 KiB at WA = 2)
+  constexpr int PW = NG * (RT / 8) / 4;                            // staging pieces per wave and tile
+  extern __shared__ __attribute__((aligned(16))) char s_dyn[];     // ring of three tiles
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave / WB, wb = wave % WB;
+  const int nbb = cb / (128 * WB);
+  const int blk_a = (int)blockIdx.y / nbb, blk_b = (int)blockIdx.y % nbb;
+  const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_split;
+  const int64_t t_end = min(tiles, t_begin + tiles_per_split);
+  if (t_begin >= t_end) return;
+
+  const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(x, x_bytes);
+  const __amdgpu_buffer_rsrc_t rs_g = make_rsrc(g, g_bytes);
+  const uint32_t xp = (uint32_t)ca * 2u, gp = (uint32_t)cb * 2u;
+  const int rl = lane >> 3;
+  // source chunk of the lane: its LDS chunk, with the halves swapped for rows 2, 3 (mod 4)
+  const uint32_t sc = (((uint32_t)(lane & 7) ^ (uint32_t)(4 * ((rl >> 1) & 1))) << 4);
+  auto stage = [&](int64_t tile, char* buf) {                      // every wave issues exactly PW loads
+    const uint32_t row0 = (uint32_t)min(tile, tiles) * RT;        // past the range: past the rows, zeros
+#pragma unroll
+    for (int j = 0; j < PW; ++j) {
+      const int i = wave + 4 * j;
+      const int grp = i >> 2, rg = i & 3;
+      char* dst = buf + (grp * RT + 8 * rg) * 128;
+      const uint32_t row = row0 + 8 * rg + rl;
+      if (grp < GA) dr_dma16(rs_x, dst, row * xp + (uint32_t)((blk_a * GA + grp) * 128) + sc);
+      else dr_dma16(rs_g, dst, row * gp + (uint32_t)((blk_b * GB + grp - GA) * 128) + sc);
+    }
+  };
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[m][n][r] = 0.f;
+
+  // lane (i16, gq): rows 8 q + 4 h + i16 / 4 of a 16-row step, channels 16 (gq & 1) + 4 (i16 & 3) ..
+  const int i16 = lane & 15, gq = lane >> 4, q = lane >> 5, rs = i16 >> 2;
+  const uint32_t byte0 = 32u * (gq & 1) + 8u * (i16 & 3);
+  const uint32_t rowb = (uint32_t)(8 * q + rs) * 128u + byte0;
+  const uint32_t hsw = 64u * ((rs >> 1) & 1);                      // where the first half of this row lives
+  const uint32_t xe = rowb + hsw + (uint32_t)(2 * wa) * (RT * 128), xo = rowb + (64u - hsw) + (uint32_t)(2 * wa) * (RT * 128);
+  const uint32_t ge = rowb + hsw + (uint32_t)(GA + 2 * wb) * (RT * 128), go = rowb + (64u - hsw) + (uint32_t)(GA + 2 * wb) * (RT * 128);
+
+  struct Ops { u32x2 a[4][2], b[4][2]; };
+  auto fetch = [&](const char* buf, int sn, Ops& o) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t off = (uint32_t)((m >> 1) * (RT * 128) + sn * 2048 + h * 512);
+        o.a[m][h] = Mma<T>::read_tr((const T*)(buf + ((m & 1) ? xo : xe) + off));
+        o.b[m][h] = Mma<T>::read_tr((const T*)(buf + ((m & 1) ? go : ge) + off));
+      }
+  };
+  auto mma = [&](const Ops& o) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const u32x4 av = u32x4{o.a[m][0][0], o.a[m][0][1], o.a[m][1][0], o.a[m][1][1]};
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        const u32x4 bv = u32x4{o.b[n][0][0], o.b[n][0][1], o.b[n][1][0], o.b[n][1][1]};
+        acc[m][n] = Mma32<T>::run(av, bv, acc[m][n]);
+      }
+    }
+  };
+
+  // ---- ring of three: tile i is multiplied while i + 1 and i + 2 are in flight ----
+  stage(t_begin, s_dyn);
+  stage(t_begin + 1, s_dyn + TILE);
+  int slot = 0;
+  for (int64_t tile = t_begin; tile < t_end; ++tile) {
+    // own pieces of this tile have landed (those of the next one may be in flight), then
+    // everyone's; every wave is also done with the tile before, whose buffer is filled next
+    if (PW == 10) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __syncthreads();
+    const int s2 = slot >= 1 ? slot - 1 : 2;                       // (slot + 2) % 3
+    stage(tile + 2, s_dyn + s2 * TILE);
+    const char* buf = s_dyn + slot * TILE;
+    Ops o0, o1;
+    fetch(buf, 0, o0);
+    fetch(buf, 1, o1);
+    mma(o0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(o1);
+    __builtin_amdgcn_sched_barrier(0);
+    slot = slot == 2 ? 0 : slot + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
+
+  // ---- per-range sums -> partial[split][a][b] ----
+  float* dst = partial + (int64_t)blockIdx.x * ca * cb;
+  const int a_base = blk_a * 128 * WA + 128 * wa, b_base = blk_b * 128 * WB + 128 * wb;
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int a = a_base + 32 * m + 8 * (r >> 2) + 4 * q + (r & 3);
+        dst[(int64_t)a * cb + b_base + 32 * n + (lane & 31)] = acc[m][n][r];
+      }
+}
+
+}  // namespace ocnn
+
+using namespace ocnn;
+
+static int dr_cu_count() {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+    n_cu = prop.multiProcessorCount;
+  }
+  return n_cu;
+}
+
+// 32-channel output blocks per wave: as many as registers allow (weights cin / 16 * MB * 4
+// registers, sums 2 * MB * 16) among those that divide the output channels
+static int dr_mb(int cin, int cout) {
+  if (cin != 64 && cin != 128 && cin != 256 && cin != 512) return 0;
+  if (cout % 128 != 0) return 0;
+  for (int mb = 4; mb >= 1; mb >>= 1)
+    if (cin * mb <= 512 && cout % (128 * mb) == 0) return mb;
+  return 0;
+}
+
+extern "C" int ocnn_conv_dense_rw_supported(int dtype, int64_t rows, int cin, int cout) {
+  if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
+  if (dr_mb(cin, cout) == 0 || cout > 4096) return 0;
+  if (((int64_t)rows + 128) * std::max(cin, cout) * 2 > 0xfff00000ll) return 0;
+  return 1;
+}
+
+template <typename T, int NKS, int MB>
+static void launch_dense_rw(const void* in, int64_t rows, int cout, const void* ws, const void* bias, void* out,
+                            int n_cu, hipStream_t st) {
+  const int lds = ((NKS / 4) >= 8 ? 2 : 4) * (NKS / 4) * 64 * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)conv_dense_rw_kernel<T, NKS, MB>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    attr_set = true;
+  }
+  const int ny = cout / (128 * MB);
+  const int64_t tiles = cdiv(rows, 64);
+  int64_t wgs = std::min<int64_t>(tiles, std::max(1, n_cu / ny));
+  const int64_t per = cdiv(tiles, wgs);
+  wgs = cdiv(tiles, per);
+  hipLaunchKernelGGL((conv_dense_rw_kernel<T, NKS, MB>), dim3((unsigned)wgs, (unsigned)ny), dim3(256), lds, st,
+                     (const T*)in, (uint32_t)(rows * NKS * 32), (const T*)ws, (const T*)bias, (T*)out, rows, cout,
+                     tiles, per);
+}
+
+template <typename T>
+__global__ void pack_weights_dense_kernel(const T* __restrict__ w, T* __restrict__ out, int cin, int cout,
+                                          int transposed) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= (int64_t)cin * cout) return;
+  int j = (int)(e & 7);
+  int lane = (int)((e >> 3) & 63);
+  int s = (int)((e >> 9) & 3);
+  int64_t rest = e >> 11;
+  const int ncg = cout >> 5;
+  int cg = (int)(rest % ncg);
+  int cc = (int)(rest / ncg);
+  int q = lane >> 5, m = lane & 31;
+  int chan = 64 * cc + 16 * s + 8 * q + j;
+  // M index m = 8 a + 4 q + b is register 4 a + b of the lanes with lane / 32 = q
+  int a = m >> 3;
+  int co = 32 * cg + 16 * (a >> 1) + 8 * ((m >> 2) & 1) + 4 * (a & 1) + (m & 3);
+  out[e] = transposed ? w[(int64_t)co * cin + chan] : w[(int64_t)chan * cout + co];
+}
+
+template <typename T>
+static int run_dense_rw(const void* in, int64_t rows, const void* w, int cin, int cout, int w_transposed,
+                        const void* bias, void* out, void* ws, hipStream_t st) {
+  const int n_cu = dr_cu_count();
+  if (n_cu <= 0) {
+    set_error("conv_dense_rw: cannot query the device");
+    return OCNN_ERR_HIP;
+  }
+  hipLaunchKernelGGL(pack_weights_dense_kernel<T>, dim3((unsigned)cdiv((int64_t)cin * cout, 256)), dim3(256), 0, st,
+                     (const T*)w, (T*)ws, cin, cout, w_transposed);
+  const int mb = dr_mb(cin, cout);
+#define OCNN_DRW(CIN_, MB_) \
+  if (cin == CIN_ && mb == MB_) { launch_dense_rw<T, CIN_ / 16, MB_>(in, rows, cout, ws, bias, out, n_cu, st); return check_launch("conv_dense_rw"); }
+  OCNN_DRW(512, 1) OCNN_DRW(256, 1) OCNN_DRW(256, 2) OCNN_DRW(128, 1) OCNN_DRW(128, 2) OCNN_DRW(128, 4)
+  OCNN_DRW(64, 1) OCNN_DRW(64, 2) OCNN_DRW(64, 4)
+#undef OCNN_DRW
+  set_error("conv_dense_rw: no kernel for cin=%d mb=%d", cin, mb);
+  return OCNN_ERR_ARG;
+}
+
+extern "C" int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
+                                  int w_transposed, const void* bias, void* out, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+  OCNN_REQUIRE(ocnn_conv_dense_rw_supported(dtype, rows, cin, cout), "conv_dense_rw: shape not supported");
+  if (rows <= 0) return OCNN_OK;
+  if (workspace_bytes < (int64_t)cin * cout * 2) {
+    set_error("conv_dense_rw: workspace too small");
+    return OCNN_ERR_WORKSPACE;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == OCNN_F16) return run_dense_rw<f16>(in, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+  return run_dense_rw<bf16>(in, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+}
+
+// ---- weight gradient ----
+// waves along the x channels of a workgroup's block, or 0 if the shape is not taken
+static int dr_wa(int ca, int cb) {
+  if (ca % 512 == 0 && cb % 128 == 0) return 4;
+  if (ca % 256 == 0 && cb % 256 == 0) return 2;
+  if (ca % 128 == 0 && cb % 512 == 0) return 1;
+  return 0;
+}
+
+static int dr_wgrad_splits(int ca, int cb, int n_cu) {
+  const int blocks = ca * cb / 65536;
+  return std::max(1, n_cu / blocks);
+}
+
+extern "C" int ocnn_conv_dense_wgrad_rw_supported(int dtype, int64_t rows, int ca, int cb) {
+  if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
+  if (dr_wa(ca, cb) == 0 || ca > 4096 || cb > 4096) return 0;
+  if (((int64_t)rows + 128) * std::max(ca, cb) * 2 > 0xfff00000ll) return 0;
+  return 1;
+}
+
+extern "C" int64_t ocnn_conv_dense_wgrad_rw_workspace_bytes(int ca, int cb) {
+  const int n_cu = dr_cu_count();
+  if (dr_wa(ca, cb) == 0) return 0;
+  return align_up((int64_t)dr_wgrad_splits(ca, cb, n_cu > 0 ? n_cu : 1024) * ca * cb * 4, 256);
+}
+
+template <typename T, int WA>
+static void launch_dense_wgrad(const void* x, const void* g, int64_t rows, int ca, int cb, int nsplit, int64_t per,
+                               int64_t tiles, float* partial, hipStream_t st) {
+  const int lds = 3 * (2 * WA + 2 * (4 / WA)) * 32 * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)conv_dense_wgrad_rw_kernel<T, WA>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((conv_dense_wgrad_rw_kernel<T, WA>), dim3((unsigned)nsplit, (unsigned)(ca * cb / 65536)),
+                     dim3(256), lds, st, (const T*)x, (uint32_t)(rows * ca * 2), (const T*)g,
+                     (uint32_t)(rows * cb * 2), ca, cb, tiles, per, partial);
+}
+
+template <typename T>
+static int run_dense_wgrad(const void* x, const void* g, int64_t rows, int ca, int cb, int out_transposed, void* gw,
+                           void* ws, int64_t ws_bytes, hipStream_t st) {
+  const int n_cu = dr_cu_count();
+  if (n_cu <= 0) {
+    set_error("conv_dense_wgrad_rw: cannot query the device");
+    return OCNN_ERR_HIP;
+  }
+  const int64_t tiles = cdiv(rows, 32);
+  const int nsplit = dr_wgrad_splits(ca, cb, n_cu);
+  const int64_t per = std::max<int64_t>(1, cdiv(tiles, nsplit));
+  const int used = (int)cdiv(tiles, per);
+  if (ws_bytes < (int64_t)used * ca * cb * 4) {
+    set_error("conv_dense_wgrad_rw: workspace too small");
+    return OCNN_ERR_WORKSPACE;
+  }
+  float* partial = (float*)ws;
+  if (rows > 0) {
+    const int wa = dr_wa(ca, cb);
+    if (wa == 4) launch_dense_wgrad<T, 4>(x, g, rows, ca, cb, used, per, tiles, partial, st);
+    else if (wa == 2) launch_dense_wgrad<T, 2>(x, g, rows, ca, cb, used, per, tiles, partial, st);
+    else launch_dense_wgrad<T, 1>(x, g, rows, ca, cb, used, per, tiles, partial, st);
+  }
+  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, 1, ca, cb, out_transposed, (T*)gw, st);
+  return check_launch("conv_dense_wgrad_rw");
+}
+
+extern "C" int ocnn_conv_dense_wgrad_rw(int dtype, const void* x, const void* g, int64_t rows, int ca, int cb,
+                                        int out_transposed, void* gw, void* workspace, int64_t workspace_bytes,
+                                        void* stream) {
+  OCNN_REQUIRE(ocnn_conv_dense_wgrad_rw_supported(dtype, rows, ca, cb), "conv_dense_wgrad_rw: shape not supported");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == OCNN_F16)
+    return run_dense_wgrad<f16>(x, g, rows, ca, cb, out_transposed, gw, workspace, workspace_bytes, st);
+  return run_dense_wgrad<bf16>(x, g, rows, ca, cb, out_transposed, gw, workspace, workspace_bytes, st);
+}

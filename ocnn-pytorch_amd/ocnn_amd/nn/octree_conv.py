@@ -53,6 +53,10 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   code = _lib.dtype_code(data)
   nbytes = L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout)
   ws = _lib.workspace(nbytes, data.device)
+  if dense and K == 1 and rows == rows_in and L.ocnn_conv_dense_rw_supported(code, rows, cin, cout):
+    _lib.check(L.ocnn_conv_dense_rw(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed),
+                                    _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return out
   # (many input channels into few output channels: the row tile that fits LDS is small and
   # the weights are streamed once per tile; the plan-free kernel is no slower there)
   if (dense and K == 1 and rows == rows_in and not (cin >= 512 and cout < 256) and
@@ -87,9 +91,10 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   return out
 
 
-def conv_wgrad(x, g, table, out_transposed=False, plan=None):
+def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
   """gW (K, ca, cb) [or (K, cb, ca)] = sum_i x[T[i,k]]^T (x) g[i].  With a tile
-  plan of the same table (and a supported shape) the staged kernel runs."""
+  plan of the same table (and a supported shape) the staged kernel runs.
+  dense: the table is the one-slot identity (row i reads row i)."""
   _lib.require_gpu(x, g, table)
   L = _lib.lib()
   x, g, table = x.contiguous(), g.contiguous(), table.contiguous()
@@ -103,6 +108,12 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None):
   shape = (K, cb, ca) if out_transposed else (K, ca, cb)
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
   code = _lib.DTYPE_CODE.get(x.dtype, -1)
+  if (dense and K == 1 and x.shape[0] == rows and
+      L.ocnn_conv_dense_wgrad_rw_supported(code, rows, ca, cb)):
+    ws = _lib.workspace(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(ca, cb), x.device)
+    _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x), _lib.ptr(g), rows, ca, cb, int(out_transposed),
+                                          _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return gw
   if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
                                                               plan.umax):
     ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K, ca, cb), x.device)
@@ -246,7 +257,7 @@ class OctreeConvBase:
     if self.dense_children:
       P = self.neigh.shape[0]
       gw = conv_wgrad(data.view(P, 8 * self.in_conv), grad, self._identity(P, data.device), False,
-                      None).view(8, self.in_conv, self.out_conv)
+                      None, dense=True).view(8, self.in_conv, self.out_conv)
       return gw.transpose(1, 2).contiguous() if out_transposed else gw
     plan = self._plan(data, self.in_conv, self.out_conv)
     return conv_wgrad(data, grad, self.neigh, out_transposed, plan)

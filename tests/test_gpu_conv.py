@@ -426,6 +426,50 @@ def test_dense_rows_kernel(dtype, cin, cout):
       assert rel_err(out, want) < TOL[dtype]
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('cin,cout', [(64, 128), (64, 512), (128, 128), (128, 256), (128, 512), (256, 128), (256, 256),
+                                      (512, 128), (512, 384), (1024, 128), (128, 1024)])
+def test_dense_rows_register_kernels(dtype, cin, cout):
+  """The persistent kernels for one-slot identity tables: out = in W + bias with the weights
+  in registers (every input width / output blocking they are built with, both weight layouts),
+  and gw = x^T g with the sums in registers (every block shape), ragged row counts, fewer
+  tiles than the ring of buffers holds."""
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(3 * cin + cout)
+  code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+  for rows in (1, 130, 4133, 64 * 300):
+    say('dense rows rw', dtype, cin, cout, rows)
+    x = torch.randn(rows, cin, generator=g).to(dtype)
+    gr = torch.randn(rows, cout, generator=g).to(dtype)
+    xd, gd = x.to(DEV), gr.to(DEV)
+    if L.ocnn_conv_dense_rw_supported(code, rows, cin, cout):
+      w = (torch.randn(cin, cout, generator=g) / cin ** 0.5).to(dtype)
+      b = torch.randn(cout, generator=g).to(dtype)
+      want = f64(x) @ f64(w) + f64(b)
+      for transposed in (0, 1):
+        wd = (w.t().contiguous() if transposed else w).to(DEV)
+        out = torch.full((rows + 1, cout), 7.0, dtype=dtype, device=DEV)      # one guard row
+        ws = torch.empty(cin * cout * 2, dtype=torch.uint8, device=DEV)
+        bd = b.to(DEV)
+        _lib.check(L.ocnn_conv_dense_rw(code, _lib.ptr(xd), rows, _lib.ptr(wd), cin, cout, transposed,
+                                        _lib.ptr(bd), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+        assert rel_err(out[:rows], want) < TOL[dtype]
+        assert bool((out[rows] == 7.0).all())
+    else:
+      assert cin > 512
+    if L.ocnn_conv_dense_wgrad_rw_supported(code, rows, cin, cout):
+      want = f64(x).T @ f64(gr)
+      ws = torch.empty(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(cin, cout), dtype=torch.uint8, device=DEV)
+      got = []
+      for transposed in (0, 1, 0):
+        gw = torch.empty((cout, cin) if transposed else (cin, cout), dtype=dtype, device=DEV)
+        _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(xd), _lib.ptr(gd), rows, cin, cout, transposed,
+                                              _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+        got.append(gw.t() if transposed else gw)
+        assert rel_err(got[-1], want) < TOL[dtype]
+      assert torch.equal(got[0], got[1].contiguous()) and torch.equal(got[0], got[2])
+
+
 def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
   """ocnn_conv_gather_wide through the C ABI (the Python layer picks it only for plans with
   enough reuse)."""
