@@ -4,7 +4,8 @@ MI355X (the headline number is bench.py's; these lines are supporting data).
   config 2: depth-8 batch of 8 (100k points each), bf16: OctreeConv 2x2x2 stride 2
             64->128 (depth 8->7), OctreeDeconv 2x2x2 stride 2 128->64 (7->8),
             OctreeDWConv 3x3x3 on 128 channels at depth 7; also the 3x3x3 64->64 layer
-            with nempty=True.
+            with nempty=True, and the pieces a U-Net adds around the convolutions (point
+            interpolation at the 800k input points, 2x2x2 max pooling).
   config 3: batch of 4, depth 9, 250k points each (planes + spheres), bf16:
             OctreeConv 3x3x3 32->32 at depth 9 and 256->256 at depth 6; build_octree and
             construct_all_neigh on the 1M points.
@@ -94,6 +95,51 @@ def main():
         'algorithmic_bytes': bytes_, 'frac_hbm_peak_at_algorithmic_bytes': bytes_ / ms / 1e6 / 8000.0,
     }), flush=True)
 
+  def run_op(tag, step, bytes_, extra):
+    for _ in range(args.warmup):
+      step()
+    torch.cuda.synchronize()
+    s = torch.cuda.Event(enable_timing=True)
+    e = torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(args.steps):
+      step()
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / args.steps
+    d = {'op': tag, 'ms_fwd_bwd': ms, 'algorithmic_bytes': bytes_,
+         'frac_hbm_peak_at_algorithmic_bytes': bytes_ / ms / 1e6 / 8000.0}
+    d.update(extra)
+    print(json.dumps(d), flush=True)
+
+  def ops(o, depth, pts, bid):
+    """The pieces a U-Net adds around the convolutions: point interpolation of the output
+    features, max pooling (non-empty nodes, as the networks use them)."""
+    from ocnn_amd.nn import octree_linear_pts, octree_nearest_pts, octree_max_pool
+    g = torch.Generator().manual_seed(9)
+    rows = int(o.nnum_nempty[depth])
+    q = torch.cat([(pts.to(dev) + 1.0) * (2 ** (depth - 1)), bid.to(dev).float().view(-1, 1)], 1)
+    n = q.shape[0]
+    for c, dt in ((64, torch.float32), (64, torch.bfloat16)):
+      es = 4 if dt == torch.float32 else 2
+      data = torch.randn(rows, c, generator=g).to(dt).to(dev).requires_grad_()
+      gout = torch.randn(n, c, generator=g).to(dt).to(dev)
+      for name, fn in (('linear', octree_linear_pts), ('nearest', octree_nearest_pts)):
+        def step():
+          data.grad = None
+          fn(data, o, depth, q, nempty=True).backward(gout)
+        run_op('interp %s %d ch d%d nempty %s' % (name, c, depth, str(dt).replace('torch.', '')), step,
+               2 * (es * (n * c + rows * c) + 16 * n), {'points': n, 'rows': rows})
+    data = torch.randn(rows, 64, generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    prow = int(o.nnum_nempty[depth - 1])
+    gout = torch.randn(prow, 64, generator=g).to(torch.bfloat16).to(dev)
+
+    def step():
+      data.grad = None
+      octree_max_pool(data, o, depth, nempty=True).backward(gout)
+    run_op('max pool 64 ch d%d->%d nempty bfloat16' % (depth, depth - 1), step,
+           2 * 2 * (rows * 64 + prow * 64) + 2 * 8 * prow * 64, {'rows': rows, 'parents': prow})
+
   bf = torch.bfloat16
   if '2' in args.configs.split(','):
     o, b_ms, n_ms, npts = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
@@ -111,6 +157,8 @@ def main():
         o._table(8, '333', 1, True), bf)
     run('conv 3x3x3 s1 64->64 d8', OctreeConv(64, 64, [3], 1), o, 8, nn8, 64, 64,
         o._table(8, '333', 1, False), bf)
+    pts, _, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 8, 1001, n=100000)
+    ops(o, 8, pts, bid)
     del o
   if '3' in args.configs.split(','):
     o, b_ms, n_ms, npts = build(synthetic.planes_cloud, 4, 1003, 250000, 9)

@@ -321,6 +321,50 @@ int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const vo
                               int channels, void* gw, void* workspace, int64_t workspace_bytes,
                               void* stream);
 
+/* Key search, ocnn/octree/octree.py:448-488 (search_key / search_xyzb): out[i] = position of
+ * query[i] in the ascending `keys`, or -1.  ocnn_search_points takes float (x, y, z, b) rows,
+ * truncates and encodes them like xyz2key (ocnn/octree/shuffled_key.py:60-90) and, with
+ * bound_check, rejects coordinates outside [0, 2^depth) (ocnn/nn/octree_interp.py:38-42). */
+int ocnn_search_key(const int64_t* keys, int64_t n, const int64_t* query, int64_t m,
+                    int64_t* out, void* stream);
+int ocnn_search_points(const float* pts, int64_t m, int depth, const int64_t* keys, int64_t n,
+                       int bound_check, int32_t* out, void* stream);
+
+/* Trilinear interpolation, ocnn/nn/octree_interp.py:49-103 (octree_linear_pts), in two steps:
+ * the 8 neighbour rows idx (m, 8) (-1 = none), their weights w (m, 8) and the weight sum
+ * norm (m) of every point (lines 60-88), then out = (sum_j w_j data[idx_j]) / (norm + 1e-12)
+ * as ocnn_csr_rows with 8 entries per row (lines 90-102).  ocnn_csr_rows is the product of
+ * a sparse matrix in row form with a dense one, out[r] = (sum_e val[e] data[col[e]]) /
+ * (rowdiv[r] + 1e-12): entries rowptr[r] .. rowptr[r+1]-1, or kfixed per row when rowptr is
+ * NULL; val NULL = ones, rowdiv NULL = no division, col < 0 = no entry.  With the transposed
+ * matrix it is the gradient with respect to data (no atomics, fixed summation order). */
+int ocnn_interp_linear_prepare(const float* pts, int64_t m, int depth, const int64_t* keys,
+                               int64_t n, int bound_check, int32_t* idx, float* w, float* norm,
+                               void* stream);
+int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const int32_t* col,
+                  const float* val, const void* data, int channels, const float* rowdiv,
+                  void* out, int64_t rows, void* stream);
+
+/* 2x2x2 max pooling, ocnn/nn/octree_pool.py:16-65.
+ * ocnn_max_pool: maximum over the children 8p .. 8p+7 of the p-th non-empty node (first on
+ * ties) and its index (indices (parents, c) int64).  fine_child = children of the fine
+ * level when data holds non-empty nodes only (an empty child counts as -inf), NULL when it
+ * holds all nodes; coarse_child = children of the coarse level when the output has a row
+ * for every coarse node (zeros for empty ones, the octree_pad of line 36), NULL when it
+ * has one per non-empty node.
+ * ocnn_max_unpool: out row r = child q % 8 of parent q / 8 (q = out_node[r] or r) takes
+ * src[src_row[p] or p] where indices say so, else 0 (lines 40-65; also d pool / d data).
+ * ocnn_max_gather: out[p] = src[row of child 8p + indices[p]] (d unpool / d data). */
+int ocnn_max_pool(int dtype, const void* data, const int32_t* fine_child,
+                  const int32_t* coarse_child, int64_t out_rows, int channels, void* out,
+                  int64_t* indices, void* stream);
+int ocnn_max_unpool(int dtype, const void* src, const int64_t* indices, const int32_t* out_node,
+                    const int32_t* src_row, int64_t out_rows, int channels, void* out,
+                    void* stream);
+int ocnn_max_gather(int dtype, const void* src, const int64_t* indices,
+                    const int32_t* fine_child, int64_t parents, int channels, void* out,
+                    void* stream);
+
 /* ocnn/nn/octree_pad.py:13-39.  pad: out (n, c) = val except out[q] =
  * data[children[q]] where children[q] >= 0; depad: out[children[q]] = data[q]. */
 int ocnn_pad(int dtype, const void* data, const int32_t* children, int64_t n,

@@ -72,6 +72,13 @@ SIGNATURES = {
     'ocnn_dwconv_wgrad_planned_supported': (_i, [_i, _l, _l, _i, _i, _i]),
     'ocnn_dwconv_wgrad_planned_workspace_bytes': (_l, [_i, _i]),
     'ocnn_dwconv_wgrad_planned': (_i, [_i, _p, _l, _p, _p, _p, _p, _i, _l, _l, _i, _i, _p, _p, _l, _p]),
+    'ocnn_search_key': (_i, [_p, _l, _p, _l, _p, _p]),
+    'ocnn_search_points': (_i, [_p, _l, _i, _p, _l, _i, _p, _p]),
+    'ocnn_interp_linear_prepare': (_i, [_p, _l, _i, _p, _l, _i, _p, _p, _p, _p]),
+    'ocnn_csr_rows': (_i, [_i, _p, _i, _p, _p, _p, _i, _p, _p, _l, _p]),
+    'ocnn_max_pool': (_i, [_i, _p, _p, _p, _l, _i, _p, _p, _p]),
+    'ocnn_max_unpool': (_i, [_i, _p, _p, _p, _p, _l, _i, _p, _p]),
+    'ocnn_max_gather': (_i, [_i, _p, _p, _p, _l, _i, _p, _p]),
     'ocnn_dwconv_wgrad_workspace_bytes': (_l, [_l, _i, _i]),
     'ocnn_dwconv_wgrad': (_i, [_i, _p, _l, _p, _p, _l, _i, _i, _p, _p, _l, _p]),
     'ocnn_pad': (_i, [_i, _p, _p, _l, _i, _f, _p, _p]),

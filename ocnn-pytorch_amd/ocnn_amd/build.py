@@ -26,6 +26,7 @@ SOURCES = {
     'wgrad_planned.hip': [],
     'plan.hip': [],
     'misc.hip': [],
+    'interp.hip': ['-ffp-contract=off'],
 }
 
 COMMON = ['-O3', '--offload-arch=gfx950', '-fPIC', '-std=c++17', '-I', INCLUDE, '-I', CSRC,

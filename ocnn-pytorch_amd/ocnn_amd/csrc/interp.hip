@@ -1,0 +1,315 @@
+// Key search, point interpolation (nearest / trilinear) and 2x2x2 max pooling on octrees.
+//
+// All of it is index arithmetic plus row gathers: HBM / L2-latency bound.  Every output
+// element is produced by exactly one thread from a fixed list of inputs (gather form), so
+// nothing here needs atomics and every result is reproducible bit for bit.
+#include <algorithm>
+
+#include "common.hpp"
+#include "morton.hpp"
+
+namespace ocnn {
+
+// first position whose key is >= q (keys ascending)
+__device__ __forceinline__ int64_t lower_bound_key(const int64_t* __restrict__ keys, int64_t n, int64_t q) {
+  int64_t lo = 0, len = n;
+  while (len > 0) {
+    const int64_t half = len >> 1;
+    const bool less = keys[lo + half] < q;
+    lo = less ? lo + half + 1 : lo;
+    len = less ? len - half - 1 : half;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ int64_t find_key(const int64_t* __restrict__ keys, int64_t n, int64_t q) {
+  const int64_t i = lower_bound_key(keys, n, q);
+  return (i < n && keys[i] == q) ? i : -1;
+}
+
+__global__ void search_key_kernel(const int64_t* __restrict__ keys, int64_t n,
+                                  const int64_t* __restrict__ query, int64_t m, int64_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < m) out[i] = find_key(keys, n, query[i]);
+}
+
+// key of a float (x, y, z, b): truncation toward zero like Tensor.long(), then the masks of
+// every key (a coordinate outside the volume wraps; bound_check is what rejects it)
+__device__ __forceinline__ int64_t key_of(float x, float y, float z, float b, int depth) {
+  return encode((int64_t)x, (int64_t)y, (int64_t)z, depth) | ((int64_t)b << 48);
+}
+
+__global__ void search_points_kernel(const float* __restrict__ pts, int64_t m, int depth,
+                                     const int64_t* __restrict__ keys, int64_t n, int bound_check,
+                                     int32_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= m) return;
+  const float x = pts[4 * i], y = pts[4 * i + 1], z = pts[4 * i + 2], b = pts[4 * i + 3];
+  int64_t r = find_key(keys, n, key_of(x, y, z, b, depth));
+  const float hi = (float)(1 << depth);
+  if (bound_check && !(x >= 0.f && x < hi && y >= 0.f && y < hi && z >= 0.f && z < hi)) r = -1;
+  out[i] = (int32_t)r;
+}
+
+// Trilinear weights: values sit at voxel centres, so f = p - 0.5, corner = floor(f), and the
+// neighbour j = (gx, gy, gz) weighs |((1 - gx) - frac_x) ((1 - gy) - frac_y) ((1 - gz) - frac_z)|.
+// One thread per (point, neighbour); the 8 threads of a point add their weights in neighbour
+// order for the normalisation.
+__global__ void interp_linear_prepare_kernel(const float* __restrict__ pts, int64_t m, int depth,
+                                             const int64_t* __restrict__ keys, int64_t n, int bound_check,
+                                             int32_t* __restrict__ idx, float* __restrict__ w,
+                                             float* __restrict__ norm) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t i = t >> 3;
+  const int j = (int)(t & 7);
+  float wj = 0.f;
+  int32_t r = -1;
+  if (i < m) {
+    const float gx = (float)(j >> 2), gy = (float)((j >> 1) & 1), gz = (float)(j & 1);
+    const float fx = pts[4 * i] - 0.5f, fy = pts[4 * i + 1] - 0.5f, fz = pts[4 * i + 2] - 0.5f;
+    const float ix = floorf(fx), iy = floorf(fy), iz = floorf(fz);
+    const float nx = ix + gx, ny = iy + gy, nz = iz + gz;
+    int64_t f = find_key(keys, n, key_of(nx, ny, nz, pts[4 * i + 3], depth));
+    const float hi = (float)(1 << depth);
+    if (bound_check && !(nx >= 0.f && nx < hi && ny >= 0.f && ny < hi && nz >= 0.f && nz < hi)) f = -1;
+    if (f >= 0) {
+      const float tx = (1.0f - gx) - (fx - ix), ty = (1.0f - gy) - (fy - iy), tz = (1.0f - gz) - (fz - iz);
+      wj = fabsf((tx * ty) * tz);
+      r = (int32_t)f;
+    }
+    idx[t] = r;
+    w[t] = wj;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) s += __shfl(wj, (threadIdx.x & ~7) + k, 64);
+  if (i < m && j == 0) norm[i] = s;
+}
+
+// out[r][c] = (sum_e val[e] * data[col[e]][c]) / (rowdiv[r] + 1e-12), e over the entries of
+// row r: rowptr[r] .. rowptr[r + 1] - 1, or kfixed entries per row.  col < 0 = no entry.
+// fp32 sums in entry order.
+template <typename T, int VEC>
+__global__ void csr_rows_kernel(const int32_t* __restrict__ rowptr, int kfixed, const int32_t* __restrict__ col,
+                                const float* __restrict__ val, const T* __restrict__ data, int C,
+                                const float* __restrict__ rowdiv, T* __restrict__ out, int64_t rows) {
+  const int lpr = C / VEC;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= rows * lpr) return;
+  const int64_t r = t / lpr;
+  const int c0 = (int)(t - r * lpr) * VEC;
+  const int64_t e0 = rowptr ? rowptr[r] : r * kfixed;
+  const int64_t e1 = rowptr ? rowptr[r + 1] : e0 + kfixed;
+  float acc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+  for (int64_t e = e0; e < e1; ++e) {
+    const int32_t cidx = col[e];
+    if (cidx < 0) continue;
+    const float we = val ? val[e] : 1.0f;
+    const T* src = data + (int64_t)cidx * C + c0;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] += we * to_f32(src[v]);
+  }
+  const float div = rowdiv ? rowdiv[r] + 1e-12f : 1.0f;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) out[r * C + c0 + v] = from_f32<T>(rowdiv ? acc[v] / div : acc[v]);
+}
+
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PoolVec { T v[VEC]; };
+
+// Max over the 8 children of a node (first one on ties) and which child it was.
+//   out row r: node r of the coarse level when `coarse_child` is given (rows of empty
+//   nodes are zeros), else the r-th non-empty node;
+//   child q = 8 p + j of the p-th non-empty node: data row fine_child[q] (< 0: -inf) when
+//   `fine_child` is given, else row q.
+// A thread owns VEC consecutive channels of an output row.
+template <typename T, int VEC>
+__global__ void max_pool_kernel(const T* __restrict__ data, const int32_t* __restrict__ fine_child,
+                                const int32_t* __restrict__ coarse_child, int64_t out_rows, int C,
+                                T* __restrict__ out, int64_t* __restrict__ indices) {
+  typedef PoolVec<T, VEC> V;
+  const int lpr = C / VEC;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= out_rows * lpr) return;
+  const int64_t r = t / lpr;
+  const int c = (int)(t - r * lpr) * VEC;
+  const int64_t p = coarse_child ? coarse_child[r] : r;
+  V o;
+  if (p < 0) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o.v[v] = from_f32<T>(0.f);
+    *(V*)(out + r * C + c) = o;
+    return;
+  }
+  V x[8];
+  int64_t row[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int64_t q = 8 * p + j;
+    row[j] = fine_child ? fine_child[q] : q;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (row[j] >= 0) x[j] = *(const V*)(data + row[j] * C + c);
+  float best[VEC];
+  int bj[VEC];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float val = row[j] >= 0 ? to_f32(x[j].v[v]) : -INFINITY;
+      if (j == 0 || val > best[v]) {
+        best[v] = val;
+        bj[v] = j;
+      }
+    }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    o.v[v] = from_f32<T>(best[v]);
+    indices[p * C + c + v] = bj[v];
+  }
+  *(V*)(out + r * C + c) = o;
+}
+
+// out row r is child j = q % 8 of parent p = q / 8 (q = out_node[r], or r): it takes
+// src[src_row[p] or p][c] if indices[p][c] == j, else zero.  (Unpooling, and the gradient
+// of pooling.)
+template <typename T, int VEC>
+__global__ void max_unpool_kernel(const T* __restrict__ src, const int64_t* __restrict__ indices,
+                                  const int32_t* __restrict__ out_node, const int32_t* __restrict__ src_row,
+                                  int64_t out_rows, int C, T* __restrict__ out) {
+  typedef PoolVec<T, VEC> V;
+  const int lpr = C / VEC;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= out_rows * lpr) return;
+  const int64_t r = t / lpr;
+  const int c = (int)(t - r * lpr) * VEC;
+  const int64_t q = out_node ? out_node[r] : r;
+  const int64_t p = q >> 3;
+  const int j = (int)(q & 7);
+  const int64_t s = src_row ? src_row[p] : p;
+  const V x = *(const V*)(src + s * C + c);
+  V o;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) o.v[v] = indices[p * C + c + v] == j ? x.v[v] : from_f32<T>(0.f);
+  *(V*)(out + r * C + c) = o;
+}
+
+// out[p][c] = src[row of child 8 p + indices[p][c]][c] (row = fine_child[q], < 0: zero, or q).
+// (The gradient of unpooling.)
+template <typename T>
+__global__ void max_gather_kernel(const T* __restrict__ src, const int64_t* __restrict__ indices,
+                                  const int32_t* __restrict__ fine_child, int64_t parents, int C,
+                                  T* __restrict__ out) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= parents * C) return;
+  const int64_t p = t / C;
+  const int c = (int)(t - p * C);
+  const int64_t q = 8 * p + indices[t];
+  const int64_t row = fine_child ? fine_child[q] : q;
+  out[t] = row >= 0 ? src[row * C + c] : from_f32<T>(0.f);
+}
+
+}  // namespace ocnn
+
+using namespace ocnn;
+
+#define OCNN_DISPATCH_DTYPE(dtype, ...)                      \
+  do {                                                       \
+    if (dtype == OCNN_F32) { typedef float T; __VA_ARGS__; } \
+    else if (dtype == OCNN_F16) { typedef f16 T; __VA_ARGS__; } \
+    else { typedef bf16 T; __VA_ARGS__; }                    \
+  } while (0)
+
+extern "C" int ocnn_search_key(const int64_t* keys, int64_t n, const int64_t* query, int64_t m, int64_t* out,
+                               void* stream) {
+  OCNN_REQUIRE(n >= 0 && m >= 0, "search_key: bad sizes");
+  if (m == 0) return OCNN_OK;
+  hipLaunchKernelGGL(search_key_kernel, dim3((unsigned)cdiv(m, 256)), dim3(256), 0, (hipStream_t)stream, keys, n,
+                     query, m, out);
+  return check_launch("search_key");
+}
+
+extern "C" int ocnn_search_points(const float* pts, int64_t m, int depth, const int64_t* keys, int64_t n,
+                                  int bound_check, int32_t* out, void* stream) {
+  OCNN_REQUIRE(n >= 0 && n < (1ll << 31) && m >= 0 && depth >= 0 && depth <= 16, "search_points: bad arguments");
+  if (m == 0) return OCNN_OK;
+  hipLaunchKernelGGL(search_points_kernel, dim3((unsigned)cdiv(m, 256)), dim3(256), 0, (hipStream_t)stream, pts, m,
+                     depth, keys, n, bound_check, out);
+  return check_launch("search_points");
+}
+
+extern "C" int ocnn_interp_linear_prepare(const float* pts, int64_t m, int depth, const int64_t* keys, int64_t n,
+                                          int bound_check, int32_t* idx, float* w, float* norm, void* stream) {
+  OCNN_REQUIRE(n >= 0 && n < (1ll << 31) && m >= 0 && m < (1ll << 28) && depth >= 0 && depth <= 16,
+               "interp_linear_prepare: bad arguments");
+  if (m == 0) return OCNN_OK;
+  hipLaunchKernelGGL(interp_linear_prepare_kernel, dim3((unsigned)cdiv(m * 8, 256)), dim3(256), 0,
+                     (hipStream_t)stream, pts, m, depth, keys, n, bound_check, idx, w, norm);
+  return check_launch("interp_linear_prepare");
+}
+
+extern "C" int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const int32_t* col, const float* val,
+                             const void* data, int channels, const float* rowdiv, void* out, int64_t rows,
+                             void* stream) {
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && rows >= 0 && (rowptr || kfixed >= 1),
+               "csr_rows: bad arguments");
+  if (rows == 0) return OCNN_OK;
+  hipStream_t st = (hipStream_t)stream;
+  OCNN_DISPATCH_DTYPE(dtype, {
+    if (channels % 4 == 0)
+      hipLaunchKernelGGL((csr_rows_kernel<T, 4>), dim3((unsigned)cdiv(rows * (channels / 4), 256)), dim3(256), 0, st,
+                         rowptr, kfixed, col, val, (const T*)data, channels, rowdiv, (T*)out, rows);
+    else
+      hipLaunchKernelGGL((csr_rows_kernel<T, 1>), dim3((unsigned)cdiv(rows * channels, 256)), dim3(256), 0, st,
+                         rowptr, kfixed, col, val, (const T*)data, channels, rowdiv, (T*)out, rows);
+  });
+  return check_launch("csr_rows");
+}
+
+extern "C" int ocnn_max_pool(int dtype, const void* data, const int32_t* fine_child, const int32_t* coarse_child,
+                             int64_t out_rows, int channels, void* out, int64_t* indices, void* stream) {
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && out_rows >= 0, "max_pool: bad arguments");
+  if (out_rows == 0) return OCNN_OK;
+  hipStream_t st = (hipStream_t)stream;
+  OCNN_DISPATCH_DTYPE(dtype, {
+    constexpr int VEC = 16 / sizeof(T);
+    if (channels % VEC == 0)
+      hipLaunchKernelGGL((max_pool_kernel<T, VEC>), dim3((unsigned)cdiv(out_rows * (channels / VEC), 256)), dim3(256),
+                         0, st, (const T*)data, fine_child, coarse_child, out_rows, channels, (T*)out, indices);
+    else
+      hipLaunchKernelGGL((max_pool_kernel<T, 1>), dim3((unsigned)cdiv(out_rows * channels, 256)), dim3(256), 0, st,
+                         (const T*)data, fine_child, coarse_child, out_rows, channels, (T*)out, indices);
+  });
+  return check_launch("max_pool");
+}
+
+extern "C" int ocnn_max_unpool(int dtype, const void* src, const int64_t* indices, const int32_t* out_node,
+                               const int32_t* src_row, int64_t out_rows, int channels, void* out, void* stream) {
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && out_rows >= 0, "max_unpool: bad arguments");
+  if (out_rows == 0) return OCNN_OK;
+  hipStream_t st = (hipStream_t)stream;
+  OCNN_DISPATCH_DTYPE(dtype, {
+    constexpr int VEC = 16 / sizeof(T);
+    if (channels % VEC == 0)
+      hipLaunchKernelGGL((max_unpool_kernel<T, VEC>), dim3((unsigned)cdiv(out_rows * (channels / VEC), 256)),
+                         dim3(256), 0, st, (const T*)src, indices, out_node, src_row, out_rows, channels, (T*)out);
+    else
+      hipLaunchKernelGGL((max_unpool_kernel<T, 1>), dim3((unsigned)cdiv(out_rows * channels, 256)), dim3(256), 0, st,
+                         (const T*)src, indices, out_node, src_row, out_rows, channels, (T*)out);
+  });
+  return check_launch("max_unpool");
+}
+
+extern "C" int ocnn_max_gather(int dtype, const void* src, const int64_t* indices, const int32_t* fine_child,
+                               int64_t parents, int channels, void* out, void* stream) {
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && parents >= 0, "max_gather: bad arguments");
+  if (parents == 0) return OCNN_OK;
+  hipStream_t st = (hipStream_t)stream;
+  OCNN_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL(max_gather_kernel<T>, dim3((unsigned)cdiv(parents * channels, 256)), dim3(256), 0, st,
+                       (const T*)src, indices, fine_child, parents, channels, (T*)out);
+  });
+  return check_launch("max_gather");
+}

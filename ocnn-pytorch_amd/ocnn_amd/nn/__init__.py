@@ -5,8 +5,13 @@ from .octree_dwconv import OctreeDWConv, octree_dwconv
 from .octree_conv_t import (OctreeConvTriton, OctreeConvT, octree_conv_triton,
                             convert_conv_triton, conv_fwd_implicit_gemm_splitk,
                             conv_bwd_implicit_gemm_splitk)
+from .octree_pool import (octree_max_pool, octree_max_unpool, OctreeMaxPool, OctreeMaxUnpool)
+from .octree_interp import (octree_nearest_pts, octree_linear_pts, OctreeInterp,
+                            octree_nearest_upsample, OctreeUpsample)
 
 __all__ = ['octree_pad', 'octree_depad', 'OctreeConv', 'OctreeDeconv', 'octree_conv',
            'octree_deconv', 'OctreeDWConv', 'octree_dwconv', 'OctreeConvTriton', 'OctreeConvT',
            'octree_conv_triton', 'convert_conv_triton', 'conv_fwd_implicit_gemm_splitk',
-           'conv_bwd_implicit_gemm_splitk']
+           'conv_bwd_implicit_gemm_splitk', 'octree_max_pool', 'octree_max_unpool', 'OctreeMaxPool',
+           'OctreeMaxUnpool', 'octree_nearest_pts', 'octree_linear_pts', 'OctreeInterp',
+           'octree_nearest_upsample', 'OctreeUpsample']

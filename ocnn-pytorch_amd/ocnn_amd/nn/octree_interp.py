@@ -1,0 +1,169 @@
+"""Point interpolation and upsampling with the API of ocnn/nn/octree_interp.py on HIP
+kernels: the neighbour search and the weights in one kernel, the weighted row gather (and
+its transpose for the gradient) in another.  No atomics: the gradient with respect to the
+data runs over the transposed sparse matrix in row form."""
+
+from typing import Optional, Union
+
+import torch
+import torch.nn
+
+from .. import _lib
+from .octree_pad import octree_depad
+
+
+def _csr_rows(data, col, val, rowptr, kfixed, rowdiv, rows):
+  out = torch.empty((rows, data.shape[1]), dtype=data.dtype, device=data.device)
+  _lib.check(_lib.lib().ocnn_csr_rows(_lib.dtype_code(data), _lib.ptr(rowptr), kfixed, _lib.ptr(col),
+                                      _lib.ptr(val), _lib.ptr(data), data.shape[1], _lib.ptr(rowdiv),
+                                      _lib.ptr(out), rows, _lib.stream()))
+  return out
+
+
+def _transpose(idx, w, rows):
+  """Row form of the transposed matrix of (point, neighbour) entries: for every data row the
+  points that read it (ascending) and their weights."""
+  flat = idx.reshape(-1)
+  k = idx.shape[1]
+  valid = flat >= 0
+  order = torch.argsort(torch.where(valid, flat, torch.full_like(flat, rows)), stable=True)
+  n = int(valid.sum())
+  order = order[:n]
+  col = torch.div(order, k, rounding_mode='floor').to(torch.int32)
+  val = None if w is None else w.reshape(-1)[order].contiguous()
+  counts = torch.bincount(flat[order].long(), minlength=rows)
+  rowptr = torch.zeros(rows + 1, dtype=torch.int32, device=idx.device)
+  rowptr[1:] = counts.cumsum(0)
+  return rowptr, col.contiguous(), val
+
+
+class _Interp(torch.autograd.Function):
+  """out[p] = (sum_j w[p, j] data[idx[p, j]]) / (norm[p] + 1e-12)   (norm None: no division)."""
+
+  @staticmethod
+  def forward(ctx, data, idx, w, norm):
+    data = data.contiguous()
+    ctx.save_for_backward(idx, w, norm)
+    ctx.rows = data.shape[0]
+    return _csr_rows(data, idx, w, None, idx.shape[1], norm, idx.shape[0])
+
+  @staticmethod
+  def backward(ctx, grad):
+    idx, w, norm = ctx.saved_tensors
+    grad = grad.contiguous()
+    if norm is not None:
+      grad = (grad / (norm.unsqueeze(1) + 1e-12).to(grad.dtype)).contiguous()
+    rowptr, col, val = _transpose(idx, w, ctx.rows)
+    return _csr_rows(grad, col, val, rowptr, 0, None, ctx.rows), None, None, None
+
+
+def _keys(octree, depth, nempty):
+  return octree.key(depth, nempty).contiguous()
+
+
+def _pts(pts):
+  _lib.require_gpu(pts)
+  assert pts.dim() == 2 and pts.shape[1] == 4, 'pts: (N, 4) rows of (x, y, z, batch)'
+  return pts.to(torch.float32).contiguous()
+
+
+def _check_rows(data, octree, depth, nempty):
+  nnum = octree.nnum_nempty[depth] if nempty else octree.nnum[depth]
+  assert data.shape[0] == nnum, 'The shape of input data is wrong.'
+
+
+def octree_nearest_pts(data: torch.Tensor, octree, depth: int, pts: torch.Tensor,
+                       nempty: bool = False, bound_check: bool = False):
+  """Nearest-neighbour interpolation at points scaled to [0, 2^depth)
+  (ocnn/nn/octree_interp.py:15-46): the row of the node that holds the point, zeros where
+  there is none."""
+  _check_rows(data, octree, depth, nempty)
+  pts = _pts(pts)
+  keys = _keys(octree, depth, nempty)
+  idx = torch.empty((pts.shape[0], 1), dtype=torch.int32, device=pts.device)
+  _lib.check(_lib.lib().ocnn_search_points(_lib.ptr(pts), pts.shape[0], depth, _lib.ptr(keys),
+                                           keys.numel(), int(bound_check), _lib.ptr(idx), _lib.stream()))
+  return _Interp.apply(data, idx, None, None)
+
+
+def octree_linear_pts(data: torch.Tensor, octree, depth: int, pts: torch.Tensor,
+                      nempty: bool = False, bound_check: bool = False):
+  """Trilinear interpolation over the (up to 8) existing neighbours, normalised by their
+  weight sum (ocnn/nn/octree_interp.py:49-103)."""
+  _check_rows(data, octree, depth, nempty)
+  pts = _pts(pts)
+  keys = _keys(octree, depth, nempty)
+  m = pts.shape[0]
+  idx = torch.empty((m, 8), dtype=torch.int32, device=pts.device)
+  w = torch.empty((m, 8), dtype=torch.float32, device=pts.device)
+  norm = torch.empty(m, dtype=torch.float32, device=pts.device)
+  _lib.check(_lib.lib().ocnn_interp_linear_prepare(_lib.ptr(pts), m, depth, _lib.ptr(keys), keys.numel(),
+                                                   int(bound_check), _lib.ptr(idx), _lib.ptr(w),
+                                                   _lib.ptr(norm), _lib.stream()))
+  return _Interp.apply(data, idx, w, norm)
+
+
+class OctreeInterp(torch.nn.Module):
+  """ocnn/nn/octree_interp.py:106-141."""
+
+  def __init__(self, method: str = 'linear', nempty: bool = False, bound_check: bool = False,
+               rescale_pts: bool = True):
+    super().__init__()
+    self.method = method
+    self.nempty = nempty
+    self.bound_check = bound_check
+    self.rescale_pts = rescale_pts
+    self.func = octree_linear_pts if method == 'linear' else octree_nearest_pts
+
+  def forward(self, data: torch.Tensor, octree, depth: int, pts: torch.Tensor,
+              bbmin: Union[torch.Tensor, float] = -1, bbmax: Union[torch.Tensor, float] = 1):
+    # points from [bbmin, bbmax] to [0, 2^depth], in place like the reference
+    if self.rescale_pts:
+      box_size = bbmax - bbmin
+      if type(box_size) is torch.Tensor:
+        box_size = box_size.max().item()
+      assert box_size > 0, 'The bounding box size must be greater than 0.'
+      pts[:, :3] = (pts[:, :3] - bbmin) * (2 ** depth / box_size)
+    return self.func(data, octree, depth, pts, self.nempty, self.bound_check)
+
+  def extra_repr(self) -> str:
+    return 'method={}, nempty={}, bound_check={}, rescale_pts={}'.format(
+        self.method, self.nempty, self.bound_check, self.rescale_pts)
+
+
+def octree_nearest_upsample(data: torch.Tensor, octree, depth: int, nempty: bool = False):
+  """depth -> depth + 1, every child takes its parent's row (ocnn/nn/octree_interp.py:144-167)."""
+  _check_rows(data, octree, depth, nempty)
+  out = data
+  if not nempty:
+    out = octree_depad(out, octree, depth)
+  out = out.unsqueeze(1).repeat(1, 8, 1).flatten(end_dim=1)
+  if nempty:
+    out = octree_depad(out, octree, depth + 1)
+  return out
+
+
+class OctreeUpsample(torch.nn.Module):
+  """depth -> target_depth (ocnn/nn/octree_interp.py:170-200)."""
+
+  def __init__(self, method: str = 'linear', nempty: bool = False):
+    super().__init__()
+    self.method = method
+    self.nempty = nempty
+    self.func = octree_linear_pts if method == 'linear' else octree_nearest_pts
+
+  def forward(self, data: torch.Tensor, octree, depth: int, target_depth: Optional[int] = None):
+    if target_depth is None:
+      target_depth = depth + 1
+    if target_depth == depth:
+      return data
+    assert target_depth >= depth, 'target_depth must be larger than depth'
+    if target_depth == depth + 1 and self.method == 'nearest':
+      return octree_nearest_upsample(data, octree, depth, self.nempty)
+    xyzb = octree.xyzb(target_depth, self.nempty)
+    pts = torch.stack(xyzb, dim=1).float()
+    pts[:, :3] = (pts[:, :3] + 0.5) * (2 ** (depth - target_depth))
+    return self.func(data, octree, depth, pts, self.nempty)
+
+  def extra_repr(self) -> str:
+    return 'method={}, nempty={}'.format(self.method, self.nempty)

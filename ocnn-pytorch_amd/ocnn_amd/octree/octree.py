@@ -447,12 +447,12 @@ class Octree:
     return self.search_key(key, depth, nempty)
 
   def search_key(self, query: torch.Tensor, depth: int, nempty: bool = False):
-    key = self.key(depth, nempty)
-    idx = torch.searchsorted(key, query)
-    valid = idx < key.shape[0]
-    found = torch.zeros_like(valid)
-    found[valid] = key[idx[valid]] == query[valid]
-    idx[found.logical_not()] = -1
+    key = self.key(depth, nempty).contiguous()
+    _lib.require_gpu(key, query)
+    query = query.to(torch.long).contiguous()
+    idx = torch.empty(query.shape, dtype=torch.long, device=query.device)
+    _lib.check(_lib.lib().ocnn_search_key(_lib.ptr(key), key.numel(), _lib.ptr(query), query.numel(),
+                                          _lib.ptr(idx), _lib.stream()))
     return idx
 
   # ---- tables for the layers ------------------------------------------------

@@ -1,0 +1,194 @@
+"""GPU parity of key search, point interpolation, upsampling and max pooling: the HIP path
+(through the C ABI) against the reference's data files and the numpy oracle."""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import ocnn_amd
+from ocnn_amd import synthetic
+from ocnn_amd.nn import (octree_depad, octree_linear_pts, octree_max_pool, octree_max_unpool,
+                         octree_nearest_pts, octree_nearest_upsample, OctreeInterp, OctreeMaxPool,
+                         OctreeMaxUnpool, OctreeUpsample)
+from ocnn_amd.octree import Octree, Points
+from oracle import interp_ref as I
+from test_gpu_octree import merged_octree, oracle_batch
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+TOL = {torch.float32: 1e-6, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}
+
+
+def say(*a):
+  print(*a, flush=True)
+  sys.stdout.flush()
+
+
+def np_(t):
+  return t.detach().float().cpu().numpy() if t.is_floating_point() else t.detach().cpu().numpy()
+
+
+def test_interp_against_reference_fixture(ref_data):
+  """test/test_octree_interp.py:21-43 through the HIP path, with the reference's tolerance."""
+  say('interp: reference fixture')
+  t = np.load(os.path.join(ref_data, 'interp.npz'))
+  o = merged_octree(ref_data)
+  w = oracle_batch(ref_data)
+  depth = 5
+  data = torch.from_numpy(t['data']).to(DEV)
+  pts = torch.from_numpy(t['pts']).to(DEV)
+  data_ne = octree_depad(data, o, depth)
+  got = {'linear': octree_linear_pts(data, o, depth, pts, nempty=False),
+         'linear_ne': octree_linear_pts(data_ne, o, depth, pts, nempty=True),
+         'near': octree_nearest_pts(data, o, depth, pts, nempty=False),
+         'near_ne': octree_nearest_pts(data_ne, o, depth, pts, nempty=True)}
+  for k, v in got.items():
+    assert np.allclose(np_(v), t[k], atol=1e-6), k
+  # and the oracle, also with the bounds check on points pushed out of the volume
+  far = t['pts'].copy()
+  far[::3, 1] -= 40.0
+  for ne in (False, True):
+    d = t['data'] if not ne else I.octree_depad(w, t['data'], depth)
+    dg = data_ne if ne else data
+    for bc in (False, True):
+      fg = torch.from_numpy(far).to(DEV)
+      assert np.allclose(np_(octree_linear_pts(dg, o, depth, fg, ne, bc)), I.linear_pts(w, d, depth, far, ne, bc), atol=1e-6)
+      assert np.array_equal(np_(octree_nearest_pts(dg, o, depth, fg, ne, bc)), I.nearest_pts(w, d, depth, far, ne, bc))
+
+
+@pytest.mark.parametrize('nempty', [False, True])
+def test_nearest_upsample_and_modules(ref_data, nempty):
+  """test/test_octree_interp.py:45-73, and the module forms against the oracle."""
+  say('upsample', nempty)
+  o = merged_octree(ref_data)
+  w = oracle_batch(ref_data)
+  depth = 4
+  rows = int(o.nnum_nempty[depth] if nempty else o.nnum[depth])
+  data = torch.rand(rows, 4, generator=torch.Generator().manual_seed(1)).to(DEV)
+  out = octree_nearest_upsample(data, o, depth, nempty)
+  xyzb = o.xyzb(depth + 1, nempty)
+  pts = torch.stack(xyzb, dim=1).float()
+  pts[:, :3] = (pts[:, :3] + 0.5) * 0.5
+  ref = octree_nearest_pts(data, o, depth, pts, nempty, bound_check=True)
+  assert torch.equal(out, ref)
+  assert np.array_equal(np_(out), I.nearest_upsample(w, np_(data), depth, nempty))
+  assert torch.equal(OctreeUpsample('nearest', nempty)(data, o, depth), out)
+  for target in (depth + 1, depth + 2):
+    got = OctreeUpsample('linear', nempty)(data, o, depth, target)
+    assert np.allclose(np_(got), I.upsample(w, np_(data), depth, target, 'linear', nempty), atol=1e-6)
+    got = OctreeUpsample('nearest', nempty)(data, o, depth, target)
+    assert np.array_equal(np_(got), I.upsample(w, np_(data), depth, target, 'nearest', nempty))
+  assert OctreeUpsample('linear', nempty)(data, o, depth, depth) is data
+  # OctreeInterp rescales the points from the bounding box in place
+  p = (torch.rand(300, 4, generator=torch.Generator().manual_seed(2)) * 2 - 1)
+  p[:, 3] = (p[:, 3] > 0).float()
+  pg = p.clone().to(DEV)
+  got = OctreeInterp('linear', nempty, bound_check=True)(data, o, depth, pg)
+  scaled = p.numpy().copy()
+  scaled[:, :3] = (scaled[:, :3] + 1.0) * (2 ** depth / 2.0)
+  assert np.allclose(np_(pg), scaled, atol=1e-6)
+  assert np.allclose(np_(got), I.linear_pts(w, np_(data), depth, scaled, nempty, True), atol=1e-6)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_interp_gradients_and_dtypes(ref_data, dtype):
+  """Gradient with respect to the data (the transposed sparse product, no atomics): against
+  the oracle, and the same bits on a second run; 16-bit data against the fp32 definition."""
+  say('interp gradients', dtype)
+  t = np.load(os.path.join(ref_data, 'interp.npz'))
+  o = merged_octree(ref_data)
+  w = oracle_batch(ref_data)
+  depth = 5
+  g = torch.Generator().manual_seed(3)
+  for ne in (False, True):
+    rows = int(o.nnum_nempty[depth] if ne else o.nnum[depth])
+    pts = torch.from_numpy(t['pts']).to(DEV)
+    data = torch.randn(rows, 8, generator=g).to(dtype).to(DEV).requires_grad_()
+    grad = torch.randn(pts.shape[0], 8, generator=g).to(dtype).to(DEV)
+    out = octree_linear_pts(data, o, depth, pts, ne)
+    assert out.dtype == dtype
+    want = I.linear_pts(w, np_(data), depth, t['pts'], ne)
+    assert np.abs(np_(out) - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
+    out.backward(grad)
+    gd = data.grad.clone()
+    wantg = I.linear_pts_grad(w, np_(grad), depth, t['pts'], rows, ne)
+    assert np.abs(np_(gd) - wantg).max() <= max(TOL[dtype], 1e-5) * max(1.0, np.abs(wantg).max())
+    data.grad = None
+    octree_linear_pts(data, o, depth, pts, ne).backward(grad)
+    assert torch.equal(data.grad, gd)
+    # nearest: every point passes its gradient to the one row it read
+    data.grad = None
+    octree_nearest_pts(data, o, depth, pts, ne).backward(grad)
+    idx = I.search_xyzb(w, t['pts'], depth, ne)
+    wantn = np.zeros((rows, 8))
+    np.add.at(wantn, idx[idx >= 0], np_(grad).astype(np.float64)[idx >= 0])
+    assert np.abs(np_(data.grad) - wantn).max() <= max(TOL[dtype], 1e-5) * max(1.0, np.abs(wantn).max())
+
+
+@pytest.mark.parametrize('nempty', [False, True])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_max_pool_unpool_vs_oracle(ref_data, nempty, dtype):
+  """octree_max_pool / octree_max_unpool and their gradients, depths with full and sparse
+  parents, against the oracle (values are copies: exact in every dtype)."""
+  say('max pool', nempty, dtype)
+  o = merged_octree(ref_data)
+  w = oracle_batch(ref_data)
+  g = torch.Generator().manual_seed(4)
+  for depth in (3, 4, 6):
+    rows = int(o.nnum_nempty[depth] if nempty else o.nnum[depth])
+    data = torch.randn(rows, 5, generator=g).to(dtype)
+    dg = data.to(DEV).requires_grad_()
+    out, idx = octree_max_pool(dg, o, depth, nempty, return_indices=True)
+    want, widx = I.max_pool(w, data.float().numpy(), depth, nempty)
+    assert np.array_equal(np_(out), want) and np.array_equal(np_(idx), widx)
+    assert idx.dtype == torch.long
+    assert torch.equal(OctreeMaxPool(nempty)(dg, o, depth), out)
+    # gradient of pooling = unpooling of the gradient
+    grad = torch.randn(out.shape, generator=g).to(dtype)
+    out.backward(grad.to(DEV))
+    assert np.array_equal(np_(dg.grad), I.max_unpool(w, grad.float().numpy(), widx, depth - 1, nempty))
+    # unpooling, module form, and its gradient (a gather at the indices)
+    pooled = out.detach().clone().requires_grad_()
+    up = OctreeMaxUnpool(nempty)(pooled, idx, o, depth - 1)
+    assert np.array_equal(np_(up), I.max_unpool(w, want, widx, depth - 1, nempty))
+    gu = torch.randn(up.shape, generator=g).to(dtype)
+    up.backward(gu.to(DEV))
+    full = gu.float().numpy() if not nempty else I.octree_pad(w, gu.float().numpy(), depth)
+    picked = np.take_along_axis(full.reshape(-1, 8, 5), widx[:, None, :], 1)[:, 0]
+    wantg = picked if nempty else I.octree_pad(w, picked, depth - 1)
+    assert np.array_equal(np_(pooled.grad), wantg)
+
+
+def test_interp_and_pool_at_full_size():
+  """The benchmark octree (8 x 100k points, depth 8): properties that need no oracle run.
+  A constant field interpolates to the constant wherever a neighbour exists; interpolating
+  at the node centres returns the node values; nearest upsampling followed by max pooling
+  is the identity on non-empty nodes; pooling picks a value that is present."""
+  say('interp / pool: full size')
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 8, 1001, n=100000)
+  o = Octree(8, 2, batch_size=8)
+  o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=8))
+  depth = 8
+  rows = int(o.nnum_nempty[depth])
+  q = torch.cat([(pts.to(DEV) + 1.0) * 128.0, bid.to(DEV).float().view(-1, 1)], 1)
+  const = torch.full((rows, 3), 2.5, device=DEV)
+  out = octree_linear_pts(const, o, depth, q, nempty=True)
+  assert torch.allclose(out, torch.full_like(out, 2.5), atol=1e-5)          # every point lies in a leaf
+  near = octree_nearest_pts(const, o, depth, q, nempty=True)
+  assert bool((near == 2.5).all())
+  data = torch.randn(rows, 16, generator=torch.Generator().manual_seed(6)).to(DEV)
+  x, y, z, b = o.xyzb(depth, nempty=True)
+  centres = torch.stack([x + 0.5, y + 0.5, z + 0.5, b], 1).float()
+  assert torch.equal(octree_nearest_pts(data, o, depth, centres, nempty=True), data)
+  assert torch.allclose(octree_linear_pts(data, o, depth, centres, nempty=True), data, atol=1e-5)
+  coarse = torch.randn(int(o.nnum_nempty[depth - 1]), 16, generator=torch.Generator().manual_seed(7)).to(DEV)
+  up = octree_nearest_upsample(coarse, o, depth - 1, nempty=True)
+  assert torch.equal(octree_max_pool(up, o, depth, nempty=True), coarse)
+  pooled, idx = octree_max_pool(data, o, depth, nempty=True, return_indices=True)
+  back = octree_max_unpool(pooled, idx, o, depth - 1, nempty=True)
+  hit = back != 0
+  assert torch.equal(back[hit], data[hit])
+  assert int(hit.sum()) == pooled.numel() - int((pooled == 0).sum())       # (a maximum may be exactly 0)
