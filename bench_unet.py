@@ -1,0 +1,140 @@
+"""Forward + backward of the reference's segmentation U-Net (ocnn/models/unet.py:16-105: encoder
+channels 32-32-64-128-256 with 2/3/4/6 residual blocks, decoder 256-256-128-96-96 with 2 each,
+2x2x2 stride-2 (de)convolutions between levels, trilinear interpolation of the last features at
+the query points, a 1x1 head) assembled from this package's layers and torch's BatchNorm1d, on
+one MI355X.  Supporting data for the pieces around the convolutions (the headline number is
+bench.py's): synthetic batch of 8 clouds x 150 000 points at depth 9, input signal 'ND'
+(normals + displacement), 10 classes, random weights, cross-entropy against random labels.
+
+One JSON line: ms per forward + backward, and the share of the step spent in each kind of
+kernel when --profile is given (torch profiler, device time).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, 'ocnn-pytorch_amd')):
+  if p not in sys.path:
+    sys.path.insert(0, p)
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--steps', type=int, default=10)
+  ap.add_argument('--warmup', type=int, default=3)
+  ap.add_argument('--batch', type=int, default=8)
+  ap.add_argument('--points', type=int, default=150000)
+  ap.add_argument('--depth', type=int, default=9)
+  ap.add_argument('--dtype', default='bfloat16')
+  ap.add_argument('--nempty', type=int, default=1)
+  ap.add_argument('--profile', action='store_true')
+  args = ap.parse_args()
+  import torch
+  from ocnn_amd import modules, synthetic
+  from ocnn_amd.nn import OctreeInterp
+  from ocnn_amd.octree import Octree, Points
+  assert torch.cuda.is_available(), 'bench_unet.py needs a GPU'
+  dev = 'cuda:0'
+  torch.cuda.set_device(0)
+  dtype = getattr(torch, args.dtype)
+  nempty = bool(args.nempty)
+
+  class UNet(torch.nn.Module):
+    def __init__(self, cin, cout):
+      super().__init__()
+      enc, dec = [32, 32, 64, 128, 256], [256, 256, 128, 96, 96]
+      eb, db = [2, 3, 4, 6], [2, 2, 2, 2]
+      self.stages = len(eb)
+      self.conv1 = modules.OctreeConvBnRelu(cin, enc[0], nempty=nempty)
+      self.downsample = torch.nn.ModuleList(
+          [modules.OctreeConvBnRelu(enc[i], enc[i + 1], [2], 2, nempty) for i in range(4)])
+      self.encoder = torch.nn.ModuleList(
+          [modules.OctreeResBlocks(enc[i + 1], enc[i + 1], eb[i], 1, nempty) for i in range(4)])
+      self.upsample = torch.nn.ModuleList(
+          [modules.OctreeDeconvBnRelu(dec[i], dec[i + 1], [2], 2, nempty) for i in range(4)])
+      self.decoder = torch.nn.ModuleList(
+          [modules.OctreeResBlocks(dec[i + 1] + enc[-i - 2], dec[i + 1], db[i], 1, nempty) for i in range(4)])
+      self.octree_interp = OctreeInterp('linear', nempty, rescale_pts=False)
+      self.header = torch.nn.Sequential(modules.Conv1x1BnRelu(dec[-1], 64), modules.Conv1x1(64, cout, use_bias=True))
+
+    def forward(self, data, octree, depth, query):
+      convd = {depth: self.conv1(data, octree, depth)}
+      for i in range(self.stages):
+        d = depth - i
+        convd[d - 1] = self.encoder[i](self.downsample[i](convd[d], octree, d), octree, d - 1)
+      d0 = depth - self.stages
+      x = convd[d0]
+      for i in range(self.stages):
+        d = d0 + i
+        x = torch.cat([convd[d + 1], self.upsample[i](x, octree, d)], dim=1)
+        x = self.decoder[i](x, octree, d + 1)
+      return self.header(self.octree_interp(x, octree, depth, query))
+
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, args.batch, 1004, n=args.points)
+  pc = Points(pts.to(dev), nrm.to(dev), batch_id=bid.to(dev), batch_size=args.batch)
+  octree = Octree(args.depth, 2, batch_size=args.batch)
+  octree.build_octree(pc)
+  octree.construct_all_neigh()
+  feat = octree.get_input_feature('ND', nempty).to(dtype)
+  query = torch.cat([(pts.to(dev) + 1.0) * (2 ** (args.depth - 1)), bid.to(dev).float().view(-1, 1)], 1)
+  labels = torch.randint(0, 10, (query.shape[0],), generator=torch.Generator().manual_seed(5)).to(dev)
+  torch.manual_seed(0)
+  net = UNet(feat.shape[1], 10).to(dev).to(dtype)
+  params = [p for p in net.parameters()]
+
+  def step():
+    for p in params:
+      p.grad = None
+    logits = net(feat, octree, args.depth, query)
+    torch.nn.functional.cross_entropy(logits.float(), labels).backward()
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  ms = (time.perf_counter() - t0) / args.steps * 1e3
+  out = {'net': 'U-Net (ocnn/models/unet.py), forward + backward', 'ms_per_step': ms, 'dtype': args.dtype,
+         'nempty': nempty, 'batch': args.batch, 'points': int(pts.shape[0]), 'depth': args.depth,
+         'rows_per_depth': (octree.nnum_nempty if nempty else octree.nnum).tolist(),
+         'parameters': sum(p.numel() for p in params)}
+  if args.profile:
+    from torch.profiler import profile, ProfilerActivity
+    with profile(activities=[ProfilerActivity.CUDA, ProfilerActivity.CPU]) as prof:
+      step()
+      torch.cuda.synchronize()
+    groups = {}
+    for e in prof.key_averages():
+      t = getattr(e, 'device_time_total', 0) or getattr(e, 'cuda_time_total', 0)
+      if e.device_type is not None and 'cuda' in str(e.device_type).lower() or 'kernel' in e.key.lower():
+        pass
+      name = e.key
+      if t <= 0 or not any(k in name for k in ('ocnn', 'Kernel', 'kernel', 'Cijk', 'gemm')):
+        continue
+      if 'conv_' in name or 'wgrad' in name or 'pack_weights' in name:
+        k = 'octree conv kernels'
+      elif 'batch_norm' in name or 'BatchNorm' in name:
+        k = 'batch norm'
+      elif 'interp' in name or 'csr_rows' in name or 'search' in name:
+        k = 'interpolation'
+      elif 'pad' in name and 'ocnn' in name:
+        k = 'pad / depad'
+      elif 'tile_plan' in name or 'neigh' in name:
+        k = 'tables / plans'
+      elif 'Cijk' in name or 'gemm' in name:
+        k = 'dense GEMM (1x1)'
+      else:
+        k = 'elementwise / other'
+      groups[k] = groups.get(k, 0.0) + t / 1e3
+    out['device_ms_by_kind'] = {k: round(v, 3) for k, v in sorted(groups.items(), key=lambda kv: -kv[1])}
+  print(json.dumps(out), flush=True)
+
+
+if __name__ == '__main__':
+  main()

@@ -212,11 +212,12 @@ int ocnn_conv_gather_rw(int dtype, const void* in, int64_t rows_in, const uint16
                         int w_transposed, int reverse_slots, const void* bias, void* out,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
-/* ocnn_conv_gather for wide layers (cin a multiple of 64, cout a multiple of 128, any
+/* ocnn_conv_gather for wide layers (cin >= 64 and cout >= 96, multiples of 32, any
  * K <= 27) over the tile plan: the distinct rows of a tile are staged in LDS 64 input
  * channels at a time, the weights stream from L2 into registers in the MFMA operand
  * layout, the four waves of a workgroup split the output channels.  Same arguments and
- * result as ocnn_conv_gather_rw; plan_max_distinct <= 416. */
+ * result as ocnn_conv_gather_rw; plan_max_distinct <= 416; workspace K * cin64 * cout * 2 bytes
+ * with cin64 = cin rounded up to a multiple of 64. */
 int ocnn_conv_gather_wide_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                     int plan_max_distinct);
 int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,

@@ -33,11 +33,12 @@ static __device__ __forceinline__ void wd_dma16(__amdgpu_buffer_rsrc_t rs, char*
 //   input channel  = 64 cc + 16 s + 8 (lane / 32) + j
 //   output channel = 32 cg + perm(lane % 32), perm(8a + 4q + b) = 16 q + 4 a + b,
 // so that a lane ends with 16 consecutive output channels per M tile.
+// Input channels are padded to whole chunks of 64 with zero weights.
 template <typename T>
 __global__ void pack_weights_wide_kernel(const T* __restrict__ w, T* __restrict__ out, int K, int cin,
                                          int cout, int transposed, int reverse) {
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= (int64_t)K * cin * cout) return;
+  if (e >= (int64_t)K * ((cin + 63) & ~63) * cout) return;
   int j = (int)(e & 7);
   int lane = (int)((e >> 3) & 63);
   int s = (int)((e >> 9) & 3);
@@ -51,11 +52,14 @@ __global__ void pack_weights_wide_kernel(const T* __restrict__ w, T* __restrict_
   int chan = 64 * cc + 16 * s + 8 * q + j;
   int co = 32 * cg + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
   int kk = reverse ? K - 1 - k : k;
-  out[e] = transposed ? w[((int64_t)kk * cout + co) * cin + chan] : w[((int64_t)kk * cin + chan) * cout + co];
+  if (chan >= cin) out[e] = (T)0.f;
+  else out[e] = transposed ? w[((int64_t)kk * cout + co) * cin + chan] : w[((int64_t)kk * cin + chan) * cout + co];
 }
 
 // One workgroup: one tile of 128 rows x 128 MB output channels (blockIdx.y); wave w owns
-// the output channels 32 MB w .. of that block.
+// the output channels 32 MB w .. of that block.  Channel counts are multiples of 32: the
+// last 64-channel chunk of the input may be half a chunk (its other half is staged as zeros
+// and meets zero weights), and waves whose output channels lie past the end idle.
 template <typename T, int MB>
 __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const uint16_t* __restrict__ loc,
@@ -71,7 +75,8 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int q = lane >> 5, r32 = lane & 31;
-  const int ncc = cin >> 6;
+  const int ncc = (cin + 63) >> 6;
+  const int ncg = cout >> 5;
   const int cg0 = ((int)blockIdx.y * 4 + wave) * MB;        // first 32-channel group of this wave
   const uint32_t pitch = (uint32_t)cin * 2u;
 
@@ -90,6 +95,7 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   // a lane's 16-byte chunk c of LDS row p lands at chunk c ^ ((p >> 1) & 7) (bank swizzle)
   const uint32_t st_c = (uint32_t)(((lane & 7) ^ (((lane >> 4) + 4 * wave) & 7)) * 16);
   const int st_p = 8 * wave + (lane >> 3);                  // LDS row of piece 0; piece i: + 32 i
+  const bool half_oob = (cin & 63) != 0 && st_c >= 64;      // this lane's piece of a half chunk at the end
   constexpr int kRowPieces = (kWdCap + 1 + 31) / 32;
 
   f32x16 acc[4][MB];
@@ -102,14 +108,15 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
 
   // ---- operands ----
   // A: weights of (chunk, slot) kk = cc K + k, k-step s; one 16-byte load per lane and M tile
-  const int64_t kstride = (int64_t)(cout >> 5) * 2048;       // elements between consecutive kk
-  const T* wbase = wpk + (int64_t)cg0 * 2048 + lane * 8;
+  const int64_t kstride = (int64_t)ncg * 2048;               // elements between consecutive kk
+  const T* wbase = wpk + lane * 8;
   const int kk_last = ncc * K - 1;
+  const bool active = cg0 < ncg;                             // (wave-uniform)
   u32x4 A[4][MB];                                            // ring over the k-steps
   auto load_a = [&](int kk, int s, u32x4 (&a)[MB]) {
     const T* p = wbase + (int64_t)min(kk, kk_last) * kstride + s * 512;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) a[mb] = *(const u32x4*)(p + mb * 2048);
+    for (int mb = 0; mb < MB; ++mb) a[mb] = *(const u32x4*)(p + (int64_t)min(cg0 + mb, ncg - 1) * 2048);
   };
   // B: a lane reads 16 bytes (8 input channels) of the neighbour row of row 32 rb + r32.
   // pv = byte address of the row in s_rows with the swizzle of k-step 0 folded in.
@@ -140,7 +147,9 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
       const int g = wave + 4 * i;
       if (g < groups) {
         const int32_t id = s_u[st_p + 32 * i];               // -1: out of range, loads zeros
-        wd_dma16(rs_in, (char*)s_rows + g * 1024, (uint32_t)id * pitch + ((uint32_t)cc * 128u + st_c));
+        uint32_t off = (uint32_t)id * pitch + ((uint32_t)cc * 128u + st_c);
+        if (cc == ncc - 1 && half_oob) off = 0xffffff00u;    // past the row's channels: zeros, not the next row
+        wd_dma16(rs_in, (char*)s_rows + g * 1024, off);
       }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -156,10 +165,12 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
         load_a(kk + (s >= 2 ? 1 : 0), (s + 2) & 3, A[(s + 2) & 3]);
         if (s < 3) read_b(pvc, s + 1, Bb[(s + 1) & 1]);
         else read_b(pvn, 0, Bb[0]);                          // (past the last slot: unused)
+        if (active) {
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb)
+          for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[s][mb], Bb[s & 1][rb], acc[rb][mb]);
+            for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[s][mb], Bb[s & 1][rb], acc[rb][mb]);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -170,6 +181,7 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   // ---- epilogue: a lane holds 16 consecutive output channels of a row per M tile ----
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
+    if (cg0 + mb >= ncg) continue;
     const int co = 32 * (cg0 + mb) + 16 * q;
     float bv[16];
 #pragma unroll
@@ -306,7 +318,7 @@ using namespace ocnn;
 extern "C" int ocnn_conv_gather_wide_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                                int plan_max_distinct) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (cin < 64 || cin % 64 != 0 || cout < 128 || cout % 128 != 0 || cin > 2048 || cout > 2048) return 0;
+  if (cin < 64 || cin % 32 != 0 || cout < 96 || cout % 32 != 0 || cin > 2048 || cout > 2048) return 0;
   if (K < 1 || K > 27) return 0;
   if (plan_max_distinct > kWdCap) return 0;
   if ((int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
@@ -317,7 +329,7 @@ template <typename T>
 static int run_wide(const void* in, int64_t rows_in, const uint16_t* loc, const int32_t* uptr,
                     const int32_t* urows, int64_t rows_out, int K, int cin, int cout, const void* w,
                     int w_transposed, int reverse, const void* bias, void* out, void* ws, hipStream_t st) {
-  const int64_t total = (int64_t)K * cin * cout;
+  const int64_t total = (int64_t)K * align_up(cin, 64) * cout;
   hipLaunchKernelGGL(pack_weights_wide_kernel<T>, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, st,
                      (const T*)w, (T*)ws, K, cin, cout, w_transposed, reverse);
   const int64_t tiles = cdiv(rows_out, kWdRows);
@@ -328,7 +340,7 @@ static int run_wide(const void* in, int64_t rows_in, const uint16_t* loc, const 
                        dim3(256), 0, st, (const T*)in, in_bytes, loc, uptr, urows, (const T*)ws, (const T*)bias,
                        (T*)out, rows_out, K, cin, cout, tiles, per_xcd);
   else
-    hipLaunchKernelGGL((conv_gather_wide_kernel<T, 1>), dim3((unsigned)(per_xcd * 8), (unsigned)(cout / 128)),
+    hipLaunchKernelGGL((conv_gather_wide_kernel<T, 1>), dim3((unsigned)(per_xcd * 8), (unsigned)cdiv(cout, 128)),
                        dim3(256), 0, st, (const T*)in, in_bytes, loc, uptr, urows, (const T*)ws, (const T*)bias,
                        (T*)out, rows_out, K, cin, cout, tiles, per_xcd);
   return check_launch("conv_gather_wide");
@@ -344,7 +356,7 @@ extern "C" int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in,
   OCNN_REQUIRE(rows_out >= 0 && rows_out < (1ll << 31) && plan_total >= 0 && plan_total < (1ll << 29),
                "conv_gather_wide: rows out of range");
   if (rows_out == 0) return OCNN_OK;
-  if (workspace_bytes < (int64_t)K * cin * cout * 2) {
+  if (workspace_bytes < (int64_t)K * align_up(cin, 64) * cout * 2) {
     set_error("conv_gather_wide: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }

@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
   static_assert(kPieces <= 20 && (kWpCap + 1) % 16 == 0, "five steps of four pieces stage a tile");
   constexpr int RSH = 5 + H;                               // log2 of the bytes of a C-channel row
   // a block of a wider layer: rows of ca (cb) channels, this block's 64 start at xb (gb)
-  const int nbb = BLK ? cb / C : 1;
+  const int nbb = BLK ? (cb + C - 1) / C : 1;             // (channel counts are multiples of 32: the last block may be half)
   const int blk_a = BLK ? (int)blockIdx.y / nbb : 0, blk_b = BLK ? (int)blockIdx.y % nbb : 0;
   const uint32_t x_pitch = BLK ? (uint32_t)ca * 2u : (1u << RSH), g_pitch = BLK ? (uint32_t)cb * 2u : (1u << RSH);
   const uint32_t xb = (uint32_t)blk_a << RSH, gb = (uint32_t)blk_b << RSH;
@@ -395,13 +395,18 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     const int ldb = BLK ? cb : C;
     float* dst = BLK ? partial + (((int64_t)split * KK + slot) * ca + blk_a * C) * cb + blk_b * C
                      : partial + ((int64_t)split * KK + slot) * (C * C);
+    // a half block at the end of the channels: what the staging loads brought in beyond a
+    // row only reached sums that are not written
+    if (BLK && blk_a * C + 32 * ah >= ca) continue;
 #pragma unroll
-    for (int bh = 0; bh < H; ++bh)
+    for (int bh = 0; bh < H; ++bh) {
+      if (BLK && blk_b * C + 32 * bh >= cb) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int a = 32 * ah + 8 * (r >> 2) + 4 * q + (r & 3);
         dst[a * ldb + 32 * bh + b32] = acc[u][bh][r];
       }
+    }
   }
 }
 
@@ -417,7 +422,7 @@ extern "C" void ocnn_debug_set_wp_timing(long long* p) { g_wp_dbg = p; }
 
 static int wp_splits(int K, int ca, int cb, int n_cu) {
   const int groups = (K == 27 && ca >= 64) ? 2 : 1;
-  const int blocks = ca >= 64 ? (ca / 64) * (cb / 64) : 1;
+  const int blocks = ca >= 64 ? ((ca + 63) / 64) * ((cb + 63) / 64) : 1;
   int s = std::max(8, n_cu / (groups * blocks) / 8 * 8);      // a multiple of 8: ranges are dealt to the XCDs
   return std::min(s, 256);
 }
@@ -436,7 +441,7 @@ static int wp_cu_count() {
 extern "C" int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
                                                  int cb, int plan_max_distinct) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (!(ca == 32 && cb == 32) && !(ca >= 64 && cb >= 64 && ca % 64 == 0 && cb % 64 == 0 && ca <= 1024 && cb <= 1024))
+  if (!(ca == 32 && cb == 32) && !(ca >= 64 && cb >= 64 && ca % 32 == 0 && cb % 32 == 0 && ca <= 1024 && cb <= 1024))
     return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
   if (plan_max_distinct > kWpCap) return 0;
@@ -463,7 +468,7 @@ static void launch_wp(const void* x, int64_t rows_x, const void* g, const uint16
                        nsplit, ca, cb, partial, g_wp_dbg);
   else if constexpr (C == 64)
     hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS, true>),
-                       dim3(nsplit * GROUPS, (ca / C) * (cb / C)), dim3(256), 0, st, (const T*)x, xb, (const T*)g,
+                       dim3(nsplit * GROUPS, ((ca + C - 1) / C) * ((cb + C - 1) / C)), dim3(256), 0, st, (const T*)x, xb, (const T*)g,
                        gb, loc, lb, uptr, urows, ub, tiles, per, nsplit, ca, cb, partial, g_wp_dbg);
 }
 

@@ -1,0 +1,137 @@
+"""Compositions of the hot-path layers with torch's BatchNorm1d / ReLU / Linear under the
+class and attribute names of ocnn/modules/modules.py and ocnn/modules/resblocks.py, so that
+networks written against the reference (and their state_dicts) work unchanged."""
+
+from typing import List
+
+import torch
+import torch.nn
+
+from .nn import OctreeConv, OctreeDeconv
+
+
+class _LayerBn(torch.nn.Module):
+  """layer -> BatchNorm1d [-> ReLU]; `name` is the attribute the layer is stored under."""
+
+  def __init__(self, name, layer, channels, relu):
+    super().__init__()
+    self._name = name
+    setattr(self, name, layer)
+    self.bn = torch.nn.BatchNorm1d(channels)
+    if relu:
+      self.relu = torch.nn.ReLU(inplace=True)
+    self._relu = relu
+
+  def forward(self, data, *args):
+    out = self.bn(getattr(self, self._name)(data, *args))
+    return self.relu(out) if self._relu else out
+
+
+class OctreeConvBn(_LayerBn):
+  """ocnn/modules/modules.py:32-51."""
+
+  def __init__(self, in_channels: int, out_channels: int, kernel_size: List[int] = [3],
+               stride: int = 1, nempty: bool = False):
+    super().__init__('conv', OctreeConv(in_channels, out_channels, kernel_size, stride, nempty),
+                     out_channels, False)
+
+
+class OctreeConvBnRelu(_LayerBn):
+  """ocnn/modules/modules.py:54-75."""
+
+  def __init__(self, in_channels: int, out_channels: int, kernel_size: List[int] = [3],
+               stride: int = 1, nempty: bool = False):
+    super().__init__('conv', OctreeConv(in_channels, out_channels, kernel_size, stride, nempty),
+                     out_channels, True)
+
+
+class OctreeDeconvBnRelu(_LayerBn):
+  """ocnn/modules/modules.py:78-99."""
+
+  def __init__(self, in_channels: int, out_channels: int, kernel_size: List[int] = [3],
+               stride: int = 1, nempty: bool = False):
+    super().__init__('deconv', OctreeDeconv(in_channels, out_channels, kernel_size, stride, nempty),
+                     out_channels, True)
+
+
+class Conv1x1(torch.nn.Module):
+  """ocnn/modules/modules.py:102-117: a 1x1x1 convolution on (N, C) rows is a Linear."""
+
+  def __init__(self, in_channels: int, out_channels: int, use_bias: bool = False):
+    super().__init__()
+    self.linear = torch.nn.Linear(in_channels, out_channels, use_bias)
+
+  def forward(self, data: torch.Tensor):
+    return self.linear(data)
+
+
+class Conv1x1Bn(_LayerBn):
+  """ocnn/modules/modules.py:120-134."""
+
+  def __init__(self, in_channels: int, out_channels: int):
+    super().__init__('conv', Conv1x1(in_channels, out_channels, use_bias=False), out_channels, False)
+
+
+class Conv1x1BnRelu(_LayerBn):
+  """ocnn/modules/modules.py:137-153."""
+
+  def __init__(self, in_channels: int, out_channels: int):
+    super().__init__('conv', Conv1x1(in_channels, out_channels, use_bias=False), out_channels, True)
+
+
+class OctreeResBlock2(torch.nn.Module):
+  """Two 3x3x3 convolutions with a (projected) shortcut, stride 1
+  (ocnn/modules/resblocks.py:65-99)."""
+
+  def __init__(self, in_channels, out_channels, stride=1, bottleneck=1, nempty=False):
+    super().__init__()
+    assert stride == 1, 'OctreeResBlock2: stride 1 only'
+    self.in_channels, self.out_channels, self.stride = in_channels, out_channels, stride
+    mid = int(out_channels / bottleneck)
+    self.conv3x3a = OctreeConvBnRelu(in_channels, mid, nempty=nempty)
+    self.conv3x3b = OctreeConvBn(mid, out_channels, nempty=nempty)
+    if in_channels != out_channels:
+      self.conv1x1 = Conv1x1Bn(in_channels, out_channels)
+    self.relu = torch.nn.ReLU(inplace=True)
+
+  def forward(self, data: torch.Tensor, octree, depth: int):
+    out = self.conv3x3b(self.conv3x3a(data, octree, depth), octree, depth)
+    if self.in_channels != self.out_channels:
+      data = self.conv1x1(data)
+    return self.relu(out + data)
+
+
+class OctreeResBlocks(torch.nn.Module):
+  """A chain of residual blocks (ocnn/modules/resblocks.py:134-159)."""
+
+  def __init__(self, in_channels, out_channels, resblk_num, bottleneck=4, nempty=False,
+               resblk=OctreeResBlock2, use_checkpoint=False):
+    super().__init__()
+    self.resblk_num = resblk_num
+    self.use_checkpoint = use_checkpoint
+    widths = [in_channels] + [out_channels] * resblk_num
+    self.resblks = torch.nn.ModuleList(
+        [resblk(widths[i], widths[i + 1], 1, bottleneck, nempty) for i in range(resblk_num)])
+
+  def forward(self, data: torch.Tensor, octree, depth: int):
+    for blk in self.resblks:
+      if self.use_checkpoint:
+        data = torch.utils.checkpoint.checkpoint(blk, data, octree, depth, use_reentrant=False)
+      else:
+        data = blk(data, octree, depth)
+    return data
+
+
+class InputFeature(torch.nn.Module):
+  """The input signal stored in the octree (ocnn/modules/modules.py:288-305)."""
+
+  def __init__(self, feature: str = 'NDF', nempty: bool = False):
+    super().__init__()
+    self.nempty = nempty
+    self.feature = feature.upper()
+
+  def forward(self, octree):
+    return octree.get_input_feature(self.feature, self.nempty)
+
+  def extra_repr(self) -> str:
+    return 'feature={}, nempty={}'.format(self.feature, self.nempty)

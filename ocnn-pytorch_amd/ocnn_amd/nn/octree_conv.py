@@ -209,8 +209,11 @@ class OctreeConvBase:
   def _plan(self, data, cin, cout, inverse=False):
     """Tile plan for the staged kernel, when the shape can use it."""
     L, code = _lib.lib(), _lib.DTYPE_CODE.get(data.dtype, -1)
-    if not (L.ocnn_conv_gather_planned_supported(code, data.shape[0], cin, cout) or
-            L.ocnn_conv_gather_rw_supported(code, data.shape[0], self.kdim, cin, cout, 0)):
+    rows = data.shape[0]
+    if not (L.ocnn_conv_gather_planned_supported(code, rows, cin, cout) or
+            L.ocnn_conv_gather_rw_supported(code, rows, self.kdim, cin, cout, 0) or
+            L.ocnn_conv_gather_wide_supported(code, rows, self.kdim, cin, cout, 0) or
+            L.ocnn_conv_wgrad_planned_supported(code, rows, rows, self.kdim, cin, cout, 0)):
       return None
     return self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse,
                              self.fine_h)

@@ -479,7 +479,7 @@ def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
   code = _lib.dtype_code(x)
   assert L.ocnn_conv_gather_wide_supported(code, rows_in, K, cin, cout, plan.umax)
   out = torch.empty((rows, cout), dtype=x.dtype, device=x.device)
-  ws = torch.empty(K * cin * cout * 2, dtype=torch.uint8, device=x.device)
+  ws = torch.empty(K * (-(-cin // 64) * 64) * cout * 2, dtype=torch.uint8, device=x.device)   # whole 64-channel chunks
   _lib.check(L.ocnn_conv_gather_wide(
       code, _lib.ptr(x), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax,
       plan.total, rows, K, _lib.ptr(w), cin, cout, int(transposed), int(reverse), _lib.ptr(bias),
@@ -489,26 +489,30 @@ def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('K,cin,cout', [(27, 128, 128), (27, 64, 256), (9, 192, 128), (8, 128, 384), (3, 256, 256),
-                                        (1, 64, 128)])
+                                        (1, 64, 128), (27, 96, 96), (27, 128, 96), (9, 96, 160), (3, 160, 224)])
 def test_wide_gather_kernel(dtype, K, cin, cout):
   """Gather-GEMM for wide layers (weights streamed into registers, rows staged 64 input
-  channels at a time), both output-channel widths per workgroup, with bias, and the
-  transposed + mirrored form, against the oracle."""
+  channels at a time), both output-channel widths per workgroup, channel counts that are
+  odd multiples of 32 (half a chunk of input channels, idle waves on the output side), with
+  bias, and the transposed + mirrored form, against the oracle.  The last input row is set
+  to NaN where no table entry reads it: nothing beyond a row may leak into a result."""
   from ocnn_amd.octree.octree import TilePlan
   g = torch.Generator().manual_seed(7 * K + cin)
   for rows, rows_in in [(1000, 1000), (130, 150), (128 * 40 + 1, 3000)]:
     say('wide gather', dtype, K, cin, cout, rows, rows_in)
-    table = _local_table(rows, rows_in, K, g)
+    table = _local_table(rows, rows_in - 1, K, g)        # the last input row is never read ..
     tg = table.to(DEV)
     plan = TilePlan(tg)
     t64 = table.numpy().astype(np.int64)
     x = torch.randn(rows_in, cin, generator=g).to(dtype)
     w = (torch.randn(K, cin, cout, generator=g) / (K * cin) ** 0.5).to(dtype)
     b = torch.randn(cout, generator=g).to(dtype)
-    got = _gather_wide(x.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV))
+    xn = x.clone()
+    xn[-1] = float('nan')                                # .. and holds NaN
+    got = _gather_wide(xn.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV))
     want = C.forward_gemm(f64(x), f64(w), t64) + f64(b)
     assert rel_err(got, want) < TOL[dtype]
-    if cin % 128 == 0:                                   # the data gradient: cout -> cin
+    if cin >= 96:                                        # the data gradient: cout -> cin
       gr = torch.randn(rows_in, cout, generator=g).to(dtype)
       got = _gather_wide(gr.to(DEV), rows_in, tg, plan, w.to(DEV), cin, True, True, None)
       want = C.forward_gemm(f64(gr), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
@@ -516,7 +520,8 @@ def test_wide_gather_kernel(dtype, K, cin, cout):
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize('K,ca,cb', [(27, 128, 128), (27, 64, 192), (9, 256, 64), (8, 128, 64), (3, 192, 128)])
+@pytest.mark.parametrize('K,ca,cb', [(27, 128, 128), (27, 64, 192), (9, 256, 64), (8, 128, 64), (3, 192, 128),
+                                     (27, 96, 96), (27, 96, 128), (8, 160, 96), (3, 64, 96)])
 def test_planned_wgrad_channel_blocks(dtype, K, ca, cb):
   """Weight gradient of layers with more than 64 channels: the planned kernel sums one
   64 x 64 block of channel pairs per workgroup."""
