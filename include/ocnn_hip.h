@@ -322,6 +322,26 @@ int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const vo
                               int channels, void* gw, void* workspace, int64_t workspace_bytes,
                               void* stream);
 
+/* Batch normalisation over the rows of a (rows, c) matrix with the ReLU of the
+ * conv-bn-relu blocks fused in (ocnn/modules/modules.py:32-99: OctreeConvBn, OctreeConvBnRelu,
+ * OctreeDeconvBnRelu use torch.nn.BatchNorm1d + ReLU): per-channel mean, biased variance and
+ * 1 / sqrt(var + eps) of x; y = (x - mean) * invstd * gamma + beta [then max(., 0)]; and the
+ * gradient dx, dgamma, dbeta (training = 1: statistics of this batch; 0: fixed statistics;
+ * dx may be NULL).  gamma / beta may be NULL (no affine part).  fp32 arithmetic, two-level
+ * reductions with a fixed order.  channels a multiple of 16 bytes of elements. */
+int ocnn_batch_norm_supported(int dtype, int64_t rows, int channels);
+int64_t ocnn_batch_norm_workspace_bytes(int channels);
+int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
+                          float* mean, float* var, float* invstd, void* workspace,
+                          int64_t workspace_bytes, void* stream);
+int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
+                          const float* invstd, const float* gamma, const float* beta, int relu,
+                          void* y, void* stream);
+int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy, int64_t rows, int channels,
+                             const float* mean, const float* invstd, const float* gamma,
+                             const float* beta, int relu, int training, void* dx, float* dgamma,
+                             float* dbeta, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Key search, ocnn/octree/octree.py:448-488 (search_key / search_xyzb): out[i] = position of
  * query[i] in the ascending `keys`, or -1.  ocnn_search_points takes float (x, y, z, b) rows,
  * truncates and encodes them like xyz2key (ocnn/octree/shuffled_key.py:60-90) and, with

@@ -27,6 +27,7 @@ SOURCES = {
     'plan.hip': [],
     'misc.hip': [],
     'interp.hip': ['-ffp-contract=off'],
+    'norm.hip': ['-ffp-contract=off'],
 }
 
 COMMON = ['-O3', '--offload-arch=gfx950', '-fPIC', '-std=c++17', '-I', INCLUDE, '-I', CSRC,

@@ -1,0 +1,404 @@
+// Batch normalisation over the rows of a (rows, C) feature matrix with the ReLU that follows
+// it in every conv-bn-relu block fused in: training statistics, the normalise (+ ReLU) pass,
+// and the gradient.  Everything here is HBM-bound; the point of the fusion is the number of
+// passes over the tensor (forward 2 reads + 1 write, backward 4 reads + 1 write, the ReLU
+// costs none) and 16-byte accesses on channels-last rows.  Reductions are two-level with a
+// fixed order (per-workgroup partial sums, then one thread per channel in fp64): no atomics,
+// bit-reproducible.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace ocnn {
+
+constexpr int kBnMaxBlocks = 2048;
+
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) BnVec { T v[VEC]; };
+
+// partial[blk][0][c] = sum_r (x[r][c] - x[0][c]),  partial[blk][1][c] = sum_r (x[r][c] - x[0][c])^2
+// over the rows of the workgroup (shifting by the first row keeps the variance free of
+// cancellation when the mean is large against the spread).  Thread: VEC channels of every
+// rpp-th row.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bn_stats_kernel(const T* __restrict__ x, int64_t rows, int C,
+                                                       int64_t rows_per_blk, float* __restrict__ partial) {
+  typedef BnVec<T, VEC> V;
+  __shared__ float s_a[256 * VEC], s_b[256 * VEC];
+  const int lpr = C / VEC, rpp = 256 / lpr;
+  const int tid = threadIdx.x, rl = tid / lpr, cl = tid - rl * lpr;
+  float s1[VEC], s2[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) s1[v] = s2[v] = 0.f;
+  if (rl < rpp) {
+    const V k = *(const V*)(x + cl * VEC);
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
+    const int64_t r1 = min(rows, r0 + rows_per_blk);
+    // four rows in flight per thread (rows past the end repeat row 0, whose shifted value is 0)
+    for (int64_t r = r0 + rl; r < r1; r += 4 * rpp) {
+      V a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t ru = r + (int64_t)u * rpp;
+        a[u] = *(const V*)(x + (ru < r1 ? ru * C : 0) + cl * VEC);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float d = to_f32(a[u].v[v]) - to_f32(k.v[v]);
+          s1[v] += d;
+          s2[v] += d * d;
+        }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    s_a[tid * VEC + v] = s1[v];
+    s_b[tid * VEC + v] = s2[v];
+  }
+  __syncthreads();
+  if (tid < lpr) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      float a = 0.f, b = 0.f;
+      for (int g = 0; g < rpp; ++g) {
+        a += s_a[(g * lpr + tid) * VEC + v];
+        b += s_b[(g * lpr + tid) * VEC + v];
+      }
+      partial[((int64_t)blockIdx.x * 2 + 0) * C + tid * VEC + v] = a;
+      partial[((int64_t)blockIdx.x * 2 + 1) * C + tid * VEC + v] = b;
+    }
+  }
+}
+
+// Sum of the per-workgroup partial sums of a channel, in a fixed order: 256 threads = 16
+// lanes x 16 channels, lane l adds the partials l, l + 16, .. (fp64), then lane 0 adds the
+// 16 lane sums.  Returns the channel for the threads that hold a result, -1 for the others.
+__device__ __forceinline__ int bn_sum_partials(const float* __restrict__ partial, int nblk, int C, double& a,
+                                               double& b) {
+  __shared__ double s_pa[256], s_pb[256];
+  const int tid = threadIdx.x, l = tid >> 4;
+  const int c = blockIdx.x * 16 + (tid & 15);
+  double sa = 0.0, sb = 0.0;
+  if (c < C) {
+    for (int i = l; i < nblk; i += 64) {                     // four loads of each kind in flight
+      float va[4], vb[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int iu = i + 16 * u;
+        va[u] = iu < nblk ? partial[((int64_t)iu * 2 + 0) * C + c] : 0.f;
+        vb[u] = iu < nblk ? partial[((int64_t)iu * 2 + 1) * C + c] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        sa += (double)va[u];
+        sb += (double)vb[u];
+      }
+    }
+  }
+  s_pa[tid] = sa;
+  s_pb[tid] = sb;
+  __syncthreads();
+  if (l != 0 || c >= C) return -1;
+  a = 0.0;
+  b = 0.0;
+  for (int k = 0; k < 16; ++k) {
+    a += s_pa[16 * k + tid];
+    b += s_pb[16 * k + tid];
+  }
+  return c;
+}
+
+// mean, biased variance and 1 / sqrt(var + eps) per channel from the partial sums
+template <typename T>
+__global__ void bn_stats_finish_kernel(const float* __restrict__ partial, int nblk, const T* __restrict__ x,
+                                       int64_t rows, int C, float eps, float* __restrict__ mean,
+                                       float* __restrict__ var, float* __restrict__ invstd) {
+  double a, b;
+  const int c = bn_sum_partials(partial, nblk, C, a, b);
+  if (c < 0) return;
+  const double m = a / (double)rows;
+  const double v = fmax(b / (double)rows - m * m, 0.0);
+  mean[c] = (float)((double)to_f32(x[c]) + m);
+  var[c] = (float)v;
+  invstd[c] = (float)(1.0 / sqrt(v + (double)eps));
+}
+
+// y = (x - mean) * (invstd * gamma) + beta, then max(., 0) when relu.  A thread keeps the
+// constants of its VEC channels in registers and walks every rpp-th row of the workgroup's
+// range, four rows in flight.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, int64_t rows, int C,
+                                                       int64_t rows_per_blk,
+                                                       const float* __restrict__ mean,
+                                                       const float* __restrict__ invstd,
+                                                       const float* __restrict__ gamma,
+                                                       const float* __restrict__ beta, int relu,
+                                                       T* __restrict__ y) {
+  typedef BnVec<T, VEC> V;
+  const int lpr = C / VEC, rpp = 256 / lpr;
+  const int tid = threadIdx.x, rl = tid / lpr, cl = tid - rl * lpr;
+  if (rl >= rpp) return;
+  float m[VEC], sc[VEC], be[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    const int c = cl * VEC + v;
+    m[v] = mean[c];
+    sc[v] = invstd[c] * (gamma ? gamma[c] : 1.f);
+    be[v] = beta ? beta[c] : 0.f;
+  }
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
+  const int64_t r1 = min(rows, r0 + rows_per_blk);
+  for (int64_t r = r0 + rl; r < r1; r += 4 * rpp) {
+    V a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t ru = r + (int64_t)u * rpp;
+      if (ru < r1) a[u] = *(const V*)(x + ru * C + cl * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t ru = r + (int64_t)u * rpp;
+      if (ru >= r1) continue;
+      V o;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        float t = (to_f32(a[u].v[v]) - m[v]) * sc[v] + be[v];
+        if (relu) t = fmaxf(t, 0.f);
+        o.v[v] = from_f32<T>(t);
+      }
+      *(V*)(y + ru * C + cl * VEC) = o;
+    }
+  }
+}
+
+// partial[blk][0][c] = sum_r dy'[r][c],  partial[blk][1][c] = sum_r dy'[r][c] * xhat[r][c], with
+// xhat = (x - mean) * invstd and dy' = dy where the forward output was positive (relu) or dy.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__ x, const T* __restrict__ dy,
+                                                           int64_t rows, int C, int64_t rows_per_blk,
+                                                           const float* __restrict__ mean,
+                                                           const float* __restrict__ invstd,
+                                                           const float* __restrict__ gamma,
+                                                           const float* __restrict__ beta, int relu,
+                                                           float* __restrict__ partial) {
+  typedef BnVec<T, VEC> V;
+  __shared__ float s_a[256 * VEC], s_b[256 * VEC];
+  const int lpr = C / VEC, rpp = 256 / lpr;
+  const int tid = threadIdx.x, rl = tid / lpr, cl = tid - rl * lpr;
+  float s1[VEC], s2[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) s1[v] = s2[v] = 0.f;
+  if (rl < rpp) {
+    float m[VEC], is[VEC], ga[VEC], be[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const int c = cl * VEC + v;
+      m[v] = mean[c];
+      is[v] = invstd[c];
+      ga[v] = gamma ? gamma[c] : 1.f;
+      be[v] = beta ? beta[c] : 0.f;
+    }
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
+    const int64_t r1 = min(rows, r0 + rows_per_blk);
+    for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {          // two rows of both tensors in flight
+      V a[2], g[2];
+      bool ok[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int64_t ru = r + (int64_t)u * rpp;
+        ok[u] = ru < r1;
+        a[u] = *(const V*)(x + (ok[u] ? ru * C : 0) + cl * VEC);
+        g[u] = *(const V*)(dy + (ok[u] ? ru * C : 0) + cl * VEC);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float xc = to_f32(a[u].v[v]) - m[v];
+          const float xh = xc * is[v];
+          float d = ok[u] ? to_f32(g[u].v[v]) : 0.f;
+          if (relu && !(xc * (is[v] * ga[v]) + be[v] > 0.f)) d = 0.f;      // the forward pass's expression
+          s1[v] += d;
+          s2[v] += d * xh;
+        }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    s_a[tid * VEC + v] = s1[v];
+    s_b[tid * VEC + v] = s2[v];
+  }
+  __syncthreads();
+  if (tid < lpr) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      float a = 0.f, b = 0.f;
+      for (int g = 0; g < rpp; ++g) {
+        a += s_a[(g * lpr + tid) * VEC + v];
+        b += s_b[(g * lpr + tid) * VEC + v];
+      }
+      partial[((int64_t)blockIdx.x * 2 + 0) * C + tid * VEC + v] = a;
+      partial[((int64_t)blockIdx.x * 2 + 1) * C + tid * VEC + v] = b;
+    }
+  }
+}
+
+__global__ void bn_bwd_finish_kernel(const float* __restrict__ partial, int nblk, int C,
+                                     float* __restrict__ dbeta, float* __restrict__ dgamma) {
+  double a, b;
+  const int c = bn_sum_partials(partial, nblk, C, a, b);
+  if (c < 0) return;
+  dbeta[c] = (float)a;
+  dgamma[c] = (float)b;
+}
+
+// training: dx = gamma * invstd * (dy' - dbeta / N - xhat * dgamma / N); with fixed statistics
+// (evaluation mode): dx = gamma * invstd * dy'.  Thread layout as in bn_apply_kernel.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__ x, const T* __restrict__ dy,
+                                                           int64_t rows, int C, int64_t rows_per_blk,
+                                                           const float* __restrict__ mean,
+                                                           const float* __restrict__ invstd,
+                                                           const float* __restrict__ gamma,
+                                                           const float* __restrict__ beta, int relu,
+                                                           const float* __restrict__ dbeta,
+                                                           const float* __restrict__ dgamma, int training,
+                                                           T* __restrict__ dx) {
+  typedef BnVec<T, VEC> V;
+  const int lpr = C / VEC, rpp = 256 / lpr;
+  const int tid = threadIdx.x, rl = tid / lpr, cl = tid - rl * lpr;
+  if (rl >= rpp) return;
+  const float inv_n = 1.0f / (float)rows;
+  float m[VEC], is[VEC], sc[VEC], be[VEC], db[VEC], dg[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    const int c = cl * VEC + v;
+    m[v] = mean[c];
+    is[v] = invstd[c];
+    sc[v] = invstd[c] * (gamma ? gamma[c] : 1.f);
+    be[v] = beta ? beta[c] : 0.f;
+    db[v] = training ? dbeta[c] * inv_n : 0.f;
+    dg[v] = training ? dgamma[c] * inv_n : 0.f;
+  }
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
+  const int64_t r1 = min(rows, r0 + rows_per_blk);
+  for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {
+    V a[2], g[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int64_t ru = r + (int64_t)u * rpp;
+      if (ru < r1) {
+        a[u] = *(const V*)(x + ru * C + cl * VEC);
+        g[u] = *(const V*)(dy + ru * C + cl * VEC);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int64_t ru = r + (int64_t)u * rpp;
+      if (ru >= r1) continue;
+      V o;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        const float xc = to_f32(a[u].v[v]) - m[v];
+        float d = to_f32(g[u].v[v]);
+        if (relu && !(xc * sc[v] + be[v] > 0.f)) d = 0.f;
+        if (training) d = d - db[v] - (xc * is[v]) * dg[v];
+        o.v[v] = from_f32<T>(d * sc[v]);
+      }
+      *(V*)(dx + ru * C + cl * VEC) = o;
+    }
+  }
+}
+
+}  // namespace ocnn
+
+using namespace ocnn;
+
+#define OCNN_DISPATCH_DTYPE(dtype, ...)                      \
+  do {                                                       \
+    if (dtype == OCNN_F32) { typedef float T; __VA_ARGS__; } \
+    else if (dtype == OCNN_F16) { typedef f16 T; __VA_ARGS__; } \
+    else { typedef bf16 T; __VA_ARGS__; }                    \
+  } while (0)
+
+static int bn_vec(int dtype) { return dtype == OCNN_F32 ? 4 : 8; }
+
+extern "C" int ocnn_batch_norm_supported(int dtype, int64_t rows, int channels) {
+  if (dtype < 0 || dtype > 2) return 0;
+  const int vec = bn_vec(dtype);
+  if (channels < vec || channels % vec != 0 || channels / vec > 256) return 0;
+  return rows >= 1;
+}
+
+// rows of a workgroup (a multiple of the rows its threads cover per pass) and their number
+static void bn_blocks(int dtype, int64_t rows, int channels, int64_t* per, int* nblk) {
+  const int rpp = 256 / (channels / bn_vec(dtype));
+  *per = align_up(std::max<int64_t>(cdiv(rows, kBnMaxBlocks), 4 * rpp), rpp);
+  *nblk = (int)cdiv(rows, *per);
+}
+
+extern "C" int64_t ocnn_batch_norm_workspace_bytes(int channels) {
+  return align_up((int64_t)kBnMaxBlocks * 2 * channels * 4, 256);
+}
+
+extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
+                                     float* mean, float* var, float* invstd, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+  OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_stats: shape not supported");
+  OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels), "batch_norm_stats: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  int64_t per;
+  int nblk;
+  bn_blocks(dtype, rows, channels, &per, &nblk);
+  float* partial = (float*)workspace;
+  OCNN_DISPATCH_DTYPE(dtype, {
+    constexpr int VEC = 16 / sizeof(T);
+    hipLaunchKernelGGL((bn_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
+                       partial);
+    hipLaunchKernelGGL(bn_stats_finish_kernel<T>, dim3((unsigned)cdiv(channels, 16)), dim3(256), 0, st, partial, nblk,
+                       (const T*)x, rows, channels, eps, mean, var, invstd);
+  });
+  return check_launch("batch_norm_stats");
+}
+
+extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
+                                     const float* invstd, const float* gamma, const float* beta, int relu,
+                                     void* y, void* stream) {
+  OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_apply: shape not supported");
+  hipStream_t st = (hipStream_t)stream;
+  int64_t per;
+  int nblk;
+  bn_blocks(dtype, rows, channels, &per, &nblk);
+  OCNN_DISPATCH_DTYPE(dtype, {
+    constexpr int VEC = 16 / sizeof(T);
+    hipLaunchKernelGGL((bn_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
+                       mean, invstd, gamma, beta, relu, (T*)y);
+  });
+  return check_launch("batch_norm_apply");
+}
+
+extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy, int64_t rows, int channels,
+                                        const float* mean, const float* invstd, const float* gamma,
+                                        const float* beta, int relu, int training, void* dx, float* dgamma,
+                                        float* dbeta, void* workspace, int64_t workspace_bytes, void* stream) {
+  OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_backward: shape not supported");
+  OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels),
+               "batch_norm_backward: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  int64_t per;
+  int nblk;
+  bn_blocks(dtype, rows, channels, &per, &nblk);
+  float* partial = (float*)workspace;
+  OCNN_DISPATCH_DTYPE(dtype, {
+    constexpr int VEC = 16 / sizeof(T);
+    hipLaunchKernelGGL((bn_bwd_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
+                       channels, per, mean, invstd, gamma, beta, relu, partial);
+    hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3((unsigned)cdiv(channels, 16)), dim3(256), 0, st, partial, nblk,
+                       channels, dbeta, dgamma);
+    if (dx)
+      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
+                         channels, per, mean, invstd, gamma, beta, relu, dbeta, dgamma, training, (T*)dx);
+  });
+  return check_launch("batch_norm_backward");
+}

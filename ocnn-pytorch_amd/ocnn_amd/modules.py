@@ -1,6 +1,7 @@
-"""Compositions of the hot-path layers with torch's BatchNorm1d / ReLU / Linear under the
-class and attribute names of ocnn/modules/modules.py and ocnn/modules/resblocks.py, so that
-networks written against the reference (and their state_dicts) work unchanged."""
+"""Compositions of the hot-path layers with batch norm / ReLU / Linear under the class and
+attribute names of ocnn/modules/modules.py and ocnn/modules/resblocks.py, so that networks
+written against the reference (and their state_dicts) work unchanged.  The batch norm is a
+BatchNorm1d subclass that runs on fused HIP kernels (statistics, normalise + ReLU in one pass)."""
 
 from typing import List
 
@@ -8,6 +9,7 @@ import torch
 import torch.nn
 
 from .nn import OctreeConv, OctreeDeconv
+from .nn.batchnorm import BatchNormRelu1d
 
 
 class _LayerBn(torch.nn.Module):
@@ -17,14 +19,12 @@ class _LayerBn(torch.nn.Module):
     super().__init__()
     self._name = name
     setattr(self, name, layer)
-    self.bn = torch.nn.BatchNorm1d(channels)
+    self.bn = BatchNormRelu1d(channels, relu=relu)          # BatchNorm1d with the ReLU fused in
     if relu:
-      self.relu = torch.nn.ReLU(inplace=True)
-    self._relu = relu
+      self.relu = torch.nn.ReLU(inplace=True)               # (kept for the module tree; applied by bn)
 
   def forward(self, data, *args):
-    out = self.bn(getattr(self, self._name)(data, *args))
-    return self.relu(out) if self._relu else out
+    return self.bn(getattr(self, self._name)(data, *args))
 
 
 class OctreeConvBn(_LayerBn):

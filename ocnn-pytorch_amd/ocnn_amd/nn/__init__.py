@@ -5,6 +5,7 @@ from .octree_dwconv import OctreeDWConv, octree_dwconv
 from .octree_conv_t import (OctreeConvTriton, OctreeConvT, octree_conv_triton,
                             convert_conv_triton, conv_fwd_implicit_gemm_splitk,
                             conv_bwd_implicit_gemm_splitk)
+from .batchnorm import BatchNormRelu1d
 from .octree_pool import (octree_max_pool, octree_max_unpool, OctreeMaxPool, OctreeMaxUnpool)
 from .octree_interp import (octree_nearest_pts, octree_linear_pts, OctreeInterp,
                             octree_nearest_upsample, OctreeUpsample)
@@ -14,4 +15,4 @@ __all__ = ['octree_pad', 'octree_depad', 'OctreeConv', 'OctreeDeconv', 'octree_c
            'octree_conv_triton', 'convert_conv_triton', 'conv_fwd_implicit_gemm_splitk',
            'conv_bwd_implicit_gemm_splitk', 'octree_max_pool', 'octree_max_unpool', 'OctreeMaxPool',
            'OctreeMaxUnpool', 'octree_nearest_pts', 'octree_linear_pts', 'OctreeInterp',
-           'octree_nearest_upsample', 'OctreeUpsample']
+           'octree_nearest_upsample', 'OctreeUpsample', 'BatchNormRelu1d']

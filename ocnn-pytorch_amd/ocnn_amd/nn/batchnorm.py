@@ -1,0 +1,97 @@
+"""torch.nn.BatchNorm1d on (rows, C) feature matrices with an optional fused ReLU, on HIP
+kernels (same parameters, buffers and state_dict keys as BatchNorm1d).  What the reference
+builds from BatchNorm1d + ReLU(inplace) after every convolution
+(ocnn/modules/modules.py:32-99, 120-153)."""
+
+import torch
+import torch.nn
+
+from .. import _lib
+
+
+def _f32(t):
+  return None if t is None else t.detach().to(torch.float32).contiguous()
+
+
+class _BatchNormRelu(torch.autograd.Function):
+  @staticmethod
+  def forward(ctx, x, weight, bias, running_mean, running_var, use_batch_stats, factor, eps, relu):
+    L = _lib.lib()
+    x = x.contiguous()
+    rows, c = x.shape
+    code = _lib.dtype_code(x)
+    dev = x.device
+    gamma, beta = _f32(weight), _f32(bias)
+    if use_batch_stats:
+      mean = torch.empty(c, dtype=torch.float32, device=dev)
+      var = torch.empty(c, dtype=torch.float32, device=dev)
+      invstd = torch.empty(c, dtype=torch.float32, device=dev)
+      ws = _lib.workspace(L.ocnn_batch_norm_workspace_bytes(c), dev)
+      _lib.check(L.ocnn_batch_norm_stats(code, _lib.ptr(x), rows, c, float(eps), _lib.ptr(mean), _lib.ptr(var),
+                                         _lib.ptr(invstd), _lib.ptr(ws), ws.numel(), _lib.stream()))
+      if running_mean is not None and factor is not None:
+        # the running variance is the unbiased one (torch.nn.functional.batch_norm)
+        unbiased = var * (rows / max(rows - 1, 1))
+        running_mean.mul_(1 - factor).add_(mean.to(running_mean.dtype), alpha=factor)
+        running_var.mul_(1 - factor).add_(unbiased.to(running_var.dtype), alpha=factor)
+    else:
+      mean = _f32(running_mean)
+      invstd = torch.rsqrt(_f32(running_var) + eps)
+    y = torch.empty_like(x)
+    _lib.check(L.ocnn_batch_norm_apply(code, _lib.ptr(x), rows, c, _lib.ptr(mean), _lib.ptr(invstd),
+                                       _lib.ptr(gamma), _lib.ptr(beta), int(relu), _lib.ptr(y), _lib.stream()))
+    ctx.save_for_backward(x, mean, invstd, gamma, beta)
+    ctx.relu, ctx.training = relu, use_batch_stats
+    ctx.wdtype = None if weight is None else weight.dtype
+    ctx.bdtype = None if bias is None else bias.dtype
+    return y
+
+  @staticmethod
+  def backward(ctx, dy):
+    L = _lib.lib()
+    x, mean, invstd, gamma, beta = ctx.saved_tensors
+    dy = dy.contiguous()
+    rows, c = x.shape
+    dev = x.device
+    dgamma = torch.empty(c, dtype=torch.float32, device=dev)
+    dbeta = torch.empty(c, dtype=torch.float32, device=dev)
+    dx = torch.empty_like(x) if ctx.needs_input_grad[0] else None
+    ws = _lib.workspace(L.ocnn_batch_norm_workspace_bytes(c), dev)
+    _lib.check(L.ocnn_batch_norm_backward(
+        _lib.dtype_code(x), _lib.ptr(x), _lib.ptr(dy), rows, c, _lib.ptr(mean), _lib.ptr(invstd), _lib.ptr(gamma),
+        _lib.ptr(beta), int(ctx.relu), int(ctx.training), _lib.ptr(dx), _lib.ptr(dgamma), _lib.ptr(dbeta),
+        _lib.ptr(ws), ws.numel(), _lib.stream()))
+    gw = dgamma.to(ctx.wdtype) if ctx.wdtype is not None and ctx.needs_input_grad[1] else None
+    gb = dbeta.to(ctx.bdtype) if ctx.bdtype is not None and ctx.needs_input_grad[2] else None
+    return dx, gw, gb, None, None, None, None, None, None
+
+
+class BatchNormRelu1d(torch.nn.BatchNorm1d):
+  """BatchNorm1d [+ ReLU] in one pass over (rows, C) inputs on the GPU; anything else (3-D
+  inputs, CPU tensors, channel counts that are not a multiple of 16 bytes) takes torch's own
+  batch norm followed by a ReLU."""
+
+  def __init__(self, num_features: int, relu: bool = False, **kwargs):
+    super().__init__(num_features, **kwargs)
+    self.fused_relu = relu
+
+  def forward(self, input: torch.Tensor) -> torch.Tensor:
+    code = _lib.DTYPE_CODE.get(input.dtype, -1)
+    if not (input.dim() == 2 and input.is_cuda and code >= 0 and input.shape[0] > 1 and
+            _lib.lib().ocnn_batch_norm_supported(code, input.shape[0], input.shape[1])):
+      out = super().forward(input)
+      return torch.relu(out) if self.fused_relu else out
+    # the bookkeeping of torch.nn.modules.batchnorm._BatchNorm.forward
+    factor = 0.0 if self.momentum is None else self.momentum
+    if self.training and self.track_running_stats and self.num_batches_tracked is not None:
+      self.num_batches_tracked.add_(1)
+      factor = 1.0 / float(self.num_batches_tracked) if self.momentum is None else self.momentum
+    use_batch_stats = self.training or (self.running_mean is None and self.running_var is None)
+    track = self.training and self.track_running_stats
+    return _BatchNormRelu.apply(input, self.weight, self.bias,
+                                self.running_mean if (not use_batch_stats or track) else None,
+                                self.running_var if (not use_batch_stats or track) else None,
+                                use_batch_stats, factor if track else None, self.eps, self.fused_relu)
+
+  def extra_repr(self) -> str:
+    return super().extra_repr() + ', relu={}'.format(self.fused_relu)

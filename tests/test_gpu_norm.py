@@ -1,0 +1,101 @@
+"""GPU parity of the fused batch norm (+ ReLU) against torch.nn.BatchNorm1d + ReLU evaluated
+in fp64 on the CPU: outputs, running statistics, all three gradients, training and evaluation
+mode, every dtype."""
+
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from ocnn_amd.nn import BatchNormRelu1d
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+TOL = {torch.float32: 2e-5, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}
+
+
+def say(*a):
+  print(*a, flush=True)
+  sys.stdout.flush()
+
+
+def _ref(x, w, b, relu, training, rm, rv, momentum, eps, dy):
+  """fp64 torch reference on the CPU; returns y, dx, dw, db and the updated running stats."""
+  bn = torch.nn.BatchNorm1d(x.shape[1], eps=eps, momentum=momentum).double()
+  with torch.no_grad():
+    bn.weight.copy_(w.double()); bn.bias.copy_(b.double())
+    bn.running_mean.copy_(rm.double()); bn.running_var.copy_(rv.double())
+  bn.train(training)
+  xd = x.double().requires_grad_()
+  y = bn(xd)
+  if relu:
+    y = torch.relu(y)
+  y.backward(dy.double())
+  return y.detach(), xd.grad, bn.weight.grad, bn.bias.grad, bn.running_mean.clone(), bn.running_var.clone()
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('relu', [False, True])
+@pytest.mark.parametrize('training', [True, False])
+def test_batch_norm_relu_vs_torch(dtype, relu, training):
+  g = torch.Generator().manual_seed(11)
+  for rows, c in [(1000, 32), (4133, 96), (257, 8), (20000, 256), (3, 64)]:
+    say('batch norm', dtype, relu, training, rows, c)
+    x = (torch.randn(rows, c, generator=g) * 1.5 + 3.0).to(dtype)          # a mean well away from zero
+    w = (torch.rand(c, generator=g) + 0.5).to(dtype).float()               # parameters the dtype holds exactly
+    b = (torch.randn(c, generator=g) * 0.3).to(dtype).float()
+    rm = (torch.randn(c, generator=g) * 0.1 + 3.0).to(dtype).float()
+    rv = (torch.rand(c, generator=g) + 1.5).to(dtype).float()
+    dy = torch.randn(rows, c, generator=g).to(dtype)
+    want = _ref(x.float(), w, b, relu, training, rm, rv, 0.1, 1e-5, dy.float())
+    bn = BatchNormRelu1d(c, relu=relu).to(DEV)
+    with torch.no_grad():
+      bn.weight.copy_(w); bn.bias.copy_(b); bn.running_mean.copy_(rm); bn.running_var.copy_(rv)
+    bn = bn.to(dtype) if dtype != torch.float32 else bn
+    bn.train(training)
+    xg = x.to(DEV).requires_grad_()
+    y = bn(xg)
+    assert y.dtype == dtype
+    y.backward(dy.to(DEV))
+    tol = TOL[dtype]
+    scale = lambda t: max(1.0, float(t.abs().max()))
+    assert float((y.detach().double().cpu() - want[0]).abs().max()) <= tol * scale(want[0])
+    # where the pre-activation is within rounding of zero the ReLU mask is a coin toss
+    sure = torch.ones_like(want[0], dtype=torch.bool)
+    if relu:
+      mu = want[4] if not training else x.double().mean(0)
+      sd = (want[5] + 1e-5).sqrt() if not training else (x.double().var(0, unbiased=False) + 1e-5).sqrt()
+      z = (x.double() - (rm.double() if not training else mu)) / ((rv.double() + 1e-5).sqrt() if not training else sd) * w.double() + b.double()
+      sure = z.abs() > 1e-3
+    assert float(((xg.grad.double().cpu() - want[1]) * sure).abs().max()) <= 4 * tol * scale(want[1])
+    assert int((~sure).sum()) < 0.01 * sure.numel()
+    # parameter gradients are sums over the rows: relative to their size
+    assert float((bn.weight.grad.double().cpu() - want[2]).abs().max()) <= 4 * tol * scale(want[2])
+    assert float((bn.bias.grad.double().cpu() - want[3]).abs().max()) <= 4 * tol * scale(want[3])
+    assert float((bn.running_mean.double().cpu() - want[4]).abs().max()) <= max(tol, 1e-3 if dtype != torch.float32 else 0) * scale(want[4])
+    assert float((bn.running_var.double().cpu() - want[5]).abs().max()) <= max(tol, 1e-2 if dtype != torch.float32 else 0) * scale(want[5])
+    assert int(bn.num_batches_tracked) == (1 if training else 0)
+    # the same bits on a second run (fixed reduction order)
+    bn.zero_grad()
+    x2 = x.to(DEV).requires_grad_()
+    y2 = bn(x2) if not training else None
+    if y2 is not None:
+      assert torch.equal(y2, y)
+
+
+def test_batch_norm_fallbacks_and_state_dict():
+  """3-D inputs and odd channel counts take torch's path; the state_dict is BatchNorm1d's."""
+  bn = BatchNormRelu1d(6, relu=True).to(DEV)
+  ref = torch.nn.BatchNorm1d(6).to(DEV)
+  ref.load_state_dict(bn.state_dict())
+  x = torch.randn(50, 6, device=DEV)
+  assert torch.allclose(bn(x), torch.relu(ref(x)), atol=1e-6)
+  bn2 = BatchNormRelu1d(16, relu=False).to(DEV)
+  ref2 = torch.nn.BatchNorm1d(16).to(DEV)
+  ref2.load_state_dict(bn2.state_dict())
+  x = torch.randn(200, 16, device=DEV)
+  assert torch.allclose(bn2(x), ref2(x), atol=1e-5)
+  assert torch.allclose(bn2.running_var, ref2.running_var, atol=1e-6)
+  x3 = torch.randn(4, 16, 10, device=DEV)
+  assert torch.allclose(bn2(x3), ref2(x3), atol=1e-5)
