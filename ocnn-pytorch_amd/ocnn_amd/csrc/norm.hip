@@ -11,7 +11,8 @@
 
 namespace ocnn {
 
-constexpr int kBnMaxBlocks = 2048;
+constexpr int kBnMaxBlocks = 512;     // workgroups of a reduction (their partial sums are added by one more kernel)
+constexpr int kBnApplyBlocks = 2048;  // workgroups of an elementwise pass
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) BnVec { T v[VEC]; };
 
@@ -71,21 +72,21 @@ __global__ __launch_bounds__(256) void bn_stats_kernel(const T* __restrict__ x, 
   }
 }
 
-// Sum of the per-workgroup partial sums of a channel, in a fixed order: 256 threads = 16
-// lanes x 16 channels, lane l adds the partials l, l + 16, .. (fp64), then lane 0 adds the
-// 16 lane sums.  Returns the channel for the threads that hold a result, -1 for the others.
+// Sum of the per-workgroup partial sums of a channel, in a fixed order: 256 threads = 64
+// lanes x 4 channels, lane l adds the partials l, l + 64, .. (fp64), then lane 0 adds the
+// 64 lane sums.  Returns the channel for the threads that hold a result, -1 for the others.
 __device__ __forceinline__ int bn_sum_partials(const float* __restrict__ partial, int nblk, int C, double& a,
                                                double& b) {
   __shared__ double s_pa[256], s_pb[256];
-  const int tid = threadIdx.x, l = tid >> 4;
-  const int c = blockIdx.x * 16 + (tid & 15);
+  const int tid = threadIdx.x, l = tid >> 2;
+  const int c = blockIdx.x * 4 + (tid & 3);
   double sa = 0.0, sb = 0.0;
   if (c < C) {
-    for (int i = l; i < nblk; i += 64) {                     // four loads of each kind in flight
+    for (int i = l; i < nblk; i += 256) {                    // four loads of each kind in flight
       float va[4], vb[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int iu = i + 16 * u;
+        const int iu = i + 64 * u;
         va[u] = iu < nblk ? partial[((int64_t)iu * 2 + 0) * C + c] : 0.f;
         vb[u] = iu < nblk ? partial[((int64_t)iu * 2 + 1) * C + c] : 0.f;
       }
@@ -102,9 +103,9 @@ __device__ __forceinline__ int bn_sum_partials(const float* __restrict__ partial
   if (l != 0 || c >= C) return -1;
   a = 0.0;
   b = 0.0;
-  for (int k = 0; k < 16; ++k) {
-    a += s_pa[16 * k + tid];
-    b += s_pb[16 * k + tid];
+  for (int k = 0; k < 64; ++k) {
+    a += s_pa[4 * k + tid];
+    b += s_pb[4 * k + tid];
   }
   return c;
 }
@@ -332,9 +333,9 @@ extern "C" int ocnn_batch_norm_supported(int dtype, int64_t rows, int channels) 
 }
 
 // rows of a workgroup (a multiple of the rows its threads cover per pass) and their number
-static void bn_blocks(int dtype, int64_t rows, int channels, int64_t* per, int* nblk) {
+static void bn_blocks(int dtype, int64_t rows, int channels, int max_blocks, int64_t* per, int* nblk) {
   const int rpp = 256 / (channels / bn_vec(dtype));
-  *per = align_up(std::max<int64_t>(cdiv(rows, kBnMaxBlocks), 4 * rpp), rpp);
+  *per = align_up(std::max<int64_t>(cdiv(rows, max_blocks), 4 * rpp), rpp);
   *nblk = (int)cdiv(rows, *per);
 }
 
@@ -350,13 +351,13 @@ extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
   int nblk;
-  bn_blocks(dtype, rows, channels, &per, &nblk);
+  bn_blocks(dtype, rows, channels, kBnMaxBlocks, &per, &nblk);
   float* partial = (float*)workspace;
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
                        partial);
-    hipLaunchKernelGGL(bn_stats_finish_kernel<T>, dim3((unsigned)cdiv(channels, 16)), dim3(256), 0, st, partial, nblk,
+    hipLaunchKernelGGL(bn_stats_finish_kernel<T>, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
                        (const T*)x, rows, channels, eps, mean, var, invstd);
   });
   return check_launch("batch_norm_stats");
@@ -369,7 +370,7 @@ extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
   int nblk;
-  bn_blocks(dtype, rows, channels, &per, &nblk);
+  bn_blocks(dtype, rows, channels, kBnApplyBlocks, &per, &nblk);
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
@@ -388,17 +389,20 @@ extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
   int nblk;
-  bn_blocks(dtype, rows, channels, &per, &nblk);
+  int64_t per_a;
+  int nblk_a;
+  bn_blocks(dtype, rows, channels, kBnMaxBlocks, &per, &nblk);
+  bn_blocks(dtype, rows, channels, kBnApplyBlocks, &per_a, &nblk_a);
   float* partial = (float*)workspace;
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_bwd_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
                        channels, per, mean, invstd, gamma, beta, relu, partial);
-    hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3((unsigned)cdiv(channels, 16)), dim3(256), 0, st, partial, nblk,
+    hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
                        channels, dbeta, dgamma);
     if (dx)
-      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
-                         channels, per, mean, invstd, gamma, beta, relu, dbeta, dgamma, training, (T*)dx);
+      hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), dim3(nblk_a), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
+                         channels, per_a, mean, invstd, gamma, beta, relu, dbeta, dgamma, training, (T*)dx);
   });
   return check_launch("batch_norm_backward");
 }

@@ -9,6 +9,7 @@ import torch
 import torch.nn
 
 from .nn import OctreeConv, OctreeDeconv
+from .nn.octree_conv import conv_gather, conv_wgrad, column_sum
 from .nn.batchnorm import BatchNormRelu1d
 
 
@@ -54,15 +55,65 @@ class OctreeDeconvBnRelu(_LayerBn):
                      out_channels, True)
 
 
+_IDENTITY = {}
+
+
+def _identity_table(rows, device):
+  """(rows, 1) table [0, 1, ..]: row i reads row i."""
+  key = (rows, str(device))
+  if key not in _IDENTITY:
+    if len(_IDENTITY) > 16:
+      _IDENTITY.clear()
+    _IDENTITY[key] = torch.arange(rows, dtype=torch.int32, device=device).view(rows, 1)
+  return _IDENTITY[key]
+
+
+class _RowsLinear(torch.autograd.Function):
+  """y = x W^T + b on many rows through the one-slot form of the convolution kernels
+  (weights (out, in) as torch.nn.Linear holds them)."""
+
+  @staticmethod
+  def forward(ctx, x, weight, bias):
+    x = x.contiguous()
+    w = weight.to(x.dtype).contiguous()
+    ctx.save_for_backward(x, w)
+    ctx.has_bias = bias is not None
+    ctx.wdtype = weight.dtype
+    rows = x.shape[0]
+    return conv_gather(x, rows, _identity_table(rows, x.device), w.view(1, w.shape[0], w.shape[1]),
+                       w.shape[0], True, False, None if bias is None else bias.to(x.dtype), None, dense=True)
+
+  @staticmethod
+  def backward(ctx, grad):
+    x, w = ctx.saved_tensors
+    grad = grad.contiguous()
+    rows = x.shape[0]
+    table = _identity_table(rows, x.device)
+    gx = gw = gb = None
+    if ctx.needs_input_grad[0]:
+      gx = conv_gather(grad, rows, table, w.view(1, w.shape[0], w.shape[1]), w.shape[1], False, False,
+                       None, None, dense=True)
+    if ctx.needs_input_grad[1]:
+      gw = conv_wgrad(x, grad, table, True, None, dense=True).view(w.shape).to(ctx.wdtype)
+    if ctx.has_bias and ctx.needs_input_grad[2]:
+      gb = column_sum(grad)
+    return gx, gw, gb
+
+
 class Conv1x1(torch.nn.Module):
-  """ocnn/modules/modules.py:102-117: a 1x1x1 convolution on (N, C) rows is a Linear."""
+  """ocnn/modules/modules.py:102-117: a 1x1x1 convolution on (N, C) rows is a Linear (same
+  parameters as torch.nn.Linear; large 16-bit inputs run on this package's GEMM kernels)."""
 
   def __init__(self, in_channels: int, out_channels: int, use_bias: bool = False):
     super().__init__()
     self.linear = torch.nn.Linear(in_channels, out_channels, use_bias)
 
   def forward(self, data: torch.Tensor):
-    return self.linear(data)
+    lin = self.linear
+    if (data.dim() == 2 and data.is_cuda and data.dtype in (torch.float16, torch.bfloat16) and
+        data.shape[0] >= 4096 and lin.in_features % 32 == 0 and lin.out_features % 16 == 0):
+      return _RowsLinear.apply(data, lin.weight, lin.bias)
+    return lin(data)
 
 
 class Conv1x1Bn(_LayerBn):

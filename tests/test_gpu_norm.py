@@ -99,3 +99,36 @@ def test_batch_norm_fallbacks_and_state_dict():
   assert torch.allclose(bn2.running_var, ref2.running_var, atol=1e-6)
   x3 = torch.randn(4, 16, 10, device=DEV)
   assert torch.allclose(bn2(x3), ref2(x3), atol=1e-5)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('cin,cout,bias', [(96, 64, False), (64, 16, True), (256, 128, False), (128, 512, True)])
+def test_conv1x1_on_package_kernels(dtype, cin, cout, bias):
+  """modules.Conv1x1 on many rows (the package's GEMM kernels) against torch.nn.Linear in fp64:
+  output and all gradients."""
+  from ocnn_amd import modules
+  g = torch.Generator().manual_seed(cin + cout)
+  rows = 5000
+  m = modules.Conv1x1(cin, cout, use_bias=bias).to(DEV).to(dtype)
+  x = torch.randn(rows, cin, generator=g).to(dtype)
+  dy = torch.randn(rows, cout, generator=g).to(dtype)
+  ref = torch.nn.Linear(cin, cout, bias).double()
+  with torch.no_grad():
+    ref.weight.copy_(m.linear.weight.double().cpu())
+    if bias:
+      ref.bias.copy_(m.linear.bias.double().cpu())
+  xd = x.double().requires_grad_()
+  ref(xd).backward(dy.double())
+  xg = x.to(DEV).requires_grad_()
+  y = m(xg)
+  y.backward(dy.to(DEV))
+  tol = 4e-3 if dtype == torch.float16 else 2e-2
+  rel = lambda a, b: float((a.double().cpu() - b).abs().max() / b.abs().max())
+  assert rel(y.detach(), ref(x.double()).detach()) < tol
+  assert rel(xg.grad, xd.grad) < tol
+  assert rel(m.linear.weight.grad, ref.weight.grad) < tol
+  if bias:
+    assert rel(m.linear.bias.grad, ref.bias.grad) < tol
+  # few rows: torch's Linear
+  small = torch.randn(10, cin, generator=g).to(dtype).to(DEV)
+  assert torch.equal(m(small), m.linear(small))
