@@ -6,7 +6,8 @@ from .octree_conv_t import (OctreeConvTriton, OctreeConvT, octree_conv_triton,
                             convert_conv_triton, conv_fwd_implicit_gemm_splitk,
                             conv_bwd_implicit_gemm_splitk)
 from .batchnorm import BatchNormRelu1d
-from .octree_pool import (octree_max_pool, octree_max_unpool, OctreeMaxPool, OctreeMaxUnpool)
+from .octree_pool import (octree_max_pool, octree_max_unpool, OctreeMaxPool, OctreeMaxUnpool,
+                          octree_avg_pool, octree_global_pool, OctreeAvgPool, OctreeGlobalPool)
 from .octree_interp import (octree_nearest_pts, octree_linear_pts, OctreeInterp,
                             octree_nearest_upsample, OctreeUpsample)
 
@@ -15,4 +16,5 @@ __all__ = ['octree_pad', 'octree_depad', 'OctreeConv', 'OctreeDeconv', 'octree_c
            'octree_conv_triton', 'convert_conv_triton', 'conv_fwd_implicit_gemm_splitk',
            'conv_bwd_implicit_gemm_splitk', 'octree_max_pool', 'octree_max_unpool', 'OctreeMaxPool',
            'OctreeMaxUnpool', 'octree_nearest_pts', 'octree_linear_pts', 'OctreeInterp',
-           'octree_nearest_upsample', 'OctreeUpsample', 'BatchNormRelu1d']
+           'octree_nearest_upsample', 'OctreeUpsample', 'BatchNormRelu1d', 'octree_avg_pool',
+           'octree_global_pool', 'OctreeAvgPool', 'OctreeGlobalPool']

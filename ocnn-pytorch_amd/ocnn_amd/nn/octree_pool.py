@@ -1,9 +1,13 @@
-"""2x2x2 max pooling / unpooling with the API of ocnn/nn/octree_pool.py on HIP kernels."""
+"""Pooling with the API of ocnn/nn/octree_pool.py on HIP kernels: 2x2x2 max pooling /
+unpooling, average pooling over a neighbour table, global average pooling per batch element."""
+
+from typing import List
 
 import torch
 import torch.nn
 
 from .. import _lib
+from ..utils import list2str, resize_with_last_val
 from .octree_pad import octree_pad
 
 
@@ -130,6 +134,82 @@ class OctreeMaxUnpool(torch.nn.Module):
 
   def forward(self, data: torch.Tensor, indices: torch.Tensor, octree, depth: int):
     return octree_max_unpool(data, indices, octree, depth, self.nempty)
+
+  def extra_repr(self) -> str:
+    return 'kernel_size={}, stride={}, nempty={}'.format(self.kernel_size, self.stride, self.nempty)
+
+
+def octree_avg_pool(data: torch.Tensor, octree, depth: int, kernel: str, stride: int = 2,
+                    nempty: bool = False):
+  """Average over the existing neighbours of the table (ocnn/nn/octree_pool.py:68-101): the
+  row-gather kernel of the interpolation with unit weights, divided by the neighbour count;
+  the gradient runs over the transposed table (no atomics)."""
+  from .octree_interp import _Interp
+  table = octree._table(depth, kernel, stride, nempty)
+  count = (table >= 0).sum(1).to(torch.float32)
+  return _Interp.apply(data, table, None, count)
+
+
+class _GlobalPool(torch.autograd.Function):
+  @staticmethod
+  def forward(ctx, data, bounds, batch_id, batch_size):
+    from .octree_conv import column_sum
+    data = data.contiguous()
+    out = torch.zeros((batch_size, data.shape[1]), dtype=data.dtype, device=data.device)
+    counts = []
+    for b in range(batch_size):
+      lo, hi = bounds[b], bounds[b + 1]
+      counts.append(max(hi - lo, 1))                    # (an element may have no node)
+      if hi > lo:
+        out[b] = (column_sum(data[lo:hi]).float() / counts[-1]).to(data.dtype)
+    ctx.count = torch.tensor(counts, dtype=torch.float32, device=data.device)
+    ctx.save_for_backward(batch_id)
+    return out
+
+  @staticmethod
+  def backward(ctx, grad):
+    batch_id, = ctx.saved_tensors
+    g = (grad.float() / ctx.count.unsqueeze(1)).to(grad.dtype)
+    return g.index_select(0, batch_id), None, None, None
+
+
+def octree_global_pool(data: torch.Tensor, octree, depth: int, nempty: bool = False):
+  """Mean over the nodes of every batch element (ocnn/nn/octree_pool.py:104-125).  The nodes of
+  an element are consecutive rows (the batch index is the top of the key), so each mean is a
+  column sum with a fixed reduction order."""
+  batch_id = octree.batch_id(depth, nempty)
+  batch_size = octree.batch_size
+  edges = torch.searchsorted(batch_id, torch.arange(batch_size + 1, device=batch_id.device))
+  return _GlobalPool.apply(data, edges.tolist(), batch_id, batch_size)
+
+
+class OctreeAvgPool(torch.nn.Module):
+  """ocnn/nn/octree_pool.py:190-200."""
+
+  def __init__(self, kernel_size: List[int], stride: int, nempty: bool = False):
+    super().__init__()
+    self.kernel_size = resize_with_last_val(kernel_size)
+    self.kernel = list2str(self.kernel_size)
+    self.stride = stride
+    self.nempty = nempty
+
+  def forward(self, data: torch.Tensor, octree, depth: int):
+    return octree_avg_pool(data, octree, depth, self.kernel, self.stride, self.nempty)
+
+  def extra_repr(self) -> str:
+    return 'kernel_size={}, stride={}, nempty={}'.format(self.kernel_size, self.stride, self.nempty)
+
+
+class OctreeGlobalPool(torch.nn.Module):
+  """ocnn/nn/octree_pool.py:174-187."""
+
+  def __init__(self, nempty: bool = False):
+    super().__init__()
+    self.kernel_size, self.kernel, self.stride = [-1, -1, -1], '-1-1-1', -1
+    self.nempty = nempty
+
+  def forward(self, data: torch.Tensor, octree, depth: int):
+    return octree_global_pool(data, octree, depth, self.nempty)
 
   def extra_repr(self) -> str:
     return 'kernel_size={}, stride={}, nempty={}'.format(self.kernel_size, self.stride, self.nempty)

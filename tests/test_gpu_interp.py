@@ -192,3 +192,59 @@ def test_interp_and_pool_at_full_size():
   hit = back != 0
   assert torch.equal(back[hit], data[hit])
   assert int(hit.sum()) == pooled.numel() - int((pooled == 0).sum())       # (a maximum may be exactly 0)
+
+
+def _to_voxels(data, o, depth):
+  x, y, z, b = o.xyzb(depth, False)
+  n = 1 << depth
+  vox = data.new_zeros([o.batch_size, n, n, n, data.shape[1]])
+  vox[b, x, y, z] = data
+  return vox
+
+
+def test_avg_pool_is_avg_pool3d_on_a_full_layer(ref_data):
+  """test/test_octree_pool.py:39-61: on a full layer the average over the existing neighbours
+  is torch.nn.AvgPool3d without the padding counted; and the gradient is its adjoint."""
+  from ocnn_amd.nn import OctreeAvgPool, octree_avg_pool
+  say('avg pool')
+  o = merged_octree(ref_data)
+  depth, c = 3, 33
+  data = torch.rand(int(o.nnum[depth]), c, generator=torch.Generator().manual_seed(8)).to(DEV)
+  grid = _to_voxels(data, o, depth)
+  for kernel, stride, pad in [(3, 1, 1), (3, 2, 1), (2, 2, 0)]:
+    want = torch.nn.AvgPool3d(kernel, stride, pad, count_include_pad=False)(grid.permute(0, 4, 1, 2, 3)).permute(0, 2, 3, 4, 1)
+    out = OctreeAvgPool([kernel], stride, nempty=False)(data, o, depth)
+    got = _to_voxels(out, o, depth - 1 if stride == 2 else depth)
+    assert torch.allclose(got, want, atol=1e-6), (kernel, stride)
+  # sparse level, gradient: <pool(x), g> = <x, pool^T(g)>
+  depth = 5
+  x = torch.randn(int(o.nnum_nempty[depth]), 6, generator=torch.Generator().manual_seed(9)).to(DEV).requires_grad_()
+  y = octree_avg_pool(x, o, depth, '333', 1, nempty=True)
+  g = torch.randn(y.shape, generator=torch.Generator().manual_seed(10)).to(DEV)
+  y.backward(g)
+  t = o.get_neigh(depth, '333', 1, True)
+  cnt = (t >= 0).sum(1).clamp(min=1).float()
+  want = torch.zeros_like(x)
+  for k in range(27):
+    v = t[:, k] >= 0
+    want.index_add_(0, t[v, k], g[v] / cnt[v, None])
+  assert torch.allclose(x.grad, want, atol=1e-5)
+
+
+@pytest.mark.parametrize('nempty', [False, True])
+def test_global_pool(ref_data, nempty):
+  from ocnn_amd.nn import OctreeGlobalPool
+  say('global pool', nempty)
+  o = merged_octree(ref_data)
+  depth = 5
+  rows = int(o.nnum_nempty[depth] if nempty else o.nnum[depth])
+  x = torch.randn(rows, 7, generator=torch.Generator().manual_seed(12)).to(DEV).requires_grad_()
+  out = OctreeGlobalPool(nempty)(x, o, depth)
+  bid = o.batch_id(depth, nempty)
+  assert out.shape == (2, 7)
+  for b in range(2):
+    assert torch.allclose(out[b], x.detach()[bid == b].mean(0), atol=1e-5)
+  g = torch.randn(2, 7, generator=torch.Generator().manual_seed(13)).to(DEV)
+  out.backward(g)
+  cnt = torch.bincount(bid, minlength=2).float()
+  assert torch.allclose(x.grad, (g / cnt[:, None])[bid], atol=1e-6)
