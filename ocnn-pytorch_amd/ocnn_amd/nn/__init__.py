@@ -2,6 +2,7 @@ from .octree_pad import octree_pad, octree_depad
 from .octree_conv import (OctreeConv, OctreeDeconv, OctreeConvBase, octree_conv, octree_deconv,
                           conv_gather, conv_wgrad, column_sum)
 from .octree_dwconv import OctreeDWConv, octree_dwconv
+from .octree_gconv import OctreeGroupConv
 from .octree_conv_t import (OctreeConvTriton, OctreeConvT, octree_conv_triton,
                             convert_conv_triton, conv_fwd_implicit_gemm_splitk,
                             conv_bwd_implicit_gemm_splitk)
@@ -17,4 +18,4 @@ __all__ = ['octree_pad', 'octree_depad', 'OctreeConv', 'OctreeDeconv', 'octree_c
            'conv_bwd_implicit_gemm_splitk', 'octree_max_pool', 'octree_max_unpool', 'OctreeMaxPool',
            'OctreeMaxUnpool', 'octree_nearest_pts', 'octree_linear_pts', 'OctreeInterp',
            'octree_nearest_upsample', 'OctreeUpsample', 'BatchNormRelu1d', 'octree_avg_pool',
-           'octree_global_pool', 'OctreeAvgPool', 'OctreeGlobalPool']
+           'octree_global_pool', 'OctreeAvgPool', 'OctreeGlobalPool', 'OctreeGroupConv']

@@ -689,3 +689,22 @@ def test_odd_channels_on_large_layers(medium):
       say('padded channels', dtype, kind, ks, stride, ne, cin, cout)
       errs = run_layer(kind, medium, depth, ks, stride, ne, cin, cout, dtype)
       assert max(errs.values()) < TOL[dtype], (dtype, kind, ks, stride, ne, cin, cout, errs)
+
+
+def test_group_conv_is_a_block_diagonal_conv(small):
+  """OctreeGroupConv (ocnn/nn/octree_gconv.py): its output equals the oracle's convolution
+  with the block-diagonal weights put together from the per-group layers."""
+  from ocnn_amd.nn import OctreeGroupConv
+  depth, cin, cout, group = 5, 12, 18, 3
+  g = torch.Generator().manual_seed(21)
+  mod = OctreeGroupConv(cin, cout, [3], 1, nempty=True, use_bias=True, group=group).to(DEV)
+  x = torch.randn(rows_of(small.ref, depth, True), cin, generator=g)
+  out = mod(x.to(DEV), small.gpu, depth)
+  w = np.zeros((27, cin, cout))
+  b = np.zeros(cout)
+  ci, co = cin // group, cout // group
+  for i, conv in enumerate(mod.convs):
+    w[:, i * ci:(i + 1) * ci, i * co:(i + 1) * co] = f64(conv.weights)
+    b[i * co:(i + 1) * co] = f64(conv.bias)
+  want = C.conv_layer(small.ref, f64(x), w, depth, [3, 3, 3], 1, True, bias=b)
+  assert rel_err(out, want) < 1e-4
