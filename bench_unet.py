@@ -109,17 +109,15 @@ def main():
     with profile(activities=[ProfilerActivity.CUDA, ProfilerActivity.CPU]) as prof:
       step()
       torch.cuda.synchronize()
-    groups = {}
+    groups, top = {}, []
     for e in prof.key_averages():
       t = getattr(e, 'device_time_total', 0) or getattr(e, 'cuda_time_total', 0)
-      if e.device_type is not None and 'cuda' in str(e.device_type).lower() or 'kernel' in e.key.lower():
-        pass
       name = e.key
       if t <= 0 or not any(k in name for k in ('ocnn', 'Kernel', 'kernel', 'Cijk', 'gemm')):
         continue
       if 'conv_' in name or 'wgrad' in name or 'pack_weights' in name:
         k = 'octree conv kernels'
-      elif 'batch_norm' in name or 'BatchNorm' in name:
+      elif 'batch_norm' in name or 'BatchNorm' in name or 'bn_' in name:
         k = 'batch norm'
       elif 'interp' in name or 'csr_rows' in name or 'search' in name:
         k = 'interpolation'
@@ -132,7 +130,9 @@ def main():
       else:
         k = 'elementwise / other'
       groups[k] = groups.get(k, 0.0) + t / 1e3
+      top.append((round(t / 1e3, 3), e.count, name[:90]))
     out['device_ms_by_kind'] = {k: round(v, 3) for k, v in sorted(groups.items(), key=lambda kv: -kv[1])}
+    out['top_kernels_ms_calls'] = sorted(top, reverse=True)[:24]
   print(json.dumps(out), flush=True)
 
 

@@ -226,6 +226,30 @@ int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint
                           int w_transposed, int reverse_slots, const void* bias, void* out,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ocnn_conv_gather for sparse tables (few of the K slots of a row hold a neighbour, as on the
+ * non-empty nodes of a deep level): the work follows the (row, neighbour) pairs.  On top of
+ * the tile plan (uptr, urows) it takes the pair plan of the table: the slots in an order
+ * slot_order (device array of K slot numbers; the first n_first of them form slot group 0,
+ * the others group 1, at most ocnn_conv_gather_sparse_max_slots(K) each - balance the pairs),
+ * cptr (tiles * K + 1 block offsets, tile-major, slots in that order) and ent (16 entries per
+ * block: position of the input row in the tile's list + 1, | (128 r + 16 (r & 7)) << 16 for
+ * row r of the tile; blocks are filled up with position 0, r = 128); max_blocks = the largest
+ * number of blocks of one tile.  Weights stay in registers, a workgroup serves 32 output
+ * channels over many tiles, results are added in a fixed order.  f16 / bf16, cin in
+ * {32, 64, 96, 128}, cout % 32 == 0, K <= 27; same result as ocnn_conv_gather.
+ * workspace: K * cin * cout * 2 bytes. */
+int ocnn_conv_gather_sparse_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
+                                      int plan_max_distinct);
+int ocnn_conv_gather_sparse_max_slots(int K);
+int ocnn_conv_gather_sparse(int dtype, const void* in, int64_t rows_in, const int32_t* uptr,
+                            const int32_t* urows, int plan_max_distinct, int64_t plan_total,
+                            const int32_t* cptr, const uint32_t* ent, int64_t n_blocks,
+                            int max_blocks, const int32_t* slot_order, int n_first,
+                            int64_t rows_out, int K,
+                            const void* w, int cin, int cout, int w_transposed, int reverse_slots,
+                            const void* bias, void* out, void* workspace, int64_t workspace_bytes,
+                            void* stream);
+
 /* out (rows, cout) = in (rows, cin) W (+ bias): ocnn_conv_gather with the one-slot identity
  * table, the form that the 2x2x2 stride-2 layers over all nodes take on the (parents, 8 C)
  * view of the children (ocnn/nn/octree_conv.py:115-168 with neigh[p] = 8p .. 8p+7).
@@ -327,20 +351,26 @@ int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const vo
  * OctreeDeconvBnRelu use torch.nn.BatchNorm1d + ReLU): per-channel mean, biased variance and
  * 1 / sqrt(var + eps) of x; y = (x - mean) * invstd * gamma + beta [then max(., 0)]; and the
  * gradient dx, dgamma, dbeta (training = 1: statistics of this batch; 0: fixed statistics;
- * dx may be NULL).  gamma / beta may be NULL (no affine part).  fp32 arithmetic, two-level
- * reductions with a fixed order.  channels a multiple of 16 bytes of elements. */
+ * dx may be NULL).  gamma / beta (dtype param_dtype) may be NULL (no affine part); the
+ * statistics kernel also moves running_mean / running_var (dtype running_dtype, may be NULL)
+ * towards the batch statistics by `factor`, the running variance towards the unbiased one
+ * (torch.nn.functional.batch_norm); dgamma / dbeta are fp32, grad_gamma / grad_beta the same
+ * sums in param_dtype (may be NULL).  fp32 arithmetic, two-level reductions with a fixed order.
+ * channels a multiple of 16 bytes of elements. */
 int ocnn_batch_norm_supported(int dtype, int64_t rows, int channels);
 int64_t ocnn_batch_norm_workspace_bytes(int channels);
 int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
-                          float* mean, float* var, float* invstd, void* workspace,
+                          float* mean, float* var, float* invstd, void* running_mean,
+                          void* running_var, int running_dtype, float factor, void* workspace,
                           int64_t workspace_bytes, void* stream);
 int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
-                          const float* invstd, const float* gamma, const float* beta, int relu,
-                          void* y, void* stream);
+                          const float* invstd, const void* gamma, const void* beta,
+                          int param_dtype, int relu, void* y, void* stream);
 int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy, int64_t rows, int channels,
-                             const float* mean, const float* invstd, const float* gamma,
-                             const float* beta, int relu, int training, void* dx, float* dgamma,
-                             float* dbeta, void* workspace, int64_t workspace_bytes, void* stream);
+                             const float* mean, const float* invstd, const void* gamma,
+                             const void* beta, int param_dtype, int relu, int training, void* dx,
+                             float* dgamma, float* dbeta, void* grad_gamma, void* grad_beta,
+                             void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Key search, ocnn/octree/octree.py:448-488 (search_key / search_xyzb): out[i] = position of
  * query[i] in the ascending `keys`, or -1.  ocnn_search_points takes float (x, y, z, b) rows,

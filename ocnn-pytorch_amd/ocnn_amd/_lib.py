@@ -49,6 +49,10 @@ SIGNATURES = {
     'ocnn_conv_gather_rw': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                  _p, _l, _p]),
     'ocnn_conv_gather_wide_supported': (_i, [_i, _l, _i, _i, _i, _i]),
+    'ocnn_conv_gather_sparse_supported': (_i, [_i, _l, _i, _i, _i, _i]),
+    'ocnn_conv_gather_sparse_max_slots': (_i, [_i]),
+    'ocnn_conv_gather_sparse': (_i, [_i, _p, _l, _p, _p, _i, _l, _p, _p, _l, _i, _p, _i, _l, _i, _p, _i, _i, _i, _i,
+                                     _p, _p, _p, _l, _p]),
     'ocnn_conv_gather_wide': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                    _p, _l, _p]),
     'ocnn_conv_dense_supported': (_i, [_i, _l, _i, _i]),
@@ -74,9 +78,10 @@ SIGNATURES = {
     'ocnn_dwconv_wgrad_planned': (_i, [_i, _p, _l, _p, _p, _p, _p, _i, _l, _l, _i, _i, _p, _p, _l, _p]),
     'ocnn_batch_norm_supported': (_i, [_i, _l, _i]),
     'ocnn_batch_norm_workspace_bytes': (_l, [_i]),
-    'ocnn_batch_norm_stats': (_i, [_i, _p, _l, _i, _f, _p, _p, _p, _p, _l, _p]),
-    'ocnn_batch_norm_apply': (_i, [_i, _p, _l, _i, _p, _p, _p, _p, _i, _p, _p]),
-    'ocnn_batch_norm_backward': (_i, [_i, _p, _p, _l, _i, _p, _p, _p, _p, _i, _i, _p, _p, _p, _p, _l, _p]),
+    'ocnn_batch_norm_stats': (_i, [_i, _p, _l, _i, _f, _p, _p, _p, _p, _p, _i, _f, _p, _l, _p]),
+    'ocnn_batch_norm_apply': (_i, [_i, _p, _l, _i, _p, _p, _p, _p, _i, _i, _p, _p]),
+    'ocnn_batch_norm_backward': (_i, [_i, _p, _p, _l, _i, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _p, _p,
+                                      _p, _l, _p]),
     'ocnn_search_key': (_i, [_p, _l, _p, _l, _p, _p]),
     'ocnn_search_points': (_i, [_p, _l, _i, _p, _l, _i, _p, _p]),
     'ocnn_interp_linear_prepare': (_i, [_p, _l, _i, _p, _l, _i, _p, _p, _p, _p]),

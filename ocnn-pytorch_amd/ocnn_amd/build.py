@@ -21,6 +21,7 @@ SOURCES = {
     'conv_staged.hip': [],
     'conv_rw.hip': [],
     'conv_wide.hip': [],
+    'conv_sparse.hip': [],
     'dense_rw.hip': [],
     'dw_planned.hip': [],
     'wgrad_planned.hip': [],

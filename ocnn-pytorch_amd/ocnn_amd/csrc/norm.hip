@@ -16,6 +16,20 @@ constexpr int kBnApplyBlocks = 2048;  // workgroups of an elementwise pass
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) BnVec { T v[VEC]; };
 
+// element c of a per-channel parameter held as f32 / f16 / bf16 (p == nullptr: dflt)
+__device__ __forceinline__ float bn_param(const void* p, int dtype, int c, float dflt) {
+  if (!p) return dflt;
+  if (dtype == OCNN_F32) return ((const float*)p)[c];
+  if (dtype == OCNN_F16) return to_f32(((const f16*)p)[c]);
+  return to_f32(((const bf16*)p)[c]);
+}
+
+__device__ __forceinline__ void bn_store(void* p, int dtype, int c, float v) {
+  if (dtype == OCNN_F32) ((float*)p)[c] = v;
+  else if (dtype == OCNN_F16) ((f16*)p)[c] = from_f32<f16>(v);
+  else ((bf16*)p)[c] = from_f32<bf16>(v);
+}
+
 // partial[blk][0][c] = sum_r (x[r][c] - x[0][c]),  partial[blk][1][c] = sum_r (x[r][c] - x[0][c])^2
 // over the rows of the workgroup (shifting by the first row keeps the variance free of
 // cancellation when the mean is large against the spread).  Thread: VEC channels of every
@@ -111,10 +125,13 @@ __device__ __forceinline__ int bn_sum_partials(const float* __restrict__ partial
 }
 
 // mean, biased variance and 1 / sqrt(var + eps) per channel from the partial sums
+// running_mean / running_var (dtype rdtype), when given, move towards the batch statistics by
+// `factor` (the running variance towards the unbiased one), as torch.nn.functional.batch_norm.
 template <typename T>
 __global__ void bn_stats_finish_kernel(const float* __restrict__ partial, int nblk, const T* __restrict__ x,
                                        int64_t rows, int C, float eps, float* __restrict__ mean,
-                                       float* __restrict__ var, float* __restrict__ invstd) {
+                                       float* __restrict__ var, float* __restrict__ invstd,
+                                       void* running_mean, void* running_var, int rdtype, float factor) {
   double a, b;
   const int c = bn_sum_partials(partial, nblk, C, a, b);
   if (c < 0) return;
@@ -123,6 +140,11 @@ __global__ void bn_stats_finish_kernel(const float* __restrict__ partial, int nb
   mean[c] = (float)((double)to_f32(x[c]) + m);
   var[c] = (float)v;
   invstd[c] = (float)(1.0 / sqrt(v + (double)eps));
+  if (running_mean) {
+    const float unbiased = (float)(v * ((double)rows / (double)max(rows - 1, (int64_t)1)));
+    bn_store(running_mean, rdtype, c, (1.f - factor) * bn_param(running_mean, rdtype, c, 0.f) + factor * mean[c]);
+    bn_store(running_var, rdtype, c, (1.f - factor) * bn_param(running_var, rdtype, c, 0.f) + factor * unbiased);
+  }
 }
 
 // y = (x - mean) * (invstd * gamma) + beta, then max(., 0) when relu.  A thread keeps the
@@ -133,8 +155,8 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
                                                        int64_t rows_per_blk,
                                                        const float* __restrict__ mean,
                                                        const float* __restrict__ invstd,
-                                                       const float* __restrict__ gamma,
-                                                       const float* __restrict__ beta, int relu,
+                                                       const void* __restrict__ gamma,
+                                                       const void* __restrict__ beta, int pdtype, int relu,
                                                        T* __restrict__ y) {
   typedef BnVec<T, VEC> V;
   const int lpr = C / VEC, rpp = 256 / lpr;
@@ -145,8 +167,8 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
   for (int v = 0; v < VEC; ++v) {
     const int c = cl * VEC + v;
     m[v] = mean[c];
-    sc[v] = invstd[c] * (gamma ? gamma[c] : 1.f);
-    be[v] = beta ? beta[c] : 0.f;
+    sc[v] = invstd[c] * bn_param(gamma, pdtype, c, 1.f);
+    be[v] = bn_param(beta, pdtype, c, 0.f);
   }
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
   const int64_t r1 = min(rows, r0 + rows_per_blk);
@@ -180,8 +202,8 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
                                                            int64_t rows, int C, int64_t rows_per_blk,
                                                            const float* __restrict__ mean,
                                                            const float* __restrict__ invstd,
-                                                           const float* __restrict__ gamma,
-                                                           const float* __restrict__ beta, int relu,
+                                                           const void* __restrict__ gamma,
+                                                           const void* __restrict__ beta, int pdtype, int relu,
                                                            float* __restrict__ partial) {
   typedef BnVec<T, VEC> V;
   __shared__ float s_a[256 * VEC], s_b[256 * VEC];
@@ -197,8 +219,8 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
       const int c = cl * VEC + v;
       m[v] = mean[c];
       is[v] = invstd[c];
-      ga[v] = gamma ? gamma[c] : 1.f;
-      be[v] = beta ? beta[c] : 0.f;
+      ga[v] = bn_param(gamma, pdtype, c, 1.f);
+      be[v] = bn_param(beta, pdtype, c, 0.f);
     }
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
     const int64_t r1 = min(rows, r0 + rows_per_blk);
@@ -245,13 +267,17 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
   }
 }
 
+// (gw / gb: the same sums in the parameters' dtype, when given)
 __global__ void bn_bwd_finish_kernel(const float* __restrict__ partial, int nblk, int C,
-                                     float* __restrict__ dbeta, float* __restrict__ dgamma) {
+                                     float* __restrict__ dbeta, float* __restrict__ dgamma, void* gw, void* gb,
+                                     int pdtype) {
   double a, b;
   const int c = bn_sum_partials(partial, nblk, C, a, b);
   if (c < 0) return;
   dbeta[c] = (float)a;
   dgamma[c] = (float)b;
+  if (gw) bn_store(gw, pdtype, c, (float)b);
+  if (gb) bn_store(gb, pdtype, c, (float)a);
 }
 
 // training: dx = gamma * invstd * (dy' - dbeta / N - xhat * dgamma / N); with fixed statistics
@@ -261,8 +287,8 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__
                                                            int64_t rows, int C, int64_t rows_per_blk,
                                                            const float* __restrict__ mean,
                                                            const float* __restrict__ invstd,
-                                                           const float* __restrict__ gamma,
-                                                           const float* __restrict__ beta, int relu,
+                                                           const void* __restrict__ gamma,
+                                                           const void* __restrict__ beta, int pdtype, int relu,
                                                            const float* __restrict__ dbeta,
                                                            const float* __restrict__ dgamma, int training,
                                                            T* __restrict__ dx) {
@@ -277,8 +303,8 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__
     const int c = cl * VEC + v;
     m[v] = mean[c];
     is[v] = invstd[c];
-    sc[v] = invstd[c] * (gamma ? gamma[c] : 1.f);
-    be[v] = beta ? beta[c] : 0.f;
+    sc[v] = invstd[c] * bn_param(gamma, pdtype, c, 1.f);
+    be[v] = bn_param(beta, pdtype, c, 0.f);
     db[v] = training ? dbeta[c] * inv_n : 0.f;
     dg[v] = training ? dgamma[c] * inv_n : 0.f;
   }
@@ -344,7 +370,8 @@ extern "C" int64_t ocnn_batch_norm_workspace_bytes(int channels) {
 }
 
 extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
-                                     float* mean, float* var, float* invstd, void* workspace,
+                                     float* mean, float* var, float* invstd, void* running_mean,
+                                     void* running_var, int running_dtype, float factor, void* workspace,
                                      int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_stats: shape not supported");
   OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels), "batch_norm_stats: workspace too small");
@@ -358,14 +385,15 @@ extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int
     hipLaunchKernelGGL((bn_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
                        partial);
     hipLaunchKernelGGL(bn_stats_finish_kernel<T>, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
-                       (const T*)x, rows, channels, eps, mean, var, invstd);
+                       (const T*)x, rows, channels, eps, mean, var, invstd, running_mean, running_var, running_dtype,
+                       factor);
   });
   return check_launch("batch_norm_stats");
 }
 
 extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
-                                     const float* invstd, const float* gamma, const float* beta, int relu,
-                                     void* y, void* stream) {
+                                     const float* invstd, const void* gamma, const void* beta, int param_dtype,
+                                     int relu, void* y, void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_apply: shape not supported");
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
@@ -374,15 +402,16 @@ extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
-                       mean, invstd, gamma, beta, relu, (T*)y);
+                       mean, invstd, gamma, beta, param_dtype, relu, (T*)y);
   });
   return check_launch("batch_norm_apply");
 }
 
 extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy, int64_t rows, int channels,
-                                        const float* mean, const float* invstd, const float* gamma,
-                                        const float* beta, int relu, int training, void* dx, float* dgamma,
-                                        float* dbeta, void* workspace, int64_t workspace_bytes, void* stream) {
+                                        const float* mean, const float* invstd, const void* gamma,
+                                        const void* beta, int param_dtype, int relu, int training, void* dx,
+                                        float* dgamma, float* dbeta, void* grad_gamma, void* grad_beta,
+                                        void* workspace, int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_backward: shape not supported");
   OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels),
                "batch_norm_backward: workspace too small");
@@ -397,12 +426,13 @@ extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_bwd_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
-                       channels, per, mean, invstd, gamma, beta, relu, partial);
+                       channels, per, mean, invstd, gamma, beta, param_dtype, relu, partial);
     hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
-                       channels, dbeta, dgamma);
+                       channels, dbeta, dgamma, grad_gamma, grad_beta, param_dtype);
     if (dx)
       hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), dim3(nblk_a), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
-                         channels, per_a, mean, invstd, gamma, beta, relu, dbeta, dgamma, training, (T*)dx);
+                         channels, per_a, mean, invstd, gamma, beta, param_dtype, relu, dbeta, dgamma, training,
+                         (T*)dx);
   });
   return check_launch("batch_norm_backward");
 }

@@ -9,8 +9,14 @@ import torch.nn
 from .. import _lib
 
 
-def _f32(t):
-  return None if t is None else t.detach().to(torch.float32).contiguous()
+def _param(t):
+  """A per-channel parameter as the kernels read it (f32 / f16 / bf16, contiguous)."""
+  if t is None:
+    return None
+  t = t.detach()
+  if t.dtype not in _lib.DTYPE_CODE:
+    t = t.float()
+  return t.contiguous()
 
 
 class _BatchNormRelu(torch.autograd.Function):
@@ -21,27 +27,36 @@ class _BatchNormRelu(torch.autograd.Function):
     rows, c = x.shape
     code = _lib.dtype_code(x)
     dev = x.device
-    gamma, beta = _f32(weight), _f32(bias)
+    gamma, beta = _param(weight), _param(bias)
+    if beta is not None and gamma is not None and beta.dtype != gamma.dtype:
+      beta = beta.to(gamma.dtype)
+    pcode = _lib.DTYPE_CODE[(gamma if gamma is not None else beta).dtype] if (gamma is not None or beta is not None) else 0
     if use_batch_stats:
       mean = torch.empty(c, dtype=torch.float32, device=dev)
       var = torch.empty(c, dtype=torch.float32, device=dev)
       invstd = torch.empty(c, dtype=torch.float32, device=dev)
       ws = _lib.workspace(L.ocnn_batch_norm_workspace_bytes(c), dev)
-      _lib.check(L.ocnn_batch_norm_stats(code, _lib.ptr(x), rows, c, float(eps), _lib.ptr(mean), _lib.ptr(var),
-                                         _lib.ptr(invstd), _lib.ptr(ws), ws.numel(), _lib.stream()))
-      if running_mean is not None and factor is not None:
-        # the running variance is the unbiased one (torch.nn.functional.batch_norm)
+      track = running_mean is not None and factor is not None
+      in_place = track and running_mean.dtype in _lib.DTYPE_CODE and running_mean.dtype == running_var.dtype \
+          and running_mean.is_contiguous() and running_var.is_contiguous()
+      _lib.check(L.ocnn_batch_norm_stats(
+          code, _lib.ptr(x), rows, c, float(eps), _lib.ptr(mean), _lib.ptr(var), _lib.ptr(invstd),
+          _lib.ptr(running_mean) if in_place else None, _lib.ptr(running_var) if in_place else None,
+          _lib.DTYPE_CODE[running_mean.dtype] if in_place else 0, float(factor) if in_place else 0.0,
+          _lib.ptr(ws), ws.numel(), _lib.stream()))
+      if track and not in_place:
         unbiased = var * (rows / max(rows - 1, 1))
         running_mean.mul_(1 - factor).add_(mean.to(running_mean.dtype), alpha=factor)
         running_var.mul_(1 - factor).add_(unbiased.to(running_var.dtype), alpha=factor)
     else:
-      mean = _f32(running_mean)
-      invstd = torch.rsqrt(_f32(running_var) + eps)
+      mean = running_mean.detach().float().contiguous()
+      invstd = torch.rsqrt(running_var.detach().float() + eps)
     y = torch.empty_like(x)
     _lib.check(L.ocnn_batch_norm_apply(code, _lib.ptr(x), rows, c, _lib.ptr(mean), _lib.ptr(invstd),
-                                       _lib.ptr(gamma), _lib.ptr(beta), int(relu), _lib.ptr(y), _lib.stream()))
+                                       _lib.ptr(gamma), _lib.ptr(beta), pcode, int(relu), _lib.ptr(y),
+                                       _lib.stream()))
     ctx.save_for_backward(x, mean, invstd, gamma, beta)
-    ctx.relu, ctx.training = relu, use_batch_stats
+    ctx.relu, ctx.training, ctx.pcode = relu, use_batch_stats, pcode
     ctx.wdtype = None if weight is None else weight.dtype
     ctx.bdtype = None if bias is None else bias.dtype
     return y
@@ -56,20 +71,29 @@ class _BatchNormRelu(torch.autograd.Function):
     dgamma = torch.empty(c, dtype=torch.float32, device=dev)
     dbeta = torch.empty(c, dtype=torch.float32, device=dev)
     dx = torch.empty_like(x) if ctx.needs_input_grad[0] else None
+    # the parameter gradients come out in the parameters' dtype where the kernels hold it
+    gw = gb = None
+    if gamma is not None and ctx.needs_input_grad[1] and ctx.wdtype == gamma.dtype:
+      gw = torch.empty(c, dtype=gamma.dtype, device=dev)
+    if beta is not None and ctx.needs_input_grad[2] and ctx.bdtype == beta.dtype and \
+        (gamma is None or beta.dtype == gamma.dtype):
+      gb = torch.empty(c, dtype=beta.dtype, device=dev)
     ws = _lib.workspace(L.ocnn_batch_norm_workspace_bytes(c), dev)
     _lib.check(L.ocnn_batch_norm_backward(
         _lib.dtype_code(x), _lib.ptr(x), _lib.ptr(dy), rows, c, _lib.ptr(mean), _lib.ptr(invstd), _lib.ptr(gamma),
-        _lib.ptr(beta), int(ctx.relu), int(ctx.training), _lib.ptr(dx), _lib.ptr(dgamma), _lib.ptr(dbeta),
-        _lib.ptr(ws), ws.numel(), _lib.stream()))
-    gw = dgamma.to(ctx.wdtype) if ctx.wdtype is not None and ctx.needs_input_grad[1] else None
-    gb = dbeta.to(ctx.bdtype) if ctx.bdtype is not None and ctx.needs_input_grad[2] else None
+        _lib.ptr(beta), ctx.pcode, int(ctx.relu), int(ctx.training), _lib.ptr(dx), _lib.ptr(dgamma),
+        _lib.ptr(dbeta), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    if gw is None and ctx.wdtype is not None and ctx.needs_input_grad[1]:
+      gw = dgamma.to(ctx.wdtype)
+    if gb is None and ctx.bdtype is not None and ctx.needs_input_grad[2]:
+      gb = dbeta.to(ctx.bdtype)
     return dx, gw, gb, None, None, None, None, None, None
 
 
 class BatchNormRelu1d(torch.nn.BatchNorm1d):
-  """BatchNorm1d [+ ReLU] in one pass over (rows, C) inputs on the GPU; anything else (3-D
-  inputs, CPU tensors, channel counts that are not a multiple of 16 bytes) takes torch's own
-  batch norm followed by a ReLU."""
+  """BatchNorm1d [+ ReLU] in one pass over (rows, C) inputs on the GPU.  Inputs the kernels do
+  not take (3-D, channel counts that are not a multiple of 16 bytes, a single row, tensors
+  that are not on the GPU) go through torch.nn.BatchNorm1d itself, followed by a ReLU."""
 
   def __init__(self, num_features: int, relu: bool = False, **kwargs):
     super().__init__(num_features, **kwargs)

@@ -25,6 +25,9 @@ from .octree_pad import octree_depad, octree_pad
 
 PAD_MIN_ROWS = 16384     # from this many table rows on, odd channel counts are zero-padded
 USE_WIDE = True          # the wide-layer gather kernel (switch for comparisons)
+USE_SPARSE = True        # the pair-list gather kernel for sparse tables
+SPARSE_MAX_OCCUPANCY = 0.3   # share of table entries that hold a row, up to which it is used
+SPARSE_MIN_ROWS = 32768      # (a workgroup loads its weights once and needs many tiles to pay for it)
 
 
 def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False):
@@ -69,6 +72,15 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
         int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return out
+  if (plan is not None and USE_SPARSE and plan.occupancy <= SPARSE_MAX_OCCUPANCY and
+      rows >= SPARSE_MIN_ROWS and L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)):
+    pp = plan.pairs()
+    _lib.check(L.ocnn_conv_gather_sparse(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax, plan.total,
+        _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.order), pp.n_first, rows, K,
+        _lib.ptr(W), cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
+        ws.numel(), _lib.stream()))
     return out
   if plan is not None and plan.reuse >= 2.0 and USE_WIDE and L.ocnn_conv_gather_wide_supported(
       code, rows_in, K, cin, cout, plan.umax):
@@ -213,6 +225,7 @@ class OctreeConvBase:
     if not (L.ocnn_conv_gather_planned_supported(code, rows, cin, cout) or
             L.ocnn_conv_gather_rw_supported(code, rows, self.kdim, cin, cout, 0) or
             L.ocnn_conv_gather_wide_supported(code, rows, self.kdim, cin, cout, 0) or
+            L.ocnn_conv_gather_sparse_supported(code, rows, self.kdim, cin, cout, 0) or
             L.ocnn_conv_wgrad_planned_supported(code, rows, rows, self.kdim, cin, cout, 0)):
       return None
     return self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse,

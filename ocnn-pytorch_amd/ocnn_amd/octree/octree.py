@@ -131,6 +131,63 @@ class TilePlan:
     _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(uptr),
                                      _lib.ptr(self.urows), _lib.ptr(self.loc), st))
     self.rows, self.K, self.total, self.umax = rows, K, total, umax
+    self.nnz = nnz
+    self._pairs = None
+
+  @property
+  def occupancy(self):
+    """Share of the table's entries that hold a row."""
+    return self.nnz / max(self.rows * self.K, 1)
+
+  def pairs(self):
+    """Pair plan of the table for ocnn_conv_gather_sparse (built on first use): per tile
+    and slot the rows that have a neighbour, in blocks of 16 entries."""
+    if self._pairs is None:
+      self._pairs = PairPlan(self)
+    return self._pairs
+
+
+class PairPlan:
+  """Blocks of 16 entries per (tile, slot), the slots dealt to two groups of about equal
+  numbers of pairs.  Entry: position of the input row in the tile's list + 1, | (128 r +
+  16 (r & 7)) << 16 for row r of the tile; blocks are filled up with position 0, r = 128."""
+
+  def __init__(self, plan: TilePlan):
+    L = _lib.lib()
+    tiles, K, R = plan.loc.shape
+    dev = plan.loc.device
+    loc = plan.loc.to(torch.int32) & 0xffff                       # (tiles, K, R), 0 = empty
+    valid = loc > 0
+    per_slot = valid.sum((0, 2)).tolist()
+    # slots to the two groups: largest first, each to the lighter group that still has room
+    cap = L.ocnn_conv_gather_sparse_max_slots(K)
+    groups, load = ([], []), [0, 0]
+    for k in sorted(range(K), key=lambda k: -per_slot[k]):
+      g = 0 if load[0] <= load[1] else 1
+      if len(groups[g]) >= cap:
+        g = 1 - g
+      groups[g].append(k)
+      load[g] += per_slot[k]
+    order = groups[0] + groups[1]
+    self.n_first = len(groups[0])
+    self.order = torch.tensor(order, dtype=torch.int32, device=dev)
+    idx = self.order.long()
+    loc, valid = loc[:, idx, :], valid[:, idx, :]
+    count = valid.sum(2)                                          # (tiles, K)
+    nblk = (count + 15) // 16
+    cptr = torch.zeros(tiles * K + 1, dtype=torch.int64, device=dev)
+    cptr[1:] = torch.cumsum(nblk.reshape(-1), 0)
+    self.n_blocks = int(cptr[-1])
+    self.max_blocks = int(nblk.sum(1).max()) if tiles > 0 else 0
+    acc = torch.arange(R + 1, dtype=torch.int32, device=dev)
+    acc = (128 * acc + 16 * (acc & 7)) << 16                      # where a row's sums live in the kernel
+    ent = torch.full((max(self.n_blocks, 1) * 16,), int(acc[R]), dtype=torch.int32, device=dev)   # filling
+    slot = torch.cumsum(valid, 2) - 1                             # place of a pair in its list
+    dest = cptr[:-1].view(tiles, K, 1) * 16 + slot
+    val = loc | acc[:R].view(1, 1, R)
+    ent[dest[valid]] = val[valid]
+    self.ent = ent
+    self.cptr = cptr.to(torch.int32)
 
 
 class Octree:

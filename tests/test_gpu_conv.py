@@ -519,6 +519,90 @@ def test_wide_gather_kernel(dtype, K, cin, cout):
       assert rel_err(got, want) < TOL[dtype]
 
 
+def _gather_sparse(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
+  """ocnn_conv_gather_sparse through the C ABI (the Python layer picks it only for large,
+  sparse tables)."""
+  L = _lib.lib()
+  rows, K = table.shape
+  cin = x.shape[1]
+  code = _lib.dtype_code(x)
+  assert L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)
+  pp = plan.pairs()
+  out = torch.empty((rows, cout), dtype=x.dtype, device=x.device)
+  ws = torch.empty(K * cin * cout * 2, dtype=torch.uint8, device=x.device)
+  _lib.check(L.ocnn_conv_gather_sparse(
+      code, _lib.ptr(x), rows_in, _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax, plan.total,
+      _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.order), pp.n_first, rows, K,
+      _lib.ptr(w), cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
+      ws.numel(), _lib.stream()))
+  return out
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('K,cin,cout', [(27, 96, 96), (27, 128, 96), (27, 32, 64), (27, 64, 32), (9, 96, 128),
+                                        (8, 128, 160), (8, 32, 32), (3, 64, 96), (1, 32, 32)])
+def test_sparse_gather_kernel(dtype, K, cin, cout):
+  """Gather-GEMM over the pair plan (blocks of 16 (row, neighbour) pairs per tile and slot,
+  weights resident in registers, fp32 sums in LDS), at several occupancies incl. a table
+  with empty slots and empty tiles, ragged row counts, with bias, and the transposed +
+  mirrored form of the data gradient, against the oracle; twice, bit-identical.  The last
+  input row holds NaN and is never read."""
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(11 * K + cin + cout)
+  for rows, rows_in, empty in [(1000, 1000, 0.85), (130, 150, 0.5), (128 * 40 + 1, 3000, 0.9), (128 * 300 + 77, 40000, 0.8)]:
+    say('sparse gather', dtype, K, cin, cout, rows, rows_in, empty)
+    table = _local_table(rows, rows_in - 1, K, g, empty=empty)
+    if K > 2:
+      table[:, 1] = -1                                   # a slot without pairs
+      table[256:384] = -1                                # a tile without pairs
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    pp = plan.pairs()
+    assert pp.n_first <= _lib.lib().ocnn_conv_gather_sparse_max_slots(K)
+    t64 = table.numpy().astype(np.int64)
+    x = torch.randn(rows_in, cin, generator=g).to(dtype)
+    w = (torch.randn(K, cin, cout, generator=g) / (K * cin * (1 - empty)) ** 0.5).to(dtype)
+    b = torch.randn(cout, generator=g).to(dtype)
+    xn = x.clone()
+    xn[-1] = float('nan')
+    got = _gather_sparse(xn.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV))
+    again = _gather_sparse(xn.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV))
+    assert torch.equal(got, again)
+    want = C.forward_gemm(f64(x), f64(w), t64) + f64(b)
+    assert rel_err(got, want) < TOL[dtype]
+    if cout <= 128:                                      # the data gradient: cout -> cin
+      gr = torch.randn(rows_in, cout, generator=g).to(dtype)
+      got = _gather_sparse(gr.to(DEV), rows_in, tg, plan, w.to(DEV), cin, True, True, None)
+      want = C.forward_gemm(f64(gr), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
+      assert rel_err(got, want) < TOL[dtype]
+
+
+def test_sparse_gather_large_tiles():
+  """Tiles near the staging limits of the pair-plan kernel (many distinct rows: one
+  workgroup per CU, the wider row-number buffers) and the refusal beyond them."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(3)
+  dtype = torch.bfloat16
+  code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+  for cin, spread in [(96, 200), (128, 170), (32, 250)]:
+    rows = rows_in = 6000
+    table = _local_table(rows, rows_in, 27, g, spread=spread, empty=0.85)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    say('sparse gather, large tiles', cin, plan.umax)
+    assert plan.umax > 256
+    assert L.ocnn_conv_gather_sparse_supported(code, rows_in, 27, cin, 64, plan.umax)
+    x = torch.randn(rows_in, cin, generator=g).to(dtype)
+    w = (torch.randn(27, cin, 64, generator=g) / (4 * cin) ** 0.5).to(dtype)
+    got = _gather_sparse(x.to(DEV), rows_in, tg, plan, w.to(DEV), 64, False, False, None)
+    want = C.forward_gemm(f64(x), f64(w), table.numpy().astype(np.int64))
+    assert rel_err(got, want) < TOL[dtype]
+  assert not L.ocnn_conv_gather_sparse_supported(code, 6000, 27, 128, 64, 511)
+  assert not L.ocnn_conv_gather_sparse_supported(code, 6000, 27, 96, 64, 600)
+  assert not L.ocnn_conv_gather_sparse_supported(code, 6000, 27, 160, 64, 100)
+
+
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('K,ca,cb', [(27, 128, 128), (27, 64, 192), (9, 256, 64), (8, 128, 64), (3, 192, 128),
                                      (27, 96, 96), (27, 96, 128), (8, 160, 96), (3, 64, 96)])
