@@ -226,6 +226,27 @@ int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint
                           int w_transposed, int reverse_slots, const void* bias, void* out,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Pair plan of a table, on top of its tile plan (loc: tiles x K x ocnn_tile_plan_rows()):
+ * what ocnn_conv_gather_sparse walks over.  No counterpart in the reference.
+ *   slot_counts: slot_count[k] (device, K x int64) = table entries of slot k that hold a row;
+ *   order (host only): deals the slots to two groups of about equal numbers of pairs, at
+ *          most max_slots each (ocnn_conv_gather_sparse_max_slots(K)); order[0 .. n_first)
+ *          = group 0, the rest group 1.  slot_count and order are host arrays here;
+ *   count: nblk[tile * K + j] = blocks of 16 pairs of slot slot_order[j] in the tile
+ *          (slot_order: device array, or NULL for 0 .. K - 1);
+ *   fill : cptr (tiles * K + 1) = exclusive prefix sum of nblk, made by the caller;
+ *          ent (16 entries per block): position of the pair's input row in the tile's list
+ *          + 1, | (128 r + 16 (r & 7)) << 16 for row r of the tile; the last block of a
+ *          list is filled up with position 0, r = 128. */
+int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,
+                               void* stream);
+int ocnn_pair_plan_order(int K, const int64_t* slot_count, int max_slots, int32_t* order,
+                         int* n_first);
+int ocnn_pair_plan_count(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
+                         int32_t* nblk, void* stream);
+int ocnn_pair_plan_fill(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
+                        const int32_t* cptr, uint32_t* ent, void* stream);
+
 /* ocnn_conv_gather for sparse tables (few of the K slots of a row hold a neighbour, as on the
  * non-empty nodes of a deep level): the work follows the (row, neighbour) pairs.  On top of
  * the tile plan (uptr, urows) it takes the pair plan of the table: the slots in an order

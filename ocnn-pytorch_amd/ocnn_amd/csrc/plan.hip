@@ -1,7 +1,10 @@
 // Tile plan of a neighbour table: for every tile of kPlanRows consecutive table
 // rows, the sorted list of distinct rows the tile reads (so a kernel can stage
 // each of them once in LDS) and, per table entry, its position in that list.
+#include <algorithm>
+
 #include "common.hpp"
+#include "mma.hpp"
 
 namespace ocnn {
 
@@ -171,6 +174,59 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
   }
 }
 
+// Pair plan of a table, on top of its tile plan: per (tile, slot) the rows of the tile that
+// have a neighbour, in blocks of 16 entries (position of the neighbour in the tile's list
+// | where the row's sums live in the pair-plan gather kernel << 16).  One wave per (tile,
+// slot in plan order); mode 0 counts the blocks, mode 1 writes the entries and fills the
+// last block up.  slot_count: pairs per slot of the whole table (mode 0, optional).
+__global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles, int K,
+                                 const int32_t* __restrict__ order, int mode, int32_t* __restrict__ nblk,
+                                 const int32_t* __restrict__ cptr, uint32_t* __restrict__ ent) {
+  const int lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);   // tile * K + j
+  if (item >= tiles * K) return;
+  const int64_t tile = item / K;
+  const int j = (int)(item - tile * K);
+  const int k = order ? order[j] : j;
+  const uint16_t* p = loc + (tile * K + k) * kPlanRows;
+  const uint32_t l0 = p[lane], l1 = p[lane + 64];
+  const unsigned long long m0 = __ballot(l0 != 0), m1 = __ballot(l1 != 0);
+  const int n0 = __popcll(m0), n = n0 + __popcll(m1);
+  if (mode == 0) {
+    if (lane == 0) nblk[item] = (n + 15) >> 4;
+    return;
+  }
+  uint32_t* e = ent + (int64_t)cptr[item] * 16;
+  const unsigned long long below = (1ull << lane) - 1ull;
+  auto entry = [](uint32_t pos, int r) { return pos | ((uint32_t)(128 * r + 16 * (r & 7)) << 16); };
+  if (l0 != 0) e[__popcll(m0 & below)] = entry(l0, lane);
+  if (l1 != 0) e[n0 + __popcll(m1 & below)] = entry(l1, lane + 64);
+  const int padded = (n + 15) & ~15;
+  if (n + lane < padded) e[n + lane] = entry(0u, kPlanRows);                 // the zero row, to a spare row
+}
+
+__global__ void pair_plan_slot_count_kernel(const uint16_t* __restrict__ loc, int64_t tiles, int K,
+                                            unsigned long long* __restrict__ slot_count) {
+  // one workgroup per slot: the sum over all tiles in a fixed order
+  __shared__ unsigned long long s_part[256];
+  const int k = blockIdx.x;
+  unsigned long long acc = 0;
+  for (int64_t t = threadIdx.x; t < tiles * (kPlanRows / 8); t += blockDim.x) {
+    const int64_t tile = t / (kPlanRows / 8);
+    const int c = (int)(t - tile * (kPlanRows / 8));
+    const u32x4 v = *(const u32x4*)(loc + (tile * K + k) * kPlanRows + 8 * c);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc += ((v[i] & 0xffffu) != 0) + ((v[i] >> 16) != 0);
+  }
+  s_part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) s_part[threadIdx.x] += s_part[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) slot_count[k] = s_part[0];
+}
+
 }  // namespace ocnn
 
 using namespace ocnn;
@@ -195,4 +251,52 @@ extern "C" int ocnn_tile_plan_count(const int32_t* table, int64_t rows, int K, i
 extern "C" int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
                                    int32_t* urows, uint16_t* loc, void* stream) {
   return plan_launch(table, rows, K, 1, nullptr, uptr, urows, loc, stream);
+}
+
+extern "C" int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,
+                                          void* stream) {
+  OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 24), "pair_plan: bad shape");
+  hipLaunchKernelGGL(pair_plan_slot_count_kernel, dim3((unsigned)K), dim3(256), 0, (hipStream_t)stream, loc,
+                     tiles, K, (unsigned long long*)slot_count);
+  return check_launch("pair_plan_slot_counts");
+}
+
+extern "C" int ocnn_pair_plan_order(int K, const int64_t* slot_count, int max_slots, int32_t* order,
+                                    int* n_first) {
+  OCNN_REQUIRE(K >= 1 && K <= 27 && max_slots >= 1 && 2 * max_slots >= K, "pair_plan_order: bad arguments");
+  // slots to the two groups: largest first, each to the lighter group that still has room
+  int idx[27];
+  for (int k = 0; k < K; ++k) idx[k] = k;
+  std::stable_sort(idx, idx + K, [&](int a, int b) { return slot_count[a] > slot_count[b]; });
+  int grp[2][27], cnt[2] = {0, 0};
+  int64_t load[2] = {0, 0};
+  for (int i = 0; i < K; ++i) {
+    int g = load[0] <= load[1] ? 0 : 1;
+    if (cnt[g] >= max_slots) g = 1 - g;
+    grp[g][cnt[g]++] = idx[i];
+    load[g] += slot_count[idx[i]];
+  }
+  for (int i = 0; i < cnt[0]; ++i) order[i] = grp[0][i];
+  for (int i = 0; i < cnt[1]; ++i) order[cnt[0] + i] = grp[1][i];
+  *n_first = cnt[0];
+  return OCNN_OK;
+}
+
+static int pair_plan_launch(const uint16_t* loc, int64_t tiles, int K, const int32_t* order, int mode,
+                            int32_t* nblk, const int32_t* cptr, uint32_t* ent, void* stream) {
+  OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 24), "pair_plan: bad shape");
+  if (tiles == 0) return OCNN_OK;
+  hipLaunchKernelGGL(pair_plan_kernel, dim3((unsigned)cdiv(tiles * K, 4)), dim3(256), 0, (hipStream_t)stream, loc,
+                     tiles, K, order, mode, nblk, cptr, ent);
+  return check_launch("pair_plan");
+}
+
+extern "C" int ocnn_pair_plan_count(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
+                                    int32_t* nblk, void* stream) {
+  return pair_plan_launch(loc, tiles, K, slot_order, 0, nblk, nullptr, nullptr, stream);
+}
+
+extern "C" int ocnn_pair_plan_fill(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
+                                   const int32_t* cptr, uint32_t* ent, void* stream) {
+  return pair_plan_launch(loc, tiles, K, slot_order, 1, nullptr, cptr, ent, stream);
 }

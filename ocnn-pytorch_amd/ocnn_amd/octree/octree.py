@@ -148,46 +148,33 @@ class TilePlan:
 
 
 class PairPlan:
-  """Blocks of 16 entries per (tile, slot), the slots dealt to two groups of about equal
-  numbers of pairs.  Entry: position of the input row in the tile's list + 1, | (128 r +
-  16 (r & 7)) << 16 for row r of the tile; blocks are filled up with position 0, r = 128."""
+  """Blocks of 16 (row, neighbour) pairs per (tile, slot) of a table, the slots dealt to two
+  groups of about equal numbers of pairs (see ocnn_pair_plan_* in the C ABI)."""
 
   def __init__(self, plan: TilePlan):
+    import ctypes
     L = _lib.lib()
-    tiles, K, R = plan.loc.shape
+    tiles, K, _ = plan.loc.shape
     dev = plan.loc.device
-    loc = plan.loc.to(torch.int32) & 0xffff                       # (tiles, K, R), 0 = empty
-    valid = loc > 0
-    per_slot = valid.sum((0, 2)).tolist()
-    # slots to the two groups: largest first, each to the lighter group that still has room
-    cap = L.ocnn_conv_gather_sparse_max_slots(K)
-    groups, load = ([], []), [0, 0]
-    for k in sorted(range(K), key=lambda k: -per_slot[k]):
-      g = 0 if load[0] <= load[1] else 1
-      if len(groups[g]) >= cap:
-        g = 1 - g
-      groups[g].append(k)
-      load[g] += per_slot[k]
-    order = groups[0] + groups[1]
-    self.n_first = len(groups[0])
-    self.order = torch.tensor(order, dtype=torch.int32, device=dev)
-    idx = self.order.long()
-    loc, valid = loc[:, idx, :], valid[:, idx, :]
-    count = valid.sum(2)                                          # (tiles, K)
-    nblk = (count + 15) // 16
-    cptr = torch.zeros(tiles * K + 1, dtype=torch.int64, device=dev)
-    cptr[1:] = torch.cumsum(nblk.reshape(-1), 0)
-    self.n_blocks = int(cptr[-1])
-    self.max_blocks = int(nblk.sum(1).max()) if tiles > 0 else 0
-    acc = torch.arange(R + 1, dtype=torch.int32, device=dev)
-    acc = (128 * acc + 16 * (acc & 7)) << 16                      # where a row's sums live in the kernel
-    ent = torch.full((max(self.n_blocks, 1) * 16,), int(acc[R]), dtype=torch.int32, device=dev)   # filling
-    slot = torch.cumsum(valid, 2) - 1                             # place of a pair in its list
-    dest = cptr[:-1].view(tiles, K, 1) * 16 + slot
-    val = loc | acc[:R].view(1, 1, R)
-    ent[dest[valid]] = val[valid]
-    self.ent = ent
-    self.cptr = cptr.to(torch.int32)
+    st = _lib.stream()
+    counts = torch.zeros(K, dtype=torch.int64, device=dev)
+    _lib.check(L.ocnn_pair_plan_slot_counts(_lib.ptr(plan.loc), tiles, K, _lib.ptr(counts), st))
+    per_slot = (ctypes.c_int64 * K)(*counts.tolist())
+    order = (ctypes.c_int32 * K)()
+    n_first = ctypes.c_int(0)
+    _lib.check(L.ocnn_pair_plan_order(K, ctypes.addressof(per_slot), L.ocnn_conv_gather_sparse_max_slots(K),
+                                      ctypes.addressof(order), ctypes.addressof(n_first)))
+    self.n_first = n_first.value
+    self.order = torch.tensor(list(order), dtype=torch.int32, device=dev)
+    nblk = torch.zeros(max(tiles * K, 1), dtype=torch.int32, device=dev)
+    _lib.check(L.ocnn_pair_plan_count(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.order), _lib.ptr(nblk), st))
+    self.cptr = torch.zeros(tiles * K + 1, dtype=torch.int32, device=dev)
+    self.cptr[1:] = torch.cumsum(nblk[:tiles * K], 0)
+    self.n_blocks, self.max_blocks = (int(v) for v in torch.stack(
+        [self.cptr[-1], nblk[:tiles * K].view(tiles, K).sum(1).max().int()]).tolist()) if tiles > 0 else (0, 0)
+    self.ent = torch.empty(max(self.n_blocks, 1) * 16, dtype=torch.int32, device=dev)
+    _lib.check(L.ocnn_pair_plan_fill(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.order), _lib.ptr(self.cptr),
+                                     _lib.ptr(self.ent), st))
 
 
 class Octree:

@@ -111,3 +111,29 @@ def test_points_normalize_and_merge():
   assert m.batch_id.dtype == torch.float32
   with pytest.raises(AssertionError):
     Points(torch.zeros(2, 2))
+
+
+def test_pair_plan_slot_order():
+  """ocnn_pair_plan_order (host only): every slot once, at most max_slots per group, the
+  heavier group no more than the largest slot above the lighter one."""
+  L = _lib.lib()
+  rng = np.random.default_rng(3)
+  for K in (1, 3, 8, 9, 27):
+    cap = L.ocnn_conv_gather_sparse_max_slots(K)
+    assert 2 * cap >= K
+    for trial in range(20):
+      counts = rng.integers(0, 1000, size=K).astype(np.int64)
+      if trial % 3 == 0:
+        counts[rng.integers(0, K)] = 50000                  # one dominant slot (the centre)
+      order = (ctypes.c_int32 * K)()
+      n_first = ctypes.c_int(0)
+      c = (ctypes.c_int64 * K)(*counts.tolist())
+      assert L.ocnn_pair_plan_order(K, ctypes.addressof(c), cap, ctypes.addressof(order),
+                                    ctypes.addressof(n_first)) == 0
+      order = list(order)
+      assert sorted(order) == list(range(K))
+      n0 = n_first.value
+      assert 0 <= n0 <= cap and K - n0 <= cap
+      a, b = counts[order[:n0]].sum(), counts[order[n0:]].sum()
+      if K <= cap:                                          # no group ever ran out of room
+        assert abs(int(a) - int(b)) <= counts.max()

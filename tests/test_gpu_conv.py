@@ -538,6 +538,43 @@ def _gather_sparse(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
   return out
 
 
+@pytest.mark.parametrize('K', [27, 8, 3, 1])
+def test_pair_plan_lists(K):
+  """The pair plan against its definition, from the tile plan's positions: per (tile, slot in
+  plan order) the rows with a neighbour in ascending order, entry = position | (128 r +
+  16 (r & 7)) << 16, lists filled up to whole blocks of 16 with position 0 and r = 128."""
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(K)
+  table = _local_table(128 * 9 + 50, 900, K, g, empty=0.8)
+  if K > 2:
+    table[:, 1] = -1
+  plan = TilePlan(table.to(DEV))
+  pp = plan.pairs()
+  loc = plan.loc.cpu().numpy().astype(np.int64) & 0xffff      # (tiles, K, 128)
+  tiles = loc.shape[0]
+  order = pp.order.cpu().numpy()
+  cptr = pp.cptr.cpu().numpy()
+  ent = pp.ent.cpu().numpy().astype(np.int64) & 0xffffffff
+  assert sorted(order.tolist()) == list(range(K))
+  per_slot = (loc > 0).sum((0, 2))
+  assert abs(int(per_slot[order[:pp.n_first]].sum()) - int(per_slot[order[pp.n_first:]].sum())) <= per_slot.max()
+  filler = (128 * 128) << 16
+  at = 0
+  most = 0
+  for t in range(tiles):
+    blocks = 0
+    for j in range(K):
+      assert cptr[t * K + j] == at
+      rows = np.nonzero(loc[t, order[j]])[0]
+      want = [int(loc[t, order[j], r]) | ((128 * r + 16 * (r & 7)) << 16) for r in rows]
+      want += [filler] * (-len(want) % 16)
+      assert ent[16 * at:16 * at + len(want)].tolist() == want
+      at += len(want) // 16
+      blocks += len(want) // 16
+    most = max(most, blocks)
+  assert cptr[tiles * K] == at == pp.n_blocks and most == pp.max_blocks
+
+
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('K,cin,cout', [(27, 96, 96), (27, 128, 96), (27, 32, 64), (27, 64, 32), (9, 96, 128),
                                         (8, 128, 160), (8, 32, 32), (3, 64, 96), (1, 32, 32)])
