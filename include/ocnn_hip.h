@@ -271,6 +271,24 @@ int ocnn_conv_gather_sparse(int dtype, const void* in, int64_t rows_in, const in
                             const void* bias, void* out, void* workspace, int64_t workspace_bytes,
                             void* stream);
 
+/* Weight gradient over the pair plan of a sparse table (the counterpart of
+ * ocnn_conv_gather_sparse; same sums as ocnn_conv_wgrad):
+ *   D[k][i][j] = sum over the table rows r with table[r][k] >= 0 of a[table[r][k]][i] * b[r][j]
+ * a: (rows_a, ca), the rows the table points at; b: (rows_b, cb), the rows of the table,
+ * cb <= 96; ca, cb multiples of 32; f16 / bf16.  out: (K, ca, cb) with a_major, (K, cb, ca)
+ * without.  slot_count and slot_order are the HOST arrays of ocnn_pair_plan_slot_counts /
+ * ocnn_pair_plan_order.  A workgroup keeps the fp32 sums of all slots for 32 a-channels in
+ * registers over a range of tiles; the ranges are added in a fixed order. */
+int ocnn_conv_wgrad_sparse_supported(int dtype, int64_t rows_a, int64_t rows_b, int K, int ca, int cb,
+                                     int plan_max_distinct);
+int64_t ocnn_conv_wgrad_sparse_workspace_bytes(int64_t rows_b, int K, int ca, int cb);
+int ocnn_conv_wgrad_sparse(int dtype, const void* a, int64_t rows_a, int ca, const void* b,
+                           int64_t rows_b, int cb, const int32_t* uptr, const int32_t* urows,
+                           int plan_max_distinct, int64_t plan_total, const int32_t* cptr,
+                           const uint32_t* ent, int64_t n_blocks, const int64_t* slot_count,
+                           const int32_t* slot_order, int K, int a_major, void* out, void* workspace,
+                           int64_t workspace_bytes, void* stream);
+
 /* out (rows, cout) = in (rows, cin) W (+ bias): ocnn_conv_gather with the one-slot identity
  * table, the form that the 2x2x2 stride-2 layers over all nodes take on the (parents, 8 C)
  * view of the children (ocnn/nn/octree_conv.py:115-168 with neigh[p] = 8p .. 8p+7).

@@ -22,6 +22,7 @@ SOURCES = {
     'conv_rw.hip': [],
     'conv_wide.hip': [],
     'conv_sparse.hip': [],
+    'wgrad_sparse.hip': [],
     'dense_rw.hip': [],
     'dw_planned.hip': [],
     'wgrad_planned.hip': [],

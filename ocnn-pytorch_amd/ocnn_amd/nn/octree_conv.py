@@ -11,6 +11,7 @@ table is centrally symmetric (stride 1, every kernel but 2x2x2) and through
 the inverse table otherwise, so no atomics are involved anywhere.
 """
 
+import ctypes
 from typing import List
 
 import torch
@@ -50,7 +51,7 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
     Wk = W.view(K, cout, cin) if transposed else W.view(K, cin, cout)
     pad_w = (0, cin_p - cin, 0, cout_p - cout) if transposed else (0, cout_p - cout, 0, cin_p - cin)
     out = conv_gather(F.pad(data, (0, cin_p - cin)), rows_in, table, F.pad(Wk, pad_w), cout_p,
-                      transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), None)
+                      transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), plan)
     return out[:, :cout].contiguous()
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
   code = _lib.dtype_code(data)
@@ -115,7 +116,7 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
   assert g.shape[0] == rows and x.dtype == g.dtype and table.dtype == torch.int32
   if rows >= PAD_MIN_ROWS and (ca % 32 or cb % 32) and x.dtype in _lib.DTYPE_CODE:
     ca_p, cb_p = -(-ca // 32) * 32, -(-cb // 32) * 32
-    gw = conv_wgrad(F.pad(x, (0, ca_p - ca)), F.pad(g, (0, cb_p - cb)), table, out_transposed, None)
+    gw = conv_wgrad(F.pad(x, (0, ca_p - ca)), F.pad(g, (0, cb_p - cb)), table, out_transposed, plan)
     return (gw[:, :cb, :ca] if out_transposed else gw[:, :ca, :cb]).contiguous()
   shape = (K, cb, ca) if out_transposed else (K, ca, cb)
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
@@ -125,6 +126,18 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
     ws = _lib.workspace(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(ca, cb), x.device)
     _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x), _lib.ptr(g), rows, ca, cb, int(out_transposed),
                                           _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    return gw
+  # (32 x 32 and 64 x 64 have kernels of their own on the tile plan that are faster still)
+  if (plan is not None and USE_SPARSE and plan.occupancy <= SPARSE_MAX_OCCUPANCY and rows >= SPARSE_MIN_ROWS and
+      not (ca == cb and ca in (32, 64)) and
+      L.ocnn_conv_wgrad_sparse_supported(code, x.shape[0], rows, K, ca, cb, plan.umax)):
+    pp = plan.pairs()
+    ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, K, ca, cb), x.device)
+    _lib.check(L.ocnn_conv_wgrad_sparse(
+        code, _lib.ptr(x), x.shape[0], ca, _lib.ptr(g), rows, cb, _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
+        plan.umax, plan.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks,
+        ctypes.addressof(pp.slot_count_host), ctypes.addressof(pp.order_host), K, int(not out_transposed),
+        _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw
   if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
                                                               plan.umax):
@@ -139,6 +152,33 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
   _lib.check(L.ocnn_conv_wgrad(
       _lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
       int(out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  return gw
+
+
+def conv_wgrad_inverse(x, g, plan_t, out_transposed=False):
+  """The same sums as conv_wgrad, taken over the INVERSE table (row j, slot k -> the row i
+  with table[i][k] == j; plan_t is its tile plan): gW[k] = sum_j x[j]^T (x) g[Tt[j,k]].  For
+  tables in which every row is pointed at from one slot only (2x2x2 stride 2: a node has one
+  parent) the inverse has 1 / K of its entries set and tiles of few distinct rows, which is
+  what the pair-plan kernel is made for.  None when the kernel does not take the shape."""
+  _lib.require_gpu(x, g)
+  L = _lib.lib()
+  x, g = x.contiguous(), g.contiguous()
+  K = plan_t.K
+  cx, cg = x.shape[1], g.shape[1]
+  code = _lib.DTYPE_CODE.get(x.dtype, -1)
+  if not (USE_SPARSE and plan_t.rows == x.shape[0] and plan_t.rows >= SPARSE_MIN_ROWS and
+          plan_t.occupancy <= SPARSE_MAX_OCCUPANCY and x.dtype == g.dtype and
+          L.ocnn_conv_wgrad_sparse_supported(code, g.shape[0], x.shape[0], K, cg, cx, plan_t.umax)):
+    return None
+  pp = plan_t.pairs()
+  gw = torch.empty((K, cg, cx) if out_transposed else (K, cx, cg), dtype=x.dtype, device=x.device)
+  ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(x.shape[0], K, cg, cx), x.device)
+  _lib.check(L.ocnn_conv_wgrad_sparse(
+      code, _lib.ptr(g), g.shape[0], cg, _lib.ptr(x), x.shape[0], cx, _lib.ptr(plan_t.uptr),
+      _lib.ptr(plan_t.urows), plan_t.umax, plan_t.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks,
+      ctypes.addressof(pp.slot_count_host), ctypes.addressof(pp.order_host), K, int(out_transposed),
+      _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
   return gw
 
 
@@ -222,6 +262,8 @@ class OctreeConvBase:
     """Tile plan for the staged kernel, when the shape can use it."""
     L, code = _lib.lib(), _lib.DTYPE_CODE.get(data.dtype, -1)
     rows = data.shape[0]
+    if self.neigh.shape[0] >= PAD_MIN_ROWS:               # odd channel counts run zero-padded
+      cin, cout = -(-cin // 32) * 32, -(-cout // 32) * 32
     if not (L.ocnn_conv_gather_planned_supported(code, rows, cin, cout) or
             L.ocnn_conv_gather_rw_supported(code, rows, self.kdim, cin, cout, 0) or
             L.ocnn_conv_gather_wide_supported(code, rows, self.kdim, cin, cout, 0) or
@@ -275,6 +317,13 @@ class OctreeConvBase:
       gw = conv_wgrad(data.view(P, 8 * self.in_conv), grad, self._identity(P, data.device), False,
                       None, dense=True).view(8, self.in_conv, self.out_conv)
       return gw.transpose(1, 2).contiguous() if out_transposed else gw
+    if self.stride == 2 and self.kernel == '222' and self.neigh.shape[0] >= SPARSE_MIN_ROWS // 8 and \
+        _lib.lib().ocnn_conv_wgrad_sparse_supported(_lib.DTYPE_CODE.get(data.dtype, -1), grad.shape[0],
+                                                    data.shape[0], self.kdim, grad.shape[1], data.shape[1], 0):
+      plan_t = self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, True, self.fine_h)
+      gw = conv_wgrad_inverse(data, grad, plan_t, out_transposed)
+      if gw is not None:
+        return gw
     plan = self._plan(data, self.in_conv, self.out_conv)
     return conv_wgrad(data, grad, self.neigh, out_transposed, plan)
 

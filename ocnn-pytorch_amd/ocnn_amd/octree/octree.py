@@ -165,6 +165,7 @@ class PairPlan:
     _lib.check(L.ocnn_pair_plan_order(K, ctypes.addressof(per_slot), L.ocnn_conv_gather_sparse_max_slots(K),
                                       ctypes.addressof(order), ctypes.addressof(n_first)))
     self.n_first = n_first.value
+    self.slot_count_host, self.order_host = per_slot, order       # (kept alive: the C ABI reads them)
     self.order = torch.tensor(list(order), dtype=torch.int32, device=dev)
     nblk = torch.zeros(max(tiles * K, 1), dtype=torch.int32, device=dev)
     _lib.check(L.ocnn_pair_plan_count(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.order), _lib.ptr(nblk), st))

@@ -614,6 +614,81 @@ def test_sparse_gather_kernel(dtype, K, cin, cout):
       assert rel_err(got, want) < TOL[dtype]
 
 
+def _wgrad_sparse(x, g, table, plan, transposed):
+  """ocnn_conv_wgrad_sparse through the C ABI."""
+  import ctypes
+  L = _lib.lib()
+  rows, K = table.shape
+  ca, cb = x.shape[1], g.shape[1]
+  code = _lib.dtype_code(x)
+  assert L.ocnn_conv_wgrad_sparse_supported(code, x.shape[0], rows, K, ca, cb, plan.umax)
+  pp = plan.pairs()
+  gw = torch.empty((K, cb, ca) if transposed else (K, ca, cb), dtype=x.dtype, device=x.device)
+  ws = torch.empty(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, K, ca, cb), dtype=torch.uint8, device=x.device)
+  _lib.check(L.ocnn_conv_wgrad_sparse(
+      code, _lib.ptr(x), x.shape[0], ca, _lib.ptr(g), rows, cb, _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax,
+      plan.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, ctypes.addressof(pp.slot_count_host),
+      ctypes.addressof(pp.order_host), K, int(not transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(),
+      _lib.stream()))
+  return gw
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('K,ca,cb', [(27, 96, 96), (27, 128, 96), (27, 32, 64), (27, 64, 32), (27, 256, 32),
+                                     (9, 96, 64), (8, 128, 96), (8, 32, 32), (3, 64, 96), (1, 32, 32)])
+def test_sparse_wgrad_kernel(dtype, K, ca, cb):
+  """Weight gradient over the pair plan (all slots of 32 x-channels in the registers of a
+  workgroup, heavy slots cut into units, per-range sums added in a fixed order), at several
+  occupancies incl. a slot and a tile without pairs and ragged row counts, both output
+  layouts, against the oracle; twice, bit-identical.  The last x row holds NaN and is never
+  read."""
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(5 * K + ca + cb)
+  for rows, rows_in, empty in [(1000, 1000, 0.85), (130, 150, 0.5), (128 * 40 + 1, 3000, 0.9), (128 * 300 + 77, 40000, 0.8)]:
+    say('sparse wgrad', dtype, K, ca, cb, rows, rows_in, empty)
+    table = _local_table(rows, rows_in - 1, K, g, empty=empty)
+    if K > 2:
+      table[:, 1] = -1
+      table[256:384] = -1
+    if K == 27:
+      table[:, 13] = torch.arange(rows, dtype=torch.int32).clamp_(max=rows_in - 2)   # a slot with all the rows
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    t64 = table.numpy().astype(np.int64)
+    x = torch.randn(rows_in, ca, generator=g).to(dtype)
+    gr = (torch.randn(rows, cb, generator=g) / (rows * (1 - empty)) ** 0.5).to(dtype)
+    xn = x.clone()
+    xn[-1] = float('nan')
+    want = C.weight_gemm(f64(x), f64(gr), t64)
+    for transposed in (False, True):
+      got = _wgrad_sparse(xn.to(DEV), gr.to(DEV), tg, plan, transposed)
+      again = _wgrad_sparse(xn.to(DEV), gr.to(DEV), tg, plan, transposed)
+      assert torch.equal(got, again)
+      assert rel_err(got, want.transpose(0, 2, 1) if transposed else want) < TOL[dtype]
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_layers_on_the_sparse_kernels(medium, dtype):
+  """Whole layers (module forward + backward against the oracle) with the thresholds of the
+  Python layer lowered so that the pair-plan kernels run on the test octree: 3x3x3 and axis
+  kernels on non-empty nodes (gather, data gradient through the mirrored slots, weight
+  gradient), 2x2x2 stride-2 conv / deconv (gathers over the table and its inverse, weight
+  gradient over the inverse table)."""
+  conv_mod = sys.modules['ocnn_amd.nn.octree_conv']
+  keep = (conv_mod.SPARSE_MIN_ROWS, conv_mod.SPARSE_MAX_OCCUPANCY)
+  conv_mod.SPARSE_MIN_ROWS, conv_mod.SPARSE_MAX_OCCUPANCY = 0, 1.0
+  try:
+    for kind, ks, stride, cin, cout in [('conv', [3], 1, 96, 96), ('conv', [3], 1, 128, 96), ('conv', [3, 3, 1], 1, 32, 96),
+                                        ('conv', [2], 2, 96, 128), ('conv', [2], 2, 32, 64), ('deconv', [2], 2, 128, 96),
+                                        ('deconv', [2], 2, 96, 32), ('deconv', [3], 1, 96, 64)]:
+      depth = 6 if kind == 'deconv' and stride == 2 else 7
+      say('layers on the sparse kernels', dtype, kind, ks, stride, cin, cout)
+      errs = run_layer(kind, medium, depth, ks, stride, True, cin, cout, dtype)
+      assert max(errs.values()) < TOL[dtype], (dtype, kind, ks, stride, cin, cout, errs)
+  finally:
+    conv_mod.SPARSE_MIN_ROWS, conv_mod.SPARSE_MAX_OCCUPANCY = keep
+
+
 def test_sparse_gather_large_tiles():
   """Tiles near the staging limits of the pair-plan kernel (many distinct rows: one
   workgroup per CU, the wider row-number buffers) and the refusal beyond them."""
