@@ -227,67 +227,66 @@ int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint
                           void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Pair plan of a table, on top of its tile plan (loc: tiles x K x ocnn_tile_plan_rows()):
- * what ocnn_conv_gather_sparse walks over.  No counterpart in the reference.
+ * what ocnn_conv_gather_sparse and ocnn_conv_wgrad_sparse walk over.  It holds, per tile and
+ * LIST, the rows that have a neighbour, in blocks of 16 pairs.  A list is a slot of the
+ * table, or - for a slot with many pairs, like the centre of a 3x3x3 table - the rows
+ * r0 .. r1 - 1 of the tiles of that slot: list = slot | r0 << 8 | (r1 - 1) << 16.  No
+ * counterpart in the reference.
  *   slot_counts: slot_count[k] (device, K x int64) = table entries of slot k that hold a row;
- *   order (host only): deals the slots to two groups of about equal numbers of pairs, at
- *          most max_slots each (ocnn_conv_gather_sparse_max_slots(K)); order[0 .. n_first)
- *          = group 0, the rest group 1.  slot_count and order are host arrays here;
- *   count: nblk[tile * K + j] = blocks of 16 pairs of slot slot_order[j] in the tile
- *          (slot_order: device array, or NULL for 0 .. K - 1);
- *   fill : cptr (tiles * K + 1) = exclusive prefix sum of nblk, made by the caller;
+ *   lists (host only, host arrays): cuts heavy slots by rows, deals the lists (at most 32)
+ *          to four groups of at most 8 with about equal numbers of pairs; lists in group
+ *          order, list_count[j] = pairs of list j (estimated for cut slots), group g = lists
+ *          group_bounds[g] .. group_bounds[g + 1] - 1;
+ *   count: nblk[tile * n_lists + j] = blocks of 16 pairs of list j in the tile (lists: a
+ *          device copy of the array);
+ *   fill : cptr (tiles * n_lists + 1) = exclusive prefix sum of nblk, made by the caller;
  *          ent (16 entries per block): position of the pair's input row in the tile's list
- *          + 1, | (128 r + 16 (r & 7)) << 16 for row r of the tile; the last block of a
- *          list is filled up with position 0, r = 128. */
+ *          of rows + 1, | (128 r + 16 (r & 7)) << 16 for row r of the tile; the last block
+ *          of a list is filled up with position 0, r = 128. */
 int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,
                                void* stream);
-int ocnn_pair_plan_order(int K, const int64_t* slot_count, int max_slots, int32_t* order,
-                         int* n_first);
-int ocnn_pair_plan_count(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
-                         int32_t* nblk, void* stream);
-int ocnn_pair_plan_fill(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
-                        const int32_t* cptr, uint32_t* ent, void* stream);
+int ocnn_pair_plan_lists(int K, const int64_t* slot_count, int32_t* lists, int64_t* list_count,
+                         int32_t* group_bounds, int* n_lists);
+int ocnn_pair_plan_count(const uint16_t* loc, int64_t tiles, int K, const int32_t* lists,
+                         int n_lists, int32_t* nblk, void* stream);
+int ocnn_pair_plan_fill(const uint16_t* loc, int64_t tiles, int K, const int32_t* lists,
+                        int n_lists, const int32_t* cptr, uint32_t* ent, void* stream);
 
 /* ocnn_conv_gather for sparse tables (few of the K slots of a row hold a neighbour, as on the
  * non-empty nodes of a deep level): the work follows the (row, neighbour) pairs.  On top of
- * the tile plan (uptr, urows) it takes the pair plan of the table: the slots in an order
- * slot_order (device array of K slot numbers; the first n_first of them form slot group 0,
- * the others group 1, at most ocnn_conv_gather_sparse_max_slots(K) each - balance the pairs),
- * cptr (tiles * K + 1 block offsets, tile-major, slots in that order) and ent (16 entries per
- * block: position of the input row in the tile's list + 1, | (128 r + 16 (r & 7)) << 16 for
- * row r of the tile; blocks are filled up with position 0, r = 128); max_blocks = the largest
- * number of blocks of one tile.  Weights stay in registers, a workgroup serves 32 output
- * channels over many tiles, results are added in a fixed order.  f16 / bf16, cin in
- * {32, 64, 96, 128}, cout % 32 == 0, K <= 27; same result as ocnn_conv_gather.
- * workspace: K * cin * cout * 2 bytes. */
+ * the tile plan (uptr, urows) it takes the pair plan of the table (cptr, ent, n_blocks = all
+ * blocks, max_blocks = the most blocks of one tile, lists as a device array, group_bounds as
+ * the host array of ocnn_pair_plan_lists).  Weights stay in registers, a workgroup serves 32
+ * output channels over many tiles, results are added in a fixed order.  f16 / bf16, cin in
+ * {32, 64, 96, 128}, cout % 32 == 0, K <= 27; same result as ocnn_conv_gather. */
 int ocnn_conv_gather_sparse_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                       int plan_max_distinct);
-int ocnn_conv_gather_sparse_max_slots(int K);
+int64_t ocnn_conv_gather_sparse_workspace_bytes(int cin, int cout);
 int ocnn_conv_gather_sparse(int dtype, const void* in, int64_t rows_in, const int32_t* uptr,
                             const int32_t* urows, int plan_max_distinct, int64_t plan_total,
                             const int32_t* cptr, const uint32_t* ent, int64_t n_blocks,
-                            int max_blocks, const int32_t* slot_order, int n_first,
-                            int64_t rows_out, int K,
-                            const void* w, int cin, int cout, int w_transposed, int reverse_slots,
-                            const void* bias, void* out, void* workspace, int64_t workspace_bytes,
-                            void* stream);
+                            int max_blocks, const int32_t* lists, int n_lists,
+                            const int32_t* group_bounds, int64_t rows_out, int K, const void* w,
+                            int cin, int cout, int w_transposed, int reverse_slots, const void* bias,
+                            void* out, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Weight gradient over the pair plan of a sparse table (the counterpart of
  * ocnn_conv_gather_sparse; same sums as ocnn_conv_wgrad):
  *   D[k][i][j] = sum over the table rows r with table[r][k] >= 0 of a[table[r][k]][i] * b[r][j]
  * a: (rows_a, ca), the rows the table points at; b: (rows_b, cb), the rows of the table,
  * cb <= 96; ca, cb multiples of 32; f16 / bf16.  out: (K, ca, cb) with a_major, (K, cb, ca)
- * without.  slot_count and slot_order are the HOST arrays of ocnn_pair_plan_slot_counts /
- * ocnn_pair_plan_order.  A workgroup keeps the fp32 sums of all slots for 32 a-channels in
- * registers over a range of tiles; the ranges are added in a fixed order. */
+ * without.  lists and list_count are the HOST arrays of ocnn_pair_plan_lists.  A workgroup
+ * keeps the fp32 sums of all lists for 32 a-channels in registers over a range of tiles; the
+ * ranges are added in a fixed order. */
 int ocnn_conv_wgrad_sparse_supported(int dtype, int64_t rows_a, int64_t rows_b, int K, int ca, int cb,
                                      int plan_max_distinct);
-int64_t ocnn_conv_wgrad_sparse_workspace_bytes(int64_t rows_b, int K, int ca, int cb);
+int64_t ocnn_conv_wgrad_sparse_workspace_bytes(int64_t rows_b, int ca, int cb);
 int ocnn_conv_wgrad_sparse(int dtype, const void* a, int64_t rows_a, int ca, const void* b,
                            int64_t rows_b, int cb, const int32_t* uptr, const int32_t* urows,
                            int plan_max_distinct, int64_t plan_total, const int32_t* cptr,
-                           const uint32_t* ent, int64_t n_blocks, const int64_t* slot_count,
-                           const int32_t* slot_order, int K, int a_major, void* out, void* workspace,
-                           int64_t workspace_bytes, void* stream);
+                           const uint32_t* ent, int64_t n_blocks, const int32_t* lists,
+                           const int64_t* list_count, int n_lists, int K, int a_major, void* out,
+                           void* workspace, int64_t workspace_bytes, void* stream);
 
 /* out (rows, cout) = in (rows, cin) W (+ bias): ocnn_conv_gather with the one-slot identity
  * table, the form that the 2x2x2 stride-2 layers over all nodes take on the (parents, 8 C)

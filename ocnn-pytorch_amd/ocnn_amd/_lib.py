@@ -50,17 +50,17 @@ SIGNATURES = {
                                  _p, _l, _p]),
     'ocnn_conv_gather_wide_supported': (_i, [_i, _l, _i, _i, _i, _i]),
     'ocnn_pair_plan_slot_counts': (_i, [_p, _l, _i, _p, _p]),
-    'ocnn_pair_plan_order': (_i, [_i, _p, _i, _p, _p]),
-    'ocnn_pair_plan_count': (_i, [_p, _l, _i, _p, _p, _p]),
-    'ocnn_pair_plan_fill': (_i, [_p, _l, _i, _p, _p, _p, _p]),
+    'ocnn_pair_plan_lists': (_i, [_i, _p, _p, _p, _p, _p]),
+    'ocnn_pair_plan_count': (_i, [_p, _l, _i, _p, _i, _p, _p]),
+    'ocnn_pair_plan_fill': (_i, [_p, _l, _i, _p, _i, _p, _p, _p]),
     'ocnn_conv_wgrad_sparse_supported': (_i, [_i, _l, _l, _i, _i, _i, _i]),
-    'ocnn_conv_wgrad_sparse_workspace_bytes': (_l, [_l, _i, _i, _i]),
-    'ocnn_conv_wgrad_sparse': (_i, [_i, _p, _l, _i, _p, _l, _i, _p, _p, _i, _l, _p, _p, _l, _p, _p, _i, _i, _p, _p,
-                                    _l, _p]),
+    'ocnn_conv_wgrad_sparse_workspace_bytes': (_l, [_l, _i, _i]),
+    'ocnn_conv_wgrad_sparse': (_i, [_i, _p, _l, _i, _p, _l, _i, _p, _p, _i, _l, _p, _p, _l, _p, _p, _i, _i, _i, _p,
+                                    _p, _l, _p]),
     'ocnn_conv_gather_sparse_supported': (_i, [_i, _l, _i, _i, _i, _i]),
-    'ocnn_conv_gather_sparse_max_slots': (_i, [_i]),
-    'ocnn_conv_gather_sparse': (_i, [_i, _p, _l, _p, _p, _i, _l, _p, _p, _l, _i, _p, _i, _l, _i, _p, _i, _i, _i, _i,
-                                     _p, _p, _p, _l, _p]),
+    'ocnn_conv_gather_sparse_workspace_bytes': (_l, [_i, _i]),
+    'ocnn_conv_gather_sparse': (_i, [_i, _p, _l, _p, _p, _i, _l, _p, _p, _l, _i, _p, _i, _p, _l, _i, _p, _i, _i, _i,
+                                     _i, _p, _p, _p, _l, _p]),
     'ocnn_conv_gather_wide': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                    _p, _l, _p]),
     'ocnn_conv_dense_supported': (_i, [_i, _l, _i, _i]),

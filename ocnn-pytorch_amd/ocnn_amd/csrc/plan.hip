@@ -2,6 +2,7 @@
 // rows, the sorted list of distinct rows the tile reads (so a kernel can stage
 // each of them once in LDS) and, per table entry, its position in that list.
 #include <algorithm>
+#include <vector>
 
 #include "common.hpp"
 #include "mma.hpp"
@@ -174,22 +175,24 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
   }
 }
 
-// Pair plan of a table, on top of its tile plan: per (tile, slot) the rows of the tile that
-// have a neighbour, in blocks of 16 entries (position of the neighbour in the tile's list
-// | where the row's sums live in the pair-plan gather kernel << 16).  One wave per (tile,
-// slot in plan order); mode 0 counts the blocks, mode 1 writes the entries and fills the
-// last block up.  slot_count: pairs per slot of the whole table (mode 0, optional).
+// Pair plan of a table, on top of its tile plan: per tile and LIST the rows that have a
+// neighbour, in blocks of 16 entries (position of the neighbour in the tile's list of rows
+// | where the row's sums live in the pair-plan gather kernel << 16).  A list is a slot, or
+// the rows r0 .. r1 - 1 of the tiles of a slot that holds many pairs (list = slot |
+// r0 << 8 | (r1 - 1) << 16).  One wave per (tile, list); mode 0 counts the blocks, mode 1
+// writes the entries and fills the last block up.
 __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles, int K,
-                                 const int32_t* __restrict__ order, int mode, int32_t* __restrict__ nblk,
+                                 const int32_t* __restrict__ lists, int nl, int mode, int32_t* __restrict__ nblk,
                                  const int32_t* __restrict__ cptr, uint32_t* __restrict__ ent) {
   const int lane = threadIdx.x & 63;
-  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);   // tile * K + j
-  if (item >= tiles * K) return;
-  const int64_t tile = item / K;
-  const int j = (int)(item - tile * K);
-  const int k = order ? order[j] : j;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);   // tile * nl + j
+  if (item >= tiles * nl) return;
+  const int64_t tile = item / nl;
+  const int32_t list = lists[(int)(item - tile * nl)];
+  const int k = list & 255, r0 = (list >> 8) & 255, r1 = ((list >> 16) & 255) + 1;
   const uint16_t* p = loc + (tile * K + k) * kPlanRows;
-  const uint32_t l0 = p[lane], l1 = p[lane + 64];
+  const uint32_t l0 = (lane >= r0 && lane < r1) ? p[lane] : 0u;
+  const uint32_t l1 = (lane + 64 >= r0 && lane + 64 < r1) ? p[lane + 64] : 0u;
   const unsigned long long m0 = __ballot(l0 != 0), m1 = __ballot(l1 != 0);
   const int n0 = __popcll(m0), n = n0 + __popcll(m1);
   if (mode == 0) {
@@ -261,42 +264,71 @@ extern "C" int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, in
   return check_launch("pair_plan_slot_counts");
 }
 
-extern "C" int ocnn_pair_plan_order(int K, const int64_t* slot_count, int max_slots, int32_t* order,
-                                    int* n_first) {
-  OCNN_REQUIRE(K >= 1 && K <= 27 && max_slots >= 1 && 2 * max_slots >= K, "pair_plan_order: bad arguments");
-  // slots to the two groups: largest first, each to the lighter group that still has room
-  int idx[27];
-  for (int k = 0; k < K; ++k) idx[k] = k;
-  std::stable_sort(idx, idx + K, [&](int a, int b) { return slot_count[a] > slot_count[b]; });
-  int grp[2][27], cnt[2] = {0, 0};
-  int64_t load[2] = {0, 0};
-  for (int i = 0; i < K; ++i) {
-    int g = load[0] <= load[1] ? 0 : 1;
-    if (cnt[g] >= max_slots) g = 1 - g;
-    grp[g][cnt[g]++] = idx[i];
-    load[g] += slot_count[idx[i]];
+extern "C" int ocnn_pair_plan_lists(int K, const int64_t* slot_count, int32_t* lists, int64_t* list_count,
+                                    int32_t* group_bounds, int* n_lists) {
+  OCNN_REQUIRE(K >= 1 && K <= 27, "pair_plan_lists: bad slot count");
+  struct List { int k, r0, r1; int64_t load; };
+  std::vector<List> all;
+  int64_t total = 0;
+  for (int k = 0; k < K; ++k) {
+    all.push_back({k, 0, kPlanRows, slot_count[k]});
+    total += slot_count[k];
   }
-  for (int i = 0; i < cnt[0]; ++i) order[i] = grp[0][i];
-  for (int i = 0; i < cnt[1]; ++i) order[cnt[0] + i] = grp[1][i];
-  *n_first = cnt[0];
+  // heavy slots (the centre of a 3x3x3 table holds a third of all pairs) are cut by rows,
+  // down to 32 rows, until no list holds more than 1/24 of the pairs or 32 lists are made
+  while ((int)all.size() < 32) {
+    int best = -1;
+    for (int i = 0; i < (int)all.size(); ++i)
+      if (all[i].r1 - all[i].r0 >= 64 && (best < 0 || all[i].load > all[best].load)) best = i;
+    if (best < 0 || all[best].load * 24 <= total) break;
+    List lo = all[best], hi = all[best];
+    lo.r1 = hi.r0 = (lo.r0 + lo.r1) / 2;
+    lo.load = all[best].load / 2;
+    hi.load = all[best].load - lo.load;
+    all[best] = lo;
+    all.push_back(hi);
+  }
+  // four groups of at most 8 lists: largest first, each to the lightest group with room
+  std::stable_sort(all.begin(), all.end(), [](const List& x, const List& y) { return x.load > y.load; });
+  std::vector<List> grp[4];
+  int64_t load[4] = {0, 0, 0, 0};
+  for (const List& l : all) {
+    int g = -1;
+    for (int c = 0; c < 4; ++c)
+      if (grp[c].size() < 8 && (g < 0 || load[c] < load[g])) g = c;
+    grp[g].push_back(l);
+    load[g] += l.load;
+  }
+  int n = 0;
+  for (int g = 0; g < 4; ++g) {
+    group_bounds[g] = n;
+    for (const List& l : grp[g]) {
+      lists[n] = l.k | (l.r0 << 8) | ((l.r1 - 1) << 16);
+      list_count[n] = l.load;
+      ++n;
+    }
+  }
+  group_bounds[4] = n;
+  *n_lists = n;
   return OCNN_OK;
 }
 
-static int pair_plan_launch(const uint16_t* loc, int64_t tiles, int K, const int32_t* order, int mode,
+static int pair_plan_launch(const uint16_t* loc, int64_t tiles, int K, const int32_t* lists, int nl, int mode,
                             int32_t* nblk, const int32_t* cptr, uint32_t* ent, void* stream) {
-  OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 24), "pair_plan: bad shape");
+  OCNN_REQUIRE(K >= 1 && K <= 27 && nl >= 1 && nl <= 32 && tiles >= 0 && tiles < (1ll << 24),
+               "pair_plan: bad shape");
   if (tiles == 0) return OCNN_OK;
-  hipLaunchKernelGGL(pair_plan_kernel, dim3((unsigned)cdiv(tiles * K, 4)), dim3(256), 0, (hipStream_t)stream, loc,
-                     tiles, K, order, mode, nblk, cptr, ent);
+  hipLaunchKernelGGL(pair_plan_kernel, dim3((unsigned)cdiv(tiles * nl, 4)), dim3(256), 0, (hipStream_t)stream, loc,
+                     tiles, K, lists, nl, mode, nblk, cptr, ent);
   return check_launch("pair_plan");
 }
 
-extern "C" int ocnn_pair_plan_count(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
+extern "C" int ocnn_pair_plan_count(const uint16_t* loc, int64_t tiles, int K, const int32_t* lists, int n_lists,
                                     int32_t* nblk, void* stream) {
-  return pair_plan_launch(loc, tiles, K, slot_order, 0, nblk, nullptr, nullptr, stream);
+  return pair_plan_launch(loc, tiles, K, lists, n_lists, 0, nblk, nullptr, nullptr, stream);
 }
 
-extern "C" int ocnn_pair_plan_fill(const uint16_t* loc, int64_t tiles, int K, const int32_t* slot_order,
+extern "C" int ocnn_pair_plan_fill(const uint16_t* loc, int64_t tiles, int K, const int32_t* lists, int n_lists,
                                    const int32_t* cptr, uint32_t* ent, void* stream) {
-  return pair_plan_launch(loc, tiles, K, slot_order, 1, nullptr, cptr, ent, stream);
+  return pair_plan_launch(loc, tiles, K, lists, n_lists, 1, nullptr, cptr, ent, stream);
 }

@@ -9,10 +9,11 @@
 // the transposing load, whose per-lane address does the gather.
 //
 // A workgroup owns 32 A channels (blockIdx.y), all B channels (<= 96) and a range of tiles,
-// and keeps the sums of ALL slots in accumulator registers for the whole range: its eight
-// waves (two per SIMD: one computes while the other waits for LDS) share the slots (a heavy
-// slot - the centre of a 3x3x3 table - is cut into several units that take every S-th
-// block; units are dealt to the waves by load on the host).
+// and keeps the sums of ALL lists of the pair plan (a list: a slot, or a range of the tiles'
+// rows of a heavy slot) in accumulator registers for the whole range: its eight waves (two
+// per SIMD: one computes while the other waits for LDS) share the lists; the units left
+// over go to the heaviest lists, which are cut into S units that take every S-th block
+// (units are dealt to the waves by load on the host).
 // Per tile it stages its 64-byte half of the distinct A rows, the B rows and the tile's
 // blocks with asynchronous global->LDS loads into the second set of buffers while the
 // blocks of the tile before are multiplied.  Per-range sums go to `partial`; a second
@@ -31,7 +32,7 @@ constexpr int kWsCap = 511;               // distinct rows per tile (+ the zero 
 constexpr int kWsEnt = 14 * 256;          // entries per tile: 27 x 8 blocks of 16 at most, in whole KiB
 
 struct WsUnits {                          // (a kernel argument)
-  int32_t unit[32];                       // per wave and unit: slot j | S << 8 | s << 16, or -1
+  int32_t unit[32];                       // per wave and unit: list j | S << 8 | s << 16, or -1
   int32_t slot[32];                       // the table slot of the unit, or -1
 };
 
@@ -69,8 +70,8 @@ static __device__ __forceinline__ void ws_stage(char* __restrict__ sa, char* __r
     ws_dma16(rs_e, se + p * 1024, t.cb * 64u + (uint32_t)(p * 1024 + lane * 16));
 }
 
-// The blocks of one tile.  unit[i] = slot j | S << 8 | s << 16 (blocks s, s + S, .. of slot
-// j), or -1.  cp: block offsets of the tile's slots.
+// The blocks of one tile.  unit[i] = list j | S << 8 | s << 16 (blocks s, s + S, .. of list
+// j), or -1.  cp: block offsets of the tile's lists.
 template <typename T, int HB, int NU>
 static __device__ __forceinline__ void ws_tile(const char* __restrict__ sa, const char* __restrict__ sb,
                                                const uint32_t* __restrict__ se, const int32_t* __restrict__ cp,
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(512, 1) void conv_wgrad_sparse_kernel(
     const T* __restrict__ a, uint32_t a_bytes, uint32_t a_pitch, const T* __restrict__ bt, uint32_t b_bytes,
     const int32_t* __restrict__ uptr, const int32_t* __restrict__ urows, uint32_t u_bytes,
     const int32_t* __restrict__ cptr, const uint32_t* __restrict__ ent, uint32_t ent_bytes,
-    WsUnits units, int64_t tiles, int64_t tiles_per_split, int K, float* __restrict__ partial) {
+    WsUnits units, int64_t tiles, int64_t tiles_per_split, int nl, float* __restrict__ partial) {
   // one array per buffer, so that the compiler can tell the buffers being filled from the
   // ones being read
   __shared__ __attribute__((aligned(16))) char s_a0[(kWsCap + 1) * 64];
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(512, 1) void conv_wgrad_sparse_kernel(
   __shared__ __attribute__((aligned(16))) uint32_t s_e1[kWsEnt];
   __shared__ int32_t s_u0[512];
   __shared__ int32_t s_u1[512];
-  __shared__ int32_t s_cp[4][32];
+  __shared__ int32_t s_cp[4][40];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(512, 1) void conv_wgrad_sparse_kernel(
   const __amdgpu_buffer_rsrc_t rs_b = make_rsrc(bt, b_bytes);
   const __amdgpu_buffer_rsrc_t rs_e = make_rsrc(ent, ent_bytes);
   const __amdgpu_buffer_rsrc_t rs_u = make_rsrc(urows, u_bytes);
-  const __amdgpu_buffer_rsrc_t rs_cp = make_rsrc(cptr, (uint32_t)((tiles * K + 1) * 4));
+  const __amdgpu_buffer_rsrc_t rs_cp = make_rsrc(cptr, (uint32_t)((tiles * nl + 1) * 4));
   const uint32_t a_col = (uint32_t)ablk * 64u;
 
   struct Meta { int32_t p0, U, cb, nb; int64_t t; };
@@ -155,8 +156,8 @@ __global__ __launch_bounds__(512, 1) void conv_wgrad_sparse_kernel(
     m.t = tc;
     m.p0 = uptr[tc];
     m.U = in ? uptr[tc + 1] - m.p0 : -16;                                // past the range: nothing to load
-    m.cb = cptr[tc * K];
-    m.nb = in ? cptr[tc * K + K] - m.cb : 0;
+    m.cb = cptr[tc * nl];
+    m.nb = in ? cptr[tc * nl + nl] - m.cb : 0;
     return m;
   };
   auto tile_of = [&](const Meta& m) {
@@ -172,14 +173,14 @@ __global__ __launch_bounds__(512, 1) void conv_wgrad_sparse_kernel(
   auto load_ids = [&](const Meta& m) {
     Ids r;
     r.u = __builtin_amdgcn_raw_buffer_load_b32(rs_u, (uint32_t)(m.p0 + tid - 1) * 4u, 0, 0);
-    r.cp = __builtin_amdgcn_raw_buffer_load_b32(rs_cp, (uint32_t)((int)m.t * K + min(tid, K)) * 4u, 0, 0);
+    r.cp = __builtin_amdgcn_raw_buffer_load_b32(rs_cp, (uint32_t)((int)m.t * nl + min(tid, nl)) * 4u, 0, 0);
     r.U = m.U;
     r.cb = m.cb;
     return r;
   };
   auto put_ids = [&](int32_t* su, int seq, const Ids& r) {
     su[tid] = (tid >= 1 && tid <= r.U) ? r.u : -1;
-    if (tid < 32) s_cp[seq & 3][tid] = r.cp - r.cb;
+    if (tid < 40) s_cp[seq & 3][tid] = r.cp - r.cb;
   };
 
   if (t_begin >= t_end) return;
@@ -256,7 +257,7 @@ __global__ void wgrad_sparse_reduce_kernel(const float* __restrict__ partial, in
 
 using namespace ocnn;
 
-static int ws_units_per_wave(int K) { return K <= 8 ? 2 : 4; }
+constexpr int kWsUnitsPerWave = 4;        // 32 units >= the lists of any plan
 
 extern "C" int ocnn_conv_wgrad_sparse_supported(int dtype, int64_t rows_a, int64_t rows_b, int K, int ca, int cb,
                                                 int plan_max_distinct) {
@@ -274,28 +275,28 @@ static int ws_splits(int64_t tiles, int ca) {
   return (int)std::max<int64_t>(1, std::min<int64_t>(tiles, std::max(1, n_cu / (ca / 32))));
 }
 
-extern "C" int64_t ocnn_conv_wgrad_sparse_workspace_bytes(int64_t rows_b, int K, int ca, int cb) {
+extern "C" int64_t ocnn_conv_wgrad_sparse_workspace_bytes(int64_t rows_b, int ca, int cb) {
   const int64_t tiles = cdiv(std::max<int64_t>(rows_b, 1), kWsRows);
-  const int nu = 8 * ws_units_per_wave(K);
+  const int nu = 8 * kWsUnitsPerWave;
   return (int64_t)ws_splits(tiles, ca) * (ca / 32) * nu * 32 * cb * 4;
 }
 
-// The units of a launch: every slot at least once, the spare units to the heaviest slots
-// (cut into S units that take every S-th block), dealt to the eight waves largest first.
-static void ws_make_units(int K, const int64_t* slot_count, const int32_t* order, int nu, int32_t* units,
+// The units of a launch: every list once, the spare units to the heaviest lists (cut into S
+// units that take every S-th block), dealt to the eight waves largest first.
+static void ws_make_units(int nl, const int32_t* lists, const int64_t* list_count, int nu, int32_t* units,
                           int32_t* unit_slot) {
-  int S[27];
-  for (int j = 0; j < K; ++j) S[j] = 1;
-  for (int spare = 8 * nu - K; spare > 0; --spare) {
+  int S[32];
+  for (int j = 0; j < nl; ++j) S[j] = 1;
+  for (int spare = 8 * nu - nl; spare > 0; --spare) {
     int best = 0;
-    for (int j = 1; j < K; ++j)
-      if (slot_count[order[j]] * S[best] > slot_count[order[best]] * S[j]) best = j;
+    for (int j = 1; j < nl; ++j)
+      if (list_count[j] * S[best] > list_count[best] * S[j]) best = j;
     ++S[best];
   }
   struct U { int j, s, S; int64_t load; };
   std::vector<U> all;
-  for (int j = 0; j < K; ++j)
-    for (int s = 0; s < S[j]; ++s) all.push_back({j, s, S[j], slot_count[order[j]] / S[j]});
+  for (int j = 0; j < nl; ++j)
+    for (int s = 0; s < S[j]; ++s) all.push_back({j, s, S[j], list_count[j] / S[j]});
   std::stable_sort(all.begin(), all.end(), [](const U& x, const U& y) { return x.load > y.load; });
   int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   int64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -305,7 +306,7 @@ static void ws_make_units(int K, const int64_t* slot_count, const int32_t* order
     for (int c = 0; c < 8; ++c)
       if (cnt[c] < nu && (w < 0 || load[c] < load[w])) w = c;
     units[w * nu + cnt[w]] = u.j | (u.S << 8) | (u.s << 16);
-    unit_slot[w * nu + cnt[w]] = order[u.j];
+    unit_slot[w * nu + cnt[w]] = lists[u.j] & 255;
     ++cnt[w];
     load[w] += u.load;
   }
@@ -314,34 +315,34 @@ static void ws_make_units(int K, const int64_t* slot_count, const int32_t* order
 template <typename T, int HB, int NU>
 static void launch_ws(const void* a, int64_t rows_a, int ca, const void* b, int64_t rows_b, const int32_t* uptr,
                       const int32_t* urows, int64_t plan_total, const int32_t* cptr, const uint32_t* ent,
-                      int64_t n_blocks, const WsUnits& units, int64_t tiles, int nsplit, int K, float* partial,
+                      int64_t n_blocks, const WsUnits& units, int64_t tiles, int nsplit, int nl, float* partial,
                       hipStream_t st) {
   hipLaunchKernelGGL((conv_wgrad_sparse_kernel<T, HB, NU>), dim3((unsigned)nsplit, (unsigned)(ca / 32)), dim3(512), 0,
                      st, (const T*)a, (uint32_t)(rows_a * ca * 2), (uint32_t)(ca * 2), (const T*)b,
                      (uint32_t)(rows_b * HB * 64), uptr, urows, (uint32_t)(plan_total * 4), cptr, ent,
-                     (uint32_t)(n_blocks * 64), units, tiles, cdiv(tiles, nsplit), K, partial);
+                     (uint32_t)(n_blocks * 64), units, tiles, cdiv(tiles, nsplit), nl, partial);
 }
 
 template <typename T>
 static int run_ws(const void* a, int64_t rows_a, int ca, const void* b, int64_t rows_b, int cb, const int32_t* uptr,
                   const int32_t* urows, int64_t plan_total, const int32_t* cptr, const uint32_t* ent,
-                  int64_t n_blocks, const int64_t* slot_count, const int32_t* order, int K, int a_major, void* out,
-                  void* ws, hipStream_t st) {
-  const int nuw = ws_units_per_wave(K), nu = 8 * nuw;
+                  int64_t n_blocks, const int32_t* lists, const int64_t* list_count, int nl, int K, int a_major,
+                  void* out, void* ws, hipStream_t st) {
+  const int nuw = kWsUnitsPerWave, nu = 8 * nuw;
   const int64_t tiles = cdiv(rows_b, kWsRows);
   const int64_t per_split = cdiv(tiles, ws_splits(tiles, ca));
   const int nsplit = (int)cdiv(tiles, per_split);          // every range holds at least one tile
   WsUnits units;
   for (int i = 0; i < 32; ++i) units.unit[i] = units.slot[i] = -1;
-  ws_make_units(K, slot_count, order, nuw, units.unit, units.slot);
+  ws_make_units(nl, lists, list_count, nuw, units.unit, units.slot);
   float* partial = (float*)ws;
   const int hb = cb / 32;
-#define OCNN_WS_CASE(HB_, NU_)                                                                              \
-  if (hb == HB_ && nuw == NU_) {                                                                            \
-    launch_ws<T, HB_, NU_>(a, rows_a, ca, b, rows_b, uptr, urows, plan_total, cptr, ent, n_blocks, units,     \
-                           tiles, nsplit, K, partial, st);                                                  \
+#define OCNN_WS_CASE(HB_)                                                                                    \
+  if (hb == HB_) {                                                                                           \
+    launch_ws<T, HB_, kWsUnitsPerWave>(a, rows_a, ca, b, rows_b, uptr, urows, plan_total, cptr, ent, n_blocks, \
+                                       units, tiles, nsplit, nl, partial, st);                               \
   }
-  OCNN_WS_CASE(1, 4) OCNN_WS_CASE(2, 4) OCNN_WS_CASE(3, 4) OCNN_WS_CASE(1, 2) OCNN_WS_CASE(2, 2) OCNN_WS_CASE(3, 2)
+  OCNN_WS_CASE(1) OCNN_WS_CASE(2) OCNN_WS_CASE(3)
 #undef OCNN_WS_CASE
   if (check_launch("conv_wgrad_sparse") != OCNN_OK) return OCNN_ERR_HIP;
   const int64_t total = (int64_t)K * ca * cb;
@@ -353,14 +354,14 @@ static int run_ws(const void* a, int64_t rows_a, int ca, const void* b, int64_t 
 extern "C" int ocnn_conv_wgrad_sparse(int dtype, const void* a, int64_t rows_a, int ca, const void* b,
                                       int64_t rows_b, int cb, const int32_t* uptr, const int32_t* urows,
                                       int plan_max_distinct, int64_t plan_total, const int32_t* cptr,
-                                      const uint32_t* ent, int64_t n_blocks, const int64_t* slot_count,
-                                      const int32_t* slot_order, int K, int a_major, void* out, void* workspace,
-                                      int64_t workspace_bytes, void* stream) {
+                                      const uint32_t* ent, int64_t n_blocks, const int32_t* lists,
+                                      const int64_t* list_count, int n_lists, int K, int a_major, void* out,
+                                      void* workspace, int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(ocnn_conv_wgrad_sparse_supported(dtype, rows_a, rows_b, K, ca, cb, plan_max_distinct),
                "conv_wgrad_sparse: shape not supported");
   OCNN_REQUIRE(rows_b >= 0 && rows_b < (1ll << 31) && plan_total >= 0 && plan_total < (1ll << 29) &&
-                   n_blocks >= 0 && n_blocks < (1ll << 25),
-               "conv_wgrad_sparse: rows out of range");
+                   n_blocks >= 0 && n_blocks < (1ll << 25) && n_lists >= 1 && n_lists <= 32,
+               "conv_wgrad_sparse: rows or lists out of range");
   hipStream_t st = (hipStream_t)stream;
   if (rows_b == 0) {                                   // nothing to add up: zeros
     WsUnits none;
@@ -374,13 +375,13 @@ extern "C" int ocnn_conv_wgrad_sparse(int dtype, const void* a, int64_t rows_a, 
                          (const float*)nullptr, 0, 0, none, K, ca, cb, a_major, (bf16*)out);
     return check_launch("wgrad_sparse_reduce");
   }
-  if (workspace_bytes < ocnn_conv_wgrad_sparse_workspace_bytes(rows_b, K, ca, cb)) {
+  if (workspace_bytes < ocnn_conv_wgrad_sparse_workspace_bytes(rows_b, ca, cb)) {
     set_error("conv_wgrad_sparse: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
   if (dtype == OCNN_F16)
-    return run_ws<f16>(a, rows_a, ca, b, rows_b, cb, uptr, urows, plan_total, cptr, ent, n_blocks, slot_count,
-                       slot_order, K, a_major, out, workspace, st);
-  return run_ws<bf16>(a, rows_a, ca, b, rows_b, cb, uptr, urows, plan_total, cptr, ent, n_blocks, slot_count,
-                      slot_order, K, a_major, out, workspace, st);
+    return run_ws<f16>(a, rows_a, ca, b, rows_b, cb, uptr, urows, plan_total, cptr, ent, n_blocks, lists,
+                       list_count, n_lists, K, a_major, out, workspace, st);
+  return run_ws<bf16>(a, rows_a, ca, b, rows_b, cb, uptr, urows, plan_total, cptr, ent, n_blocks, lists,
+                      list_count, n_lists, K, a_major, out, workspace, st);
 }

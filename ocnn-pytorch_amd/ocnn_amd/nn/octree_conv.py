@@ -77,11 +77,12 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   if (plan is not None and USE_SPARSE and plan.occupancy <= SPARSE_MAX_OCCUPANCY and
       rows >= SPARSE_MIN_ROWS and L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)):
     pp = plan.pairs()
+    ws = _lib.workspace(L.ocnn_conv_gather_sparse_workspace_bytes(cin, cout), data.device)
     _lib.check(L.ocnn_conv_gather_sparse(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax, plan.total,
-        _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.order), pp.n_first, rows, K,
-        _lib.ptr(W), cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
-        ws.numel(), _lib.stream()))
+        _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.lists), pp.n_lists,
+        ctypes.addressof(pp.group_bounds_host), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
+        _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return out
   if plan is not None and plan.reuse >= 2.0 and USE_WIDE and L.ocnn_conv_gather_wide_supported(
       code, rows_in, K, cin, cout, plan.umax):
@@ -132,12 +133,12 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
       not (ca == cb and ca in (32, 64)) and
       L.ocnn_conv_wgrad_sparse_supported(code, x.shape[0], rows, K, ca, cb, plan.umax)):
     pp = plan.pairs()
-    ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, K, ca, cb), x.device)
+    ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, ca, cb), x.device)
     _lib.check(L.ocnn_conv_wgrad_sparse(
         code, _lib.ptr(x), x.shape[0], ca, _lib.ptr(g), rows, cb, _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
         plan.umax, plan.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks,
-        ctypes.addressof(pp.slot_count_host), ctypes.addressof(pp.order_host), K, int(not out_transposed),
-        _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+        ctypes.addressof(pp.lists_host), ctypes.addressof(pp.list_count_host), pp.n_lists, K,
+        int(not out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw
   if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
                                                               plan.umax):
@@ -173,11 +174,11 @@ def conv_wgrad_inverse(x, g, plan_t, out_transposed=False):
     return None
   pp = plan_t.pairs()
   gw = torch.empty((K, cg, cx) if out_transposed else (K, cx, cg), dtype=x.dtype, device=x.device)
-  ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(x.shape[0], K, cg, cx), x.device)
+  ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(x.shape[0], cg, cx), x.device)
   _lib.check(L.ocnn_conv_wgrad_sparse(
       code, _lib.ptr(g), g.shape[0], cg, _lib.ptr(x), x.shape[0], cx, _lib.ptr(plan_t.uptr),
       _lib.ptr(plan_t.urows), plan_t.umax, plan_t.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks,
-      ctypes.addressof(pp.slot_count_host), ctypes.addressof(pp.order_host), K, int(out_transposed),
+      ctypes.addressof(pp.lists_host), ctypes.addressof(pp.list_count_host), pp.n_lists, K, int(out_transposed),
       _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
   return gw
 

@@ -148,8 +148,9 @@ class TilePlan:
 
 
 class PairPlan:
-  """Blocks of 16 (row, neighbour) pairs per (tile, slot) of a table, the slots dealt to two
-  groups of about equal numbers of pairs (see ocnn_pair_plan_* in the C ABI)."""
+  """Blocks of 16 (row, neighbour) pairs per tile and list of a table; a list is a slot, or
+  a range of the tiles' rows of a slot with many pairs; the lists are dealt to four groups
+  of about equal numbers of pairs (see ocnn_pair_plan_* in the C ABI)."""
 
   def __init__(self, plan: TilePlan):
     import ctypes
@@ -160,21 +161,24 @@ class PairPlan:
     counts = torch.zeros(K, dtype=torch.int64, device=dev)
     _lib.check(L.ocnn_pair_plan_slot_counts(_lib.ptr(plan.loc), tiles, K, _lib.ptr(counts), st))
     per_slot = (ctypes.c_int64 * K)(*counts.tolist())
-    order = (ctypes.c_int32 * K)()
-    n_first = ctypes.c_int(0)
-    _lib.check(L.ocnn_pair_plan_order(K, ctypes.addressof(per_slot), L.ocnn_conv_gather_sparse_max_slots(K),
-                                      ctypes.addressof(order), ctypes.addressof(n_first)))
-    self.n_first = n_first.value
-    self.slot_count_host, self.order_host = per_slot, order       # (kept alive: the C ABI reads them)
-    self.order = torch.tensor(list(order), dtype=torch.int32, device=dev)
-    nblk = torch.zeros(max(tiles * K, 1), dtype=torch.int32, device=dev)
-    _lib.check(L.ocnn_pair_plan_count(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.order), _lib.ptr(nblk), st))
-    self.cptr = torch.zeros(tiles * K + 1, dtype=torch.int32, device=dev)
-    self.cptr[1:] = torch.cumsum(nblk[:tiles * K], 0)
+    # host arrays, kept alive with the plan: the C ABI reads them at every call
+    self.lists_host = (ctypes.c_int32 * 32)()
+    self.list_count_host = (ctypes.c_int64 * 32)()
+    self.group_bounds_host = (ctypes.c_int32 * 5)()
+    n_lists = ctypes.c_int(0)
+    _lib.check(L.ocnn_pair_plan_lists(K, ctypes.addressof(per_slot), ctypes.addressof(self.lists_host),
+                                      ctypes.addressof(self.list_count_host),
+                                      ctypes.addressof(self.group_bounds_host), ctypes.addressof(n_lists)))
+    nl = self.n_lists = n_lists.value
+    self.lists = torch.tensor(list(self.lists_host)[:nl], dtype=torch.int32, device=dev)
+    nblk = torch.zeros(max(tiles * nl, 1), dtype=torch.int32, device=dev)
+    _lib.check(L.ocnn_pair_plan_count(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.lists), nl, _lib.ptr(nblk), st))
+    self.cptr = torch.zeros(tiles * nl + 1, dtype=torch.int32, device=dev)
+    self.cptr[1:] = torch.cumsum(nblk[:tiles * nl], 0)
     self.n_blocks, self.max_blocks = (int(v) for v in torch.stack(
-        [self.cptr[-1], nblk[:tiles * K].view(tiles, K).sum(1).max().int()]).tolist()) if tiles > 0 else (0, 0)
+        [self.cptr[-1], nblk[:tiles * nl].view(tiles, nl).sum(1).max().int()]).tolist()) if tiles > 0 else (0, 0)
     self.ent = torch.empty(max(self.n_blocks, 1) * 16, dtype=torch.int32, device=dev)
-    _lib.check(L.ocnn_pair_plan_fill(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.order), _lib.ptr(self.cptr),
+    _lib.check(L.ocnn_pair_plan_fill(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.lists), nl, _lib.ptr(self.cptr),
                                      _lib.ptr(self.ent), st))
 
 

@@ -113,27 +113,39 @@ def test_points_normalize_and_merge():
     Points(torch.zeros(2, 2))
 
 
-def test_pair_plan_slot_order():
-  """ocnn_pair_plan_order (host only): every slot once, at most max_slots per group, the
-  heavier group no more than the largest slot above the lighter one."""
+def test_pair_plan_lists_and_groups():
+  """ocnn_pair_plan_lists (host only): the lists cover every (slot, row of a tile) once, heavy
+  slots are cut by rows, at most 32 lists in four groups of at most 8 whose loads differ by
+  no more than the largest list."""
   L = _lib.lib()
   rng = np.random.default_rng(3)
   for K in (1, 3, 8, 9, 27):
-    cap = L.ocnn_conv_gather_sparse_max_slots(K)
-    assert 2 * cap >= K
     for trial in range(20):
       counts = rng.integers(0, 1000, size=K).astype(np.int64)
       if trial % 3 == 0:
-        counts[rng.integers(0, K)] = 50000                  # one dominant slot (the centre)
-      order = (ctypes.c_int32 * K)()
-      n_first = ctypes.c_int(0)
+        counts[rng.integers(0, K)] = 15000                   # one dominant slot (the centre)
       c = (ctypes.c_int64 * K)(*counts.tolist())
-      assert L.ocnn_pair_plan_order(K, ctypes.addressof(c), cap, ctypes.addressof(order),
-                                    ctypes.addressof(n_first)) == 0
-      order = list(order)
-      assert sorted(order) == list(range(K))
-      n0 = n_first.value
-      assert 0 <= n0 <= cap and K - n0 <= cap
-      a, b = counts[order[:n0]].sum(), counts[order[n0:]].sum()
-      if K <= cap:                                          # no group ever ran out of room
-        assert abs(int(a) - int(b)) <= counts.max()
+      lists = (ctypes.c_int32 * 32)()
+      loads = (ctypes.c_int64 * 32)()
+      gb = (ctypes.c_int32 * 5)()
+      nl = ctypes.c_int(0)
+      assert L.ocnn_pair_plan_lists(K, ctypes.addressof(c), ctypes.addressof(lists), ctypes.addressof(loads),
+                                    ctypes.addressof(gb), ctypes.addressof(nl)) == 0
+      nl = nl.value
+      assert K <= nl <= 32 and list(gb)[0] == 0 and list(gb)[4] == nl
+      cover = np.zeros((K, 128), int)
+      for v in list(lists)[:nl]:
+        k, r0, r1 = v & 255, (v >> 8) & 255, ((v >> 16) & 255) + 1
+        assert 0 <= k < K and 0 <= r0 < r1 <= 128 and (r1 - r0) % 32 == 0
+        cover[k, r0:r1] += 1
+      assert (cover == 1).all()
+      loads = np.array(list(loads)[:nl])
+      assert loads.sum() == counts.sum()
+      sums = []
+      for g in range(4):
+        assert 0 <= gb[g + 1] - gb[g] <= 8
+        sums.append(int(loads[gb[g]:gb[g + 1]].sum()))
+      if nl <= 28:                                           # (room in every group)
+        assert max(sums) - min(sums) <= loads.max()
+      if counts.max() * 24 > counts.sum() and K < 27:
+        assert nl > K                                        # the heavy slot was cut

@@ -527,52 +527,58 @@ def _gather_sparse(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
   cin = x.shape[1]
   code = _lib.dtype_code(x)
   assert L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)
+  import ctypes
   pp = plan.pairs()
   out = torch.empty((rows, cout), dtype=x.dtype, device=x.device)
-  ws = torch.empty(K * cin * cout * 2, dtype=torch.uint8, device=x.device)
+  ws = torch.empty(L.ocnn_conv_gather_sparse_workspace_bytes(cin, cout), dtype=torch.uint8, device=x.device)
   _lib.check(L.ocnn_conv_gather_sparse(
       code, _lib.ptr(x), rows_in, _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax, plan.total,
-      _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.order), pp.n_first, rows, K,
-      _lib.ptr(w), cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
-      ws.numel(), _lib.stream()))
+      _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.lists), pp.n_lists,
+      ctypes.addressof(pp.group_bounds_host), rows, K, _lib.ptr(w), cin, cout, int(transposed), int(reverse),
+      _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
   return out
 
 
 @pytest.mark.parametrize('K', [27, 8, 3, 1])
 def test_pair_plan_lists(K):
-  """The pair plan against its definition, from the tile plan's positions: per (tile, slot in
-  plan order) the rows with a neighbour in ascending order, entry = position | (128 r +
-  16 (r & 7)) << 16, lists filled up to whole blocks of 16 with position 0 and r = 128."""
+  """The pair plan against its definition, from the tile plan's positions: per tile and list
+  (slot, or rows r0 .. r1 - 1 of a heavy slot) the rows with a neighbour in ascending order,
+  entry = position | (128 r + 16 (r & 7)) << 16, filled up to whole blocks of 16 with
+  position 0 and r = 128."""
   from ocnn_amd.octree.octree import TilePlan
   g = torch.Generator().manual_seed(K)
   table = _local_table(128 * 9 + 50, 900, K, g, empty=0.8)
   if K > 2:
     table[:, 1] = -1
+  if K == 27:
+    table[:, 13] = torch.arange(table.shape[0], dtype=torch.int32).clamp_(max=899)
   plan = TilePlan(table.to(DEV))
   pp = plan.pairs()
   loc = plan.loc.cpu().numpy().astype(np.int64) & 0xffff      # (tiles, K, 128)
   tiles = loc.shape[0]
-  order = pp.order.cpu().numpy()
+  lists = pp.lists.cpu().numpy()
+  nl = pp.n_lists
+  assert lists.tolist() == list(pp.lists_host)[:nl]
+  if K in (27, 1):
+    assert nl > K                                              # the full slot is cut by rows
   cptr = pp.cptr.cpu().numpy()
   ent = pp.ent.cpu().numpy().astype(np.int64) & 0xffffffff
-  assert sorted(order.tolist()) == list(range(K))
-  per_slot = (loc > 0).sum((0, 2))
-  assert abs(int(per_slot[order[:pp.n_first]].sum()) - int(per_slot[order[pp.n_first:]].sum())) <= per_slot.max()
   filler = (128 * 128) << 16
   at = 0
   most = 0
   for t in range(tiles):
     blocks = 0
-    for j in range(K):
-      assert cptr[t * K + j] == at
-      rows = np.nonzero(loc[t, order[j]])[0]
-      want = [int(loc[t, order[j], r]) | ((128 * r + 16 * (r & 7)) << 16) for r in rows]
+    for j in range(nl):
+      assert cptr[t * nl + j] == at
+      k, r0, r1 = lists[j] & 255, (lists[j] >> 8) & 255, ((lists[j] >> 16) & 255) + 1
+      rows = [r for r in range(r0, r1) if loc[t, k, r] > 0]
+      want = [int(loc[t, k, r]) | ((128 * r + 16 * (r & 7)) << 16) for r in rows]
       want += [filler] * (-len(want) % 16)
       assert ent[16 * at:16 * at + len(want)].tolist() == want
       at += len(want) // 16
       blocks += len(want) // 16
     most = max(most, blocks)
-  assert cptr[tiles * K] == at == pp.n_blocks and most == pp.max_blocks
+  assert cptr[tiles * nl] == at == pp.n_blocks and most == pp.max_blocks
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
@@ -592,10 +598,10 @@ def test_sparse_gather_kernel(dtype, K, cin, cout):
     if K > 2:
       table[:, 1] = -1                                   # a slot without pairs
       table[256:384] = -1                                # a tile without pairs
+    if K == 27:                                          # a slot with all the rows (it is cut into lists)
+      table[:, 13] = torch.arange(rows, dtype=torch.int32).clamp_(max=rows_in - 2)
     tg = table.to(DEV)
     plan = TilePlan(tg)
-    pp = plan.pairs()
-    assert pp.n_first <= _lib.lib().ocnn_conv_gather_sparse_max_slots(K)
     t64 = table.numpy().astype(np.int64)
     x = torch.randn(rows_in, cin, generator=g).to(dtype)
     w = (torch.randn(K, cin, cout, generator=g) / (K * cin * (1 - empty)) ** 0.5).to(dtype)
@@ -624,12 +630,12 @@ def _wgrad_sparse(x, g, table, plan, transposed):
   assert L.ocnn_conv_wgrad_sparse_supported(code, x.shape[0], rows, K, ca, cb, plan.umax)
   pp = plan.pairs()
   gw = torch.empty((K, cb, ca) if transposed else (K, ca, cb), dtype=x.dtype, device=x.device)
-  ws = torch.empty(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, K, ca, cb), dtype=torch.uint8, device=x.device)
+  ws = torch.empty(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, ca, cb), dtype=torch.uint8, device=x.device)
   _lib.check(L.ocnn_conv_wgrad_sparse(
       code, _lib.ptr(x), x.shape[0], ca, _lib.ptr(g), rows, cb, _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax,
-      plan.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, ctypes.addressof(pp.slot_count_host),
-      ctypes.addressof(pp.order_host), K, int(not transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(),
-      _lib.stream()))
+      plan.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, ctypes.addressof(pp.lists_host),
+      ctypes.addressof(pp.list_count_host), pp.n_lists, K, int(not transposed), _lib.ptr(gw), _lib.ptr(ws),
+      ws.numel(), _lib.stream()))
   return gw
 
 
