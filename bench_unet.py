@@ -32,6 +32,7 @@ def main():
   ap.add_argument('--dtype', default='bfloat16')
   ap.add_argument('--nempty', type=int, default=1)
   ap.add_argument('--profile', action='store_true')
+  ap.add_argument('--torch-loss', action='store_true', help='torch.nn.functional.cross_entropy for the loss')
   args = ap.parse_args()
   import torch
   from ocnn_amd import modules, synthetic
@@ -90,7 +91,13 @@ def main():
     for p in params:
       p.grad = None
     logits = net(feat, octree, args.depth, query)
-    torch.nn.functional.cross_entropy(logits.float(), labels).backward()
+    if args.torch_loss:
+      loss = torch.nn.functional.cross_entropy(logits.float(), labels)
+    else:
+      # the same cross-entropy; torch's nll_loss kernels take 1.7 ms on 1.2 M x 10 logits
+      lf = logits.float()
+      loss = (torch.logsumexp(lf, 1) - lf.gather(1, labels.view(-1, 1)).squeeze(1)).mean()
+    loss.backward()
 
   for _ in range(args.warmup):
     step()

@@ -394,7 +394,11 @@ int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const vo
  * towards the batch statistics by `factor`, the running variance towards the unbiased one
  * (torch.nn.functional.batch_norm); dgamma / dbeta are fp32, grad_gamma / grad_beta the same
  * sums in param_dtype (may be NULL).  fp32 arithmetic, two-level reductions with a fixed order.
- * channels a multiple of 16 bytes of elements. */
+ * channels a multiple of 16 bytes of elements.  residual (may be NULL): a tensor like x added
+ * to the normalised values before the ReLU, each summand rounded to the dtype first (the
+ * tail of a residual block, ocnn/modules/resblocks.py:96-99); the backward pass then takes the
+ * forward output y for the ReLU's mask and writes the residual's gradient to d_residual
+ * (both may be NULL). */
 int ocnn_batch_norm_supported(int dtype, int64_t rows, int channels);
 int64_t ocnn_batch_norm_workspace_bytes(int channels);
 int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
@@ -403,12 +407,13 @@ int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, 
                           int64_t workspace_bytes, void* stream);
 int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
                           const float* invstd, const void* gamma, const void* beta,
-                          int param_dtype, int relu, void* y, void* stream);
+                          int param_dtype, int relu, const void* residual, void* y, void* stream);
 int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy, int64_t rows, int channels,
                              const float* mean, const float* invstd, const void* gamma,
-                             const void* beta, int param_dtype, int relu, int training, void* dx,
-                             float* dgamma, float* dbeta, void* grad_gamma, void* grad_beta,
-                             void* workspace, int64_t workspace_bytes, void* stream);
+                             const void* beta, int param_dtype, int relu, int training,
+                             const void* y, void* dx, void* d_residual, float* dgamma, float* dbeta,
+                             void* grad_gamma, void* grad_beta, void* workspace,
+                             int64_t workspace_bytes, void* stream);
 
 /* Key search, ocnn/octree/octree.py:448-488 (search_key / search_xyzb): out[i] = position of
  * query[i] in the ascending `keys`, or -1.  ocnn_search_points takes float (x, y, z, b) rows,

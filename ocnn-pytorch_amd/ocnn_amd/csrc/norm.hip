@@ -147,7 +147,7 @@ __global__ void bn_stats_finish_kernel(const float* __restrict__ partial, int nb
   }
 }
 
-// y = (x - mean) * (invstd * gamma) + beta, then max(., 0) when relu.  A thread keeps the
+// y = (x - mean) * (invstd * gamma) + beta (+ res), then max(., 0) when relu.  A thread keeps the
 // constants of its VEC channels in registers and walks every rpp-th row of the workgroup's
 // range, four rows in flight.
 template <typename T, int VEC>
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
                                                        const float* __restrict__ invstd,
                                                        const void* __restrict__ gamma,
                                                        const void* __restrict__ beta, int pdtype, int relu,
-                                                       T* __restrict__ y) {
+                                                       const T* __restrict__ res, T* __restrict__ y) {
   typedef BnVec<T, VEC> V;
   const int lpr = C / VEC, rpp = 256 / lpr;
   const int tid = threadIdx.x, rl = tid / lpr, cl = tid - rl * lpr;
@@ -173,11 +173,14 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
   const int64_t r1 = min(rows, r0 + rows_per_blk);
   for (int64_t r = r0 + rl; r < r1; r += 4 * rpp) {
-    V a[4];
+    V a[4], b[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int64_t ru = r + (int64_t)u * rpp;
-      if (ru < r1) a[u] = *(const V*)(x + ru * C + cl * VEC);
+      if (ru < r1) {
+        a[u] = *(const V*)(x + ru * C + cl * VEC);
+        if (res) b[u] = *(const V*)(res + ru * C + cl * VEC);
+      }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -187,6 +190,7 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         float t = (to_f32(a[u].v[v]) - m[v]) * sc[v] + be[v];
+        if (res) t = to_f32(from_f32<T>(t)) + to_f32(b[u].v[v]);      // (rounded as the separate passes would)
         if (relu) t = fmaxf(t, 0.f);
         o.v[v] = from_f32<T>(t);
       }
@@ -197,6 +201,7 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
 
 // partial[blk][0][c] = sum_r dy'[r][c],  partial[blk][1][c] = sum_r dy'[r][c] * xhat[r][c], with
 // xhat = (x - mean) * invstd and dy' = dy where the forward output was positive (relu) or dy.
+// ymask: the forward output, when it is not a function of x alone (a residual was added).
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__ x, const T* __restrict__ dy,
                                                            int64_t rows, int C, int64_t rows_per_blk,
@@ -204,6 +209,7 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
                                                            const float* __restrict__ invstd,
                                                            const void* __restrict__ gamma,
                                                            const void* __restrict__ beta, int pdtype, int relu,
+                                                           const T* __restrict__ ymask,
                                                            float* __restrict__ partial) {
   typedef BnVec<T, VEC> V;
   __shared__ float s_a[256 * VEC], s_b[256 * VEC];
@@ -225,7 +231,7 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
     const int64_t r1 = min(rows, r0 + rows_per_blk);
     for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {          // two rows of both tensors in flight
-      V a[2], g[2];
+      V a[2], g[2], ym[2];
       bool ok[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
@@ -233,6 +239,7 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
         ok[u] = ru < r1;
         a[u] = *(const V*)(x + (ok[u] ? ru * C : 0) + cl * VEC);
         g[u] = *(const V*)(dy + (ok[u] ? ru * C : 0) + cl * VEC);
+        if (ymask) ym[u] = *(const V*)(ymask + (ok[u] ? ru * C : 0) + cl * VEC);
       }
 #pragma unroll
       for (int u = 0; u < 2; ++u)
@@ -241,7 +248,8 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
           const float xc = to_f32(a[u].v[v]) - m[v];
           const float xh = xc * is[v];
           float d = ok[u] ? to_f32(g[u].v[v]) : 0.f;
-          if (relu && !(xc * (is[v] * ga[v]) + be[v] > 0.f)) d = 0.f;      // the forward pass's expression
+          if (relu && !(ymask ? to_f32(ym[u].v[v]) > 0.f
+                              : xc * (is[v] * ga[v]) + be[v] > 0.f)) d = 0.f;       // the forward pass's expression
           s1[v] += d;
           s2[v] += d * xh;
         }
@@ -291,6 +299,7 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__
                                                            const void* __restrict__ beta, int pdtype, int relu,
                                                            const float* __restrict__ dbeta,
                                                            const float* __restrict__ dgamma, int training,
+                                                           const T* __restrict__ ymask, T* __restrict__ dres,
                                                            T* __restrict__ dx) {
   typedef BnVec<T, VEC> V;
   const int lpr = C / VEC, rpp = 256 / lpr;
@@ -311,29 +320,32 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
   const int64_t r1 = min(rows, r0 + rows_per_blk);
   for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {
-    V a[2], g[2];
+    V a[2], g[2], ym[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int64_t ru = r + (int64_t)u * rpp;
       if (ru < r1) {
         a[u] = *(const V*)(x + ru * C + cl * VEC);
         g[u] = *(const V*)(dy + ru * C + cl * VEC);
+        if (ymask) ym[u] = *(const V*)(ymask + ru * C + cl * VEC);
       }
     }
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int64_t ru = r + (int64_t)u * rpp;
       if (ru >= r1) continue;
-      V o;
+      V o, gr;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         const float xc = to_f32(a[u].v[v]) - m[v];
         float d = to_f32(g[u].v[v]);
-        if (relu && !(xc * sc[v] + be[v] > 0.f)) d = 0.f;
+        if (relu && !(ymask ? to_f32(ym[u].v[v]) > 0.f : xc * sc[v] + be[v] > 0.f)) d = 0.f;
+        gr.v[v] = from_f32<T>(d);                                      // the gradient of the residual
         if (training) d = d - db[v] - (xc * is[v]) * dg[v];
         o.v[v] = from_f32<T>(d * sc[v]);
       }
       *(V*)(dx + ru * C + cl * VEC) = o;
+      if (dres) *(V*)(dres + ru * C + cl * VEC) = gr;
     }
   }
 }
@@ -393,7 +405,7 @@ extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int
 
 extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
                                      const float* invstd, const void* gamma, const void* beta, int param_dtype,
-                                     int relu, void* y, void* stream) {
+                                     int relu, const void* residual, void* y, void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_apply: shape not supported");
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
@@ -402,16 +414,18 @@ extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
-                       mean, invstd, gamma, beta, param_dtype, relu, (T*)y);
+                       mean, invstd, gamma, beta, param_dtype, relu, (const T*)residual, (T*)y);
   });
   return check_launch("batch_norm_apply");
 }
 
 extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy, int64_t rows, int channels,
                                         const float* mean, const float* invstd, const void* gamma,
-                                        const void* beta, int param_dtype, int relu, int training, void* dx,
-                                        float* dgamma, float* dbeta, void* grad_gamma, void* grad_beta,
-                                        void* workspace, int64_t workspace_bytes, void* stream) {
+                                        const void* beta, int param_dtype, int relu, int training,
+                                        const void* y, void* dx, void* d_residual, float* dgamma, float* dbeta,
+                                        void* grad_gamma, void* grad_beta, void* workspace,
+                                        int64_t workspace_bytes, void* stream) {
+  OCNN_REQUIRE(!d_residual || dx, "batch_norm_backward: d_residual needs dx");
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_backward: shape not supported");
   OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels),
                "batch_norm_backward: workspace too small");
@@ -426,13 +440,13 @@ extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
     hipLaunchKernelGGL((bn_bwd_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
-                       channels, per, mean, invstd, gamma, beta, param_dtype, relu, partial);
+                       channels, per, mean, invstd, gamma, beta, param_dtype, relu, (const T*)y, partial);
     hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
                        channels, dbeta, dgamma, grad_gamma, grad_beta, param_dtype);
     if (dx)
       hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), dim3(nblk_a), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
                          channels, per_a, mean, invstd, gamma, beta, param_dtype, relu, dbeta, dgamma, training,
-                         (T*)dx);
+                         (const T*)y, (T*)d_residual, (T*)dx);
   });
   return check_launch("batch_norm_backward");
 }

@@ -146,10 +146,11 @@ class OctreeResBlock2(torch.nn.Module):
     self.relu = torch.nn.ReLU(inplace=True)
 
   def forward(self, data: torch.Tensor, octree, depth: int):
-    out = self.conv3x3b(self.conv3x3a(data, octree, depth), octree, depth)
+    out = self.conv3x3b.conv(self.conv3x3a(data, octree, depth), octree, depth)
     if self.in_channels != self.out_channels:
       data = self.conv1x1(data)
-    return self.relu(out + data)
+    # relu(bn(out) + data): the sum and the ReLU ride on the batch norm's pass over `out`
+    return self.conv3x3b.bn(out, residual=data, relu=True)
 
 
 class OctreeResBlocks(torch.nn.Module):

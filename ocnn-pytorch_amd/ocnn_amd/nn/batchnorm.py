@@ -21,7 +21,8 @@ def _param(t):
 
 class _BatchNormRelu(torch.autograd.Function):
   @staticmethod
-  def forward(ctx, x, weight, bias, running_mean, running_var, use_batch_stats, factor, eps, relu):
+  def forward(ctx, x, weight, bias, running_mean, running_var, use_batch_stats, factor, eps, relu,
+              residual=None):
     L = _lib.lib()
     x = x.contiguous()
     rows, c = x.shape
@@ -52,10 +53,15 @@ class _BatchNormRelu(torch.autograd.Function):
       mean = running_mean.detach().float().contiguous()
       invstd = torch.rsqrt(running_var.detach().float() + eps)
     y = torch.empty_like(x)
+    if residual is not None:
+      residual = residual.contiguous()
+      assert residual.shape == x.shape and residual.dtype == x.dtype
     _lib.check(L.ocnn_batch_norm_apply(code, _lib.ptr(x), rows, c, _lib.ptr(mean), _lib.ptr(invstd),
-                                       _lib.ptr(gamma), _lib.ptr(beta), pcode, int(relu), _lib.ptr(y),
-                                       _lib.stream()))
-    ctx.save_for_backward(x, mean, invstd, gamma, beta)
+                                       _lib.ptr(gamma), _lib.ptr(beta), pcode, int(relu), _lib.ptr(residual),
+                                       _lib.ptr(y), _lib.stream()))
+    # with a residual the ReLU's mask is not a function of x alone: the output is kept for it
+    ctx.save_for_backward(x, mean, invstd, gamma, beta, y if (residual is not None and relu) else None)
+    ctx.has_residual = residual is not None
     ctx.relu, ctx.training, ctx.pcode = relu, use_batch_stats, pcode
     ctx.wdtype = None if weight is None else weight.dtype
     ctx.bdtype = None if bias is None else bias.dtype
@@ -64,13 +70,15 @@ class _BatchNormRelu(torch.autograd.Function):
   @staticmethod
   def backward(ctx, dy):
     L = _lib.lib()
-    x, mean, invstd, gamma, beta = ctx.saved_tensors
+    x, mean, invstd, gamma, beta, y = ctx.saved_tensors
     dy = dy.contiguous()
     rows, c = x.shape
     dev = x.device
     dgamma = torch.empty(c, dtype=torch.float32, device=dev)
     dbeta = torch.empty(c, dtype=torch.float32, device=dev)
-    dx = torch.empty_like(x) if ctx.needs_input_grad[0] else None
+    want_res = ctx.has_residual and ctx.needs_input_grad[9]
+    dx = torch.empty_like(x) if (ctx.needs_input_grad[0] or want_res) else None
+    dres = torch.empty_like(x) if want_res else None
     # the parameter gradients come out in the parameters' dtype where the kernels hold it
     gw = gb = None
     if gamma is not None and ctx.needs_input_grad[1] and ctx.wdtype == gamma.dtype:
@@ -81,13 +89,13 @@ class _BatchNormRelu(torch.autograd.Function):
     ws = _lib.workspace(L.ocnn_batch_norm_workspace_bytes(c), dev)
     _lib.check(L.ocnn_batch_norm_backward(
         _lib.dtype_code(x), _lib.ptr(x), _lib.ptr(dy), rows, c, _lib.ptr(mean), _lib.ptr(invstd), _lib.ptr(gamma),
-        _lib.ptr(beta), ctx.pcode, int(ctx.relu), int(ctx.training), _lib.ptr(dx), _lib.ptr(dgamma),
-        _lib.ptr(dbeta), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), ws.numel(), _lib.stream()))
+        _lib.ptr(beta), ctx.pcode, int(ctx.relu), int(ctx.training), _lib.ptr(y), _lib.ptr(dx), _lib.ptr(dres),
+        _lib.ptr(dgamma), _lib.ptr(dbeta), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), ws.numel(), _lib.stream()))
     if gw is None and ctx.wdtype is not None and ctx.needs_input_grad[1]:
       gw = dgamma.to(ctx.wdtype)
     if gb is None and ctx.bdtype is not None and ctx.needs_input_grad[2]:
       gb = dbeta.to(ctx.bdtype)
-    return dx, gw, gb, None, None, None, None, None, None
+    return dx, gw, gb, None, None, None, None, None, None, dres
 
 
 class BatchNormRelu1d(torch.nn.BatchNorm1d):
@@ -99,12 +107,17 @@ class BatchNormRelu1d(torch.nn.BatchNorm1d):
     super().__init__(num_features, **kwargs)
     self.fused_relu = relu
 
-  def forward(self, input: torch.Tensor) -> torch.Tensor:
+  def forward(self, input: torch.Tensor, residual: torch.Tensor = None, relu: bool = None) -> torch.Tensor:
+    """residual: added to the normalised values before the ReLU (the tail of a residual
+    block), in the same pass.  relu: overrides the module's setting for this call."""
+    relu = self.fused_relu if relu is None else relu
     code = _lib.DTYPE_CODE.get(input.dtype, -1)
     if not (input.dim() == 2 and input.is_cuda and code >= 0 and input.shape[0] > 1 and
             _lib.lib().ocnn_batch_norm_supported(code, input.shape[0], input.shape[1])):
       out = super().forward(input)
-      return torch.relu(out) if self.fused_relu else out
+      if residual is not None:
+        out = out + residual
+      return torch.relu(out) if relu else out
     # the bookkeeping of torch.nn.modules.batchnorm._BatchNorm.forward
     factor = 0.0 if self.momentum is None else self.momentum
     if self.training and self.track_running_stats and self.num_batches_tracked is not None:
@@ -115,7 +128,7 @@ class BatchNormRelu1d(torch.nn.BatchNorm1d):
     return _BatchNormRelu.apply(input, self.weight, self.bias,
                                 self.running_mean if (not use_batch_stats or track) else None,
                                 self.running_var if (not use_batch_stats or track) else None,
-                                use_batch_stats, factor if track else None, self.eps, self.fused_relu)
+                                use_batch_stats, factor if track else None, self.eps, relu, residual)
 
   def extra_repr(self) -> str:
     return super().extra_repr() + ', relu={}'.format(self.fused_relu)

@@ -84,6 +84,57 @@ def test_batch_norm_relu_vs_torch(dtype, relu, training):
       assert torch.equal(y2, y)
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('training', [True, False])
+def test_batch_norm_residual_relu_vs_torch(dtype, training):
+  """relu(bn(x) + residual) in one pass (the tail of a residual block) against torch's
+  BatchNorm1d + add + ReLU in fp64: output, both input gradients, parameter gradients."""
+  g = torch.Generator().manual_seed(13)
+  for rows, c in [(1000, 32), (4133, 96), (20000, 256)]:
+    say('batch norm + residual', dtype, training, rows, c)
+    x = (torch.randn(rows, c, generator=g) * 1.5 + 1.0).to(dtype)
+    res = torch.randn(rows, c, generator=g).to(dtype)
+    dy = torch.randn(rows, c, generator=g).to(dtype)
+    w = (torch.rand(c, generator=g) + 0.5).to(dtype).float()
+    b = (torch.randn(c, generator=g) * 0.3).to(dtype).float()
+    ref = torch.nn.BatchNorm1d(c).double()
+    with torch.no_grad():
+      ref.weight.copy_(w); ref.bias.copy_(b); ref.running_mean.fill_(1.0); ref.running_var.fill_(2.0)
+    ref.train(training)
+    xr, rr = x.double().requires_grad_(), res.double().requires_grad_()
+    pre = ref(xr) + rr
+    yr = torch.relu(pre)
+    yr.backward(dy.double())
+    bn = BatchNormRelu1d(c, relu=False).to(DEV)
+    with torch.no_grad():
+      bn.weight.copy_(w); bn.bias.copy_(b); bn.running_mean.fill_(1.0); bn.running_var.fill_(2.0)
+    bn = bn.to(dtype) if dtype != torch.float32 else bn
+    bn.train(training)
+    xg, rg = x.to(DEV).requires_grad_(), res.to(DEV).requires_grad_()
+    y = bn(xg, residual=rg, relu=True)
+    y.backward(dy.to(DEV))
+    tol = TOL[dtype]
+    scale = lambda t: max(1.0, float(t.abs().max()))
+    assert float((y.detach().double().cpu() - yr.detach()).abs().max()) <= 2 * tol * scale(yr)
+    sure = pre.detach().abs() > 2e-2 * (1 if dtype != torch.float32 else 1e-3)     # away from the ReLU's kink
+    assert int((~sure).sum()) < 0.05 * sure.numel()
+    assert float(((xg.grad.double().cpu() - xr.grad) * sure).abs().max()) <= 4 * tol * scale(xr.grad)
+    assert float(((rg.grad.double().cpu() - rr.grad) * sure).abs().max()) <= 4 * tol * scale(rr.grad)
+    # (parameter gradients are sums over the rows: an element at the kink may fall either way)
+    slack = ((~sure) * dy.double().abs()).sum(0)
+    assert bool(((bn.bias.grad.double().cpu() - ref.bias.grad).abs() <= 8 * tol * scale(ref.bias.grad) + slack).all())
+    assert bool(((bn.weight.grad.double().cpu() - ref.weight.grad).abs()
+                 <= 8 * tol * scale(ref.weight.grad) + 5 * slack).all())
+    # only the residual's gradient wanted: dx is still computed for it, x gets none
+    x3 = x.to(DEV)
+    r3 = res.to(DEV).requires_grad_()
+    for p_ in bn.parameters():
+      p_.requires_grad_(False)
+    y3 = bn(x3, residual=r3, relu=True)
+    y3.backward(dy.to(DEV))
+    assert torch.equal(r3.grad, rg.grad) and torch.equal(y3, y) == (not training or True)
+
+
 def test_batch_norm_fallbacks_and_state_dict():
   """3-D inputs and odd channel counts take torch's path; the state_dict is BatchNorm1d's."""
   bn = BatchNormRelu1d(6, relu=True).to(DEV)
