@@ -10,6 +10,10 @@ MI355X (the headline number is bench.py's; these lines are supporting data).
             OctreeConv 3x3x3 32->32 at depth 9 and 256->256 at depth 6; build_octree and
             construct_all_neigh on the 1M points.
 
+  config 4: the U-Net's octree (batch of 8, 150k points each, depth 9), bf16: 3x3x3 and
+            2x2x2 stride-2 layers of 96 / 128 channels on the non-empty nodes of depths 9 and
+            8 (the tables the pair-plan kernels are for).
+
 Every layer runs forward + backward through the module (autograd included); one JSON
 line per layer: ms per fwd+bwd, effective TFLOP/s over non-empty neighbours, and the
 rate at the algorithmic byte count as a fraction of 8 TB/s.
@@ -31,7 +35,7 @@ def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--steps', type=int, default=30)
   ap.add_argument('--warmup', type=int, default=5)
-  ap.add_argument('--configs', default='2,3')
+  ap.add_argument('--configs', default='2,3,4')
   args = ap.parse_args()
   import torch
   from ocnn_amd import synthetic
@@ -169,6 +173,23 @@ def main():
         o._table(9, '333', 1, False), bf)
     run('conv 3x3x3 s1 256->256 d6', OctreeConv(256, 256, [3], 1), o, 6, int(o.nnum[6]), 256, 256,
         o._table(6, '333', 1, False), bf)
+  if '4' in args.configs.split(','):
+    # the U-Net's octree (config 4: batch 8, 150k points each, depth 9), layers on the non-empty
+    # nodes of depths 9 and 8, where 14 % / 25 % of the table entries hold a neighbour
+    o, b_ms, n_ms, npts = build(synthetic.mixed_cloud, 8, 1004, 150000, 9)
+    print(json.dumps({'octree': 'config 4 (batch 8, depth 9)', 'points': npts, 'build_octree_ms': b_ms,
+                      'construct_all_neigh_ms': n_ms, 'nnum_nempty': o.nnum_nempty.tolist()}), flush=True)
+    ne9, ne8 = int(o.nnum_nempty[9]), int(o.nnum_nempty[8])
+    run('conv 3x3x3 s1 96->96 d9 nempty', OctreeConv(96, 96, [3], 1, nempty=True), o, 9, ne9, 96, 96,
+        o._table(9, '333', 1, True), bf)
+    run('conv 3x3x3 s1 96->96 d8 nempty', OctreeConv(96, 96, [3], 1, nempty=True), o, 8, ne8, 96, 96,
+        o._table(8, '333', 1, True), bf)
+    run('conv 3x3x3 s1 128->96 d9 nempty', OctreeConv(128, 96, [3], 1, nempty=True), o, 9, ne9, 128, 96,
+        o._table(9, '333', 1, True), bf)
+    run('conv 2x2x2 s2 96->96 d9->8 nempty', OctreeConv(96, 96, [2], 2, nempty=True), o, 9, ne9, 96, 96,
+        o._table(9, '222', 2, True), bf)
+    run('deconv 2x2x2 s2 96->96 d8->9 nempty', OctreeDeconv(96, 96, [2], 2, nempty=True), o, 8, ne8, 96, 96,
+        o._table(9, '222', 2, True), bf)
 
 
 if __name__ == '__main__':
