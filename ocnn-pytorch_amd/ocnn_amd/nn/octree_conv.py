@@ -35,6 +35,17 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K)).  With a
   tile plan of the same table (and a supported shape) the staged kernel runs.
   dense: the table is the one-slot identity (row i reads row i)."""
+  out, planned = _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense)
+  if planned and plan is not None and plan.overflow_rows is not None:
+    # the few tiles that are too dense for the plan: plan-free kernel, results put in place
+    sub, _ = _conv_gather(data, rows_in, plan.overflow_table, W, cout, transposed, reverse, bias, None, False)
+    out.index_copy_(0, plan.overflow_rows, sub)
+  return out
+
+
+def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense):
+  """conv_gather without the overflow rows of the plan; also returns whether a kernel on
+  the plan ran."""
   _lib.require_gpu(data, table, W)
   L = _lib.lib()
   data, W, table = data.contiguous(), W.contiguous(), table.contiguous()
@@ -52,7 +63,7 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
     pad_w = (0, cin_p - cin, 0, cout_p - cout) if transposed else (0, cout_p - cout, 0, cin_p - cin)
     out = conv_gather(F.pad(data, (0, cin_p - cin)), rows_in, table, F.pad(Wk, pad_w), cout_p,
                       transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), plan)
-    return out[:, :cout].contiguous()
+    return out[:, :cout].contiguous(), False
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
   code = _lib.dtype_code(data)
   nbytes = L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout)
@@ -60,20 +71,20 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   if dense and K == 1 and rows == rows_in and L.ocnn_conv_dense_rw_supported(code, rows, cin, cout):
     _lib.check(L.ocnn_conv_dense_rw(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed),
                                     _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out
+    return out, False
   # (many input channels into few output channels: the row tile that fits LDS is small and
   # the weights are streamed once per tile; the plan-free kernel is no slower there)
   if (dense and K == 1 and rows == rows_in and not (cin >= 512 and cout < 256) and
       L.ocnn_conv_dense_supported(code, rows, cin, cout)):
     _lib.check(L.ocnn_conv_dense(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed),
                                  _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out
+    return out, False
   if plan is not None and L.ocnn_conv_gather_rw_supported(code, rows_in, K, cin, cout, plan.umax):
     _lib.check(L.ocnn_conv_gather_rw(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
         int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out
+    return out, True
   if (plan is not None and USE_SPARSE and plan.occupancy <= SPARSE_MAX_OCCUPANCY and
       rows >= SPARSE_MIN_ROWS and L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)):
     pp = plan.pairs()
@@ -83,32 +94,44 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
         _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks, pp.max_blocks, _lib.ptr(pp.lists), pp.n_lists,
         ctypes.addressof(pp.group_bounds_host), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
         _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out
+    return out, True
   if plan is not None and plan.reuse >= 2.0 and USE_WIDE and L.ocnn_conv_gather_wide_supported(
       code, rows_in, K, cin, cout, plan.umax):
     _lib.check(L.ocnn_conv_gather_wide(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
         int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out
+    return out, True
   if plan is not None and plan.reuse >= 2.0 and L.ocnn_conv_gather_planned_supported(
       code, rows_in, cin, cout):
     _lib.check(L.ocnn_conv_gather_planned(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
         _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out
+    return out, True
   _lib.check(L.ocnn_conv_gather(
       code, _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(W),
       cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
       ws.numel(), _lib.stream()))
-  return out
+  return out, False
 
 
 def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
   """gW (K, ca, cb) [or (K, cb, ca)] = sum_i x[T[i,k]]^T (x) g[i].  With a tile
   plan of the same table (and a supported shape) the staged kernel runs.
   dense: the table is the one-slot identity (row i reads row i)."""
+  gw, planned = _conv_wgrad(x, g, table, out_transposed, plan, dense)
+  if planned and plan is not None and plan.overflow_rows is not None:
+    # the few tiles that are too dense for the plan: their share of the sums, plan-free kernel
+    more, _ = _conv_wgrad(x, g.index_select(0, plan.overflow_rows), plan.overflow_table, out_transposed, None,
+                          False)
+    gw += more
+  return gw
+
+
+def _conv_wgrad(x, g, table, out_transposed, plan, dense):
+  """conv_wgrad without the overflow rows of the plan; also returns whether a kernel on the
+  plan ran."""
   _lib.require_gpu(x, g, table)
   L = _lib.lib()
   x, g, table = x.contiguous(), g.contiguous(), table.contiguous()
@@ -118,7 +141,7 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
   if rows >= PAD_MIN_ROWS and (ca % 32 or cb % 32) and x.dtype in _lib.DTYPE_CODE:
     ca_p, cb_p = -(-ca // 32) * 32, -(-cb // 32) * 32
     gw = conv_wgrad(F.pad(x, (0, ca_p - ca)), F.pad(g, (0, cb_p - cb)), table, out_transposed, plan)
-    return (gw[:, :cb, :ca] if out_transposed else gw[:, :ca, :cb]).contiguous()
+    return (gw[:, :cb, :ca] if out_transposed else gw[:, :ca, :cb]).contiguous(), False
   shape = (K, cb, ca) if out_transposed else (K, ca, cb)
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
   code = _lib.DTYPE_CODE.get(x.dtype, -1)
@@ -127,7 +150,7 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
     ws = _lib.workspace(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(ca, cb), x.device)
     _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x), _lib.ptr(g), rows, ca, cb, int(out_transposed),
                                           _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return gw
+    return gw, False
   # (32 x 32 and 64 x 64 have kernels of their own on the tile plan that are faster still)
   if (plan is not None and USE_SPARSE and plan.occupancy <= SPARSE_MAX_OCCUPANCY and rows >= SPARSE_MIN_ROWS and
       not (ca == cb and ca in (32, 64)) and
@@ -139,7 +162,7 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
         plan.umax, plan.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks,
         ctypes.addressof(pp.lists_host), ctypes.addressof(pp.list_count_host), pp.n_lists, K,
         int(not out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return gw
+    return gw, True
   if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
                                                               plan.umax):
     ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K, ca, cb), x.device)
@@ -147,13 +170,13 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
         code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, ca, cb, int(out_transposed),
         _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return gw
+    return gw, True
   ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes_for(_lib.dtype_code(x), x.shape[0], rows, K,
                                                             ca, cb), x.device)
   _lib.check(L.ocnn_conv_wgrad(
       _lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
       int(out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
-  return gw
+  return gw, False
 
 
 def conv_wgrad_inverse(x, g, plan_t, out_transposed=False):
@@ -180,6 +203,10 @@ def conv_wgrad_inverse(x, g, plan_t, out_transposed=False):
       _lib.ptr(plan_t.urows), plan_t.umax, plan_t.total, _lib.ptr(pp.cptr), _lib.ptr(pp.ent), pp.n_blocks,
       ctypes.addressof(pp.lists_host), ctypes.addressof(pp.list_count_host), pp.n_lists, K, int(out_transposed),
       _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  if plan_t.overflow_rows is not None:                     # (tiles too dense for the plan)
+    more, _ = _conv_wgrad(g, x.index_select(0, plan_t.overflow_rows), plan_t.overflow_table, not out_transposed,
+                          None, False)
+    gw += more
   return gw
 
 

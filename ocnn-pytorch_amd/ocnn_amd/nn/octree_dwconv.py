@@ -31,6 +31,8 @@ def dw_gather(data, rows_in, table, w, reverse, bias=None, plan=None):
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
         plan.umax, plan.total, rows, K, _lib.ptr(w), C, int(reverse), _lib.ptr(bias), _lib.ptr(out),
         _lib.stream()))
+    if plan.overflow_rows is not None:                     # the few tiles too dense for the plan
+      out.index_copy_(0, plan.overflow_rows, dw_gather(data, rows_in, plan.overflow_table, w, reverse, bias))
     return out
   _lib.check(L.ocnn_dwconv_gather(
       _lib.dtype_code(data), _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(w), C,
@@ -55,6 +57,8 @@ def dw_wgrad(x, g, table, plan=None):
         code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, C, _lib.ptr(gw), _lib.ptr(ws), ws.numel(),
         _lib.stream()))
+    if plan.overflow_rows is not None:
+      gw += dw_wgrad(x, g.index_select(0, plan.overflow_rows), plan.overflow_table)
     return gw
   ws = _lib.workspace(L.ocnn_dwconv_wgrad_workspace_bytes(rows, K, C), x.device)
   _lib.check(L.ocnn_dwconv_wgrad(_lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g),

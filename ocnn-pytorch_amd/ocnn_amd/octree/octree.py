@@ -105,9 +105,17 @@ class _NeighTables:
 
 
 class TilePlan:
-  """Per-tile distinct-row lists of a table (see ocnn_tile_plan_* in the C ABI)."""
+  """Per-tile distinct-row lists of a table (see ocnn_tile_plan_* in the C ABI).
 
-  def __init__(self, table: torch.Tensor):
+  The kernels on the plan stage a tile's distinct rows in LDS and take tiles of up to `cap`
+  rows.  A handful of denser tiles must not send a whole level to the plan-free kernels: when
+  at most a tenth of the tiles are over the limit, those tiles are emptied in the plan (as if
+  their table rows were all -1) and their rows listed in `overflow_rows` / `overflow_table`;
+  the Python layer runs them through the plan-free kernels and puts the results in place."""
+
+  CAP = 415      # the smallest limit of the kernels on the plan
+
+  def __init__(self, table: torch.Tensor, cap: int = None):
     _lib.require_gpu(table)
     L = _lib.lib()
     table = table.contiguous()
@@ -116,8 +124,21 @@ class TilePlan:
     tiles = (rows + tile_rows - 1) // tile_rows
     dev = table.device
     st = _lib.stream()
+    cap = self.CAP if cap is None else cap
+    self.overflow_rows = self.overflow_table = None
     ucount = torch.zeros(tiles, dtype=torch.int32, device=dev)
     _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(ucount), st))
+    if tiles > 0:
+      big = ucount > cap
+      n_big = int(big.sum())
+      if 0 < n_big <= max(1, tiles // 10):
+        idx = (big.nonzero().view(-1, 1) * tile_rows + torch.arange(tile_rows, device=dev).view(1, -1)).view(-1)
+        idx = idx[idx < rows]
+        self.overflow_rows = idx
+        self.overflow_table = table.index_select(0, idx).contiguous()
+        table = table.clone()
+        table[idx] = -1
+        ucount = torch.where(big, torch.zeros_like(ucount), ucount)
     uptr = torch.zeros(tiles + 1, dtype=torch.int32, device=dev)
     uptr[1:] = torch.cumsum(ucount, 0)
     total, umax, nnz = (int(v) for v in torch.stack(

@@ -695,6 +695,50 @@ def test_layers_on_the_sparse_kernels(medium, dtype):
     conv_mod.SPARSE_MIN_ROWS, conv_mod.SPARSE_MAX_OCCUPANCY = keep
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_overflow_tiles_of_a_plan(dtype):
+  """A few tiles with more distinct rows than the kernels on the plan take: the plan empties
+  them and lists their rows, the Python layer runs those through the plan-free kernels;
+  gather, mirrored data gradient and weight gradient of several kernels against the oracle."""
+  from ocnn_amd.octree.octree import TilePlan
+  conv_mod = sys.modules['ocnn_amd.nn.octree_conv']
+  dw_mod = sys.modules['ocnn_amd.nn.octree_dwconv']
+  g = torch.Generator().manual_seed(17)
+  rows = rows_in = 128 * 60 + 31
+  table = _local_table(rows, rows_in, 27, g, spread=40, empty=0.3)
+  for t0 in (5, 33):                                       # two tiles that point all over the place
+    table[128 * t0:128 * (t0 + 1)] = torch.randint(0, rows_in, (128, 27), generator=g).to(torch.int32)
+  tg = table.to(DEV)
+  plan = TilePlan(tg)
+  assert plan.overflow_rows is not None and plan.overflow_rows.numel() == 256 and plan.umax <= TilePlan.CAP
+  assert TilePlan(tg, cap=4096).overflow_rows is None
+  t64 = table.numpy().astype(np.int64)
+  for cin, cout in [(64, 64), (32, 32), (128, 128), (96, 96)]:
+    say('overflow tiles', dtype, cin, cout)
+    x = torch.randn(rows_in, cin, generator=g).to(dtype)
+    w = (torch.randn(27, cin, cout, generator=g) / (19 * cin) ** 0.5).to(dtype)
+    b = torch.randn(cout, generator=g).to(dtype)
+    gr = (torch.randn(rows, cout, generator=g) / rows ** 0.5).to(dtype)
+    got = conv_mod.conv_gather(x.to(DEV), rows_in, tg, w.to(DEV), cout, False, False, b.to(DEV), plan)
+    assert rel_err(got, C.forward_gemm(f64(x), f64(w), t64) + f64(b)) < TOL[dtype]
+    got = conv_mod.conv_gather(gr.to(DEV), rows_in, tg, w.to(DEV), cin, True, True, None, plan)
+    want = C.forward_gemm(f64(gr), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
+    assert rel_err(got, want) < TOL[dtype]
+    got = conv_mod.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+    assert rel_err(got, C.weight_gemm(f64(x), f64(gr), t64)) < 2 * TOL[dtype]
+  # depth-wise
+  c = 64
+  x = torch.randn(rows_in, c, generator=g).to(dtype)
+  w = (torch.randn(27, 1, c, generator=g) / 19 ** 0.5).to(dtype)
+  gr = (torch.randn(rows, c, generator=g) / rows ** 0.5).to(dtype)
+  got = dw_mod.dw_gather(x.to(DEV), rows_in, tg, w.to(DEV), False, None, plan)
+  valid = (t64 >= 0)[..., None]
+  xg = f64(x)[np.maximum(t64, 0)] * valid                    # (rows, 27, c)
+  assert rel_err(got, (xg * f64(w)[:, 0][None]).sum(1)) < TOL[dtype]
+  got = dw_mod.dw_wgrad(x.to(DEV), gr.to(DEV), tg, plan)
+  assert rel_err(got, (xg * f64(gr)[:, None, :]).sum(0)[:, None, :]) < 2 * TOL[dtype]
+
+
 def test_sparse_gather_large_tiles():
   """Tiles near the staging limits of the pair-plan kernel (many distinct rows: one
   workgroup per CU, the wider row-number buffers) and the refusal beyond them."""
