@@ -137,9 +137,8 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
     for (int rb = 0; rb < 4; ++rb) b[rb] = *(const u32x4*)(rows_c + (pv[rb] ^ ((uint32_t)s << 5)));
   };
 
-  load_a(0, 0, A[0]);
-  load_a(0, 1, A[1]);
-  for (int cc = 0; cc < ncc; ++cc) {
+  // the distinct rows' channels 64 cc .. of the tile -> LDS
+  auto stage_chunk = [&](int cc) {
     // every wave is done with the chunk before (and, the first time, s_u is complete)
     __syncthreads();
 #pragma unroll
@@ -154,6 +153,12 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+  };
+  const int nfull = cin >> 6;                                // whole 64-channel chunks
+  load_a(0, 0, A[0]);
+  load_a(0, 1, A[1]);
+  for (int cc = 0; cc < nfull; ++cc) {
+    stage_chunk(cc);
     load_pos(0, pvc);
     read_b(pvc, 0, Bb[0]);
     for (int k = 0; k < K; ++k) {
@@ -175,6 +180,39 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
       }
 #pragma unroll
       for (int rb = 0; rb < 4; ++rb) pvc[rb] = pvn[rb];
+    }
+  }
+  if (nfull < ncc) {
+    // Half a chunk at the end (cin % 64 == 32): two k-steps per slot instead of four.  The
+    // weights of a slot sit in one pair of the ring while the next slot's go into the other,
+    // so the slots are taken two at a time (the chunk before left the first pair filled).
+    const int cc = nfull;
+    stage_chunk(cc);
+    load_pos(0, pvc);
+    read_b(pvc, 0, Bb[0]);
+    auto half_slot = [&](int k, auto ring) {
+      constexpr int r = decltype(ring)::value;               // this slot's pair of the ring: 0 or 2
+      const int kk = cc * K + k;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        if (s == 0) load_pos(k + 1 < K ? k + 1 : 0, pvn);
+        load_a(kk + 1, s, A[(r ^ 2) + s]);
+        if (s == 0) read_b(pvc, 1, Bb[1]);
+        else read_b(pvn, 0, Bb[0]);                          // (past the last slot: unused)
+        if (active) {
+#pragma unroll
+          for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[r + s][mb], Bb[s][rb], acc[rb][mb]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int rb = 0; rb < 4; ++rb) pvc[rb] = pvn[rb];
+    };
+    for (int k = 0; k < K; k += 2) {
+      half_slot(k, std::integral_constant<int, 0>{});
+      if (k + 1 < K) half_slot(k + 1, std::integral_constant<int, 2>{});
     }
   }
 
