@@ -7,7 +7,9 @@ bench.py's): synthetic batch of 8 clouds x 150 000 points at depth 9, input sign
 (normals + displacement), 10 classes, random weights, cross-entropy against random labels.
 
 One JSON line: ms per forward + backward, and the share of the step spent in each kind of
-kernel when --profile is given (torch profiler, device time).
+kernel when --profile is given (torch profiler, device time).  ms_per_step is the step on a
+resident octree; ms_octree_build_and_tables + ms_first_step_on_a_fresh_octree is what a step costs
+when every batch brings a new octree (the plans of its tables are built inside that step).
 """
 
 import argparse
@@ -77,9 +79,13 @@ def main():
 
   pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, args.batch, 1004, n=args.points)
   pc = Points(pts.to(dev), nrm.to(dev), batch_id=bid.to(dev), batch_size=args.batch)
-  octree = Octree(args.depth, 2, batch_size=args.batch)
-  octree.build_octree(pc)
-  octree.construct_all_neigh()
+  def build():
+    o = Octree(args.depth, 2, batch_size=args.batch)
+    o.build_octree(pc)
+    o.construct_all_neigh()
+    return o
+
+  octree = build()
   feat = octree.get_input_feature('ND', nempty).to(dtype)
   query = torch.cat([(pts.to(dev) + 1.0) * (2 ** (args.depth - 1)), bid.to(dev).float().view(-1, 1)], 1)
   labels = torch.randint(0, 10, (query.shape[0],), generator=torch.Generator().manual_seed(5)).to(dev)
@@ -87,7 +93,7 @@ def main():
   net = UNet(feat.shape[1], 10).to(dev).to(dtype)
   params = [p for p in net.parameters()]
 
-  def step():
+  def step(octree=octree):
     for p in params:
       p.grad = None
     logits = net(feat, octree, args.depth, query)
@@ -107,7 +113,21 @@ def main():
     step()
   torch.cuda.synchronize()
   ms = (time.perf_counter() - t0) / args.steps * 1e3
-  out = {'net': 'U-Net (ocnn/models/unet.py), forward + backward', 'ms_per_step': ms, 'dtype': args.dtype,
+  # a training loop sees a new octree every step: build, tables, plans and the step on it
+  fresh = []
+  for _ in range(3):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    o = build()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    step(o)
+    torch.cuda.synchronize()
+    fresh.append(((t1 - t0) * 1e3, (time.perf_counter() - t1) * 1e3))
+  fresh.sort(key=lambda v: v[0] + v[1])
+  out = {'net': 'U-Net (ocnn/models/unet.py), forward + backward', 'ms_per_step': ms,
+         'ms_octree_build_and_tables': fresh[1][0], 'ms_first_step_on_a_fresh_octree': fresh[1][1],
+         'dtype': args.dtype,
          'nempty': nempty, 'batch': args.batch, 'points': int(pts.shape[0]), 'depth': args.depth,
          'rows_per_depth': (octree.nnum_nempty if nempty else octree.nnum).tolist(),
          'parameters': sum(p.numel() for p in params)}

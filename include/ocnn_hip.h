@@ -174,8 +174,15 @@ int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
  * table rows, the ascending list of distinct rows the tile reads, and for every
  * table entry its position in that list plus one (0 for -1).  Lets a kernel bring
  * each distinct row into LDS once per tile instead of once per (row, slot).
- *   count: ucount[tile] = number of distinct rows        (tiles = ceil(rows / R))
- *   fill : uptr (tiles + 1) = exclusive prefix sum of ucount, made by the caller;
+ *   count: ucount[tile] = number of distinct rows        (tiles = ceil(rows / R));
+ *          tile_nnz[tile] (may be NULL) = entries of the tile that hold a row;
+ *   offsets: uptr (tiles + 1) = exclusive prefix sum of ucount, and what the host needs to
+ *          size the lists, stats (device, 5 x int64) = [tiles with more than cap distinct
+ *          rows, dropped (0 | 1), total, largest count, entries set].  When the tiles over
+ *          cap are few (at most a tenth of the tiles, at least one) they are dropped: they
+ *          count as empty in uptr and in the last three figures, and the caller runs their
+ *          rows without the plan;
+ *   fill : uptr as made by offsets (or by the caller);
  *          urows[uptr[tile] + u] = u-th distinct row; loc (tiles, K, R) uint16:
  *          loc[tile][k][r] = 1 + position of table[tile * R + r][k], or 0 for -1 and
  *          for the rows of the last tile past the table.
@@ -183,7 +190,9 @@ int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
  * (ocnn/nn/kernels/conv_fwd_implicit_gemm.py:57-72). */
 int ocnn_tile_plan_rows(void);
 int ocnn_tile_plan_count(const int32_t* table, int64_t rows, int K, int32_t* ucount,
-                         void* stream);
+                         int32_t* tile_nnz, void* stream);
+int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile_nnz, int64_t tiles, int cap,
+                           int32_t* uptr, int64_t* stats, void* stream);
 int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
                         int32_t* urows, uint16_t* loc, void* stream);
 

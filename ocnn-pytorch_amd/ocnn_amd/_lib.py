@@ -40,7 +40,8 @@ SIGNATURES = {
     'ocnn_conv_gather_workspace_bytes': (_l, [_i, _l, _i, _i, _i]),
     'ocnn_conv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _i, _i, _p, _p, _p, _l, _p]),
     'ocnn_tile_plan_rows': (_i, []),
-    'ocnn_tile_plan_count': (_i, [_p, _l, _i, _p, _p]),
+    'ocnn_tile_plan_count': (_i, [_p, _l, _i, _p, _p, _p]),
+    'ocnn_tile_plan_offsets': (_i, [_p, _p, _l, _i, _p, _p, _p]),
     'ocnn_tile_plan_fill': (_i, [_p, _l, _i, _p, _p, _p, _p]),
     'ocnn_conv_gather_planned_supported': (_i, [_i, _l, _i, _i]),
     'ocnn_conv_gather_planned': (_i, [_i, _p, _l, _p, _p, _p, _l, _i, _p, _i, _i, _i, _i, _p, _p,

@@ -18,7 +18,7 @@ __device__ __forceinline__ int plan_hash(int32_t v) {
   return (int)(((uint32_t)v * 2654435761u) >> 19);      // 13 bits
 }
 
-// mode 0: ucount[tile] = number of distinct valid entries
+// mode 0: ucount[tile] = number of distinct valid entries, tile_nnz[tile] = valid entries
 // mode 1: urows[uptr[tile] + u] = u-th distinct row; loc[tile][k][row in tile] = u + 1, or
 //         0 for an empty entry (also for the rows of the last tile that lie past the table)
 //
@@ -28,8 +28,9 @@ __device__ __forceinline__ int plan_hash(int32_t v) {
 __global__ __launch_bounds__(256) void tile_plan_kernel(
     const int32_t* __restrict__ table, int64_t rows, int K, int mode,
     int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, int32_t* __restrict__ urows,
-    uint16_t* __restrict__ loc) {
+    uint16_t* __restrict__ loc, int32_t* __restrict__ tile_nnz) {
   __shared__ int32_t s_key[kPlanHash];
+  __shared__ int32_t s_nnz;
   __shared__ uint16_t s_val[kPlanHash];
   __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];
   __shared__ int32_t s_scan[256];
@@ -48,10 +49,17 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
     ent[i] = (e < n && e0 + e < lim) ? table[e0 + e] : -1;
   }
   for (int i = tid; i < kPlanHash; i += 256) s_key[i] = -1;
+  if (tid == 0) s_nnz = 0;
 #pragma unroll
   for (int i = 0; i < kPer; ++i)
     if (tid + 256 * i < n) s_tab[tid + 256 * i] = ent[i];
   __syncthreads();
+  if (mode == 0 && tile_nnz != nullptr) {
+    int set = 0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) set += ent[i] >= 0 ? 1 : 0;
+    atomicAdd(&s_nnz, set);
+  }
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
     const int32_t v = ent[i];
@@ -85,7 +93,10 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
   }
   const int total = s_scan[255];
   if (mode == 0) {
-    if (tid == 0) ucount[tile] = total;
+    if (tid == 0) {
+      ucount[tile] = total;
+      if (tile_nnz != nullptr) tile_nnz[tile] = s_nnz;
+    }
     return;
   }
   int pos = s_scan[tid] - cnt;
@@ -208,13 +219,76 @@ __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles
   if (n + lane < padded) e[n + lane] = entry(0u, kPlanRows);                 // the zero row, to a spare row
 }
 
+// What the host needs to know of the counts, and the offsets of the row lists, in one
+// workgroup (a table has tens of thousands of tiles at most).  Tiles with more than `cap`
+// distinct rows are dropped (counted as empty) when they are few: at most a tenth of the
+// tiles.  stats: [tiles over cap, dropped (0 | 1), total, largest count, entries set], the
+// last three without the dropped tiles.
+__global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
+    const int32_t* __restrict__ ucount, const int32_t* __restrict__ tile_nnz, int64_t tiles, int cap,
+    int32_t* __restrict__ uptr, int64_t* __restrict__ stats) {
+  __shared__ long long s_sum[1024];
+  __shared__ int s_big, s_max;
+  __shared__ long long s_nnz;
+  const int tid = threadIdx.x;
+  const int64_t per = (tiles + 1023) / 1024;
+  const int64_t t0 = min(tiles, tid * per), t1 = min(tiles, t0 + per);
+  if (tid == 0) { s_big = 0; s_max = 0; s_nnz = 0; }
+  __syncthreads();
+  int big = 0;
+  for (int64_t t = t0; t < t1; ++t) big += ucount[t] > cap ? 1 : 0;
+  if (big) atomicAdd(&s_big, big);
+  __syncthreads();
+  const int n_big = s_big;
+  const bool drop = n_big > 0 && n_big <= max((int64_t)1, tiles / 10);
+  long long sum = 0, nnz = 0;
+  int mx = 0;
+  for (int64_t t = t0; t < t1; ++t) {
+    const int c = ucount[t];
+    if (drop && c > cap) continue;
+    sum += c;
+    mx = max(mx, c);
+    nnz += tile_nnz[t];
+  }
+  s_sum[tid] = sum;
+  atomicMax(&s_max, mx);
+  atomicAdd((unsigned long long*)&s_nnz, (unsigned long long)nnz);
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const long long v = tid >= off ? s_sum[tid - off] : 0;
+    __syncthreads();
+    s_sum[tid] += v;
+    __syncthreads();
+  }
+  long long at = s_sum[tid] - sum;
+  for (int64_t t = t0; t < t1; ++t) {
+    uptr[t] = (int32_t)at;
+    const int c = ucount[t];
+    at += (drop && c > cap) ? 0 : c;
+  }
+  if (tid == 1023) {
+    uptr[tiles] = (int32_t)s_sum[1023];
+    stats[0] = n_big;
+    stats[1] = drop ? 1 : 0;
+    stats[2] = s_sum[1023];
+    stats[3] = s_max;
+    stats[4] = s_nnz;
+  }
+}
+
+__global__ void pair_plan_zero_kernel(unsigned long long* __restrict__ slot_count, int K) {
+  if ((int)threadIdx.x < K) slot_count[threadIdx.x] = 0;
+}
+
 __global__ void pair_plan_slot_count_kernel(const uint16_t* __restrict__ loc, int64_t tiles, int K,
                                             unsigned long long* __restrict__ slot_count) {
-  // one workgroup per slot: the sum over all tiles in a fixed order
+  // workgroup (k, y): slot k over the tiles y, y + gridDim.y, ..; integer sums, so the order
+  // in which the workgroups add theirs does not show in the result
   __shared__ unsigned long long s_part[256];
   const int k = blockIdx.x;
   unsigned long long acc = 0;
-  for (int64_t t = threadIdx.x; t < tiles * (kPlanRows / 8); t += blockDim.x) {
+  const int64_t chunks = tiles * (kPlanRows / 8);
+  for (int64_t t = (int64_t)blockIdx.y * blockDim.x + threadIdx.x; t < chunks; t += (int64_t)gridDim.y * blockDim.x) {
     const int64_t tile = t / (kPlanRows / 8);
     const int c = (int)(t - tile * (kPlanRows / 8));
     const u32x4 v = *(const u32x4*)(loc + (tile * K + k) * kPlanRows + 8 * c);
@@ -227,7 +301,7 @@ __global__ void pair_plan_slot_count_kernel(const uint16_t* __restrict__ loc, in
     if ((int)threadIdx.x < s) s_part[threadIdx.x] += s_part[threadIdx.x + s];
     __syncthreads();
   }
-  if (threadIdx.x == 0) slot_count[k] = s_part[0];
+  if (threadIdx.x == 0 && s_part[0] != 0) atomicAdd(&slot_count[k], s_part[0]);
 }
 
 }  // namespace ocnn
@@ -237,29 +311,40 @@ using namespace ocnn;
 extern "C" int ocnn_tile_plan_rows(void) { return kPlanRows; }
 
 static int plan_launch(const int32_t* table, int64_t rows, int K, int mode, int32_t* ucount,
-                       const int32_t* uptr, int32_t* urows, uint16_t* loc, void* stream) {
+                       const int32_t* uptr, int32_t* urows, uint16_t* loc, int32_t* tile_nnz, void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows >= 0 && rows < (1ll << 31), "tile_plan: bad shape");
   if (rows == 0) return OCNN_OK;
   int64_t tiles = cdiv(rows, kPlanRows);
   hipLaunchKernelGGL(tile_plan_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream,
-                     table, rows, K, mode, ucount, uptr, urows, loc);
+                     table, rows, K, mode, ucount, uptr, urows, loc, tile_nnz);
   return check_launch("tile_plan");
 }
 
 extern "C" int ocnn_tile_plan_count(const int32_t* table, int64_t rows, int K, int32_t* ucount,
-                                    void* stream) {
-  return plan_launch(table, rows, K, 0, ucount, nullptr, nullptr, nullptr, stream);
+                                    int32_t* tile_nnz, void* stream) {
+  return plan_launch(table, rows, K, 0, ucount, nullptr, nullptr, nullptr, tile_nnz, stream);
+}
+
+extern "C" int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile_nnz, int64_t tiles, int cap,
+                                      int32_t* uptr, int64_t* stats, void* stream) {
+  OCNN_REQUIRE(tiles >= 0 && tiles < (1ll << 31) && cap >= 0, "tile_plan_offsets: bad shape");
+  hipLaunchKernelGGL(tile_plan_offsets_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ucount, tile_nnz,
+                     tiles, cap, uptr, stats);
+  return check_launch("tile_plan_offsets");
 }
 
 extern "C" int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
                                    int32_t* urows, uint16_t* loc, void* stream) {
-  return plan_launch(table, rows, K, 1, nullptr, uptr, urows, loc, stream);
+  return plan_launch(table, rows, K, 1, nullptr, uptr, urows, loc, nullptr, stream);
 }
 
 extern "C" int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,
                                           void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 24), "pair_plan: bad shape");
-  hipLaunchKernelGGL(pair_plan_slot_count_kernel, dim3((unsigned)K), dim3(256), 0, (hipStream_t)stream, loc,
+  hipLaunchKernelGGL(pair_plan_zero_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream,
+                     (unsigned long long*)slot_count, K);
+  const unsigned gy = (unsigned)std::max<int64_t>(1, std::min<int64_t>(64, cdiv(tiles, 16)));
+  hipLaunchKernelGGL(pair_plan_slot_count_kernel, dim3((unsigned)K, gy), dim3(256), 0, (hipStream_t)stream, loc,
                      tiles, K, (unsigned long long*)slot_count);
   return check_launch("pair_plan_slot_counts");
 }

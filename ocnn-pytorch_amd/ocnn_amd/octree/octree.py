@@ -111,49 +111,79 @@ class TilePlan:
   rows.  A handful of denser tiles must not send a whole level to the plan-free kernels: when
   at most a tenth of the tiles are over the limit, those tiles are emptied in the plan (as if
   their table rows were all -1) and their rows listed in `overflow_rows` / `overflow_table`;
-  the Python layer runs them through the plan-free kernels and puts the results in place."""
+  the Python layer runs them through the plan-free kernels and puts the results in place.
+
+  Building a plan needs sizes on the host (the length of the row lists); `build_many` makes
+  the plans of several tables with ONE read-back for all of them, which is what a fresh octree
+  in the middle of a training step wants: every read-back waits for the whole queue of kernels
+  before it and leaves the device idle while the host catches up."""
 
   CAP = 415      # the smallest limit of the kernels on the plan
 
   def __init__(self, table: torch.Tensor, cap: int = None):
+    self._count(table, cap)
+    self._finish([int(v) for v in self._stats.tolist()])
+
+  @classmethod
+  def build_many(cls, tables, cap: int = None):
+    """Plans of several tables with one device -> host read-back."""
+    plans = [cls.__new__(cls) for _ in tables]
+    for p, t in zip(plans, tables):
+      p._count(t, cap)
+    host = torch.stack([p._stats for p in plans]).tolist() if plans else []
+    for p, st in zip(plans, host):
+      p._finish([int(v) for v in st])
+    return plans
+
+  def _count(self, table, cap):
+    """First half: distinct rows per tile, their offsets, and the sizes the second half
+    needs on the host as one device vector."""
     _lib.require_gpu(table)
     L = _lib.lib()
     table = table.contiguous()
     rows, K = table.shape
-    tile_rows = L.ocnn_tile_plan_rows()
-    tiles = (rows + tile_rows - 1) // tile_rows
-    dev = table.device
-    st = _lib.stream()
-    cap = self.CAP if cap is None else cap
+    self._tile_rows = L.ocnn_tile_plan_rows()
+    tiles = (rows + self._tile_rows - 1) // self._tile_rows
+    self._cap = self.CAP if cap is None else cap
+    self._table = table
+    self.rows, self.K = rows, K
     self.overflow_rows = self.overflow_table = None
-    ucount = torch.zeros(tiles, dtype=torch.int32, device=dev)
-    _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(ucount), st))
-    if tiles > 0:
-      big = ucount > cap
-      n_big = int(big.sum())
-      if 0 < n_big <= max(1, tiles // 10):
-        idx = (big.nonzero().view(-1, 1) * tile_rows + torch.arange(tile_rows, device=dev).view(1, -1)).view(-1)
-        idx = idx[idx < rows]
-        self.overflow_rows = idx
-        self.overflow_table = table.index_select(0, idx).contiguous()
-        table = table.clone()
-        table[idx] = -1
-        ucount = torch.where(big, torch.zeros_like(ucount), ucount)
-    uptr = torch.zeros(tiles + 1, dtype=torch.int32, device=dev)
-    uptr[1:] = torch.cumsum(ucount, 0)
-    total, umax, nnz = (int(v) for v in torch.stack(
-        [uptr[-1], ucount.max(), (table >= 0).sum().int()]).tolist()) if tiles > 0 else (0, 0, 0)
+    self._pairs = None
+    self._on_pairs = None          # called when the pair plan is first asked for
+    dev, st = table.device, _lib.stream()
+    self._ucount = torch.empty(tiles, dtype=torch.int32, device=dev)
+    tile_nnz = torch.empty(tiles, dtype=torch.int32, device=dev)
+    self.uptr = torch.empty(tiles + 1, dtype=torch.int32, device=dev)
+    self._stats = torch.empty(5, dtype=torch.int64, device=dev)
+    _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(self._ucount), _lib.ptr(tile_nnz), st))
+    _lib.check(L.ocnn_tile_plan_offsets(_lib.ptr(self._ucount), _lib.ptr(tile_nnz), tiles, self._cap,
+                                        _lib.ptr(self.uptr), _lib.ptr(self._stats), st))
+
+  def _finish(self, stats):
+    """Second half, with the sizes on the host: row lists and positions."""
+    L = _lib.lib()
+    table, tile_rows = self._table, self._tile_rows
+    rows, K = self.rows, self.K
+    tiles = self._ucount.numel()
+    dev = table.device
+    _, dropped, total, umax, nnz = stats
+    if dropped:
+      big = self._ucount > self._cap
+      idx = (big.nonzero().view(-1, 1) * tile_rows + torch.arange(tile_rows, device=dev).view(1, -1)).view(-1)
+      idx = idx[idx < rows]
+      self.overflow_rows = idx
+      self.overflow_table = table.index_select(0, idx).contiguous()
+      table = table.clone()
+      table[idx] = -1
     # how often a staged row is used by its tile: near 1 there is nothing to gain from staging
     self.reuse = nnz / max(total, 1)
-    self.uptr = uptr
     self.urows = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
     # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"
     self.loc = torch.empty((tiles, K, tile_rows), dtype=torch.int16, device=dev)
-    _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(uptr),
-                                     _lib.ptr(self.urows), _lib.ptr(self.loc), st))
-    self.rows, self.K, self.total, self.umax = rows, K, total, umax
-    self.nnz = nnz
-    self._pairs = None
+    _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(self.uptr),
+                                     _lib.ptr(self.urows), _lib.ptr(self.loc), _lib.stream()))
+    self.total, self.umax, self.nnz = total, umax, nnz
+    self._table = self._ucount = self._stats = None
 
   @property
   def occupancy(self):
@@ -165,23 +195,54 @@ class TilePlan:
     and slot the rows that have a neighbour, in blocks of 16 entries."""
     if self._pairs is None:
       self._pairs = PairPlan(self)
+      if self._on_pairs is not None:
+        self._on_pairs()
     return self._pairs
 
 
 class PairPlan:
   """Blocks of 16 (row, neighbour) pairs per tile and list of a table; a list is a slot, or
   a range of the tiles' rows of a slot with many pairs; the lists are dealt to four groups
-  of about equal numbers of pairs (see ocnn_pair_plan_* in the C ABI)."""
+  of about equal numbers of pairs (see ocnn_pair_plan_* in the C ABI).  `build_many` makes
+  the pair plans of several tile plans with two read-backs in all."""
 
   def __init__(self, plan: TilePlan):
-    import ctypes
+    self._slot_counts(plan)
+    self._lists(self._counts.tolist())
+    self._finish([int(v) for v in self._sizes.tolist()] if self._sizes is not None else None)
+
+  @classmethod
+  def build_many(cls, plans):
+    out = [cls.__new__(cls) for _ in plans]
+    for pp, plan in zip(out, plans):
+      pp._slot_counts(plan)
+    host = torch.cat([pp._counts for pp in out]).tolist() if out else []
+    at = 0
+    for pp in out:
+      pp._lists(host[at:at + pp._K])
+      at += pp._K
+    sizes = [pp._sizes for pp in out if pp._sizes is not None]
+    host = torch.stack(sizes).tolist() if sizes else []
+    it = iter(host)
+    for pp in out:
+      pp._finish([int(v) for v in next(it)] if pp._sizes is not None else None)
+    return out
+
+  def _slot_counts(self, plan):
     L = _lib.lib()
-    tiles, K, _ = plan.loc.shape
+    self._plan = plan
+    self._tiles, self._K, _ = plan.loc.shape
+    self._counts = torch.zeros(self._K, dtype=torch.int64, device=plan.loc.device)
+    _lib.check(L.ocnn_pair_plan_slot_counts(_lib.ptr(plan.loc), self._tiles, self._K, _lib.ptr(self._counts),
+                                            _lib.stream()))
+
+  def _lists(self, counts):
+    """With the pairs per slot on the host: the lists and their groups, then the number of
+    blocks per (tile, list)."""
+    L = _lib.lib()
+    plan, tiles, K = self._plan, self._tiles, self._K
     dev = plan.loc.device
-    st = _lib.stream()
-    counts = torch.zeros(K, dtype=torch.int64, device=dev)
-    _lib.check(L.ocnn_pair_plan_slot_counts(_lib.ptr(plan.loc), tiles, K, _lib.ptr(counts), st))
-    per_slot = (ctypes.c_int64 * K)(*counts.tolist())
+    per_slot = (ctypes.c_int64 * K)(*[int(c) for c in counts])
     # host arrays, kept alive with the plan: the C ABI reads them at every call
     self.lists_host = (ctypes.c_int32 * 32)()
     self.list_count_host = (ctypes.c_int64 * 32)()
@@ -191,16 +252,24 @@ class PairPlan:
                                       ctypes.addressof(self.list_count_host),
                                       ctypes.addressof(self.group_bounds_host), ctypes.addressof(n_lists)))
     nl = self.n_lists = n_lists.value
-    self.lists = torch.tensor(list(self.lists_host)[:nl], dtype=torch.int32, device=dev)
+    self.lists = torch.tensor(list(self.lists_host)[:nl], dtype=torch.int32).to(dev, non_blocking=True)
     nblk = torch.zeros(max(tiles * nl, 1), dtype=torch.int32, device=dev)
-    _lib.check(L.ocnn_pair_plan_count(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.lists), nl, _lib.ptr(nblk), st))
+    _lib.check(L.ocnn_pair_plan_count(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.lists), nl, _lib.ptr(nblk),
+                                      _lib.stream()))
     self.cptr = torch.zeros(tiles * nl + 1, dtype=torch.int32, device=dev)
-    self.cptr[1:] = torch.cumsum(nblk[:tiles * nl], 0)
-    self.n_blocks, self.max_blocks = (int(v) for v in torch.stack(
-        [self.cptr[-1], nblk[:tiles * nl].view(tiles, nl).sum(1).max().int()]).tolist()) if tiles > 0 else (0, 0)
-    self.ent = torch.empty(max(self.n_blocks, 1) * 16, dtype=torch.int32, device=dev)
-    _lib.check(L.ocnn_pair_plan_fill(_lib.ptr(plan.loc), tiles, K, _lib.ptr(self.lists), nl, _lib.ptr(self.cptr),
-                                     _lib.ptr(self.ent), st))
+    self._sizes = None
+    if tiles > 0:
+      self.cptr[1:] = torch.cumsum(nblk[:tiles * nl], 0)
+      self._sizes = torch.stack([self.cptr[-1], nblk[:tiles * nl].view(tiles, nl).sum(1).max().int()])
+
+  def _finish(self, sizes):
+    L = _lib.lib()
+    plan = self._plan
+    self.n_blocks, self.max_blocks = sizes if sizes is not None else (0, 0)
+    self.ent = torch.empty(max(self.n_blocks, 1) * 16, dtype=torch.int32, device=plan.loc.device)
+    _lib.check(L.ocnn_pair_plan_fill(_lib.ptr(plan.loc), self._tiles, self._K, _lib.ptr(self.lists), self.n_lists,
+                                     _lib.ptr(self.cptr), _lib.ptr(self.ent), _lib.stream()))
+    self._plan = self._counts = self._sizes = None
 
 
 class Octree:
@@ -230,6 +299,7 @@ class Octree:
     self._tables = {}        # (depth, kernel, stride, nempty) -> int32 table
     self._tables_t = {}      # same key -> inverse table
     self._plans = {}         # (key, inverse) -> TilePlan
+    self._plans_prebuilt = False
 
     self.nnum = torch.zeros(num, dtype=torch.long)
     self.nnum_nempty = torch.zeros(num, dtype=torch.long)
@@ -421,6 +491,7 @@ class Octree:
     self.nempty_neighs = [None] * num
     self._nempty_indices32 = [None] * num
     self._tables, self._tables_t, self._plans = {}, {}, {}
+    self._plans_prebuilt = False
     return idx
 
   def octree_grow_full(self, depth: int, update_neigh: bool = True):
@@ -568,14 +639,53 @@ class Octree:
       self._tables_t[ck] = out
     return self._tables_t[ck]
 
+  # Plans asked for by earlier octrees of the same (depth, full_depth): a network asks every
+  # octree for the same plans, layer by layer, and each plan built on its own costs two
+  # device -> host read-backs in the middle of the step.  The first request on a fresh octree
+  # therefore builds all the plans its predecessors were asked for, together.
+  PREBUILD_PLANS = True
+  _plan_requests = {}        # (depth, full_depth) -> {plan key: {'pairs': bool}}
+
   def _plan(self, depth, kernel, stride, nempty, inverse=False, rows_in=None):
     """Tile plan of the table (or of its inverse), cached with the table."""
     ck = ((depth, kernel, stride, bool(nempty)), bool(inverse))
     if ck not in self._plans:
-      t = (self._table_t(depth, kernel, stride, nempty, rows_in) if inverse
-           else self._table(depth, kernel, stride, nempty))
-      self._plans[ck] = TilePlan(t)
+      requests = Octree._plan_requests.setdefault((self.depth, self.full_depth), {})
+      if Octree.PREBUILD_PLANS and requests and not self._plans_prebuilt:
+        self._plans_prebuilt = True
+        self._prebuild_plans(requests)
+      if ck not in self._plans:
+        t = (self._table_t(depth, kernel, stride, nempty, rows_in) if inverse
+             else self._table(depth, kernel, stride, nempty))
+        self._plans[ck] = TilePlan(t)
+      known = rows_in is None or rows_in == self._fine_rows(depth, nempty)
+      if ck not in requests and known:
+        requests[ck] = {'pairs': False}
+      if ck in requests:
+        entry = requests[ck]
+        plan = self._plans[ck]
+        if plan._pairs is None:
+          plan._on_pairs = lambda: entry.__setitem__('pairs', True)
     return self._plans[ck]
+
+  def _fine_rows(self, depth, nempty):
+    """Rows on the side of a table that its entries index (all tables of this class: the
+    nodes of `depth`, or the non-empty ones)."""
+    return int(self.nnum_nempty[depth] if nempty else self.nnum[depth])
+
+  def _prebuild_plans(self, requests):
+    keys = [ck for ck in requests if ck not in self._plans and ck[0][0] <= self.depth and
+            self.neighs.has(ck[0][0])]
+    tables = []
+    for (depth, kernel, stride, nempty), inverse in keys:
+      tables.append(self._table_t(depth, kernel, stride, nempty, self._fine_rows(depth, nempty)) if inverse
+                    else self._table(depth, kernel, stride, nempty))
+    plans = TilePlan.build_many(tables)
+    for ck, plan in zip(keys, plans):
+      self._plans[ck] = plan
+    with_pairs = [plan for ck, plan in zip(keys, plans) if requests[ck]['pairs']]
+    for plan, pp in zip(with_pairs, PairPlan.build_many(with_pairs)):
+      plan._pairs = pp
 
   @staticmethod
   def _widen(t32):

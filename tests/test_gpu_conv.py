@@ -319,6 +319,83 @@ def test_tile_plan_reconstructs_table(medium):
       assert np.array_equal(u[lb[blk >= 0] - 1], blk[blk >= 0])
 
 
+def _same_plan(a, b):
+  assert (a.rows, a.K, a.total, a.umax, a.nnz) == (b.rows, b.K, b.total, b.umax, b.nnz)
+  assert torch.equal(a.uptr, b.uptr) and torch.equal(a.urows[:a.total], b.urows[:b.total]) and torch.equal(a.loc, b.loc)
+  assert (a.overflow_rows is None) == (b.overflow_rows is None)
+  if a.overflow_rows is not None:
+    assert torch.equal(a.overflow_rows, b.overflow_rows) and torch.equal(a.overflow_table, b.overflow_table)
+
+
+def _same_pairs(a, b):
+  assert (a.n_lists, a.n_blocks, a.max_blocks) == (b.n_lists, b.n_blocks, b.max_blocks)
+  assert list(a.lists_host) == list(b.lists_host) and list(a.list_count_host) == list(b.list_count_host)
+  assert list(a.group_bounds_host) == list(b.group_bounds_host)
+  assert torch.equal(a.lists, b.lists) and torch.equal(a.cptr, b.cptr)
+  assert torch.equal(a.ent[:16 * a.n_blocks], b.ent[:16 * b.n_blocks])
+
+
+def test_plans_built_together_equal_plans_built_alone(medium):
+  say('tile plans and pair plans: one read-back for several tables gives the same plans')
+  from ocnn_amd.octree.octree import PairPlan, TilePlan
+  o = medium.gpu
+  tables = [o._table(7, '333', 1, False), o._table(7, '333', 1, True), o._table(7, '222', 2, True),
+            o._table_t(7, '222', 2, True, int(o.nnum_nempty[7])), o._table(6, '313', 1, True),
+            torch.empty((0, 27), dtype=torch.int32, device=DEV)]
+  alone = [TilePlan(t) for t in tables]
+  together = TilePlan.build_many(tables)
+  for a, b in zip(alone, together):
+    _same_plan(a, b)
+  # a low staging limit: some tiles overflow (emptied in the plan), and one table has too many
+  counts = (alone[1].uptr[1:] - alone[1].uptr[:-1]).float()
+  cap = int(torch.quantile(counts, 0.97))
+  alone = [TilePlan(t, cap=cap) for t in tables]
+  together = TilePlan.build_many(tables, cap=cap)
+  assert any(p.overflow_rows is not None for p in alone)
+  for a, b in zip(alone, together):
+    _same_plan(a, b)
+  for a, b in zip([PairPlan(p) for p in alone], PairPlan.build_many(together)):
+    _same_pairs(a, b)
+
+
+def test_fresh_octree_builds_the_plans_of_its_predecessors(medium):
+  say('plans: a fresh octree builds what earlier octrees were asked for, at its first request')
+  def fresh():
+    o = Octree(7, 2, batch_size=3)
+    pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 3, 11, n=40000)
+    o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=3))
+    o.construct_all_neigh()
+    return o
+  saved = Octree._plan_requests
+  Octree._plan_requests = {}
+  try:
+    first = fresh()
+    keys = [(7, '333', 1, True, False), (6, '333', 1, True, False), (7, '222', 2, True, False),
+            (7, '222', 2, True, True), (5, '333', 1, False, False)]
+    for d, k, s, ne, inv in keys:
+      p = first._plan(d, k, s, ne, inv, first._fine_rows(d, ne))
+      if d == 7 and k == '333':
+        p.pairs()
+    assert len(first._plans) == len(keys)
+    second = fresh()
+    assert not second._plans
+    second._plan(5, '333', 1, False, False, None)            # any request builds all of them
+    assert set(second._plans) == set(first._plans)
+    for ck, p in first._plans.items():
+      _same_plan(p, second._plans[ck])
+      assert (p._pairs is None) == (second._plans[ck]._pairs is None)
+      if p._pairs is not None:
+        _same_pairs(p._pairs, second._plans[ck]._pairs)
+    # switched off: plans are built one by one, on request
+    Octree.PREBUILD_PLANS = False
+    third = fresh()
+    third._plan(5, '333', 1, False, False, None)
+    assert len(third._plans) == 1
+  finally:
+    Octree.PREBUILD_PLANS = True
+    Octree._plan_requests = saved
+
+
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 def test_staged_kernel_many_passes(dtype):
   """A table with no locality: tiles need far more distinct rows than fit in
