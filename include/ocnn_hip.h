@@ -310,7 +310,9 @@ int ocnn_conv_dense(int dtype, const void* in, int64_t rows, const void* w, int 
 /* The same GEMM, and its weight gradient gw (ca, cb) [or (cb, ca)] = x^T g, with what is
  * reused kept in registers by persistent workgroups (weights, resp. the fp32 sums), so that
  * each tensor crosses L2 once: cin in {64, 128, 256, 512}, cout % 128 == 0; weight gradient
- * for ca % 512 == 0 and cb % 128 == 0, both % 256 == 0, or ca % 128 == 0 and cb % 512 == 0. */
+ * for any ca, cb that are multiples of 8 (summed in blocks of 512 x 128, 256 x 256 or
+ * 128 x 512 channel pairs, whichever covers ca x cb with the fewest; the channels a block
+ * has past ca or cb are staged as zeros and not written). */
 int ocnn_conv_dense_rw_supported(int dtype, int64_t rows, int cin, int cout);
 int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
                        int w_transposed, const void* bias, void* out, void* workspace,

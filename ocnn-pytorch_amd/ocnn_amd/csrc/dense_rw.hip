@@ -6,7 +6,8 @@
 //     input channels x its 32 MB output channels) and stream 64-row tiles through a ring of
 //     two to four buffers in LDS;
 //   * dW = in^T g: persistent workgroups keep a 512 x 128 (or 256 x 256, 128 x 512) block of
-//     fp32 sums in accumulator registers (256 per lane) and stream 32-row tiles of both
+//     fp32 sums in accumulator registers (256 per lane; smaller layers fill a part of one
+//     block, the rest is staged as zeros: the pass is bound by HBM) and stream 32-row tiles of both
 //     operands through a ring of three LDS buffers; per-range sums go to the split reduction
 //     (fixed order, no atomics).
 #include <algorithm>
@@ -167,6 +168,8 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
 // of the rows 2, 3 (mod 4) are swapped, so that the four rows of a transposing read fall
 // on different banks.  Both operands are read with ds_read_b64_tr_b16.
 // ---------------------------------------------------------------------------------------
+// (Blocks at the edges multiply the zeros staged past the channels like everything else:
+// skipping those 32 x 32 pieces with wave-uniform branches made the kernel slower.)
 template <typename T, int WA>
 __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
     const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes, int ca, int cb,
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave / WB, wb = wave % WB;
-  const int nbb = cb / (128 * WB);
+  const int nbb = (cb + 128 * WB - 1) / (128 * WB);   // blocks at the edges may hold fewer channels
   const int blk_a = (int)blockIdx.y / nbb, blk_b = (int)blockIdx.y % nbb;
   const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_split;
   const int64_t t_end = min(tiles, t_begin + tiles_per_split);
@@ -199,8 +202,14 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
       const int grp = i >> 2, rg = i & 3;
       char* dst = buf + (grp * RT + 8 * rg) * 128;
       const uint32_t row = row0 + 8 * rg + rl;
-      if (grp < GA) dr_dma16(rs_x, dst, row * xp + (uint32_t)((blk_a * GA + grp) * 128) + sc);
-      else dr_dma16(rs_g, dst, row * gp + (uint32_t)((blk_b * GB + grp - GA) * 128) + sc);
+      // channels past the end of a row: an offset past the buffer, which reads as zeros
+      if (grp < GA) {
+        const uint32_t cbyte = (uint32_t)((blk_a * GA + grp) * 128) + sc;
+        dr_dma16(rs_x, dst, cbyte < xp ? row * xp + cbyte : 0xffffff00u);
+      } else {
+        const uint32_t cbyte = (uint32_t)((blk_b * GB + grp - GA) * 128) + sc;
+        dr_dma16(rs_g, dst, cbyte < gp ? row * gp + cbyte : 0xffffff00u);
+      }
     }
   };
 
@@ -219,6 +228,8 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
   const uint32_t hsw = 64u * ((rs >> 1) & 1);                      // where the first half of this row lives
   const uint32_t xe = rowb + hsw + (uint32_t)(2 * wa) * (RT * 128), xo = rowb + (64u - hsw) + (uint32_t)(2 * wa) * (RT * 128);
   const uint32_t ge = rowb + hsw + (uint32_t)(GA + 2 * wb) * (RT * 128), go = rowb + (64u - hsw) + (uint32_t)(GA + 2 * wb) * (RT * 128);
+
+  const int a_base = blk_a * 128 * WA + 128 * wa, b_base = blk_b * 128 * WB + 128 * wb;
 
   struct Ops { u32x2 a[4][2], b[4][2]; };
   auto fetch = [&](const char* buf, int sn, Ops& o) {
@@ -269,7 +280,6 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
 
   // ---- per-range sums -> partial[split][a][b] ----
   float* dst = partial + (int64_t)blockIdx.x * ca * cb;
-  const int a_base = blk_a * 128 * WA + 128 * wa, b_base = blk_b * 128 * WB + 128 * wb;
 #pragma unroll
   for (int m = 0; m < 4; ++m)
 #pragma unroll
@@ -277,7 +287,8 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int a = a_base + 32 * m + 8 * (r >> 2) + 4 * q + (r & 3);
-        dst[(int64_t)a * cb + b_base + 32 * n + (lane & 31)] = acc[m][n][r];
+        const int b = b_base + 32 * n + (lane & 31);
+        if (a < ca && b < cb) dst[(int64_t)a * cb + b] = acc[m][n][r];
       }
 }
 
@@ -389,16 +400,22 @@ extern "C" int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const
 
 // ---- weight gradient ----
 // waves along the x channels of a workgroup's block, or 0 if the shape is not taken
+// blocks of 128 WA x 512 / WA channel pairs that cover ca x cb
+static int dr_wgrad_blocks(int ca, int cb, int wa) {
+  return (int)(cdiv(ca, 128 * wa) * cdiv(cb, 512 / wa));
+}
+
+// the block shape with the fewest blocks (ties: the squarer one stages less per tile)
 static int dr_wa(int ca, int cb) {
-  if (ca % 512 == 0 && cb % 128 == 0) return 4;
-  if (ca % 256 == 0 && cb % 256 == 0) return 2;
-  if (ca % 128 == 0 && cb % 512 == 0) return 1;
-  return 0;
+  if (ca < 8 || cb < 8 || ca % 8 != 0 || cb % 8 != 0) return 0;
+  int best = 2;
+  if (dr_wgrad_blocks(ca, cb, 4) < dr_wgrad_blocks(ca, cb, best)) best = 4;
+  if (dr_wgrad_blocks(ca, cb, 1) < dr_wgrad_blocks(ca, cb, best)) best = 1;
+  return best;
 }
 
 static int dr_wgrad_splits(int ca, int cb, int n_cu) {
-  const int blocks = ca * cb / 65536;
-  return std::max(1, n_cu / blocks);
+  return std::max(1, n_cu / dr_wgrad_blocks(ca, cb, dr_wa(ca, cb)));
 }
 
 extern "C" int ocnn_conv_dense_wgrad_rw_supported(int dtype, int64_t rows, int ca, int cb) {
@@ -424,7 +441,7 @@ static void launch_dense_wgrad(const void* x, const void* g, int64_t rows, int c
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     attr_set = true;
   }
-  hipLaunchKernelGGL((conv_dense_wgrad_rw_kernel<T, WA>), dim3((unsigned)nsplit, (unsigned)(ca * cb / 65536)),
+  hipLaunchKernelGGL((conv_dense_wgrad_rw_kernel<T, WA>), dim3((unsigned)nsplit, (unsigned)dr_wgrad_blocks(ca, cb, WA)),
                      dim3(256), lds, st, (const T*)x, (uint32_t)(rows * ca * 2), (const T*)g,
                      (uint32_t)(rows * cb * 2), ca, cb, tiles, per, partial);
 }

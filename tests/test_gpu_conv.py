@@ -505,12 +505,13 @@ def test_dense_rows_kernel(dtype, cin, cout):
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('cin,cout', [(64, 128), (64, 512), (128, 128), (128, 256), (128, 512), (256, 128), (256, 256),
-                                      (512, 128), (512, 384), (1024, 128), (128, 1024)])
+                                      (512, 128), (512, 384), (1024, 128), (128, 1024), (96, 64), (768, 96),
+                                      (64, 16), (128, 96), (384, 256), (72, 40), (256, 32), (8, 8)])
 def test_dense_rows_register_kernels(dtype, cin, cout):
   """The persistent kernels for one-slot identity tables: out = in W + bias with the weights
   in registers (every input width / output blocking they are built with, both weight layouts),
-  and gw = x^T g with the sums in registers (every block shape), ragged row counts, fewer
-  tiles than the ring of buffers holds."""
+  and gw = x^T g with the sums in registers (every block shape, also channel counts that fill
+  only a part of a block), ragged row counts, fewer tiles than the ring of buffers holds."""
   L = _lib.lib()
   g = torch.Generator().manual_seed(3 * cin + cout)
   code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
@@ -533,8 +534,9 @@ def test_dense_rows_register_kernels(dtype, cin, cout):
         assert rel_err(out[:rows], want) < TOL[dtype]
         assert bool((out[rows] == 7.0).all())
     else:
-      assert cin > 512
-    if L.ocnn_conv_dense_wgrad_rw_supported(code, rows, cin, cout):
+      assert cin not in (64, 128, 256, 512) or cout % 128
+    assert L.ocnn_conv_dense_wgrad_rw_supported(code, rows, cin, cout)     # any multiples of 8
+    if True:
       want = f64(x).T @ f64(gr)
       ws = torch.empty(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(cin, cout), dtype=torch.uint8, device=DEV)
       got = []
