@@ -7,6 +7,7 @@ from typing import List
 
 import torch
 import torch.nn
+import torch.nn.functional as F
 
 from .nn import OctreeConv, OctreeDeconv
 from .nn.octree_conv import conv_gather, conv_wgrad, column_sum
@@ -100,6 +101,35 @@ class _RowsLinear(torch.autograd.Function):
     return gx, gw, gb
 
 
+class _RowsLinearNarrow(torch.autograd.Function):
+  """y = x W^T + b for few output channels (a classification head: 64 -> 10 on a million
+  rows).  Output and input gradient are the library's GEMMs; the weight gradient, a sum over
+  all rows into a handful of numbers, is where the library's choice of kernel is slow (0.89 ms
+  for 1.2 M x 64 x 10) and runs on this package's split reduction instead (fixed order)."""
+
+  @staticmethod
+  def forward(ctx, x, weight, bias):
+    x = x.contiguous()
+    ctx.save_for_backward(x, weight)
+    ctx.has_bias = bias is not None
+    return F.linear(x, weight.to(x.dtype), None if bias is None else bias.to(x.dtype))
+
+  @staticmethod
+  def backward(ctx, grad):
+    x, weight = ctx.saved_tensors
+    grad = grad.contiguous()
+    rows = x.shape[0]
+    gx = gw = gb = None
+    if ctx.needs_input_grad[0]:
+      gx = grad @ weight.to(grad.dtype)
+    if ctx.needs_input_grad[1]:
+      gw = conv_wgrad(x, grad, _identity_table(rows, x.device), True, None, dense=True)
+      gw = gw.view(weight.shape).to(weight.dtype)
+    if ctx.has_bias and ctx.needs_input_grad[2]:
+      gb = column_sum(grad)
+    return gx, gw, gb
+
+
 class Conv1x1(torch.nn.Module):
   """ocnn/modules/modules.py:102-117: a 1x1x1 convolution on (N, C) rows is a Linear (same
   parameters as torch.nn.Linear; large 16-bit inputs run on this package's GEMM kernels)."""
@@ -113,6 +143,9 @@ class Conv1x1(torch.nn.Module):
     if (data.dim() == 2 and data.is_cuda and data.dtype in (torch.float16, torch.bfloat16) and
         data.shape[0] >= 4096 and lin.in_features % 32 == 0 and lin.out_features % 16 == 0):
       return _RowsLinear.apply(data, lin.weight, lin.bias)
+    if (data.dim() == 2 and data.is_cuda and data.dtype in (torch.float16, torch.bfloat16) and
+        data.shape[0] >= 65536 and lin.in_features % 32 == 0 and lin.out_features < 16):
+      return _RowsLinearNarrow.apply(data, lin.weight, lin.bias)
     return lin(data)
 
 

@@ -183,3 +183,37 @@ def test_conv1x1_on_package_kernels(dtype, cin, cout, bias):
   # few rows: torch's Linear
   small = torch.randn(10, cin, generator=g).to(dtype).to(DEV)
   assert torch.equal(m(small), m.linear(small))
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_conv1x1_narrow_head(dtype):
+  """modules.Conv1x1 with few output channels on many rows (64 -> 10, a classification head):
+  torch's GEMMs for output and input gradient, the package's split reduction for the weight
+  gradient; against torch.nn.Linear in fp64, and the same bits on a second run."""
+  from ocnn_amd import modules
+  g = torch.Generator().manual_seed(7)
+  rows, cin, cout = 70000, 64, 10
+  m = modules.Conv1x1(cin, cout, use_bias=True).to(DEV).to(dtype)
+  x = torch.randn(rows, cin, generator=g).to(dtype)
+  dy = torch.randn(rows, cout, generator=g).to(dtype)
+  ref = torch.nn.Linear(cin, cout, True).double()
+  with torch.no_grad():
+    ref.weight.copy_(m.linear.weight.double().cpu())
+    ref.bias.copy_(m.linear.bias.double().cpu())
+  xd = x.double().requires_grad_()
+  ref(xd).backward(dy.double())
+  grads = []
+  for _ in range(2):
+    m.zero_grad()
+    xg = x.to(DEV).requires_grad_()
+    y = m(xg)
+    assert y.grad_fn is not None and 'RowsLinearNarrow' in type(y.grad_fn).__name__
+    y.backward(dy.to(DEV))
+    grads.append(m.linear.weight.grad.clone())
+  tol = 4e-3 if dtype == torch.float16 else 2e-2
+  rel = lambda a, b: float((a.double().cpu() - b).abs().max() / b.abs().max())
+  assert rel(y.detach(), ref(x.double()).detach()) < tol
+  assert rel(xg.grad, xd.grad) < tol
+  assert rel(m.linear.weight.grad, ref.weight.grad) < tol
+  assert rel(m.linear.bias.grad, ref.bias.grad) < tol
+  assert torch.equal(grads[0], grads[1])
