@@ -403,7 +403,8 @@ int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const vo
  * dx may be NULL).  gamma / beta (dtype param_dtype) may be NULL (no affine part); the
  * statistics kernel also moves running_mean / running_var (dtype running_dtype, may be NULL)
  * towards the batch statistics by `factor`, the running variance towards the unbiased one
- * (torch.nn.functional.batch_norm); dgamma / dbeta are fp32, grad_gamma / grad_beta the same
+ * (torch.nn.functional.batch_norm) and adds one to *batches_tracked (device, may be NULL: the
+ * module's num_batches_tracked); dgamma / dbeta are fp32, grad_gamma / grad_beta the same
  * sums in param_dtype (may be NULL).  fp32 arithmetic, two-level reductions with a fixed order.
  * channels a multiple of 16 bytes of elements.  residual (may be NULL): a tensor like x added
  * to the normalised values before the ReLU, each summand rounded to the dtype first (the
@@ -414,8 +415,9 @@ int ocnn_batch_norm_supported(int dtype, int64_t rows, int channels);
 int64_t ocnn_batch_norm_workspace_bytes(int channels);
 int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
                           float* mean, float* var, float* invstd, void* running_mean,
-                          void* running_var, int running_dtype, float factor, void* workspace,
-                          int64_t workspace_bytes, void* stream);
+                          void* running_var, int running_dtype, float factor,
+                          int64_t* batches_tracked, void* workspace, int64_t workspace_bytes,
+                          void* stream);
 int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int channels, const float* mean,
                           const float* invstd, const void* gamma, const void* beta,
                           int param_dtype, int relu, const void* residual, void* y, void* stream);

@@ -87,7 +87,7 @@ SIGNATURES = {
     'ocnn_dwconv_wgrad_planned': (_i, [_i, _p, _l, _p, _p, _p, _p, _i, _l, _l, _i, _i, _p, _p, _l, _p]),
     'ocnn_batch_norm_supported': (_i, [_i, _l, _i]),
     'ocnn_batch_norm_workspace_bytes': (_l, [_i]),
-    'ocnn_batch_norm_stats': (_i, [_i, _p, _l, _i, _f, _p, _p, _p, _p, _p, _i, _f, _p, _l, _p]),
+    'ocnn_batch_norm_stats': (_i, [_i, _p, _l, _i, _f, _p, _p, _p, _p, _p, _i, _f, _p, _p, _l, _p]),
     'ocnn_batch_norm_apply': (_i, [_i, _p, _l, _i, _p, _p, _p, _p, _i, _i, _p, _p, _p]),
     'ocnn_batch_norm_backward': (_i, [_i, _p, _p, _l, _i, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p,
                                       _p, _l, _p]),

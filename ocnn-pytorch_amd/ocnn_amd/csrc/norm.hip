@@ -131,7 +131,10 @@ template <typename T>
 __global__ void bn_stats_finish_kernel(const float* __restrict__ partial, int nblk, const T* __restrict__ x,
                                        int64_t rows, int C, float eps, float* __restrict__ mean,
                                        float* __restrict__ var, float* __restrict__ invstd,
-                                       void* running_mean, void* running_var, int rdtype, float factor) {
+                                       void* running_mean, void* running_var, int rdtype, float factor,
+                                       long long* batches_tracked) {
+  // (the module's count of training batches, kept here to spare a launch of its own)
+  if (batches_tracked != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *batches_tracked += 1;
   double a, b;
   const int c = bn_sum_partials(partial, nblk, C, a, b);
   if (c < 0) return;
@@ -383,8 +386,9 @@ extern "C" int64_t ocnn_batch_norm_workspace_bytes(int channels) {
 
 extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int channels, float eps,
                                      float* mean, float* var, float* invstd, void* running_mean,
-                                     void* running_var, int running_dtype, float factor, void* workspace,
-                                     int64_t workspace_bytes, void* stream) {
+                                     void* running_var, int running_dtype, float factor,
+                                     int64_t* batches_tracked, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_stats: shape not supported");
   OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels), "batch_norm_stats: workspace too small");
   hipStream_t st = (hipStream_t)stream;
@@ -398,7 +402,7 @@ extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int
                        partial);
     hipLaunchKernelGGL(bn_stats_finish_kernel<T>, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
                        (const T*)x, rows, channels, eps, mean, var, invstd, running_mean, running_var, running_dtype,
-                       factor);
+                       factor, (long long*)batches_tracked);
   });
   return check_launch("batch_norm_stats");
 }

@@ -22,7 +22,7 @@ def _param(t):
 class _BatchNormRelu(torch.autograd.Function):
   @staticmethod
   def forward(ctx, x, weight, bias, running_mean, running_var, use_batch_stats, factor, eps, relu,
-              residual=None):
+              residual=None, batches_tracked=None):
     L = _lib.lib()
     x = x.contiguous()
     rows, c = x.shape
@@ -44,12 +44,13 @@ class _BatchNormRelu(torch.autograd.Function):
           code, _lib.ptr(x), rows, c, float(eps), _lib.ptr(mean), _lib.ptr(var), _lib.ptr(invstd),
           _lib.ptr(running_mean) if in_place else None, _lib.ptr(running_var) if in_place else None,
           _lib.DTYPE_CODE[running_mean.dtype] if in_place else 0, float(factor) if in_place else 0.0,
-          _lib.ptr(ws), ws.numel(), _lib.stream()))
+          _lib.ptr(batches_tracked), _lib.ptr(ws), ws.numel(), _lib.stream()))
       if track and not in_place:
         unbiased = var * (rows / max(rows - 1, 1))
         running_mean.mul_(1 - factor).add_(mean.to(running_mean.dtype), alpha=factor)
         running_var.mul_(1 - factor).add_(unbiased.to(running_var.dtype), alpha=factor)
     else:
+      assert batches_tracked is None
       mean = running_mean.detach().float().contiguous()
       invstd = torch.rsqrt(running_var.detach().float() + eps)
     y = torch.empty_like(x)
@@ -95,7 +96,7 @@ class _BatchNormRelu(torch.autograd.Function):
       gw = dgamma.to(ctx.wdtype)
     if gb is None and ctx.bdtype is not None and ctx.needs_input_grad[2]:
       gb = dbeta.to(ctx.bdtype)
-    return dx, gw, gb, None, None, None, None, None, None, dres
+    return dx, gw, gb, None, None, None, None, None, None, dres, None
 
 
 class BatchNormRelu1d(torch.nn.BatchNorm1d):
@@ -120,15 +121,20 @@ class BatchNormRelu1d(torch.nn.BatchNorm1d):
       return torch.relu(out) if relu else out
     # the bookkeeping of torch.nn.modules.batchnorm._BatchNorm.forward
     factor = 0.0 if self.momentum is None else self.momentum
+    counter = None
     if self.training and self.track_running_stats and self.num_batches_tracked is not None:
-      self.num_batches_tracked.add_(1)
-      factor = 1.0 / float(self.num_batches_tracked) if self.momentum is None else self.momentum
+      nbt = self.num_batches_tracked
+      if (self.momentum is not None and nbt.is_cuda and nbt.dtype == torch.long and nbt.device == input.device):
+        counter = nbt                        # counted by the statistics kernel: no launch of its own
+      else:
+        nbt.add_(1)
+        factor = 1.0 / float(nbt) if self.momentum is None else self.momentum
     use_batch_stats = self.training or (self.running_mean is None and self.running_var is None)
     track = self.training and self.track_running_stats
     return _BatchNormRelu.apply(input, self.weight, self.bias,
                                 self.running_mean if (not use_batch_stats or track) else None,
                                 self.running_var if (not use_batch_stats or track) else None,
-                                use_batch_stats, factor if track else None, self.eps, relu, residual)
+                                use_batch_stats, factor if track else None, self.eps, relu, residual, counter)
 
   def extra_repr(self) -> str:
     return super().extra_repr() + ', relu={}'.format(self.fused_relu)
