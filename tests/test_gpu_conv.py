@@ -1033,3 +1033,49 @@ def test_group_conv_is_a_block_diagonal_conv(small):
     b[i * co:(i + 1) * co] = f64(conv.bias)
   want = C.conv_layer(small.ref, f64(x), w, depth, [3, 3, 3], 1, True, bias=b)
   assert rel_err(out, want) < 1e-4
+
+
+@pytest.mark.parametrize('first', [0, 40, 80])
+def test_random_shapes_through_the_dispatch(first):
+  """Random tables (local or scattered entries, 5 % .. 100 % set, ragged row counts, a stretch
+  of empty rows), channel counts (multiples of 32, and 4 / 8 / 10 / 16 / 48) and slot counts
+  through conv_gather / conv_wgrad, which pick the kernel per shape and plan: output, the
+  transposed-weight form and both weight-gradient layouts against the oracle."""
+  from ocnn_amd.octree.octree import TilePlan
+  chans = [32, 64, 96, 128, 160, 192, 256, 48, 16, 8, 4, 10, 384]
+  for case in range(first, first + 40):
+    rng = np.random.default_rng(case)
+    dtype = [torch.float16, torch.bfloat16][case % 2]
+    K = int(rng.choice([1, 3, 8, 9, 27]))
+    cin, cout = int(rng.choice(chans)), int(rng.choice(chans))
+    rows = int(rng.choice([1, 5, 127, 129, 1000, 5000, 20000, 33000, 70000]))
+    rows_in = int(rng.choice([1, 7, 300, 5000, 20000, 40000])) if rng.random() < 0.5 else rows
+    p = float(rng.choice([0.05, 0.15, 0.3, 0.6, 1.0]))
+    local = rng.random() < 0.7
+    if local:                                   # entries near the row: plans with reuse
+      t = (np.arange(rows)[:, None] * rows_in // max(rows, 1) + rng.integers(-40, 41, size=(rows, K))) % rows_in
+    else:
+      t = rng.integers(0, rows_in, size=(rows, K))
+    t = np.where(rng.random((rows, K)) < p, t, -1).astype(np.int32)
+    if rng.random() < 0.3 and rows > 200:
+      t[100:200] = -1
+    x = torch.from_numpy(rng.standard_normal((rows_in, cin)).astype(np.float32)).to(dtype)
+    w = torch.from_numpy((rng.standard_normal((K, cin, cout)) / np.sqrt(K * cin)).astype(np.float32)).to(dtype)
+    b = torch.from_numpy(rng.standard_normal(cout).astype(np.float32)).to(dtype) if rng.random() < 0.5 else None
+    gr = torch.from_numpy(rng.standard_normal((rows, cout)).astype(np.float32)).to(dtype)
+    use_plan = rng.random() < 0.8
+    say('random case', case, dtype, 'K', K, cin, '->', cout, 'rows', rows, 'rows_in', rows_in, 'set', p,
+        'local', local, 'plan', use_plan, 'bias', b is not None)
+    td = torch.from_numpy(t).to(DEV)
+    plan = TilePlan(td) if use_plan else None
+    t64 = t.astype(np.int64)
+    xd, wd, gd = x.to(DEV), w.to(DEV), gr.to(DEV)
+    want = C.forward_gemm(f64(x), f64(w), t64)
+    out = ocnn_amd.nn.conv_gather(xd, rows_in, td, wd, cout, False, False, None if b is None else b.to(DEV), plan)
+    assert rel_err(out, want + (0 if b is None else f64(b))) < TOL[dtype]
+    out = ocnn_amd.nn.conv_gather(xd, rows_in, td, w.transpose(1, 2).contiguous().to(DEV), cout, True, False,
+                                  None, plan)
+    assert rel_err(out, want) < TOL[dtype]
+    want = C.weight_gemm(f64(x), f64(gr), t64)
+    assert rel_err(ocnn_amd.nn.conv_wgrad(xd, gd, td, False, plan), want) < TOL[dtype]
+    assert rel_err(ocnn_amd.nn.conv_wgrad(xd, gd, td, True, plan).transpose(1, 2), want) < TOL[dtype]
