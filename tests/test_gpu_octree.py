@@ -314,3 +314,58 @@ def test_full_size_invariants():
   p = (pts.to(DEV) + 1.0) * 128.0
   key = xyz2key(p[:, 0], p[:, 1], p[:, 2], bid.to(DEV).view(-1), 8)
   assert torch.equal(leaf_key[idx], key)
+
+
+def test_random_octrees_vs_oracle():
+  """Random depth / full depth / batch size / point counts (1 .. 40 000) and point
+  distributions (uniform, a sphere, clusters with duplicates, grid-aligned coordinates up to the
+  box faces): keys, children, counts, point -> leaf map, leaf signals and all neighbour tables
+  bit exact against the oracle."""
+  for case in range(60):
+    rng = np.random.default_rng(case)
+    depth = int(rng.integers(2, 10))
+    full = max(1, min(int(rng.integers(1, 5)), depth - 1))
+    n = int(rng.choice([1, 2, 17, 500, 5000, 40000]))
+    batch = min(int(rng.choice([1, 1, 2, 3, 5])), n)
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+      pts = rng.uniform(-0.99, 0.99, (n, 3))
+    elif kind == 1:
+      v = rng.standard_normal((n, 3))
+      pts = 0.9 * v / np.linalg.norm(v, axis=1, keepdims=True)
+    elif kind == 2:
+      c = rng.uniform(-0.8, 0.8, (5, 3))
+      pts = c[rng.integers(0, 5, n)] + rng.normal(0, 0.01, (n, 3)) * (rng.random((n, 1)) < 0.7)
+    else:
+      pts = rng.integers(-2 ** depth // 2, 2 ** depth // 2, (n, 3)) / (2.0 ** (depth - 1))
+    pts = np.clip(pts, -1.0, 0.999999).astype(np.float32)
+    nrm = rng.standard_normal((n, 3)).astype(np.float32)
+    fea = rng.standard_normal((n, 2)).astype(np.float32) if rng.random() < 0.5 else None
+    bid = None
+    if batch > 1:
+      bid = rng.integers(0, batch, n)
+      bid[:batch] = np.arange(batch)                         # every element has a point
+      bid = np.sort(bid).astype(np.int64)
+    say('random octree', case, 'depth', depth, 'full', full, 'batch', batch, 'points', n, 'kind', kind)
+    pc = Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV),
+                None if fea is None else torch.from_numpy(fea).to(DEV),
+                batch_id=None if bid is None else torch.from_numpy(bid).view(-1, 1).to(DEV), batch_size=batch)
+    o = Octree(depth, full, batch_size=batch)
+    idx = o.build_octree(pc)
+    o.construct_all_neigh()
+    w, widx = R.build_octree(pts, nrm, fea, bid, depth, full, batch)
+    R.construct_all_neigh(w)
+    assert np.array_equal(o.nnum.numpy(), w.nnum) and np.array_equal(o.nnum_nempty.numpy(), w.nnum_nempty)
+    assert np.array_equal(np_(idx), widx)
+    for d in range(depth + 1):
+      assert np.array_equal(np_(o.keys[d]), w.keys[d]), d
+      assert np.array_equal(np_(o.children[d]), w.children[d]), d
+      if d:
+        assert np.array_equal(np_(o.neighs[d]), w.neighs[d]), d
+    assert np.array_equal(np_(o.points[depth]), w.points[depth])
+    if fea is not None:
+      assert np.array_equal(np_(o.features[depth]), w.features[depth])
+    assert np.allclose(np_(o.normals[depth]), w.normals[depth], atol=1e-6)
+    for kern, stride, ne in [('333', 1, True), ('222', 2, False), ('222', 2, True), ('333', 2, True),
+                             ('313', 1, False), ('131', 2, True)]:
+      assert np.array_equal(np_(o._table(depth, kern, stride, ne)), w.get_neigh(depth, kern, stride, ne))
