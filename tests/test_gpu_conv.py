@@ -1079,3 +1079,36 @@ def test_random_shapes_through_the_dispatch(first):
     want = C.weight_gemm(f64(x), f64(gr), t64)
     assert rel_err(ocnn_amd.nn.conv_wgrad(xd, gd, td, False, plan), want) < TOL[dtype]
     assert rel_err(ocnn_amd.nn.conv_wgrad(xd, gd, td, True, plan).transpose(1, 2), want) < TOL[dtype]
+
+
+def test_random_layers_vs_oracle():
+  """Random module configurations (conv / deconv / depth-wise, all eight kernel shapes, both
+  strides, all or non-empty nodes, channel counts incl. 4 / 10 / 16 / 48, f16 / bf16 / fp32, with
+  and without bias) on octrees of depth 5 to 8: forward and all gradients against the oracle."""
+  octs = [(5, 2, 3000, 1), (6, 3, 8000, 2), (7, 2, 30000, 3), (7, 1, 60000, 4), (8, 2, 50000, 5)]
+  kerns = ['333', '222', '311', '131', '113', '331', '313', '133']
+  chans = [32, 64, 96, 128, 48, 16, 4, 10, 160, 256]
+  pairs = {}
+  for case in range(48):
+    rng = np.random.default_rng(case)
+    kind = ['conv', 'deconv', 'dwconv'][int(rng.integers(0, 3))]
+    depth, batch, n, seed = octs[int(rng.integers(0, len(octs)))]
+    kern = kerns[int(rng.integers(0, 8))] if rng.random() < 0.5 else ['333', '222'][int(rng.integers(0, 2))]
+    stride = int(rng.choice([1, 2])) if kern != '222' else 2
+    ne = bool(rng.integers(0, 2))
+    cin, cout = int(rng.choice(chans)), int(rng.choice(chans))
+    dtype = [torch.float16, torch.bfloat16, torch.float32][int(rng.choice([0, 1, 1, 0, 2]))]
+    if dtype == torch.float32:
+      cin, cout = min(cin, 32), min(cout, 32)
+    if kind == 'dwconv':
+      cout = cin
+    if (depth, batch) not in pairs:
+      pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, batch, seed, n=n)
+      pairs[(depth, batch)] = Pair(pts, nrm, bid if batch > 1 else None, depth, 2, batch)
+    d = depth - 1 if (kind == 'deconv' and stride == 2) else depth
+    bias = bool(rng.integers(0, 2))
+    say('random layer', case, kind, kern, 'stride', stride, 'nempty', ne, cin, '->', cout, dtype, 'depth', d,
+        'of', depth, 'batch', batch, 'bias', bias)
+    errs = run_layer(kind, pairs[(depth, batch)], d, [int(c) for c in kern], stride, ne, cin, cout, dtype,
+                     seed=case, use_bias=bias)
+    assert max(errs.values()) < TOL[dtype], (case, errs)
