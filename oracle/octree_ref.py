@@ -158,6 +158,34 @@ class OctreeRef:
       return neigh[:, LUT_KERNEL[kernel]]
     raise ValueError('Unsupported kernel {}'.format(kernel))
 
+  # octree.py:525-568 ------------------------------------------------------
+  def get_input_feature(self, feature, nempty=False):
+    """N: leaf normals; D: displacement = <local point, normal>; L: local point = frac(p) - 0.5;
+    P: point scaled to [-1, 1]; F: leaf features; all fp32, in this order; zero rows for the
+    empty leaves unless nempty."""
+    d = self.depth
+    feature = feature.upper()
+    parts = []
+    pts = self.points[d].astype(np.float32)
+    # torch's frac() is x - trunc(x); the leaf points are non-negative
+    local = (pts - np.trunc(pts)).astype(np.float32) - np.float32(0.5)
+    if 'N' in feature:
+      parts.append(self.normals[d].astype(np.float32))
+    if 'D' in feature:
+      parts.append((local * self.normals[d].astype(np.float32)).sum(1, keepdims=True, dtype=np.float32))
+    if 'L' in feature:
+      parts.append(local)
+    if 'P' in feature:
+      parts.append(pts * np.float32(2.0 ** (1 - d)) - np.float32(1.0))
+    if 'F' in feature:
+      parts.append(self.features[d].astype(np.float32))
+    out = np.concatenate(parts, 1)
+    if not nempty:
+      full = np.zeros((int(self.nnum[d]), out.shape[1]), np.float32)
+      full[self.nempty_index(d)] = out
+      out = full
+    return out
+
   # octree.py:464-488 ------------------------------------------------------
   def search_key(self, query, depth, nempty=False):
     key = self.keys[depth]

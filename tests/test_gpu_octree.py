@@ -369,3 +369,32 @@ def test_random_octrees_vs_oracle():
     for kern, stride, ne in [('333', 1, True), ('222', 2, False), ('222', 2, True), ('333', 2, True),
                              ('313', 1, False), ('131', 2, True)]:
       assert np.array_equal(np_(o._table(depth, kern, stride, ne)), w.get_neigh(depth, kern, stride, ne))
+
+
+def test_input_feature_vs_oracle():
+  """Octree.get_input_feature (ocnn/octree/octree.py:525-568) and modules.InputFeature: every
+  letter and combinations, all nodes (zero rows for empty leaves) and non-empty nodes; the
+  pieces are closed forms of the leaf signals: D = <L, N>, P = points / 2^(depth - 1) - 1."""
+  from ocnn_amd.modules import InputFeature
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 3, 21, n=20000)
+  fea = torch.randn(pts.shape[0], 4, generator=torch.Generator().manual_seed(2))
+  o = Octree(6, 2, batch_size=3)
+  o.build_octree(Points(pts.to(DEV), nrm.to(DEV), fea.to(DEV), batch_id=bid.to(DEV), batch_size=3))
+  w, _ = R.build_octree(pts.numpy(), nrm.numpy(), fea.numpy(), bid.numpy(), 6, 2, 3)
+  for feature in ['N', 'D', 'L', 'P', 'F', 'ND', 'NDF', 'lpf', 'FPLDN']:
+    for ne in (False, True):
+      say('input feature', feature, 'nempty', ne)
+      got = np_(o.get_input_feature(feature, ne))
+      want = w.get_input_feature(feature, ne)
+      assert got.shape == want.shape and got.dtype == np.float32
+      assert np.abs(got - want).max() <= 2e-6, (feature, ne)
+      assert np.array_equal(got, np_(InputFeature(feature, ne)(o)))
+  nd = np_(o.get_input_feature('NDL', True))
+  assert np.allclose(nd[:, 3], (nd[:, 4:7] * nd[:, 0:3]).sum(1), atol=1e-6)     # D = <L, N>
+  assert np.abs(nd[:, 4:7]).max() <= 0.5
+  empty = np_(o.children[6]) < 0
+  assert not np_(o.get_input_feature('ND', False))[empty].any()
+  # to_points: the leaf signals back as a point cloud in [-1, 1]
+  back = o.to_points()
+  assert np.allclose(np_(back.points), w.points[6] * 2.0 ** (1 - 6) - 1.0, atol=1e-6)
+  assert np.array_equal(np_(back.normals), np_(o.normals[6]))

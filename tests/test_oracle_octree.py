@@ -237,3 +237,21 @@ def test_search_key_fixture(ref_data):
   key = R.xyz2key(q[:, 0], q[:, 1], q[:, 2], q[:, 3], 5)
   assert np.array_equal(oct.search_key(key, 5, False), d['idx'])
   assert np.array_equal(oct.search_key(key, 5, True), d['idx_ne'])
+
+
+@pytest.mark.parametrize('i', [1, 2, 3, 4, 5])
+def test_input_feature_against_reference_fixture(ref_data, i):
+  """get_input_feature('ND') (ocnn/octree/octree.py:525-568) on the reference's octree files:
+  their `feature` array holds the leaf normals and, in its fourth column, the displacement
+  <local point, normal> as the tool that wrote the files scaled it, by 2 / sqrt(3) (the current
+  Python code of the reference has no such factor).  Pins the leaf averages of the points, the
+  local coordinates and the order of the channels."""
+  d = np.load(os.path.join(ref_data, 'octree/test_%03d.npz' % i))
+  w, _ = R.build_octree(d['points'], d['normals'], None, None, int(d['depth']), int(d['full_depth']), 1)
+  f = w.get_input_feature('ND', nempty=True)
+  assert f.shape == d['feature'].shape and f.dtype == np.float32
+  assert np.allclose(f[:, :3], d['feature'][:, :3])
+  assert np.abs(d['feature'][:, 3] - 2.0 / np.sqrt(3.0) * f[:, 3]).max() < 2e-6
+  full = w.get_input_feature('ND', nempty=False)
+  assert full.shape[0] == int(d['nnum'][-1]) and np.array_equal(full[w.nempty_index(w.depth)], f)
+  assert not full[w.children[w.depth] < 0].any()
