@@ -217,3 +217,80 @@ def test_conv1x1_narrow_head(dtype):
   assert rel(m.linear.weight.grad, ref.weight.grad) < tol
   assert rel(m.linear.bias.grad, ref.bias.grad) < tol
   assert torch.equal(grads[0], grads[1])
+
+
+@pytest.mark.parametrize('cin,cout', [(32, 32), (32, 64)])
+@pytest.mark.parametrize('nempty', [False, True])
+def test_residual_block_is_its_parts(cin, cout, nempty):
+  """modules.OctreeResBlock2 / OctreeResBlocks (ocnn/modules/resblocks.py:65-99, 134-159): the
+  block with its fused tail (sum with the shortcut and ReLU inside the last batch norm's pass)
+  against the same layers put together from torch.nn.BatchNorm1d, torch.nn.Linear and separate
+  additions, fp32, training mode: output, input gradient, every parameter gradient and the
+  running statistics."""
+  import copy
+  from ocnn_amd import modules, synthetic
+  from ocnn_amd.nn import OctreeConv
+  from ocnn_amd.octree import Octree, Points
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 2, 31, n=6000)
+  o = Octree(5, 2, batch_size=2)
+  o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=2))
+  o.construct_all_neigh()
+  depth = 5
+  rows = int(o.nnum_nempty[depth] if nempty else o.nnum[depth])
+  torch.manual_seed(cin + cout)
+  blk = modules.OctreeResBlocks(cin, cout, 2, bottleneck=1, nempty=nempty).to(DEV)
+  for p in blk.parameters():
+    if p.dim() == 1:
+      p.data.uniform_(0.5, 1.5)
+  say('residual blocks', cin, cout, 'nempty', nempty, 'rows', rows)
+
+  class Parts(torch.nn.Module):
+    """One block from library layers; the parameters are those of `b`."""
+    def __init__(self, b):
+      super().__init__()
+      self.ca, self.cb = copy.deepcopy(b.conv3x3a.conv), copy.deepcopy(b.conv3x3b.conv)
+      def bn_of(m):
+        t = torch.nn.BatchNorm1d(m.num_features, m.eps, m.momentum).to(DEV)
+        t.load_state_dict({k: v.clone() for k, v in m.state_dict().items()})
+        return t
+      self.ba, self.bb = bn_of(b.conv3x3a.bn), bn_of(b.conv3x3b.bn)
+      self.proj = None
+      if hasattr(b, 'conv1x1'):
+        self.proj = copy.deepcopy(b.conv1x1.conv.linear)
+        self.bp = bn_of(b.conv1x1.bn)
+    def forward(self, x, octree, depth):
+      y = torch.relu(self.ba(self.ca(x, octree, depth)))
+      y = self.bb(self.cb(y, octree, depth))
+      s = x if self.proj is None else self.bp(self.proj(x))
+      return torch.relu(y + s)
+
+  parts = torch.nn.ModuleList([Parts(b) for b in blk.resblks])
+  x = torch.randn(rows, cin, device=DEV)
+  dy = torch.randn(rows, cout, device=DEV)
+  xa = x.clone().requires_grad_()
+  ya = blk(xa, o, depth)
+  ya.backward(dy)
+  xb = x.clone().requires_grad_()
+  yb = xb
+  for p in parts:
+    yb = p(yb, o, depth)
+  yb.backward(dy)
+  # (in the 2-norm: a pre-activation within rounding of zero may fall on either side of the
+  # ReLU in the two forms, which moves single entries of the gradients by O(1))
+  # (the gradients before a batch norm amplify this by 1 / sigma: 5e-3; a wiring error is O(1))
+  close = lambda a, b: float((a.detach() - b.detach()).norm()) <= 5e-3 * float(b.detach().norm())
+  assert close(ya, yb) and close(xa.grad, xb.grad)
+  for b, p in zip(blk.resblks, parts):
+    pairs = [(b.conv3x3a.conv.weights, p.ca.weights), (b.conv3x3b.conv.weights, p.cb.weights),
+             (b.conv3x3a.bn.weight, p.ba.weight), (b.conv3x3a.bn.bias, p.ba.bias),
+             (b.conv3x3b.bn.weight, p.bb.weight), (b.conv3x3b.bn.bias, p.bb.bias)]
+    stats = [(b.conv3x3a.bn, p.ba), (b.conv3x3b.bn, p.bb)]
+    if p.proj is not None:
+      pairs += [(b.conv1x1.conv.linear.weight, p.proj.weight), (b.conv1x1.bn.weight, p.bp.weight),
+                (b.conv1x1.bn.bias, p.bp.bias)]
+      stats.append((b.conv1x1.bn, p.bp))
+    for i, (u, v) in enumerate(pairs):
+      assert close(u.grad, v.grad), (i, float((u.grad - v.grad).norm()), float(v.grad.norm()))
+    for u, v in stats:
+      assert close(u.running_mean, v.running_mean) and close(u.running_var, v.running_var)
+      assert int(u.num_batches_tracked) == int(v.num_batches_tracked) == 1
