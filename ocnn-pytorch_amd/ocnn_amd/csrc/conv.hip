@@ -566,7 +566,7 @@ static WgradPlan plan_wgrad(int dtype, int64_t rows_x, int64_t rows, int K, int 
   int64_t s = std::min<int64_t>(want, cdiv(rows, min_rows));
   int64_t cap = std::max<int64_t>(1, (48ll << 20) / ((int64_t)K * ca * cb * 4));   // <= 48 MiB of partials
   s = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(s, cap), 256));
-  p.rows_per_split = align_up(cdiv(rows, s), 32);
+  p.rows_per_split = std::max<int64_t>(32, align_up(cdiv(rows, s), 32));   // (rows may be 0)
   p.splits = (int)cdiv(rows, p.rows_per_split);
   return p;
 }

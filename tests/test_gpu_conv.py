@@ -1112,3 +1112,29 @@ def test_random_layers_vs_oracle():
     errs = run_layer(kind, pairs[(depth, batch)], d, [int(c) for c in kern], stride, ne, cin, cout, dtype,
                      seed=case, use_bias=bias)
     assert max(errs.values()) < TOL[dtype], (case, errs)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_empty_inputs(dtype):
+  """Tables without rows, and tables whose entries are all -1 over an input without rows: empty
+  outputs, resp. zeros (+ bias), and zero weight gradients, with and without a plan."""
+  from ocnn_amd.octree.octree import TilePlan
+  for K, cin, cout in [(27, 64, 64), (27, 96, 96), (8, 128, 128), (1, 64, 128), (27, 5, 7)]:
+    say('empty inputs', dtype, K, cin, cout)
+    w = torch.randn(K, cin, cout, device=DEV).to(dtype)
+    b = torch.randn(cout, device=DEV).to(dtype)
+    t0 = torch.empty((0, K), dtype=torch.int32, device=DEV)
+    x = torch.randn(10, cin, device=DEV).to(dtype)
+    g0 = torch.empty((0, cout), device=DEV).to(dtype)
+    t1 = torch.full((300, K), -1, dtype=torch.int32, device=DEV)
+    x0 = torch.empty((0, cin), device=DEV).to(dtype)
+    g1 = torch.randn(300, cout, device=DEV).to(dtype)
+    for plan0, plan1 in [(None, None), (TilePlan(t0), TilePlan(t1))]:
+      out = ocnn_amd.nn.conv_gather(x, 10, t0, w, cout, False, False, b, plan0)
+      assert tuple(out.shape) == (0, cout)
+      gw = ocnn_amd.nn.conv_wgrad(x, g0, t0, False, plan0)
+      assert tuple(gw.shape) == (K, cin, cout) and not gw.any()
+      out = ocnn_amd.nn.conv_gather(x0, 0, t1, w, cout, False, False, b, plan1)
+      assert torch.equal(out, b.view(1, -1).expand(300, cout))
+      gw = ocnn_amd.nn.conv_wgrad(x0, g1, t1, True, plan1)
+      assert tuple(gw.shape) == (K, cout, cin) and not gw.any()
