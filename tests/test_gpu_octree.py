@@ -438,3 +438,45 @@ def test_random_octrees_regrown_from_split_masks():
       assert np.array_equal(np_(o.children[d]), np_(built.children[d])), d
       if d:
         assert np.array_equal(np_(o.neighs[d]), np_(built.neighs[d])), d
+
+
+def test_random_merge_equals_batched_build():
+  """merge_octrees of separately built octrees == build_octree on the merged cloud with batch
+  ids (the identity the reference's test_octree.py:115-123 checks on its two files), on random
+  clouds of unequal sizes: keys, children, counts, leaf signals, neighbour tables, batch_nnum."""
+  for case in range(12):
+    rng = np.random.default_rng(2000 + case)
+    depth = int(rng.integers(3, 8))
+    full = max(1, min(int(rng.integers(1, 4)), depth - 1))
+    batch = int(rng.integers(2, 5))
+    clouds = []
+    for b in range(batch):
+      n = int(rng.choice([1, 30, 2000, 15000]))
+      c = rng.uniform(-0.5, 0.5, 3)
+      v = rng.standard_normal((n, 3))
+      pts = np.clip(c + rng.uniform(0.1, 0.4) * v / np.linalg.norm(v, axis=1, keepdims=True), -0.99, 0.99)
+      clouds.append((pts.astype(np.float32), v.astype(np.float32), rng.standard_normal((n, 2)).astype(np.float32)))
+    say('merge', case, 'depth', depth, 'full', full, 'sizes', [len(c[0]) for c in clouds])
+    singles, parts = [], []
+    for pts, nrm, fea in clouds:
+      pc = Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV), torch.from_numpy(fea).to(DEV))
+      parts.append(pc)
+      o = Octree(depth, full)
+      o.build_octree(pc)
+      singles.append(o)
+    merged = merge_octrees(singles)
+    merged.construct_all_neigh()
+    whole = Octree(depth, full, batch_size=batch)
+    whole.build_octree(merge_points(parts))
+    whole.construct_all_neigh()
+    assert np.array_equal(merged.nnum.numpy(), whole.nnum.numpy())
+    assert np.array_equal(merged.nnum_nempty.numpy(), whole.nnum_nempty.numpy())
+    assert merged.batch_nnum.sum(1).tolist() == merged.nnum.tolist()
+    assert merged.batch_nnum_nempty.sum(1).tolist() == merged.nnum_nempty.tolist()
+    for d in range(depth + 1):
+      assert np.array_equal(np_(merged.keys[d]), np_(whole.keys[d])), d
+      assert np.array_equal(np_(merged.children[d]), np_(whole.children[d])), d
+      if d:
+        assert np.array_equal(np_(merged.neighs[d]), np_(whole.neighs[d])), d
+    for name in ('points', 'normals', 'features'):
+      assert np.array_equal(np_(getattr(merged, name)[depth]), np_(getattr(whole, name)[depth])), name
