@@ -221,6 +221,22 @@ int ocnn_conv_gather_rw(int dtype, const void* in, int64_t rows_in, const uint16
                         int w_transposed, int reverse_slots, const void* bias, void* out,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ocnn_conv_gather_rw without a workspace argument and without any allocation.  No
+ * counterpart in the reference: it is for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The
+ * packed weights go to a device array built into the library, K * cin * cout * 2 bytes of
+ * it, at most ocnn_conv_gather_rw_static_max_weight_bytes() = 221 184 (27 x 64 x 64); a
+ * larger layer is rejected with OCNN_ERR_ARG.  Every GPU the library runs on holds its own
+ * copy of the array until the process ends; all calls on one GPU share it, so calls that
+ * overlap on one GPU (different streams or threads) race.  Same arguments otherwise, same
+ * result bit for bit as ocnn_conv_gather_rw. */
+int64_t ocnn_conv_gather_rw_static_max_weight_bytes(void);
+int ocnn_conv_gather_rw_static(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,
+                               const int32_t* uptr, const int32_t* urows, int plan_max_distinct,
+                               int64_t plan_total, int64_t rows_out, int K, const void* w, int cin,
+                               int cout, int w_transposed, int reverse_slots, const void* bias,
+                               void* out, void* stream);
+
 /* ocnn_conv_gather for wide layers (cin >= 64 and cout >= 96, multiples of 32, any
  * K <= 27) over the tile plan: the distinct rows of a tile are staged in LDS 64 input
  * channels at a time, the weights stream from L2 into registers in the MFMA operand

@@ -49,6 +49,9 @@ SIGNATURES = {
     'ocnn_conv_gather_rw_supported': (_i, [_i, _l, _i, _i, _i, _i]),
     'ocnn_conv_gather_rw': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                  _p, _l, _p]),
+    'ocnn_conv_gather_rw_static_max_weight_bytes': (_l, []),
+    'ocnn_conv_gather_rw_static': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
+                                        _p]),
     'ocnn_conv_gather_wide_supported': (_i, [_i, _l, _i, _i, _i, _i]),
     'ocnn_pair_plan_slot_counts': (_i, [_p, _l, _i, _p, _p]),
     'ocnn_pair_plan_lists': (_i, [_i, _p, _p, _p, _p, _p]),

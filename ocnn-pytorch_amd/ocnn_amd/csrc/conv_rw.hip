@@ -11,6 +11,7 @@
 // units (v_mfma_f32_32x32x16, M = 64 output channels, N = 128 rows), and the four
 // partial sums are added through LDS in wave order (deterministic).
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -686,4 +687,58 @@ extern "C" int ocnn_conv_gather_rw(int dtype, const void* in, int64_t rows_in, c
                        bias, out, workspace, st);
   return run_rw<bf16>(in, rows_in, loc, uptr, urows, plan_total, rows_out, K, cin, w, w_transposed, reverse_slots, bias,
                       out, workspace, st);
+}
+
+// ---------------------------------------------------------------------------------------
+// Entry point that allocates nothing and takes no workspace.  The packed weights (what the
+// workspace of ocnn_conv_gather_rw holds) go to a file-scope device array instead.  Its
+// address on the current device is looked up once per device; host code never uses the
+// array's name for anything else.  Every call on a GPU shares that GPU's array: calls that
+// overlap on one GPU (two streams, two threads) race.  The pre-pass rewrites all K * cin *
+// cout elements that the kernel reads, so nothing needs clearing between calls.
+// ---------------------------------------------------------------------------------------
+constexpr int64_t kRwScratchBytes = 27 * 64 * 64 * 2;          // the largest shape: 216 KiB
+static __device__ __align__(256) unsigned char scratch[kRwScratchBytes];
+
+constexpr int kRwMaxDevices = 64;
+static void* g_rw_scratch_ptr[kRwMaxDevices];
+static std::mutex g_rw_scratch_mutex;
+
+static int rw_scratch_of_current_device(void** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kRwMaxDevices) {
+    set_error("conv_gather_rw_static: cannot tell the current device");
+    return OCNN_ERR_HIP;
+  }
+  std::lock_guard<std::mutex> lock(g_rw_scratch_mutex);
+  if (g_rw_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("conv_gather_rw_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      return OCNN_ERR_HIP;
+    }
+    g_rw_scratch_ptr[dev] = p;
+  }
+  *ptr = g_rw_scratch_ptr[dev];
+  return OCNN_OK;
+}
+
+extern "C" int64_t ocnn_conv_gather_rw_static_max_weight_bytes(void) { return kRwScratchBytes; }
+
+extern "C" int ocnn_conv_gather_rw_static(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,
+                                          const int32_t* uptr, const int32_t* urows, int plan_max_distinct,
+                                          int64_t plan_total, int64_t rows_out, int K, const void* w, int cin,
+                                          int cout, int w_transposed, int reverse_slots, const void* bias,
+                                          void* out, void* stream) {
+  OCNN_REQUIRE(ocnn_conv_gather_rw_supported(dtype, rows_in, K, cin, cout, plan_max_distinct),
+               "conv_gather_rw_static: shape not supported");
+  OCNN_REQUIRE((int64_t)K * cin * cout * 2 <= kRwScratchBytes,
+               "conv_gather_rw_static: %lld bytes of weights exceed the built-in buffer of %lld bytes",
+               (long long)K * cin * cout * 2, (long long)kRwScratchBytes);
+  void* ws = nullptr;
+  int rc = rw_scratch_of_current_device(&ws);
+  if (rc != OCNN_OK) return rc;
+  return ocnn_conv_gather_rw(dtype, in, rows_in, loc, uptr, urows, plan_max_distinct, plan_total, rows_out, K, w,
+                             cin, cout, w_transposed, reverse_slots, bias, out, ws, kRwScratchBytes, stream);
 }
