@@ -1,8 +1,7 @@
 """Forward + backward of the reference's segmentation U-Net (ocnn/models/unet.py:16-105: encoder
 channels 32-32-64-128-256 with 2/3/4/6 residual blocks, decoder 256-256-128-96-96 with 2 each,
 2x2x2 stride-2 (de)convolutions between levels, trilinear interpolation of the last features at
-the query points, a 1x1 head) assembled from this package's layers and torch's BatchNorm1d, on
-one MI355X.  Supporting data for the pieces around the convolutions (the headline number is
+the query points, a 1x1 head) as this package assembles it (ocnn_amd/unet.py), on one MI355X.  Supporting data for the pieces around the convolutions (the headline number is
 bench.py's): synthetic batch of 8 clouds x 150 000 points at depth 9, input signal 'ND'
 (normals + displacement), 10 classes, random weights, cross-entropy against random labels.
 
@@ -38,45 +37,14 @@ def main():
   ap.add_argument('--torch-loss', action='store_true', help='torch.nn.functional.cross_entropy for the loss')
   args = ap.parse_args()
   import torch
-  from ocnn_amd import modules, synthetic
-  from ocnn_amd.nn import OctreeInterp
+  from ocnn_amd import synthetic
+  from ocnn_amd.unet import UNet
   from ocnn_amd.octree import Octree, Points
   assert torch.cuda.is_available(), 'bench_unet.py needs a GPU'
   dev = 'cuda:0'
   torch.cuda.set_device(0)
   dtype = getattr(torch, args.dtype)
   nempty = bool(args.nempty)
-
-  class UNet(torch.nn.Module):
-    def __init__(self, cin, cout):
-      super().__init__()
-      enc, dec = [32, 32, 64, 128, 256], [256, 256, 128, 96, 96]
-      eb, db = [2, 3, 4, 6], [2, 2, 2, 2]
-      self.stages = len(eb)
-      self.conv1 = modules.OctreeConvBnRelu(cin, enc[0], nempty=nempty)
-      self.downsample = torch.nn.ModuleList(
-          [modules.OctreeConvBnRelu(enc[i], enc[i + 1], [2], 2, nempty) for i in range(4)])
-      self.encoder = torch.nn.ModuleList(
-          [modules.OctreeResBlocks(enc[i + 1], enc[i + 1], eb[i], 1, nempty) for i in range(4)])
-      self.upsample = torch.nn.ModuleList(
-          [modules.OctreeDeconvBnRelu(dec[i], dec[i + 1], [2], 2, nempty) for i in range(4)])
-      self.decoder = torch.nn.ModuleList(
-          [modules.OctreeResBlocks(dec[i + 1] + enc[-i - 2], dec[i + 1], db[i], 1, nempty) for i in range(4)])
-      self.octree_interp = OctreeInterp('linear', nempty, rescale_pts=False)
-      self.header = torch.nn.Sequential(modules.Conv1x1BnRelu(dec[-1], 64), modules.Conv1x1(64, cout, use_bias=True))
-
-    def forward(self, data, octree, depth, query):
-      convd = {depth: self.conv1(data, octree, depth)}
-      for i in range(self.stages):
-        d = depth - i
-        convd[d - 1] = self.encoder[i](self.downsample[i](convd[d], octree, d), octree, d - 1)
-      d0 = depth - self.stages
-      x = convd[d0]
-      for i in range(self.stages):
-        d = d0 + i
-        x = torch.cat([convd[d + 1], self.upsample[i](x, octree, d)], dim=1)
-        x = self.decoder[i](x, octree, d + 1)
-      return self.header(self.octree_interp(x, octree, depth, query))
 
   pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, args.batch, 1004, n=args.points)
   pc = Points(pts.to(dev), nrm.to(dev), batch_id=bid.to(dev), batch_size=args.batch)
@@ -88,16 +56,16 @@ def main():
 
   octree = build()
   feat = octree.get_input_feature('ND', nempty).to(dtype)
-  query = torch.cat([(pts.to(dev) + 1.0) * (2 ** (args.depth - 1)), bid.to(dev).float().view(-1, 1)], 1)
+  query = torch.cat([pts.to(dev), bid.to(dev).float().view(-1, 1)], 1)     # xyz in [-1, 1], batch index
   labels = torch.randint(0, 10, (query.shape[0],), generator=torch.Generator().manual_seed(5)).to(dev)
   torch.manual_seed(0)
-  net = UNet(feat.shape[1], 10).to(dev).to(dtype)
+  net = UNet(feat.shape[1], 10, 'linear', nempty).to(dev).to(dtype)
   params = [p for p in net.parameters()]
 
   def step(octree=octree):
     for p in params:
       p.grad = None
-    logits = net(feat, octree, args.depth, query)
+    logits = net(feat, octree, args.depth, query.clone())   # (the interpolation rescales its points in place)
     if args.torch_loss:
       loss = torch.nn.functional.cross_entropy(logits.float(), labels)
     else:

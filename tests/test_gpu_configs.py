@@ -1,0 +1,208 @@
+"""GPU parity on the workloads the benchmark configurations name, each on its own octree.
+
+  configs[0]  one sphere cloud of 20 000 points, depth 6, OctreeConv 3x3x3 32 -> 32 in fp32:
+              the whole layer (out, data gradient, weight gradient) against the fp64 oracle,
+              octree and neighbour table bit exact against the oracle
+  configs[1]  batch 8 x 100 000 points, depth 8, 64 -> 64 in fp16 / bf16: every slot of the
+              weight gradient and sampled rows of the output and of the data gradient against
+              the fp64 definition (the adjoint scalars alone would let a few wrong rows pass)
+  configs[3]  batch 4 x 250 000 points (planes + spheres), depth 9: integer invariants of
+              the build and the tables, then 32 -> 32 at depth 9 and 256 -> 256 at depth 6 in
+              bf16 the same way
+
+Tolerances: fp32 1e-4, 16-bit 2e-2 of the largest magnitude of the expected tensor (the bound
+the task states); the sampled rows are also held row by row to the same fraction of the
+row's own largest expected magnitude x 4 (a wrong row cannot hide behind a large one).
+
+The full-size definitions are evaluated in fp64 with plain torch indexing and matmul on the
+device (no kernel of this package): the data gradient in its scatter form, from the table
+entries that point at a sampled row, so that it does not lean on the table's symmetry.
+"""
+
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from ocnn_amd import synthetic
+from ocnn_amd.nn import OctreeConv
+from ocnn_amd.octree import Octree, Points, xyz2key
+from oracle import conv_ref as C
+from oracle import octree_ref as R
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+TOL = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+
+
+def say(*a):
+  print(*a, flush=True)
+  sys.stdout.flush()
+
+
+def f64(t):
+  return t.detach().double().cpu().numpy()
+
+
+def rel(got, want):
+  """max |got - want| over the largest |want| (both torch, any device)."""
+  want = want.double()
+  return float((got.double() - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def rel_rows(got, want):
+  """worst row: max |got - want| of the row over the row's own largest |want|."""
+  want = want.double()
+  scale = want.abs().amax(1).clamp_min(1e-30)
+  return float(((got.double() - want).abs().amax(1) / scale).max())
+
+
+def build(maker, batch, seed, n, depth):
+  if batch == 1:
+    pts, nrm = maker(n, seed=seed)
+    bid = None
+  else:
+    pts, nrm, bid = synthetic.batch_clouds(maker, batch, seed, n=n)
+  pc = Points(pts.to(DEV), nrm.to(DEV), batch_id=None if bid is None else bid.to(DEV), batch_size=batch)
+  o = Octree(depth, 2, batch_size=batch)
+  idx = o.build_octree(pc)
+  o.construct_all_neigh()
+  return o, idx, pts, nrm, bid
+
+
+def integer_invariants(o, idx, pts, bid, depth):
+  """What must hold of any octree and its tables, whatever the size."""
+  assert int(idx.max()) + 1 == int(o.nnum_nempty[depth])
+  for d in range(3, depth + 1):
+    k = o.keys[d]
+    assert bool((k[1:] > k[:-1]).all())                                 # sorted, unique
+    assert int(o.nnum[d]) == 8 * int(o.nnum_nempty[d - 1])
+    c = o.children[d]
+    assert torch.equal(c[c >= 0].long(), torch.arange(int(o.nnum_nempty[d]), device=DEV))
+    t = o._table(d, '333', 1, False).long()
+    n = t.shape[0]
+    assert torch.equal(t[:, 13], torch.arange(n, device=DEV))            # centre slot = itself
+    rows, slots = torch.nonzero(t >= 0, as_tuple=True)
+    assert torch.equal(t[t[rows, slots], 26 - slots], rows)              # central symmetry
+    del rows, slots, t
+    assert torch.equal(o.keys[d] >> 3 & ((1 << 45) - 1),
+                       (o.keys[d - 1][o.nempty_index(d - 1)] & ((1 << 48) - 1)).repeat_interleave(8))
+    t2 = o._table(d, '222', 2, False).long()
+    assert torch.equal(t2, (torch.arange(n // 8, device=DEV) * 8).unsqueeze(1) + torch.arange(8, device=DEV))
+  leaf_key = o.keys[depth][o.nempty_index(depth)]
+  p = (pts.to(DEV) + 1.0) * float(2 ** (depth - 1))
+  b = None if bid is None else bid.to(DEV).view(-1)
+  assert torch.equal(leaf_key[idx], xyz2key(p[:, 0], p[:, 1], p[:, 2], b, depth))
+
+
+def definition_checks(o, depth, ch, dtype, nempty, seed, samples=512):
+  """One OctreeConv 3x3x3 ch -> ch forward + backward through the module; every slot of the
+  weight gradient, `samples` rows of the output and of the data gradient against fp64."""
+  g = torch.Generator().manual_seed(seed)
+  t = o._table(depth, '333', 1, nempty)
+  rows = t.shape[0]
+  conv = OctreeConv(ch, ch, [3], 1, nempty=nempty)
+  with torch.no_grad():
+    conv.weights.copy_(torch.randn(conv.weights.shape, generator=g) / (27 * ch) ** 0.5)
+  conv = conv.to(DEV).to(dtype)
+  x = torch.randn(rows, ch, generator=g).to(dtype).to(DEV).requires_grad_()
+  gout = torch.randn(rows, ch, generator=g).to(dtype).to(DEV)
+  out = conv(x, o, depth)
+  out.backward(gout)
+  assert out.dtype == dtype and x.grad.dtype == dtype and conv.weights.grad.dtype == dtype
+  W = conv.weights.detach().double()
+  xd = x.detach()
+  tol = TOL[dtype]
+
+  # every slot of the weight gradient: gW[k] = sum_i [t_ik >= 0] x[t_ik]^T (x) g[i]
+  want_w = torch.empty(27, ch, ch, dtype=torch.float64, device=DEV)
+  for k in range(27):
+    v = torch.nonzero(t[:, k] >= 0).squeeze(1)
+    want_w[k] = xd[t[v, k].long()].double().T @ gout[v].double()
+  err_w = rel(conv.weights.grad, want_w)
+  err_w_slot = max(rel(conv.weights.grad[k], want_w[k]) for k in range(27))
+
+  # sampled rows of the output: out[i] = sum_k [t_ik >= 0] x[t_ik] @ W[k]
+  sel = torch.randint(0, rows, (samples,), generator=g).to(DEV)
+  ts = t[sel].long()
+  want_o = torch.zeros(samples, ch, dtype=torch.float64, device=DEV)
+  for k in range(27):
+    v = ts[:, k] >= 0
+    want_o[v] += xd[ts[v, k]].double() @ W[k]
+  err_o, err_o_row = rel(out[sel], want_o), rel_rows(out[sel], want_o)
+
+  # sampled rows of the data gradient, scatter form: gin[j] = sum over the entries (i, k) of
+  # the WHOLE table that hold j of g[i] @ W[k]^T
+  sel = torch.unique(torch.randint(0, rows, (samples,), generator=g)).to(DEV)
+  where = torch.full((rows,), -1, dtype=torch.long, device=DEV)
+  where[sel] = torch.arange(sel.numel(), device=DEV)
+  want_g = torch.zeros(sel.numel(), ch, dtype=torch.float64, device=DEV)
+  for k in range(27):
+    tk = t[:, k].long()
+    pos = torch.where(tk >= 0, where[tk.clamp_min(0)], torch.full_like(tk, -1))
+    i = torch.nonzero(pos >= 0).squeeze(1)
+    want_g.index_add_(0, pos[i], gout[i].double() @ W[k].T)
+  err_g, err_g_row = rel(x.grad[sel], want_g), rel_rows(x.grad[sel], want_g)
+  say('   rows %d  nnz/row %.2f  rel err: gW %.2e (worst slot %.2e)  out %.2e (worst row %.2e)  '
+      'gdata %.2e (worst row %.2e)' % (rows, float((t >= 0).sum()) / rows, err_w, err_w_slot, err_o,
+                                       err_o_row, err_g, err_g_row))
+  assert err_w < tol and err_w_slot < tol
+  assert err_o < tol and err_o_row < 4 * tol
+  assert err_g < tol and err_g_row < 4 * tol
+
+
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('nempty', [False, True])
+def test_config0_sphere_depth6_fp32(nempty):
+  say('configs[0]: 20 000 points on a sphere, depth 6, 32 -> 32 fp32, nempty', nempty)
+  o, idx, pts, nrm, _ = build(synthetic.sphere_cloud, 1, 1000, 20000, 6)
+  ref, ref_idx = R.build_octree(pts.numpy(), nrm.numpy(), depth=6, full_depth=2)
+  R.construct_all_neigh(ref)
+  assert np.array_equal(torch.cat(o.keys).cpu().numpy(), np.concatenate(ref.keys))
+  assert np.array_equal(torch.cat(o.children).cpu().numpy(), np.concatenate(ref.children))
+  assert np.array_equal(idx.cpu().numpy(), ref_idx)
+  for d in range(1, 7):
+    assert np.array_equal(o.neighs[d].cpu().numpy(), ref.neighs[d]), d
+  g = torch.Generator().manual_seed(1000)
+  conv = OctreeConv(32, 32, [3], 1, nempty=nempty)
+  with torch.no_grad():
+    bound = 1.0 / (27 * 32) ** 0.5                       # the configuration's Kaiming-uniform bound
+    conv.weights.copy_((torch.rand(conv.weights.shape, generator=g) * 2 - 1) * bound)
+  conv = conv.to(DEV)
+  rows = int(ref.nnum_nempty[6] if nempty else ref.nnum[6])
+  data = torch.randn(rows, 32, generator=g)
+  gout = torch.randn(rows, 32, generator=g)
+  x = data.to(DEV).requires_grad_()
+  out = conv(x, o, 6)
+  out.backward(gout.to(DEV))
+  want = C.conv_layer(ref, f64(data), f64(conv.weights), 6, [3], 1, nempty, grad=f64(gout))
+  for name, got, exp in (('out', out, want[0]), ('gdata', x.grad, want[1]), ('gW', conv.weights.grad, want[2])):
+    exp = torch.from_numpy(exp)
+    e, er = rel(got.cpu(), exp), (rel_rows(got.cpu(), exp) if name != 'gW' else 0.0)
+    say('   %-5s rel err %.2e  worst row %.2e' % (name, e, er))
+    assert e < 1e-4 and er < 4e-4, name
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_config1_full_weight_gradient_and_sampled_rows(dtype):
+  say('configs[1]: 8 x 100 000 points, depth 8, 64 -> 64', dtype)
+  o, _, _, _, _ = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
+  definition_checks(o, 8, 64, dtype, False, 31)
+  say('configs[1], non-empty nodes only (the mode of the reference\'s published table)')
+  definition_checks(o, 8, 64, dtype, True, 32)
+
+
+def test_config3_depth9_build_and_layers():
+  say('configs[3]: 4 x 250 000 points on planes and spheres, depth 9: build and tables')
+  o, idx, pts, _, bid = build(synthetic.planes_cloud, 4, 1003, 250000, 9)
+  say('   nnum', o.nnum.tolist(), 'nnum_nempty', o.nnum_nempty.tolist())
+  integer_invariants(o, idx, pts, bid, 9)
+  say('configs[3]: 32 -> 32 at depth 9, bf16')
+  definition_checks(o, 9, 32, torch.bfloat16, False, 33)
+  say('configs[3]: 256 -> 256 at depth 6, bf16')
+  definition_checks(o, 6, 256, torch.bfloat16, False, 34)
+  say('configs[3]: the same layers on non-empty nodes')
+  definition_checks(o, 9, 32, torch.bfloat16, True, 35)
+  definition_checks(o, 6, 256, torch.bfloat16, True, 36)
