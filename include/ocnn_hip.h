@@ -339,10 +339,6 @@ int ocnn_conv_dense_wgrad_rw(int dtype, const void* x, const void* g, int64_t ro
                              int out_transposed, void* gw, void* workspace,
                              int64_t workspace_bytes, void* stream);
 
-/* Selects how the MFMA weight-gradient kernel reads its LDS tiles: 1 (default)
- * = transposing LDS loads, 0 = 16-bit loads.  Same results either way. */
-void ocnn_set_wgrad_transpose_load(int on);
-
 /* Weight gradient, ocnn/nn/octree_conv.py:170-202 (weight_gemm) and
  * ocnn/nn/kernels/conv_bwd_implicit_gemm_splitk.py:94-184,294-306:
  * gw[k][a][b] = sum_i [t[i][k] >= 0] x[t[i][k]][a] * g[i][b], computed as

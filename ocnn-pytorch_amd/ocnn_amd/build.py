@@ -9,6 +9,8 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(HERE, 'csrc')
 LIB_DIR = os.path.join(HERE, 'lib')
 LIB_PATH = os.path.join(LIB_DIR, 'libocnn_hip.so')
+# measurement probes (MFMA and LDS rates of the part), used by bench.py only: a library of their own
+PROBE_LIB_PATH = os.path.join(LIB_DIR, 'libocnn_probe.so')
 INCLUDE = os.path.join(ROOT, 'include')
 
 # file -> extra flags.  The key/build kernels must round every fp32 operation
@@ -66,6 +68,7 @@ def build_library(verbose=False):
   with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
     objs = list(pool.map(compile_one, SOURCES.items()))
   _run([hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-o', LIB_PATH] + objs)
+  _run([hipcc] + COMMON + ['-shared', os.path.join(CSRC, 'probe.hip'), '-o', PROBE_LIB_PATH])
   if verbose:
     print('built', LIB_PATH)
   return LIB_PATH

@@ -314,29 +314,21 @@ __global__ __launch_bounds__(256) void conv_gather_plain_kernel(
 // M = x channels (a), N = g channels (b), reduction = rows, 32 rows per MFMA.
 // Both operands are needed "transposed" (a lane wants 8 consecutive rows of one
 // channel): tiles are staged row-major in LDS and read with the transposing
-// LDS load (USE_TR) or with eight 16-bit reads.
-template <typename T, bool USE_TR>
+// LDS load.
+template <typename T>
 __device__ __forceinline__ u32x4 read_frag_t(const T* tile, int pitch, int c0, int lane) {
   const int g = lane >> 4, i = lane & 15;
-  if constexpr (USE_TR) {
-    // lane i of a 16-lane group addresses 4 consecutive channels of row i/4 and
-    // receives channel c0+i of rows 0..3 of the group's block
-    const T* p = tile + (8 * g + (i >> 2)) * pitch + c0 + 4 * (i & 3);
-    u32x2 lo = Mma<T>::read_tr(p);
-    u32x2 hi = Mma<T>::read_tr(p + 4 * pitch);
-    return u32x4{lo[0], lo[1], hi[0], hi[1]};
-  } else {
-    const unsigned short* p = (const unsigned short*)tile + (8 * g) * pitch + c0 + i;
-    unsigned v[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = p[j * pitch];
-    return u32x4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
-  }
+  // lane i of a 16-lane group addresses 4 consecutive channels of row i/4 and
+  // receives channel c0+i of rows 0..3 of the group's block
+  const T* p = tile + (8 * g + (i >> 2)) * pitch + c0 + 4 * (i & 3);
+  u32x2 lo = Mma<T>::read_tr(p);
+  u32x2 hi = Mma<T>::read_tr(p + 4 * pitch);
+  return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
 // TILE = 64: wave w owns x-channel tile w and all 4 g-channel tiles.
 // TILE = 32: wave w owns x-channel tile w/2 and g-channel tile w%2.
-template <typename T, int TILE, int KG, bool USE_TR>
+template <typename T, int TILE, int KG>
 __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(
     const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ gmat, uint32_t g_bytes,
     const int32_t* __restrict__ table, int64_t rows, int K, int ca, int cb,
@@ -418,11 +410,11 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(
     }
     u32x4 bf[NB];
 #pragma unroll
-    for (int n = 0; n < NB; ++n) bf[n] = read_frag_t<T, USE_TR>(s_g, PITCH, (b_t0 + n) * 16, lane);
+    for (int n = 0; n < NB; ++n) bf[n] = read_frag_t<T>(s_g, PITCH, (b_t0 + n) * 16, lane);
 #pragma unroll
     for (int q = 0; q < KG; ++q) {
       if (k0 + q < K) {
-        u32x4 af = read_frag_t<T, USE_TR>(s_x[q], PITCH, a_t * 16, lane);
+        u32x4 af = read_frag_t<T>(s_x[q], PITCH, a_t * 16, lane);
 #pragma unroll
         for (int n = 0; n < NB; ++n) acc[q][n] = Mma<T>::run(af, bf[n], acc[q][n]);
       }
@@ -549,8 +541,6 @@ struct WgradPlan {
   int64_t rows_per_split;
 };
 
-static bool g_wgrad_use_tr = true;
-
 static WgradPlan plan_wgrad(int dtype, int64_t rows_x, int64_t rows, int K, int ca, int cb) {
   WgradPlan p{false, 0, 1, rows};
   bool fits = (int64_t)rows_x * ca * 2 < 0xffff0000ll && (int64_t)rows * cb * 2 < 0xffff0000ll;
@@ -574,8 +564,6 @@ static WgradPlan plan_wgrad(int dtype, int64_t rows_x, int64_t rows, int K, int 
 }  // namespace ocnn
 
 using namespace ocnn;
-
-extern "C" void ocnn_set_wgrad_transpose_load(int on) { g_wgrad_use_tr = on != 0; }
 
 extern "C" int64_t ocnn_conv_workspace_bytes(int K, int cin, int cout) {
   return align_up((int64_t)K * cin * cout * 4, 256);
@@ -670,12 +658,12 @@ static int run_wgrad(int dtype, const void* x, int64_t rows_x, const void* g, co
       constexpr int KG = kWgradSlots;
       dim3 grid(p.splits, (unsigned)(cdiv(K, KG) * (ca / p.TILE)), (unsigned)(cb / p.TILE));
       uint32_t xb = (uint32_t)(rows_x * ca * sizeof(T)), gb = (uint32_t)(rows * cb * sizeof(T));
-#define OCNN_WGRAD_CASE(tile_, tr_)                                                             \
-  hipLaunchKernelGGL((conv_wgrad_mfma_kernel<T, tile_, KG, tr_>), grid, dim3(256), 0, st,       \
+#define OCNN_WGRAD_CASE(tile_)                                                                  \
+  hipLaunchKernelGGL((conv_wgrad_mfma_kernel<T, tile_, KG>), grid, dim3(256), 0, st,            \
                      (const T*)x, xb, (const T*)g, gb, table, rows, K, ca, cb, p.rows_per_split, \
                      partial)
-      if (p.TILE == 64) { if (g_wgrad_use_tr) OCNN_WGRAD_CASE(64, true); else OCNN_WGRAD_CASE(64, false); }
-      else              { if (g_wgrad_use_tr) OCNN_WGRAD_CASE(32, true); else OCNN_WGRAD_CASE(32, false); }
+      if (p.TILE == 64) OCNN_WGRAD_CASE(64);
+      else OCNN_WGRAD_CASE(32);
 #undef OCNN_WGRAD_CASE
     }
   }
@@ -722,10 +710,10 @@ static int run_wgrad_f32_split(const void* x, int64_t rows_x, const void* g, con
   const bf16* gs[3] = {gh, gl, gh};
   for (int i = 0; i < 3; ++i) {
     if (p.TILE == 64)
-      hipLaunchKernelGGL((conv_wgrad_mfma_kernel<bf16, 64, KG, true>), grid, dim3(256), 0, st, xs[i], xbytes,
+      hipLaunchKernelGGL((conv_wgrad_mfma_kernel<bf16, 64, KG>), grid, dim3(256), 0, st, xs[i], xbytes,
                          gs[i], gbytes, table, rows, K, ca, cb, p.rows_per_split, partial + i * pstride);
     else
-      hipLaunchKernelGGL((conv_wgrad_mfma_kernel<bf16, 32, KG, true>), grid, dim3(256), 0, st, xs[i], xbytes,
+      hipLaunchKernelGGL((conv_wgrad_mfma_kernel<bf16, 32, KG>), grid, dim3(256), 0, st, xs[i], xbytes,
                          gs[i], gbytes, table, rows, K, ca, cb, p.rows_per_split, partial + i * pstride);
   }
   int64_t per = (int64_t)K * ca * cb;

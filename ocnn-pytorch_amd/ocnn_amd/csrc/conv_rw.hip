@@ -17,10 +17,6 @@
 #include "common.hpp"
 #include "mma.hpp"
 
-#ifndef OCNN_RW_EXP
-#define OCNN_RW_EXP 0   // timing experiments: bit 0 no partial-sum writes, 1 no barriers, 2 no reads/adds, 3 no stores
-#endif
-
 namespace ocnn {
 
 constexpr int kRwRows = 128;   // rows per tile (the plan's tile size)
@@ -67,8 +63,7 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const uint16_t* __restrict__ loc,
     uint32_t loc_bytes, const int32_t* __restrict__ uptr, const int32_t* __restrict__ urows,
     uint32_t urows_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
-    T* __restrict__ out, int64_t rows_out, int K, int64_t tiles, int64_t tiles_per_wg,
-    long long* dbg) {
+    T* __restrict__ out, int64_t rows_out, int K, int64_t tiles, int64_t tiles_per_wg) {
   constexpr int kLocElems = (kRwRows * 27 * 2 + 1023) / 1024 * 512;   // whole KiB: filled 1 KiB per instruction
   // Everything a tile needs is double buffered, one array per buffer so that the compiler
   // can tell the buffer being filled from the one being read.
@@ -161,12 +156,6 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
     }
   };
 
-#ifdef OCNN_RW_TIMING
-  const bool timing = dbg != nullptr;
-#else
-  constexpr bool timing = false;
-#endif
-  long long t_main = 0, t_wait = 0, t_mark = 0;
 
   // Two accumulator sets: while a 64-row half is being multiplied into one, the partial sums
   // of the half before it (the other set) are exchanged through LDS and stored, a piece per
@@ -366,16 +355,13 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
     const uint32_t p_raw = __builtin_amdgcn_raw_buffer_load_b32(rs_p, (uint32_t)min(tile + 4, tiles) * 4u, 0, 0);
     p_nxt = p_nx2;
     p_nx2 = p_nx3;
-    if (timing) t_mark = clock64();
     half_body(std::integral_constant<int, 0>{}, rows, lc, tile > t_begin ? (tile - 1) * kRwRows + 64 : rows_out,
               0, kPieces, st);
     half_body(std::integral_constant<int, 1>{}, rows, lc, tile * kRwRows, (UPW >= 14 ? kHalfSteps : kPieces), kPieces, st);
-    if (timing) { long long t = clock64(); t_main += t - t_mark; t_mark = t; }
     // the next tile has landed (own loads, then everyone's); every wave is past its last read
     // of this tile's buffers and of s_red
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     p_nx3 = __builtin_amdgcn_readfirstlane((int32_t)p_raw);
-    if (timing) { long long t = clock64(); t_wait += t - t_mark; t_mark = t; }
   };
   for (int64_t tile = t_begin; tile < t_end; tile += 2) {
     tile_body(std::integral_constant<int, 0>{}, tile);
@@ -386,11 +372,6 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
   for (int e = 0; e < 26; ++e) {
     exch_piece(std::integral_constant<int, 1>{}, e, (t_end - 1) * kRwRows + 64, true);
     __builtin_amdgcn_sched_barrier(0);
-  }
-  if (timing && lane == 0) {
-    long long* d = dbg + ((int64_t)blockIdx.x * 4 + wave) * 8;
-    d[0] = t_main; d[1] = 0; d[2] = t_wait; d[3] = t_end - t_begin;
-    d[4] = 0; d[5] = 0; d[6] = 0; d[7] = 0;
   }
 }
 
@@ -589,12 +570,6 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
 
 using namespace ocnn;
 
-static long long* g_rw_dbg = nullptr;
-
-#ifdef OCNN_RW_TIMING
-// per-wave cycle counters of the kernel phases (development aid)
-extern "C" void ocnn_debug_set_rw_timing(long long* p) { g_rw_dbg = p; }
-#endif
 
 extern "C" int ocnn_conv_gather_rw_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                              int plan_max_distinct) {
@@ -616,7 +591,7 @@ static void launch_rw(const void* in, int64_t rows_in, const uint16_t* loc, cons
   wgs = cdiv(tiles, per);
   hipLaunchKernelGGL((conv_gather_rw_kernel<T, UPW>), dim3((unsigned)wgs), dim3(256), 0, st,
                      (const T*)in, (uint32_t)(rows_in * 128), loc, (uint32_t)(tiles * kRwRows * K * 2), uptr,
-                     urows, urows_bytes, (const T*)ws, (const T*)bias, (T*)out, rows_out, K, tiles, per, g_rw_dbg);
+                     urows, urows_bytes, (const T*)ws, (const T*)bias, (T*)out, rows_out, K, tiles, per);
 }
 
 template <typename T, int KK>

@@ -20,10 +20,6 @@
 #include "mma.hpp"
 #include "reduce.hpp"
 
-#ifndef OCNN_WP_EXP
-#define OCNN_WP_EXP 0   // timing experiments: bit 0 no staging in the steps, 1 no x reads, 2 no g reads, 3 no positions
-#endif
-
 namespace ocnn {
 
 constexpr int kWpRows = 128;   // rows per tile (the plan's tile size)
@@ -65,7 +61,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes,
     const uint16_t* __restrict__ loc, uint32_t loc_bytes, const int32_t* __restrict__ uptr,
     const int32_t* __restrict__ urows, uint32_t urows_bytes, int64_t tiles,
-    int64_t tiles_per_split, int nsplit, int ca, int cb, float* __restrict__ partial, long long* dbg) {
+    int64_t tiles_per_split, int nsplit, int ca, int cb, float* __restrict__ partial) {
   constexpr int H = C / 32;                   // 32-channel halves of a row
   constexpr int NU = H * NFULL + NHALF;       // 32 x C accumulator units per wave
   constexpr int NS = NFULL + NHALF;           // distinct slots per wave
@@ -241,16 +237,12 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     acc[u][bh] = Mma32<T>::run(av, bv, acc[u][bh]);
   };
 
-  long long t_dma = 0;
   // One step: the MFMAs of 16 rows on `oc`; between them the operand fetch of the
   // following step (rows 16 sn.. of the buffers xs/gs/lcs) into `on`, and four staging
   // pieces t0..t0+3 of the next tile (t0 < 0: none).
   auto step = [&](const WpOps& oc, WpOps& on, const char* xs, const char* gs, const char* lcs, int sn,
                   int t0, const WpStage& sg) {
     int32_t ids[4] = {0, 0, 0, 0};
-#ifdef OCNN_WP_TIMING
-    long long tq[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       mm(m, oc);
@@ -260,11 +252,11 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
         if (m < PF0) {
 #pragma unroll
           for (int t = m * IP; t < (m + 1) * IP && t < NL + 4; ++t) {
-            if (t < NL) { if (!(OCNN_WP_EXP & 8)) pf_loc(t, lcs, sn); }
-            else if (!(OCNN_WP_EXP & 4)) pf_g(t - NL, gs, sn, on);
+            if (t < NL) pf_loc(t, lcs, sn);
+            else pf_g(t - NL, gs, sn, on);
           }
         } else if (m - PF0 < NL) {
-          if (!(OCNN_WP_EXP & 2)) pf_x(m - PF0, xs, on);
+          pf_x(m - PF0, xs, on);
         }
       } else {
         if (m == 0) {
@@ -278,7 +270,7 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
           for (int t = (m - XS) * XP; t < (m - XS + 1) * XP && t < NL; ++t) pf_x(t, xs, on);
         }
       }
-      if (!(OCNN_WP_EXP & 1) && t0 >= 0) {
+      if (t0 >= 0) {
         if (m == 0) {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
@@ -288,21 +280,12 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
         for (int j = 0; j < 4; ++j) {
           const int mj = (j * NM) / 4 + 1 < NM ? (j * NM) / 4 + 1 : NM - 1;
           if (m == mj && t0 + j < kPieces) {
-#ifdef OCNN_WP_TIMING
-            if (dbg) tq[2 * j] = clock64();
-#endif
             stage_piece(t0 + j, sg, ids[j]);
-#ifdef OCNN_WP_TIMING
-            if (dbg) tq[2 * j + 1] = clock64();
-#endif
           }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-#ifdef OCNN_WP_TIMING
-    if (dbg && t0 >= 0) t_dma += (tq[1] - tq[0]) + (tq[3] - tq[2]) + (tq[5] - tq[4]) + (tq[7] - tq[6]);
-#endif
   };
   // operand fetch of a tile's first step when there is no previous step to hide it under
   auto first_fetch = [&](const char* xs, const char* gs, const char* lcs, WpOps& on) {
@@ -327,22 +310,11 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
     st = make_stage(t_begin, p_nxt - p_cur, p_nxt, p_nx2 - p_nxt, s_u0 + 4, s_u1 + 4, s_x0, s_g0, s_loc0);
 #pragma unroll
     for (int t = 0; t < kPieces; ++t) stage_piece(t, st, stage_id(t, st));     // also: list of the second tile
-#if OCNN_WP_EXP & 1
-    st.sx = (char*)s_x1; st.sg = (char*)s_g1; st.sl = (char*)s_loc1;
-#pragma unroll
-    for (int t = 0; t < tU; ++t) stage_piece(t, st, stage_id(t, st));   // timing experiment: both buffers filled
-#endif
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     first_fetch((const char*)s_x0, (const char*)s_g0, (const char*)s_loc0, ops[0]);
   }
 
-#ifdef OCNN_WP_TIMING
-  const bool timing = dbg != nullptr;
-#else
-  constexpr bool timing = false;
-#endif
-  long long t_steps = 0, t_wait = 0, t_last = 0, t_mark = 0;
   // one tile out of buffer B; stages the next tile into buffer 1 - B meanwhile
   auto tile_body = [&](auto BC, int64_t tile) {
     constexpr int B = decltype(BC)::value;
@@ -360,29 +332,21 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
         rs_p, (uint32_t)min(tile + 4, tiles) * 4u, 0, 0);
     p_nxt = p_nx2;
     p_nx2 = p_nx3;
-    if (timing) t_mark = clock64();
 #pragma unroll
     for (int s = 0; s < 7; ++s)
       step(ops[s & 1], ops[(s + 1) & 1], xs, gs, lcs, s + 1, s < 5 ? 4 * s : -1, sg);
-    if (timing) { long long t = clock64(); t_steps += t - t_mark; t_mark = t; }
     // The next tile has landed: own loads, then everyone's.  The LDS reads in flight belong
     // to this tile's buffers and need not drain, so neither barrier is a __syncthreads().
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     p_nx3 = __builtin_amdgcn_readfirstlane((int32_t)p_raw);
-    if (timing) { long long t = clock64(); t_wait += t - t_mark; t_mark = t; }
     // last step, with the first operands of the next tile fetched from the other buffer
     step(ops[1], ops[0], sg.sx, sg.sg, sg.sl, 0, -1, sg);
     asm volatile("s_barrier" ::: "memory");  // buffer B may be overwritten now: its last reads fed this step
-    if (timing) { long long t = clock64(); t_last += t - t_mark; t_mark = t; }
   };
 
   for (int64_t tile = t_begin; tile < t_end; tile += 2) {
     tile_body(std::integral_constant<int, 0>{}, tile);
     if (tile + 1 < t_end) tile_body(std::integral_constant<int, 1>{}, tile + 1);
-  }
-  if (timing && lane == 0) {
-    long long* d = dbg + ((int64_t)blockIdx.x * 4 + wave) * 8;
-    d[0] = t_dma; d[1] = t_steps; d[2] = t_wait; d[3] = t_last; d[4] = t_end - t_begin;
   }
 
   // ---- per-range sums -> partial[split][slot][a][b] ----
@@ -414,11 +378,6 @@ __global__ __launch_bounds__(256, 1) void conv_wgrad_planned_kernel(
 
 using namespace ocnn;
 
-static long long* g_wp_dbg = nullptr;
-#ifdef OCNN_WP_TIMING
-// per-wave cycle counters of the kernel phases (development aid)
-extern "C" void ocnn_debug_set_wp_timing(long long* p) { g_wp_dbg = p; }
-#endif
 
 static int wp_splits(int K, int ca, int cb, int n_cu) {
   const int groups = (K == 27 && ca >= 64) ? 2 : 1;
@@ -465,11 +424,11 @@ static void launch_wp(const void* x, int64_t rows_x, const void* g, const uint16
   if (ca == C && cb == C)
     hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS, false>), dim3(nsplit * GROUPS),
                        dim3(256), 0, st, (const T*)x, xb, (const T*)g, gb, loc, lb, uptr, urows, ub, tiles, per,
-                       nsplit, ca, cb, partial, g_wp_dbg);
+                       nsplit, ca, cb, partial);
   else if constexpr (C == 64)
     hipLaunchKernelGGL((conv_wgrad_planned_kernel<T, C, KK, NFULL, NHALF, GROUPS, true>),
                        dim3(nsplit * GROUPS, ((ca + C - 1) / C) * ((cb + C - 1) / C)), dim3(256), 0, st, (const T*)x, xb, (const T*)g,
-                       gb, loc, lb, uptr, urows, ub, tiles, per, nsplit, ca, cb, partial, g_wp_dbg);
+                       gb, loc, lb, uptr, urows, ub, tiles, per, nsplit, ca, cb, partial);
 }
 
 template <typename T>

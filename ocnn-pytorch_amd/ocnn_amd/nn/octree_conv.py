@@ -25,8 +25,6 @@ from .octree_pad import octree_depad, octree_pad
 
 
 PAD_MIN_ROWS = 16384     # from this many table rows on, odd channel counts are zero-padded
-USE_WIDE = True          # the wide-layer gather kernel (switch for comparisons)
-USE_SPARSE = True        # the pair-list gather kernel for sparse tables
 SPARSE_MAX_OCCUPANCY = 0.3   # share of table entries that hold a row, up to which it is used
 SPARSE_MIN_ROWS = 32768      # (a workgroup loads its weights once and needs many tiles to pay for it)
 
@@ -85,7 +83,7 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
         int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return out, True
-  if (plan is not None and USE_SPARSE and plan.occupancy <= SPARSE_MAX_OCCUPANCY and
+  if (plan is not None and plan.occupancy <= SPARSE_MAX_OCCUPANCY and
       rows >= SPARSE_MIN_ROWS and L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)):
     pp = plan.pairs()
     ws = _lib.workspace(L.ocnn_conv_gather_sparse_workspace_bytes(cin, cout), data.device)
@@ -95,7 +93,7 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
         ctypes.addressof(pp.group_bounds_host), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
         _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return out, True
-  if plan is not None and plan.reuse >= 2.0 and USE_WIDE and L.ocnn_conv_gather_wide_supported(
+  if plan is not None and plan.reuse >= 2.0 and L.ocnn_conv_gather_wide_supported(
       code, rows_in, K, cin, cout, plan.umax):
     _lib.check(L.ocnn_conv_gather_wide(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
@@ -157,7 +155,7 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense):
   # channel counts that are not multiples of 64 on the table-row side the pair-plan kernel, which
   # sums exactly ca x cb and only over the pairs, beats the planned kernel's zero-padded 64 x 64
   # blocks on dense tables too: 96 -> 96 on 5.0 M rows 2.3 against 3.3 ms)
-  if (plan is not None and USE_SPARSE and (plan.occupancy <= SPARSE_MAX_OCCUPANCY or cb % 64 != 0) and
+  if (plan is not None and (plan.occupancy <= SPARSE_MAX_OCCUPANCY or cb % 64 != 0) and
       rows >= SPARSE_MIN_ROWS and not (ca == cb and ca in (32, 64)) and
       L.ocnn_conv_wgrad_sparse_supported(code, x.shape[0], rows, K, ca, cb, plan.umax)):
     pp = plan.pairs()
@@ -196,7 +194,7 @@ def conv_wgrad_inverse(x, g, plan_t, out_transposed=False):
   K = plan_t.K
   cx, cg = x.shape[1], g.shape[1]
   code = _lib.DTYPE_CODE.get(x.dtype, -1)
-  if not (USE_SPARSE and plan_t.rows == x.shape[0] and plan_t.rows >= SPARSE_MIN_ROWS and
+  if not (plan_t.rows == x.shape[0] and plan_t.rows >= SPARSE_MIN_ROWS and
           plan_t.occupancy <= SPARSE_MAX_OCCUPANCY and x.dtype == g.dtype and
           L.ocnn_conv_wgrad_sparse_supported(code, g.shape[0], x.shape[0], K, cg, cx, plan_t.umax)):
     return None

@@ -13,6 +13,7 @@ nnum / nnum_nempty stay on the host, as in the reference.
 from typing import List, Union
 
 import ctypes
+import threading
 
 import torch
 import torch.nn.functional as F
@@ -270,6 +271,38 @@ class PairPlan:
     _lib.check(L.ocnn_pair_plan_fill(_lib.ptr(plan.loc), self._tiles, self._K, _lib.ptr(self.lists), self.n_lists,
                                      _lib.ptr(self.cptr), _lib.ptr(self.ent), _lib.stream()))
     self._plan = self._counts = self._sizes = None
+
+
+class PlanHistory:
+  """Which tile plans (and pair plans) octrees of a kind (depth, full_depth) were asked for.
+  Bounded (the kinds and the plans of a kind seen least recently are dropped) and safe to
+  use from several threads."""
+
+  MAX_KINDS = 16
+  MAX_PLANS = 64
+
+  def __init__(self):
+    self._lock = threading.Lock()
+    self._kinds = {}           # kind -> {plan key: pair plan wanted}, both in order of last use
+
+  def requests(self, kind):
+    """Snapshot {plan key: pair plan wanted} of a kind."""
+    with self._lock:
+      return dict(self._kinds.get(kind, {}))
+
+  def note(self, kind, key, pairs=False):
+    with self._lock:
+      plans = self._kinds.pop(kind, {})
+      plans[key] = plans.pop(key, False) or pairs
+      while len(plans) > self.MAX_PLANS:
+        plans.pop(next(iter(plans)))
+      self._kinds[kind] = plans
+      while len(self._kinds) > self.MAX_KINDS:
+        self._kinds.pop(next(iter(self._kinds)))
+
+  def clear(self):
+    with self._lock:
+      self._kinds.clear()
 
 
 class Octree:
@@ -642,15 +675,19 @@ class Octree:
   # Plans asked for by earlier octrees of the same (depth, full_depth): a network asks every
   # octree for the same plans, layer by layer, and each plan built on its own costs two
   # device -> host read-backs in the middle of the step.  The first request on a fresh octree
-  # therefore builds all the plans its predecessors were asked for, together.
+  # therefore builds all the plans that `plan_history` holds for its kind, together.  The
+  # history is an object: the default one is shared by all octrees of the process; an octree
+  # (or a data loader, for all the octrees of one network) may carry its own
+  # (`octree.plan_history = PlanHistory()`), and `clear()` forgets what was asked for.
   PREBUILD_PLANS = True
-  _plan_requests = {}        # (depth, full_depth) -> {plan key: {'pairs': bool}}
+  plan_history = None        # set below to the process-wide default PlanHistory()
 
   def _plan(self, depth, kernel, stride, nempty, inverse=False, rows_in=None):
     """Tile plan of the table (or of its inverse), cached with the table."""
     ck = ((depth, kernel, stride, bool(nempty)), bool(inverse))
     if ck not in self._plans:
-      requests = Octree._plan_requests.setdefault((self.depth, self.full_depth), {})
+      history, kind = self.plan_history, (self.depth, self.full_depth)
+      requests = history.requests(kind)
       if Octree.PREBUILD_PLANS and requests and not self._plans_prebuilt:
         self._plans_prebuilt = True
         self._prebuild_plans(requests)
@@ -658,14 +695,11 @@ class Octree:
         t = (self._table_t(depth, kernel, stride, nempty, rows_in) if inverse
              else self._table(depth, kernel, stride, nempty))
         self._plans[ck] = TilePlan(t)
-      known = rows_in is None or rows_in == self._fine_rows(depth, nempty)
-      if ck not in requests and known:
-        requests[ck] = {'pairs': False}
-      if ck in requests:
-        entry = requests[ck]
+      if rows_in is None or rows_in == self._fine_rows(depth, nempty):
+        history.note(kind, ck)
         plan = self._plans[ck]
         if plan._pairs is None:
-          plan._on_pairs = lambda: entry.__setitem__('pairs', True)
+          plan._on_pairs = lambda: history.note(kind, ck, pairs=True)
     return self._plans[ck]
 
   def _fine_rows(self, depth, nempty):
@@ -683,7 +717,7 @@ class Octree:
     plans = TilePlan.build_many(tables)
     for ck, plan in zip(keys, plans):
       self._plans[ck] = plan
-    with_pairs = [plan for ck, plan in zip(keys, plans) if requests[ck]['pairs']]
+    with_pairs = [plan for ck, plan in zip(keys, plans) if requests[ck]]
     for plan, pp in zip(with_pairs, PairPlan.build_many(with_pairs)):
       plan._pairs = pp
 
@@ -830,3 +864,7 @@ def merge_octrees(octrees: List['Octree']):
 def init_octree(depth: int, full_depth: int = 2, batch_size: int = 1,
                 device: Union[torch.device, str] = 'cpu'):
   return Octree.init_octree(depth, full_depth, batch_size, device)
+
+
+
+Octree.plan_history = PlanHistory()

@@ -149,3 +149,21 @@ def test_pair_plan_lists_and_groups():
         assert max(sums) - min(sums) <= loads.max()
       if counts.max() * 24 > counts.sum() and K < 27:
         assert nl > K                                        # the heavy slot was cut
+
+
+def test_plan_history_is_bounded_and_clearable():
+  from ocnn_amd.octree.octree import PlanHistory
+  h = PlanHistory()
+  for kind in range(PlanHistory.MAX_KINDS + 5):
+    for j in range(PlanHistory.MAX_PLANS + 7):
+      h.note((kind, 2), ((j, '333', 1, False), False), pairs=j % 2 == 0)
+  assert len(h._kinds) == PlanHistory.MAX_KINDS
+  assert (0, 2) not in h._kinds                          # the kinds used least recently are dropped
+  last = h.requests((PlanHistory.MAX_KINDS + 4, 2))
+  assert len(last) == PlanHistory.MAX_PLANS and ((0, '333', 1, False), False) not in last
+  key = ((PlanHistory.MAX_PLANS + 6, '333', 1, False), False)
+  assert last[key] is True
+  h.note((PlanHistory.MAX_KINDS + 4, 2), key)            # a later plain request keeps the pair-plan wish
+  assert h.requests((PlanHistory.MAX_KINDS + 4, 2))[key] is True
+  h.clear()
+  assert h.requests((PlanHistory.MAX_KINDS + 4, 2)) == {}

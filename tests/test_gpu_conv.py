@@ -131,20 +131,14 @@ MFMA_SHAPES = [(32, 32), (64, 64), (64, 128), (128, 64), (32, 48), (96, 16)]
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize('tr', [1, 0])
-def test_mfma_conv_333(small, medium, dtype, tr):
-  """3x3x3 stride-1 conv on the MFMA kernels, several channel shapes, both
-  nempty modes, both ways of reading the weight-gradient tiles."""
-  _lib.lib().ocnn_set_wgrad_transpose_load(tr)
-  try:
-    for cin, cout in MFMA_SHAPES:
-      for pair, depth in ((small, 6), (medium, 7), (medium, 5)):
-        for ne in (False, True):
-          say('mfma conv', dtype, 'tr', tr, cin, cout, 'depth', depth, 'nempty', ne)
-          errs = run_layer('conv', pair, depth, [3], 1, ne, cin, cout, dtype)
-          assert max(errs.values()) < TOL[dtype], (cin, cout, depth, ne, errs)
-  finally:
-    _lib.lib().ocnn_set_wgrad_transpose_load(1)
+def test_mfma_conv_333(small, medium, dtype):
+  """3x3x3 stride-1 conv on the MFMA kernels, several channel shapes, both nempty modes."""
+  for cin, cout in MFMA_SHAPES:
+    for pair, depth in ((small, 6), (medium, 7), (medium, 5)):
+      for ne in (False, True):
+        say('mfma conv', dtype, cin, cout, 'depth', depth, 'nempty', ne)
+        errs = run_layer('conv', pair, depth, [3], 1, ne, cin, cout, dtype)
+        assert max(errs.values()) < TOL[dtype], (cin, cout, depth, ne, errs)
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
@@ -366,8 +360,9 @@ def test_fresh_octree_builds_the_plans_of_its_predecessors(medium):
     o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=3))
     o.construct_all_neigh()
     return o
-  saved = Octree._plan_requests
-  Octree._plan_requests = {}
+  from ocnn_amd.octree.octree import PlanHistory
+  saved = Octree.plan_history
+  Octree.plan_history = PlanHistory()
   try:
     first = fresh()
     keys = [(7, '333', 1, True, False), (6, '333', 1, True, False), (7, '222', 2, True, False),
@@ -393,7 +388,7 @@ def test_fresh_octree_builds_the_plans_of_its_predecessors(medium):
     assert len(third._plans) == 1
   finally:
     Octree.PREBUILD_PLANS = True
-    Octree._plan_requests = saved
+    Octree.plan_history = saved
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
