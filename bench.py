@@ -1,17 +1,22 @@
 """Benchmark of the octree sparse-convolution hot path on one MI355X.
 
-One step = OctreeConv 3x3x3 stride 1, 64 -> 64 channels, forward + backward
-(data and weight gradients) at depth 8 over a batch of 8 synthetic octrees
-(100k surface points each), fp16 features/weights with fp32 accumulation.
-Inputs (octree, tables, features) are resident in HBM before the timed region.
+One step = OctreeConv 3x3x3 stride 1, 64 -> 64 channels, forward + backward (data and weight
+gradients) through the module at depth 8 over a batch of 8 synthetic octrees (100k surface
+points each), bf16 features / weights with fp32 accumulation (configs[1] of BASELINE.json, in
+the dtype its target sentence names; the same step in fp16 is reported beside it).  Inputs
+(octree, tables, tile plans, features) are resident in HBM before the timed region.
 
-Prints one JSON line; `value` is effective TFLOP/s counting only non-empty
-neighbours (6 * nnz * Cin * Cout per step).
+Prints ONE JSON line.  `value` is effective TFLOP/s counting only non-empty neighbours
+(6 * nnz * Cin * Cout per step).  Beside it: the dominant kernel against its roofline, what
+the part itself sustains (MFMA rate with N(0, 1) operands), what a step costs when every step
+brings a new octree (build, tables, plans), compact records of the layers of configs[2] and
+configs[3], and the reference's CPU execution form timed on the host cores.
 """
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -20,11 +25,12 @@ for p in (ROOT, os.path.join(ROOT, 'ocnn-pytorch_amd')):
   if p not in sys.path:
     sys.path.insert(0, p)
 
-PEAK_MFMA_16BIT_TFLOPS = 2500.0     # MI355X dense bf16 / fp16
-PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the gather-GEMM kernel at the default workload (fp16, depth 8,
-# batch 8), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy; None for
-# any other workload.  The summary under profiles/ gives the counter readings.
+from bench_common import PEAK_HBM_GBS, PEAK_MFMA_16BIT_TFLOPS, build_octree, time_layer   # noqa: E402
+
+# HBM bytes per launch of the gather-GEMM kernel at the default workload, from the rocprofv3
+# FETCH_SIZE / WRITE_SIZE passes summarised in this file under profiles/ (not measured by this
+# run: counters need the profiler); None for any other workload.
+TRAFFIC_SOURCE = 'profiles/conv_gather_rw_hbm_traffic_depth8_c64_fp16.txt'
 TRAFFIC_GATHER_DEFAULT = int((209100 * 2.0 + 235970 * 1.0) * 1024)
 
 
@@ -33,14 +39,16 @@ def parse():
   ap.add_argument('--gpus', type=int, default=1)
   ap.add_argument('--steps', type=int, default=50)
   ap.add_argument('--warmup', type=int, default=10)
-  ap.add_argument('--dtype', default='fp16', choices=['fp16', 'bf16'])
+  ap.add_argument('--dtype', default='bf16', choices=['fp16', 'bf16'])
   ap.add_argument('--nempty', type=int, default=0)
   ap.add_argument('--depth', type=int, default=8)
   ap.add_argument('--batch', type=int, default=8)
   ap.add_argument('--points', type=int, default=100000)
   ap.add_argument('--channels', type=int, default=64)
   ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
-  ap.add_argument('--cpu-rows', type=int, default=262144)
+  ap.add_argument('--no-extras', action='store_true',
+                  help='headline step only: no second dtype, other layers, probes or fresh-octree steps')
+  ap.add_argument('--cpu-rows', type=int, default=524288)
   ap.add_argument('--only', default='all', choices=['all', 'fwd', 'bwd_data', 'wgrad'],
                   help='run a single pass per step (for counter collection); the JSON line is '
                        'then not a benchmark result')
@@ -80,11 +88,14 @@ class KernelTimer:
   def count(self):
     return len(self.events)
 
+  def reset(self):
+    self.events = []
+
 
 def cpu_baseline(torch, table32, rows_in, cin, cout, sample_rows):
-  """Times the reference's CPU execution form (chunked gather -> mm ->
-  scatter_add, oracle.conv_ref.BlockGemmCPU, fp32) on the first `sample_rows`
-  rows of the same neighbour table, forward + both gradients."""
+  """Times the reference's CPU execution form (chunked gather -> mm -> scatter_add,
+  oracle.conv_ref.BlockGemmCPU, fp32) on the first `sample_rows` rows of the same neighbour
+  table, forward + both gradients: one warm-up, three timed runs, the median."""
   from oracle.conv_ref import BlockGemmCPU
   g = torch.Generator().manual_seed(7)
   table = table32[:sample_rows].long().cpu()
@@ -92,25 +103,26 @@ def cpu_baseline(torch, table32, rows_in, cin, cout, sample_rows):
   W = torch.randn(27, cin, cout, generator=g) / 40.0
   grad = torch.randn(table.shape[0], cout, generator=g)
 
-  def one(tab, gr):
-    eng = BlockGemmCPU(tab, cin)
+  def one():
+    t0 = time.perf_counter()
+    eng = BlockGemmCPU(table, cin)
     eng.forward(data, W)
-    eng.backward(gr, W, rows_in)
-    eng.weight(data, gr, tuple(W.shape))
+    eng.backward(grad, W, rows_in)
+    eng.weight(data, grad, tuple(W.shape))
+    return time.perf_counter() - t0
 
-  one(table[:8192], grad[:8192])                      # warm-up
-  t0 = time.perf_counter()
-  one(table, grad)
-  dt = time.perf_counter() - t0
+  one()                                               # warm-up
+  runs = [one() for _ in range(3)]
+  dt = statistics.median(runs)
   nnz = int((table >= 0).sum())
   return {
       'value': 6.0 * nnz * cin * cout / dt / 1e12,
       'unit': 'TFLOP/s',
       'cores': torch.get_num_threads(),
       'kind': 'port',
-      'sample': 'first {} of {} table rows, fp32, fwd+bwd-data+bwd-weight, {:.2f} s; '
-                'host cpu_count={} affinity={}'.format(
-                    table.shape[0], table32.shape[0], dt, os.cpu_count(),
+      'sample': 'first {} of {} table rows, fp32, fwd+bwd-data+bwd-weight; 1 warm-up + 3 timed runs '
+                '({}) s, median {:.2f} s; host cpu_count={} affinity={}'.format(
+                    table.shape[0], table32.shape[0], ', '.join('%.2f' % r for r in runs), dt, os.cpu_count(),
                     len(os.sched_getaffinity(0))),
       'ms_per_step_extrapolated': dt * 1e3 * table32.shape[0] / table.shape[0],
   }
@@ -125,70 +137,85 @@ def main():
   import torch
   import ocnn_amd
   from ocnn_amd import synthetic
-  from ocnn_amd.nn import OctreeConv
+  from ocnn_amd.nn import OctreeConv, OctreeDeconv, OctreeDWConv
   import importlib
   conv_mod = importlib.import_module('ocnn_amd.nn.octree_conv')
   from ocnn_amd.octree import Octree, Points
+  from ocnn_amd.octree.octree import TilePlan
 
   assert torch.cuda.is_available(), 'bench.py needs a GPU'
   dev = 'cuda:0'
   torch.cuda.set_device(0)
-  dtype = torch.float16 if args.dtype == 'fp16' else torch.bfloat16
+  DT = {'fp16': torch.float16, 'bf16': torch.bfloat16}
+  dtype = DT[args.dtype]
   C = args.channels
   nempty = bool(args.nempty)
+  depth = args.depth
+  extras = not args.no_extras and args.only == 'all'
 
   # ---- inputs: synthetic clouds -> octree (timed separately) ----------------
-  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, args.batch, 1001, n=args.points)
-  pc = Points(pts.to(dev), nrm.to(dev), batch_id=bid.to(dev) if args.batch > 1 else None,
-              batch_size=args.batch)
-
-  def build():
-    o = Octree(args.depth, 2, batch_size=args.batch)
-    o.build_octree(pc)
-    torch.cuda.synchronize()
-    t = time.perf_counter()
-    o.construct_all_neigh()
-    torch.cuda.synchronize()
-    return o, time.perf_counter() - t
-
-  build()                                              # warm-up (first-use costs)
-  torch.cuda.synchronize()
-  t0 = time.perf_counter()
-  octree, neigh_s = build()
-  build_s = time.perf_counter() - t0 - neigh_s
-
-  depth = args.depth
+  build_octree(torch, synthetic, Octree, Points, synthetic.mixed_cloud, args.batch, 1001, args.points, depth, dev, 1)
+  octree, build_ms, neigh_ms, pts, _, pc = build_octree(torch, synthetic, Octree, Points, synthetic.mixed_cloud,
+                                                        args.batch, 1001, args.points, depth, dev)
   table = octree._table(depth, '333', 1, nempty)
   rows = table.shape[0]
   nnz = int((table >= 0).sum())
+  plan_ms = []
+  for _ in range(3):                                   # one tile plan, built alone (once per octree and table)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    TilePlan(table)
+    torch.cuda.synchronize()
+    plan_ms.append((time.perf_counter() - t0) * 1e3)
+
   g = torch.Generator().manual_seed(1001)
   conv = OctreeConv(C, C, [3], 1, nempty=nempty)
   with torch.no_grad():
     bound = 1.0 / (27 * C) ** 0.5                      # Kaiming-uniform bound
     conv.weights.copy_((torch.rand(conv.weights.shape, generator=g) * 2 - 1) * bound)
-  conv = conv.to(dev).to(dtype)
-  x = torch.randn(rows, C, generator=g).to(dtype).to(dev).requires_grad_()
-  gout = torch.randn(rows, C, generator=g).to(dtype).to(dev)
+  x32 = torch.randn(rows, C, generator=g)
+  gout32 = torch.randn(rows, C, generator=g)
 
   t_gather = KernelTimer(torch, conv_mod, 'conv_gather')
   t_wgrad = KernelTimer(torch, conv_mod, 'conv_wgrad')
-
   eng = conv_mod._OctreeConv(C, C, [3], 1, nempty)
   eng.setup(octree, depth)
-  w_cast = conv.weights.detach()
 
-  def step():
-    if args.only == 'fwd':
-      eng.forward_gemm(x.detach(), w_cast)
-    elif args.only == 'bwd_data':
-      eng.backward_gemm(gout, w_cast)
-    elif args.only == 'wgrad':
-      eng.weight_gemm(x.detach(), gout)
-    else:
-      x.grad = None
-      conv.weights.grad = None
-      out = conv(x, octree, depth)
-      out.backward(gout)
+  def timed_steps(dt, steps, warmup, oct=octree, only='all'):
+    """ms per step of the layer in dtype `dt` on octree `oct` (kernel timers enabled)."""
+    m = OctreeConv(C, C, [3], 1, nempty=nempty)
+    with torch.no_grad():
+      m.weights.copy_(conv.weights)
+    m = m.to(dev).to(dt)
+    x = x32.to(dt).to(dev).requires_grad_()
+    gout = gout32.to(dt).to(dev)
+    w_cast = m.weights.detach()
+
+    def step():
+      if only == 'fwd':
+        eng.forward_gemm(x.detach(), w_cast)
+      elif only == 'bwd_data':
+        eng.backward_gemm(gout, w_cast)
+      elif only == 'wgrad':
+        eng.weight_gemm(x.detach(), gout)
+      else:
+        x.grad = None
+        m.weights.grad = None
+        m(x, oct, depth).backward(gout)
+
+    for _ in range(warmup):
+      step()
+    torch.cuda.synchronize()
+    t_gather.reset()
+    t_wgrad.reset()
+    t_gather.enabled = t_wgrad.enabled = True
+    t0 = time.perf_counter()
+    for _ in range(steps):
+      step()
+    torch.cuda.synchronize()
+    dt_s = time.perf_counter() - t0
+    t_gather.enabled = t_wgrad.enabled = False
+    return dt_s * 1e3 / steps, t_gather.mean_ms(), t_wgrad.mean_ms(), t_gather.count()
 
   if args.calib:
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -197,32 +224,22 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
-  for _ in range(args.warmup):
-    step()
-  torch.cuda.synchronize()
-  t_gather.enabled = t_wgrad.enabled = True
-  t0 = time.perf_counter()
-  for _ in range(args.steps):
-    step()
-  torch.cuda.synchronize()
-  dt = time.perf_counter() - t0
-  ms = dt * 1e3 / args.steps
-
+  # ---- the headline step ------------------------------------------------------
+  ms, gather_ms, wgrad_ms, n_gather = timed_steps(dtype, args.steps, args.warmup, only=args.only)
+  gather_ms = gather_ms or float('nan')
+  wgrad_ms = wgrad_ms or float('nan')
   flops_step = 6.0 * nnz * C * C
-  gather_ms = t_gather.mean_ms() or float('nan')
-  wgrad_ms = t_wgrad.mean_ms() or float('nan')
   flops_launch = 2.0 * nnz * C * C
   achieved = flops_launch / (gather_ms * 1e-3) / 1e12
   es = 2                                               # bytes per feature element
   bytes_gather = es * (rows * C + rows * C + 27 * C * C) + 4 * rows * 27
   bytes_wgrad = es * (rows * C + rows * C) + 4 * rows * 27 + 4 * 27 * C * C
+  default_workload = (depth, args.batch, args.points, C, nempty) == (8, 8, 100000, 64, False)
 
-  default_workload = (args.depth, args.batch, args.points, C, nempty) == (8, 8, 100000, 64, False)
-  TRAFFIC_GATHER_BYTES = TRAFFIC_GATHER_DEFAULT if default_workload else None
   result = {
       'metric': 'OctreeConv 3x3x3 64->64 fwd+bwd at depth 8 (batch 8): effective TFLOP/s '
                 'over non-empty neighbours',
-      'value': flops_step / dt * args.steps / 1e12,
+      'value': flops_step / (ms * 1e-3) / 1e12,
       'unit': 'TFLOP/s',
       'n_gpus': 1,
       'steps': args.steps,
@@ -240,6 +257,7 @@ def main():
                           args.batch, depth, args.points, C, C, args.dtype, nempty),
           'rows': rows, 'nnz': nnz, 'valid_per_row': nnz / rows,
       },
+      'fraction_of_mfma_peak_whole_step': flops_step / (ms * 1e-3) / 1e12 / PEAK_MFMA_16BIT_TFLOPS,
       'roofline': {
           'kernel': 'conv_gather_rw_kernel (forward and data gradient; mean of both launches, '
                     'each bracketed with its weight-pack pre-pass)',
@@ -248,8 +266,10 @@ def main():
           'peak': PEAK_MFMA_16BIT_TFLOPS,
           'unit': 'TFLOP/s',
           'frac': achieved / PEAK_MFMA_16BIT_TFLOPS,
-          'traffic': TRAFFIC_GATHER_BYTES,
-          'launches': t_gather.count(),
+          'traffic': TRAFFIC_GATHER_DEFAULT if default_workload else None,
+          'traffic_source': (TRAFFIC_SOURCE + ' (rocprofv3 counters of an earlier run of this command, fp16; '
+                             'not measured by this run)') if default_workload else None,
+          'launches': n_gather,
           'avg_launch_ms': gather_ms,
           'algorithmic_flops_per_launch': flops_launch,
           'algorithmic_bytes_per_launch': bytes_gather,
@@ -260,22 +280,92 @@ def main():
           'conv_wgrad_ms': wgrad_ms,
           'conv_wgrad_tflops': flops_launch / (wgrad_ms * 1e-3) / 1e12,
           'conv_wgrad_algorithmic_bytes': bytes_wgrad,
-          'sustained_mfma_note': 'v_mfma_f32_32x32x16_f16 alone sustains 1.67 PFLOP/s on this part with '
-                                 'random operands (2.38 with constant ones): clocks drop under load',
-          'fraction_of_mfma_peak_whole_step': flops_step / (ms * 1e-3) / 1e12 / PEAK_MFMA_16BIT_TFLOPS,
       },
       'octree': {
           'points': int(pts.shape[0]),
-          'build_octree_ms': build_s * 1e3,
-          'construct_all_neigh_ms': neigh_s * 1e3,
+          'build_octree_ms': build_ms,
+          'construct_all_neigh_ms': neigh_ms,
+          'tile_plan_ms_per_table': min(plan_ms),
           'nnum': octree.nnum.tolist(),
           'nnum_nempty': octree.nnum_nempty.tolist(),
       },
   }
   if args.only != 'all':
     result['note'] = 'single-pass run (--only {}): not a benchmark result'.format(args.only)
+
+  if extras:
+    # ---- the same step in the other 16-bit type ------------------------------
+    other = 'fp16' if args.dtype == 'bf16' else 'bf16'
+    oms, ogm, owm, _ = timed_steps(DT[other], args.steps, args.warmup)
+    result['other_dtype'] = {'dtype': other, 'ms_per_step': oms, 'value': flops_step / (oms * 1e-3) / 1e12,
+                             'conv_gather_ms': ogm, 'conv_wgrad_ms': owm,
+                             'fraction_of_mfma_peak_whole_step': flops_step / (oms * 1e-3) / 1e12 /
+                             PEAK_MFMA_16BIT_TFLOPS}
+
+    # ---- what the part sustains: v_mfma_f32_32x32x16 alone, all CUs ----------
+    try:
+      from ocnn_amd import probe
+      sustained = {k: probe.mfma_rate(dtype, k, 20000)['tflops'] for k in ('constant', 'normal')}
+      result['mfma_sustained'] = {
+          'tflops_constant_operands': sustained['constant'], 'tflops_normal_operands': sustained['normal'],
+          'note': 'v_mfma_f32_32x32x16 back to back on every SIMD, {}: clocks fall under matrix load with '
+                  'random operands, so this, not the published peak, bounds any kernel on N(0,1) data'.format(
+                      args.dtype),
+          'step_fraction_of_sustained_normal': flops_step / (ms * 1e-3) / 1e12 / sustained['normal'],
+          'gather_kernel_dense_fraction_of_sustained_normal':
+              (2.0 * rows * 28 * C * C / (gather_ms * 1e-3) / 1e12) / sustained['normal'],
+      }
+    except Exception as e:                              # the probe library is optional
+      result['mfma_sustained'] = {'error': repr(e)}
+
+    # ---- a new octree every step, as in training: build, tables, plans, step ---
+    fresh = []
+    for _ in range(3):
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      o = Octree(depth, 2, batch_size=args.batch)
+      o.build_octree(pc)
+      o.construct_all_neigh()
+      torch.cuda.synchronize()
+      t1 = time.perf_counter()
+      fms, _, _, _ = timed_steps(dtype, 1, 0, oct=o)
+      fresh.append(((t1 - t0) * 1e3, fms))
+    fresh.sort(key=lambda v: v[0] + v[1])
+    result['fresh_octree'] = {'build_and_tables_ms': fresh[1][0], 'first_step_with_plan_build_ms': fresh[1][1],
+                              'note': 'median of 3; the step includes the tile plan of its table (built once per '
+                                      'octree and table, shared by every layer and pass that uses the table)'}
+
+    # ---- the layers of configs[2] and configs[3], bf16, forward + backward -----
+    bf = torch.bfloat16
+    ks, kw = min(args.steps, 20), min(args.warmup, 5)
+    layers = []
+    nn8, ne8, nn7 = int(octree.nnum[8]), int(octree.nnum_nempty[8]), int(octree.nnum[7])
+    run = lambda *a, **k: layers.append(time_layer(torch, *a, steps=ks, warmup=kw, dev=dev, **k))
+    if default_workload:
+      run('configs[2] conv 2x2x2 s2 64->128 d8->7', OctreeConv(64, 128, [2], 2), octree, 8, nn8, 64, 128,
+          octree._table(8, '222', 2, False), bf)
+      run('configs[2] deconv 2x2x2 s2 128->64 d7->8', OctreeDeconv(128, 64, [2], 2), octree, 7, nn7, 128, 64,
+          octree._table(8, '222', 2, False), bf)
+      run('configs[2] dwconv 3x3x3 128 d7', OctreeDWConv(128, [3], 1), octree, 7, nn7, 128, 128,
+          octree._table(7, '333', 1, False), bf, dw=True)
+      run('configs[1] nempty=True: conv 3x3x3 s1 64->64 d8', OctreeConv(64, 64, [3], 1, nempty=True), octree, 8, ne8,
+          64, 64, octree._table(8, '333', 1, True), bf)
+      o3, b3, n3, p3, _, _ = build_octree(torch, synthetic, Octree, Points, synthetic.planes_cloud, 4, 1003, 250000,
+                                          9, dev)
+      run('configs[3] conv 3x3x3 s1 32->32 d9', OctreeConv(32, 32, [3], 1), o3, 9, int(o3.nnum[9]), 32, 32,
+          o3._table(9, '333', 1, False), bf)
+      run('configs[3] conv 3x3x3 s1 256->256 d6', OctreeConv(256, 256, [3], 1), o3, 6, int(o3.nnum[6]), 256, 256,
+          o3._table(6, '333', 1, False), bf)
+      result['configs3_octree'] = {'points': int(p3.shape[0]), 'build_octree_ms': b3, 'construct_all_neigh_ms': n3,
+                                   'nnum_depth9': int(o3.nnum[9]), 'nnum_nempty_depth9': int(o3.nnum_nempty[9])}
+      del o3
+    result['other_layers'] = [
+        {'layer': r['layer'], 'ms_fwd_bwd': round(r['ms_fwd_bwd'], 4), 'eff_tflops': round(r['eff_tflops'], 1),
+         'pct_mfma_peak': round(100 * r['frac_mfma_peak'], 2),
+         'pct_hbm_peak': round(100 * r['frac_hbm_peak_at_algorithmic_bytes'], 1)} for r in layers]
+
   if not args.no_cpu:
-    result['cpu_baseline'] = cpu_baseline(torch, table, x.shape[0], C, C, args.cpu_rows)
+    result['cpu_baseline'] = cpu_baseline(torch, table, rows, C, C, args.cpu_rows)
   print(json.dumps(result))
 
 
