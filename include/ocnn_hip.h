@@ -95,6 +95,20 @@ int ocnn_build_level_fill(const int64_t* node_key, const int32_t* pidx,
                           int64_t* keys, int32_t* children, int64_t* next_key,
                           void* stream);
 
+/* Regrowing an octree from split decisions, ocnn/octree/octree.py:323-351 (octree_split) and
+ * :353-402 (octree_grow).
+ * split_children: children[i] = ordinal of node i among the nodes with split[i] != 0, or -1;
+ *        *count (device) = their number.  A layer without any split node keeps node 0
+ *        (children[0] = 0, count 1), as the reference does.  Workspace as for
+ *        ocnn_build_level_count.
+ * grow_layer: the layer below `n_nempty` non-empty nodes (nempty_index = their rows, keys of
+ *        their layer in key_above): keys[8 p + j] = key of the p-th of them with j appended
+ *        below the batch bits, children[8 p + j] = 8 p + j. */
+int ocnn_split_children(const int32_t* split, int64_t n, void* workspace, int64_t workspace_bytes,
+                        int32_t* children, int64_t* count, void* stream);
+int ocnn_grow_layer(const int64_t* key_above, const int32_t* nempty_index, int64_t n_nempty,
+                    int64_t* keys, int32_t* children, void* stream);
+
 /* Per-leaf signal of ocnn/octree/octree.py:273-281: sequential fp32 sum of
  * the leaf's points (in point order), then mode 0: divide by the count
  * (points, features); mode 1: L2-normalise with eps 1e-12 (normals). */

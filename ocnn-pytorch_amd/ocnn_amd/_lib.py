@@ -27,6 +27,8 @@ SIGNATURES = {
     'ocnn_build_level_workspace_bytes': (_l, [_l]),
     'ocnn_build_level_count': (_i, [_p, _l, _p, _l, _p, _p, _p]),
     'ocnn_build_level_fill': (_i, [_p, _p, _l, _l, _i, _p, _p, _p, _p]),
+    'ocnn_split_children': (_i, [_p, _l, _p, _l, _p, _p, _p]),
+    'ocnn_grow_layer': (_i, [_p, _p, _l, _p, _p, _p]),
     'ocnn_leaf_average': (_i, [_p, _i, _p, _p, _l, _i, _p, _p]),
     'ocnn_neigh_full': (_i, [_i, _i, _p, _p, _p]),
     'ocnn_neigh_from_parent': (_i, [_p, _p, _p, _l, _p, _p, _p]),

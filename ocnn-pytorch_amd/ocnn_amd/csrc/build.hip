@@ -113,6 +113,37 @@ __global__ void leaf_normal_kernel(const float* src, const int32_t* perm,
   out[3 * leaf + 2] = az / d;
 }
 
+// ---- regrowing an octree from split decisions (generative decoders) ----------------------
+__global__ void split_flag_kernel(const int32_t* split, int64_t n, int32_t* flag) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) flag[i] = split[i] != 0;
+}
+
+// rank = inclusive count of the split nodes up to i.  A layer in which nothing is split keeps
+// node 0 as its one non-empty node (the reference does, so that the next layer is never empty).
+__global__ void split_children_kernel(const int32_t* flag, const int32_t* rank, int64_t n,
+                                      int32_t* children, int64_t* count) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int32_t total = rank[n - 1];
+  int32_t c = flag[i] ? rank[i] - 1 : -1;
+  if (total == 0 && i == 0) c = 0;
+  children[i] = c;
+  if (i == 0) *count = total == 0 ? 1 : total;
+}
+
+// Node 8 p + j of the new layer is child j of the p-th non-empty node of the layer above:
+// its key is that node's key with j appended below the batch bits; it is numbered as itself.
+__global__ void grow_layer_kernel(const int64_t* key_above, const int32_t* nempty_index, int64_t n_out,
+                                  int64_t* keys, int32_t* children) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_out) return;
+  const int64_t k = key_above[nempty_index[i >> 3]];
+  const int64_t low = k & ((1ll << 48) - 1);
+  keys[i] = (k - low) | (low << 3) | (i & 7);
+  children[i] = (int32_t)i;
+}
+
 struct SortLayout {
   int64_t ckey, csorted, iota, flag, uid, temp, temp_bytes, total;
 };
@@ -239,6 +270,34 @@ extern "C" int ocnn_build_level_fill(const int64_t* node_key, const int32_t* pid
                      children, next_key);
   hipLaunchKernelGGL(level_fill_child_kernel, grid, block, 0, st, node_key, pidx, n, children);
   return check_launch("build_level_fill");
+}
+
+extern "C" int ocnn_split_children(const int32_t* split, int64_t n, void* workspace, int64_t workspace_bytes,
+                                   int32_t* children, int64_t* count, void* stream) {
+  OCNN_REQUIRE(n > 0 && n < (1ll << 28), "split_children: n=%lld out of range", (long long)n);
+  LevelLayout L;
+  if (level_layout(n, &L) != OCNN_OK) { set_error("split_children: rocprim size query failed"); return OCNN_ERR_HIP; }
+  if (workspace_bytes < L.total) { set_error("split_children: workspace %lld < %lld", (long long)workspace_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  int32_t* flag = (int32_t*)(ws + L.flag);
+  int32_t* rank = (int32_t*)(ws + L.uid);
+  dim3 grid(cdiv(n, 256)), block(256);
+  hipLaunchKernelGGL(split_flag_kernel, grid, block, 0, st, split, n, flag);
+  size_t tb = (size_t)L.temp_bytes;
+  hipError_t e = rocprim::inclusive_scan(ws + L.temp, tb, flag, rank, (size_t)n, rocprim::plus<int32_t>(), st);
+  if (e != hipSuccess) { set_error("split_children: scan: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
+  hipLaunchKernelGGL(split_children_kernel, grid, block, 0, st, flag, rank, n, children, count);
+  return check_launch("split_children");
+}
+
+extern "C" int ocnn_grow_layer(const int64_t* key_above, const int32_t* nempty_index, int64_t n_nempty,
+                               int64_t* keys, int32_t* children, void* stream) {
+  OCNN_REQUIRE(n_nempty > 0 && n_nempty < (1ll << 28), "grow_layer: n_nempty=%lld out of range",
+               (long long)n_nempty);
+  hipLaunchKernelGGL(grow_layer_kernel, dim3(cdiv(8 * n_nempty, 256)), dim3(256), 0, (hipStream_t)stream,
+                     key_above, nempty_index, 8 * n_nempty, keys, children);
+  return check_launch("grow_layer");
 }
 
 extern "C" int ocnn_leaf_average(const float* src, int channels, const int32_t* perm,

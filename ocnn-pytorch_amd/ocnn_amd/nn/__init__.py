@@ -1,4 +1,5 @@
 from .octree_pad import octree_pad, octree_depad
+from .octree2col import octree2col, col2octree
 from .octree_conv import (OctreeConv, OctreeDeconv, OctreeConvBase, octree_conv, octree_deconv,
                           conv_gather, conv_wgrad, column_sum)
 from .octree_dwconv import OctreeDWConv, octree_dwconv
@@ -12,7 +13,7 @@ from .octree_pool import (octree_max_pool, octree_max_unpool, OctreeMaxPool, Oct
 from .octree_interp import (octree_nearest_pts, octree_linear_pts, OctreeInterp,
                             octree_nearest_upsample, OctreeUpsample)
 
-__all__ = ['octree_pad', 'octree_depad', 'OctreeConv', 'OctreeDeconv', 'octree_conv',
+__all__ = ['octree_pad', 'octree_depad', 'octree2col', 'col2octree', 'OctreeConv', 'OctreeDeconv', 'octree_conv',
            'octree_deconv', 'OctreeDWConv', 'octree_dwconv', 'OctreeConvTriton', 'OctreeConvT',
            'octree_conv_triton', 'convert_conv_triton', 'conv_fwd_implicit_gemm_splitk',
            'conv_bwd_implicit_gemm_splitk', 'octree_max_pool', 'octree_max_unpool', 'OctreeMaxPool',

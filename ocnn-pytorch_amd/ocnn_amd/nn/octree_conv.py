@@ -21,6 +21,7 @@ from torch.autograd import Function
 
 from .. import _lib
 from ..utils import list2str, resize_with_last_val, xavier_uniform_
+from .octree2col import col2octree, octree2col
 from .octree_pad import octree_depad, octree_pad
 
 
@@ -429,8 +430,10 @@ octree_deconv = OctreeDeconvFunction.apply
 class OctreeConv(OctreeConvBase, torch.nn.Module):
   """Octree convolution.  Constructor, parameters (`weights` (kdim, Cin, Cout),
   `bias`) and forward(data, octree, depth) follow ocnn/nn/octree_conv.py:300-431.
-  `method` and `max_buffer` are accepted and ignored: every kernel shape,
-  stride and nempty mode runs on the same HIP engine."""
+  `max_buffer` is accepted and ignored (nothing is buffered).  method='explicit_gemm' takes
+  the reference's im2col route (octree2col + torch.mm, ocnn/nn/octree_conv.py:366-376); every
+  other method name of the reference ('block_gemm', 'triton') and 'hip' run the HIP engine,
+  for every kernel shape, stride and nempty mode."""
 
   def __init__(self, in_channels: int, out_channels: int, kernel_size: List[int] = [3],
                stride: int = 1, nempty: bool = False, method: str = 'triton',
@@ -445,7 +448,12 @@ class OctreeConv(OctreeConvBase, torch.nn.Module):
   def check_method(self, method: str):
     if method not in ('explicit_gemm', 'block_gemm', 'triton', 'hip'):
       raise ValueError('Unknown method: {}'.format(method))
-    return 'hip'
+    return 'explicit_gemm' if method == 'explicit_gemm' else 'hip'
+
+  def explicit_gemm(self, data: torch.Tensor, octree, depth: int):
+    """im2col, then one matrix product (autograd differentiates the torch ops)."""
+    col = octree2col(data, octree, depth, self.kernel, self.stride, self.nempty)
+    return torch.mm(col.flatten(1), self.weights.to(data.dtype).flatten(0, 1))
 
   def reset_parameters(self):
     xavier_uniform_(self.weights)
@@ -455,8 +463,11 @@ class OctreeConv(OctreeConvBase, torch.nn.Module):
   def is_conv_layer(self): return True
 
   def forward(self, data: torch.Tensor, octree, depth: int):
-    out = octree_conv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
-                      self.kernel_size, self.stride, self.nempty, self.max_buffer)
+    if self.method == 'explicit_gemm':
+      out = self.explicit_gemm(data, octree, depth)
+    else:
+      out = octree_conv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
+                        self.kernel_size, self.stride, self.nempty, self.max_buffer)
     if self.use_bias:
       out = out + self.bias.to(out.dtype)
     if self.stride == 2 and not self.nempty:
@@ -479,8 +490,14 @@ class OctreeDeconv(OctreeConv):
   def forward(self, data: torch.Tensor, octree, depth: int):
     if self.stride == 2 and not self.nempty:
       data = octree_depad(data, octree, depth)
-    out = octree_deconv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
-                        self.kernel_size, self.stride, self.nempty, self.max_buffer)
+    if self.method == 'explicit_gemm':
+      # one product for all slots, then the adjoint of im2col (ocnn/nn/octree_conv.py:453-457)
+      col = torch.mm(data, self.weights.to(data.dtype).flatten(0, 1).t())
+      out = col2octree(col.view(col.shape[0], self.kdim, -1), octree, depth + (self.stride == 2), self.kernel,
+                       self.stride, self.nempty)
+    else:
+      out = octree_deconv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
+                          self.kernel_size, self.stride, self.nempty, self.max_buffer)
     if self.use_bias:
       out = out + self.bias.to(out.dtype)
     return out

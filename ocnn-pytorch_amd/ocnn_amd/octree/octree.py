@@ -543,44 +543,51 @@ class Octree:
       self.construct_neigh(depth)
 
   def octree_split(self, split: torch.Tensor, depth: int):
-    """Sets which nodes of `depth` are split (ocnn/octree/octree.py:323-351)."""
-    empty = split == 0
-    total = cumsum(split, dim=0, exclusive=True)
-    children, nnum_nempty = torch.split(total, [split.shape[0], 1])
-    children[empty] = -1
-    if nnum_nempty == 0:
-      nnum_nempty = 1
-      children[0] = 0
-    self.children[depth] = children.int()
-    self.nnum_nempty[depth] = nnum_nempty
+    """Declares which nodes of `depth` have children: `split` holds one number per node, non
+    zero = split (ocnn/octree/octree.py:323-351).  One scan kernel numbers the split nodes;
+    the count comes back with one read."""
+    n = int(split.shape[0])
+    assert n == int(self.nnum[depth]), 'one split decision per node of the layer'
+    L = _lib.lib()
+    flags = (split != 0).to(torch.int32).contiguous()
+    _lib.require_gpu(flags)
+    children = torch.empty(n, dtype=torch.int32, device=flags.device)
+    count = torch.zeros(1, dtype=torch.long, device=flags.device)
+    ws = _lib.workspace(L.ocnn_build_level_workspace_bytes(n), flags.device)
+    _lib.check(L.ocnn_split_children(_lib.ptr(flags), n, _lib.ptr(ws), ws.numel(), _lib.ptr(children),
+                                     _lib.ptr(count), _lib.stream()))
+    self.children[depth] = children
+    self.nnum_nempty[depth] = int(count)
     self._drop_nempty(depth)
 
-  def octree_grow(self, depth: int, update_neigh: bool = True):
-    """Adds the children layer of the split nodes (ocnn/octree/octree.py:353-402)."""
-    if depth > self.depth:
-      assert depth == self.depth + 1
-      self.depth = depth
-      for lst in (self.keys, self.children, self.features, self.normals, self.points,
-                  self.nempty_masks, self.nempty_indices, self.nempty_neighs,
-                  self._nempty_indices32):
-        lst.append(None)
-      self.neighs.append(None)
-      zero = torch.zeros(1, dtype=torch.long)
-      self.nnum = torch.cat([self.nnum, zero])
-      self.nnum_nempty = torch.cat([self.nnum_nempty, zero])
-      zero = torch.zeros([1, self.batch_size], dtype=torch.long)
-      self.batch_nnum = torch.cat([self.batch_nnum, zero], dim=0)
-      self.batch_nnum_nempty = torch.cat([self.batch_nnum_nempty, zero], dim=0)
+  def _append_layer(self):
+    """Room for one more layer in every per-depth list and count."""
+    self.depth += 1
+    for per_depth in (self.keys, self.children, self.features, self.normals, self.points, self.nempty_masks,
+                      self.nempty_indices, self.nempty_neighs, self._nempty_indices32, self.neighs):
+      per_depth.append(None)
+    self.nnum = torch.cat([self.nnum, self.nnum.new_zeros(1)])
+    self.nnum_nempty = torch.cat([self.nnum_nempty, self.nnum_nempty.new_zeros(1)])
+    self.batch_nnum = torch.cat([self.batch_nnum, self.batch_nnum.new_zeros(1, self.batch_size)])
+    self.batch_nnum_nempty = torch.cat([self.batch_nnum_nempty, self.batch_nnum_nempty.new_zeros(1, self.batch_size)])
 
-    nnum = self.nnum_nempty[depth - 1] * 8
-    self.nnum[depth] = nnum
-    self.nnum_nempty[depth] = nnum
-    key = self.key(depth - 1, nempty=True)
-    batch_id = (key >> 48) << 48
-    key = ((key & ((1 << 48) - 1)) << 3) | batch_id
-    key = key.unsqueeze(1) + torch.arange(8, device=key.device)
-    self.keys[depth] = key.view(-1)
-    self.children[depth] = torch.arange(int(nnum), dtype=torch.int32, device=self.device)
+  def octree_grow(self, depth: int, update_neigh: bool = True):
+    """Creates layer `depth` as the children of the non-empty nodes of the layer above it, all
+    of them marked non-empty until octree_split says otherwise
+    (ocnn/octree/octree.py:353-402); the octree gets one layer deeper when needed."""
+    if depth > self.depth:
+      assert depth == self.depth + 1, 'layers are grown one at a time'
+      self._append_layer()
+    parents = int(self.nnum_nempty[depth - 1])
+    total = 8 * parents
+    above = self.keys[depth - 1]
+    _lib.require_gpu(above)
+    keys = torch.empty(total, dtype=torch.long, device=above.device)
+    children = torch.empty(total, dtype=torch.int32, device=above.device)
+    _lib.check(_lib.lib().ocnn_grow_layer(_lib.ptr(above), _lib.ptr(self._nempty_index32(depth - 1)), parents,
+                                          _lib.ptr(keys), _lib.ptr(children), _lib.stream()))
+    self.keys[depth], self.children[depth] = keys, children
+    self.nnum[depth] = self.nnum_nempty[depth] = total
     self._drop_nempty(depth)
     if update_neigh:
       self.construct_neigh(depth)
@@ -742,62 +749,56 @@ class Octree:
 
   # ---- input signal (ocnn/octree/octree.py:525-568) -------------------------
   def get_input_feature(self, feature: str, nempty: bool = False):
+    """The input signal of the finest layer, one block of channels per letter of `feature`, in
+    the fixed order N D L P F whatever the order of the letters:
+      N  the leaf normals (3)             D  <offset of the leaf's mean point from the
+      L  that offset itself (3)              voxel centre, normal> (1)
+      P  the mean point in [-1, 1] (3)    F  the leaf features
+    Rows of empty nodes are zero unless nempty (ocnn/octree/octree.py:525-568)."""
     from ..nn.octree_pad import octree_pad
-    features = []
-    depth = self.depth
-    feature = feature.upper()
-    if 'N' in feature:
-      features.append(self.normals[depth])
-    if 'L' in feature or 'D' in feature:
-      local_points = self.points[depth].frac() - 0.5
-    if 'D' in feature:
-      features.append(torch.sum(local_points * self.normals[depth], dim=1, keepdim=True))
-    if 'L' in feature:
-      features.append(local_points)
-    if 'P' in feature:
-      features.append(self.points[depth] * (2 ** (1 - depth)) - 1.0)
-    if 'F' in feature:
-      features.append(self.features[depth])
-    out = torch.cat(features, dim=1)
-    if not nempty:
-      out = octree_pad(out, self, depth)
-    return out
+    depth, wanted = self.depth, set(feature.upper())
+    normals, points = self.normals[depth], self.points[depth]
+    offset = points.frac() - 0.5 if wanted & {'L', 'D'} else None
+    blocks = {
+        'N': lambda: normals,
+        'D': lambda: (offset * normals).sum(dim=1, keepdim=True),
+        'L': lambda: offset,
+        'P': lambda: points * (2.0 ** (1 - depth)) - 1.0,
+        'F': lambda: self.features[depth],
+    }
+    out = torch.cat([blocks[c]() for c in 'NDLPF' if c in wanted], dim=1)
+    return out if nempty else octree_pad(out, self, depth)
 
   def to_points(self, rescale: bool = True):
+    """The leaves as a point cloud: their mean points (voxel centres when the octree holds
+    none), in [-1, 1] when rescale, with the leaf normals and features."""
     depth = self.depth
     xyz = self.points[depth]
-    batch_id = self.batch_id(depth, nempty=True)
     if xyz is None:
       x, y, z, batch_id = self.xyzb(depth, nempty=True)
       xyz = torch.stack([x, y, z], dim=1) + 0.5
+    else:
+      batch_id = self.batch_id(depth, nempty=True)
     if rescale:
-      xyz = xyz * (2 ** (1 - depth)) - 1.0
+      xyz = xyz * (2.0 ** (1 - depth)) - 1.0
     return Points(xyz, self.normals[depth], self.features[depth], batch_id=batch_id,
                   batch_size=self.batch_size)
 
   # ---- device moves, batching (ocnn/octree/octree.py:600-752) ---------------
   def to(self, device: Union[torch.device, str], non_blocking: bool = False):
-    if isinstance(device, str):
-      device = torch.device(device)
+    """A copy on `device` (the octree itself when it is there already).  The node counts are
+    host tensors on any device, so that shape queries never wait for the GPU."""
+    device = torch.device(device)
     if self.device == device:
       return self
-
-    def mv(prop):
-      return [p.to(device, non_blocking=non_blocking) if isinstance(p, torch.Tensor) else None
-              for p in prop]
-
-    octree = Octree.init_like(self, device)
-    octree.keys = mv(self.keys)
-    octree.children = mv(self.children)
-    octree.neighs = self.neighs.moved(device, non_blocking)
-    octree.features = mv(self.features)
-    octree.normals = mv(self.normals)
-    octree.points = mv(self.points)
-    octree.nnum = self.nnum.clone()
-    octree.nnum_nempty = self.nnum_nempty.clone()
-    octree.batch_nnum = self.batch_nnum.clone()
-    octree.batch_nnum_nempty = self.batch_nnum_nempty.clone()
-    return octree
+    moved = Octree.init_like(self, device)
+    for name in ('keys', 'children', 'features', 'normals', 'points'):
+      setattr(moved, name, [None if t is None else t.to(device, non_blocking=non_blocking)
+                            for t in getattr(self, name)])
+    moved.neighs = self.neighs.moved(device, non_blocking)
+    for name in ('nnum', 'nnum_nempty', 'batch_nnum', 'batch_nnum_nempty'):
+      setattr(moved, name, getattr(self, name).clone())
+    return moved
 
   def cuda(self, non_blocking: bool = False):
     return self.to('cuda', non_blocking)

@@ -104,6 +104,22 @@ def octree_depad(data, oct, depth):
   return data[oct.nempty_index(depth)]
 
 
+def octree2col(data, table):
+  """ocnn/nn/octree2col.py:15-38 on a given table: (rows, K, C), zeros at -1 entries."""
+  out = np.zeros((table.shape[0], table.shape[1], data.shape[1]), data.dtype)
+  valid = table >= 0
+  out[valid] = data[table[valid]]
+  return out
+
+
+def col2octree(col, table, rows_in):
+  """ocnn/nn/octree2col.py:41-53: out[t_ik] += col[i, k] over the valid entries."""
+  out = np.zeros((rows_in, col.shape[2]), col.dtype)
+  valid = table >= 0
+  np.add.at(out, table[valid], col[valid])
+  return out
+
+
 # --------------------------------------------------------------------------
 # layer level: shapes as in OctreeConvBase.setup (octree_conv.py:51-100)
 # --------------------------------------------------------------------------

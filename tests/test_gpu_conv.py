@@ -216,6 +216,55 @@ def test_table_level_api(small):
   assert rel_err(mod(x.detach(), small.gpu, depth), want[0]) < 2e-2
 
 
+@pytest.mark.parametrize('nempty', [False, True])
+def test_octree2col_and_col2octree(small, nempty):
+  say('octree2col / col2octree against the oracle, all kernel shapes and strides, nempty', nempty)
+  from ocnn_amd.nn import col2octree, octree2col
+  g = torch.Generator().manual_seed(12)
+  d = 5
+  rows_in = rows_of(small.ref, d, nempty)
+  data = torch.randn(rows_in, 5, generator=g)
+  for kern in ['333', '222', '311', '131', '113', '331', '313', '133']:
+    for stride in (1, 2):
+      table = small.ref.get_neigh(d, kern, stride, nempty)
+      col = octree2col(data.to(DEV), small.gpu, d, kern, stride, nempty)
+      want = C.octree2col(f64(data), table)
+      assert col.dtype == torch.float32 and np.array_equal(f64(col), want), (kern, stride)
+      other = torch.randn(col.shape, generator=g)
+      back = col2octree(other.to(DEV), small.gpu, d, kern, stride, nempty)
+      assert rel_err(back, C.col2octree(f64(other), table, rows_in)) < 1e-6, (kern, stride)
+
+
+@pytest.mark.parametrize('kind', ['conv', 'deconv'])
+def test_explicit_gemm_equals_the_hip_engine(small, kind):
+  """The reference's own cross-check (test/test_octree_conv.py:85-163): the im2col route
+  through autograd against the engine, output, data gradient and weight gradient, over kernel
+  shapes x strides x nempty, fp32."""
+  g = torch.Generator().manual_seed(13)
+  depth, cin, cout = 5, 6, 7
+  Mod = OctreeConv if kind == 'conv' else OctreeDeconv
+  for kern, stride, ne in GRID:
+    ks = [int(c) for c in kern]
+    mods = [Mod(cin, cout, ks, stride, ne, method=m, use_bias=True).to(DEV) for m in ('explicit_gemm', 'hip')]
+    assert mods[0].method == 'explicit_gemm' and mods[1].method == 'hip'
+    with torch.no_grad():
+      mods[0].bias.copy_(torch.randn(cout, generator=g))
+      mods[1].weights.copy_(mods[0].weights)
+      mods[1].bias.copy_(mods[0].bias)
+    data = torch.randn(rows_of(small.ref, depth, ne), cin, generator=g)
+    res = []
+    for m in mods:
+      x = data.to(DEV).requires_grad_()
+      out = m(x, small.gpu, depth)
+      if not res:
+        gout = torch.randn(out.shape, generator=g).to(DEV)
+      out.backward(gout)
+      res.append((out, x.grad, m.weights.grad, m.bias.grad))
+    for name, a, b in zip(('out', 'gdata', 'gw', 'gb'), res[0], res[1]):
+      assert a.shape == b.shape, (kind, kern, stride, ne, name)
+      assert rel_err(b, f64(a)) < 1e-4, (kind, kern, stride, ne, name)
+
+
 def test_pad_depad(small):
   say('octree_pad / octree_depad')
   d = 5

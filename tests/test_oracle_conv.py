@@ -295,3 +295,27 @@ def test_block_gemm_cpu_matches_definition(oct):
 def test_shape_check(oct):
   with pytest.raises(AssertionError):
     C.conv_layer(oct, np.zeros((3, 2)), np.zeros((27, 2, 2)), 4)
+
+
+@pytest.mark.parametrize('kernel,stride,nempty', GRID)
+def test_im2col_form_equals_the_engine(oct, kernel, stride, nempty):
+  """octree2col + one matrix product is the forward pass, the product + col2octree the
+  backward one (what the reference's explicit_gemm route computes, octree_conv.py:366-376,
+  453-457), and col2octree is the adjoint of octree2col."""
+  rng = np.random.default_rng(3)
+  table = oct.get_neigh(5, kernel, stride, nempty)
+  rows_in = int(oct.nnum_nempty[5] if nempty else oct.nnum[5])
+  K = table.shape[1]
+  data = rng.standard_normal((rows_in, 3))
+  W = rng.standard_normal((K, 3, 4))
+  col = C.octree2col(data, table)
+  assert col.shape == (table.shape[0], K, 3)
+  assert np.all(col[table < 0] == 0)
+  np.testing.assert_allclose(col.reshape(len(table), -1) @ W.reshape(-1, 4), C.forward_gemm(data, W, table),
+                             atol=1e-12)
+  grad = rng.standard_normal((table.shape[0], 4))
+  gcol = (grad @ W.reshape(-1, 4).T).reshape(len(table), K, 3)
+  np.testing.assert_allclose(C.col2octree(gcol, table, rows_in), C.backward_gemm(grad, W, table, rows_in),
+                             atol=1e-12)
+  other = rng.standard_normal(col.shape)
+  assert abs((col * other).sum() - (data * C.col2octree(other, table, rows_in)).sum()) < 1e-9
