@@ -224,6 +224,18 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
+  # ---- from a cold start: the first steps, in blocks of five ----------------------
+  # The step time falls over the first 30 ms or so of sustained work (1.21 -> 1.03 ms here;
+  # it does again after a second of idling, and also right after 50 ms of matrix work that
+  # touches no memory: it is the memory side of the chip that ramps).  The reference times
+  # its layers with triton.testing.do_bench, 25 ms of warm-up before 100 ms of repetitions
+  # (test/benchmark_conv.py:115,131).  This section shows the ramp and leaves the chip where
+  # such a warm-up would; the W warm-up steps and the K timed steps of the contract follow.
+  cold = []
+  if extras:
+    for _ in range(8):
+      cold.append(timed_steps(dtype, 5, 0)[0])
+
   # ---- the headline step ------------------------------------------------------
   ms, gather_ms, wgrad_ms, n_gather = timed_steps(dtype, args.steps, args.warmup, only=args.only)
   gather_ms = gather_ms or float('nan')
@@ -294,6 +306,9 @@ def main():
     result['note'] = 'single-pass run (--only {}): not a benchmark result'.format(args.only)
 
   if extras:
+    result['cold_start'] = {'ms_per_step_blocks_of_5': [round(v, 4) for v in cold],
+                            'note': 'the first 40 steps of the process, run before the W warm-up steps: the step '
+                                    'time falls for about 30 ms of sustained work before it settles'}
     # ---- the same step in the other 16-bit type ------------------------------
     other = 'fp16' if args.dtype == 'bf16' else 'bf16'
     oms, ogm, owm, _ = timed_steps(DT[other], args.steps, args.warmup)
@@ -306,8 +321,13 @@ def main():
     try:
       from ocnn_amd import probe
       sustained = {k: probe.mfma_rate(dtype, k, 20000)['tflops'] for k in ('constant', 'normal')}
+      alone, mixed = probe.mfma_mix(False), probe.mfma_mix(True)
       result['mfma_sustained'] = {
           'tflops_constant_operands': sustained['constant'], 'tflops_normal_operands': sustained['normal'],
+          'two_chains_alone': {k: round(alone[k], 3) for k in ('tflops', 'ticks_per_mfma', 'ns_per_mfma', 'ghz')},
+          'two_chains_with_gather_kernel_side_work': {k: round(mixed[k], 3) for k in
+                                                      ('tflops', 'ticks_per_mfma', 'ns_per_mfma', 'ghz')},
+          'gather_kernel_ns_per_mfma': gather_ms * 1e6 / (-(-rows // 128) / 256.0 * 224.0),
           'note': 'v_mfma_f32_32x32x16 back to back on every SIMD, {}: clocks fall under matrix load with '
                   'random operands, so this, not the published peak, bounds any kernel on N(0,1) data'.format(
                       args.dtype),

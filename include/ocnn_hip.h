@@ -210,6 +210,38 @@ int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile_nnz, int64
 int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
                         int32_t* urows, uint16_t* loc, void* stream);
 
+/* ---- kernel selection ----------------------------------------------------
+ * Which entry point runs a gather-GEMM (forward_gemm / backward_gemm in gather form,
+ * ocnn/nn/octree_conv.py:115-168) or a weight gradient (weight_gemm, :170-202) of a given
+ * shape: the reference picks between its Triton and torch paths in Python
+ * (ocnn/nn/octree_conv.py:347-357); here the choice among the kernels is part of the ABI.
+ * A returned code names an entry point that accepts the shape (its *_supported() predicate
+ * and the row ranges it checks).  identity_table: the table is the one-slot identity (row i
+ * reads row i: the dense form of 2x2x2 stride-2 layers and 1x1 convolutions).  Without a tile
+ * plan pass has_plan = 0 (the other plan arguments are then ignored); plan_occupancy = share
+ * of the table entries that are set, plan_reuse = entries set / distinct rows summed over
+ * the tiles.  ZERO_PADDED: pad the channels with zeros to multiples of 32 (cout of a gather:
+ * 16) and choose again. */
+#define OCNN_GATHER_PLAIN 0        /* ocnn_conv_gather            */
+#define OCNN_GATHER_DENSE_RW 1     /* ocnn_conv_dense_rw          */
+#define OCNN_GATHER_DENSE 2        /* ocnn_conv_dense             */
+#define OCNN_GATHER_RW 3           /* ocnn_conv_gather_rw         */
+#define OCNN_GATHER_SPARSE 4       /* ocnn_conv_gather_sparse     */
+#define OCNN_GATHER_WIDE 5         /* ocnn_conv_gather_wide       */
+#define OCNN_GATHER_PLANNED 6      /* ocnn_conv_gather_planned    */
+#define OCNN_GATHER_ZERO_PADDED 7
+#define OCNN_WGRAD_PLAIN 0         /* ocnn_conv_wgrad             */
+#define OCNN_WGRAD_DENSE_RW 1      /* ocnn_conv_dense_wgrad_rw    */
+#define OCNN_WGRAD_SPARSE 2        /* ocnn_conv_wgrad_sparse      */
+#define OCNN_WGRAD_PLANNED 3       /* ocnn_conv_wgrad_planned     */
+#define OCNN_WGRAD_ZERO_PADDED 4
+int ocnn_conv_gather_choose(int dtype, int64_t rows_in, int64_t rows_out, int K, int cin, int cout,
+                            int identity_table, int has_plan, int plan_max_distinct,
+                            int64_t plan_total, double plan_occupancy, double plan_reuse);
+int ocnn_conv_wgrad_choose(int dtype, int64_t rows_x, int64_t rows, int K, int ca, int cb,
+                           int identity_table, int has_plan, int plan_max_distinct,
+                           int64_t plan_total, double plan_occupancy);
+
 /* ocnn_conv_gather over a tile plan (same arguments otherwise, same result).
  * Supported for f16 / bf16 with cin and cout multiples of 64 and an input
  * smaller than 4 GiB; ocnn_conv_gather_planned_supported() tells. */

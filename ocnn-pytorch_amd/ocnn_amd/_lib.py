@@ -5,13 +5,13 @@ There is no CPU fallback: if the library cannot be loaded the package raises.
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_void_p, POINTER
 
 import torch
 
 from . import build as _build
 
-_i, _l, _p, _f = c_int, c_int64, c_void_p, c_float
+_i, _l, _p, _f, _d = c_int, c_int64, c_void_p, c_float, c_double
 
 # name -> (restype, argtypes); mirrors include/ocnn_hip.h one to one
 SIGNATURES = {
@@ -41,6 +41,8 @@ SIGNATURES = {
     'ocnn_conv_workspace_bytes': (_l, [_i, _i, _i]),
     'ocnn_conv_gather_workspace_bytes': (_l, [_i, _l, _i, _i, _i]),
     'ocnn_conv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _i, _i, _p, _p, _p, _l, _p]),
+    'ocnn_conv_gather_choose': (_i, [_i, _l, _l, _i, _i, _i, _i, _i, _i, _l, _d, _d]),
+    'ocnn_conv_wgrad_choose': (_i, [_i, _l, _l, _i, _i, _i, _i, _i, _i, _l, _d]),
     'ocnn_tile_plan_rows': (_i, []),
     'ocnn_tile_plan_count': (_i, [_p, _l, _i, _p, _p, _p]),
     'ocnn_tile_plan_offsets': (_i, [_p, _p, _l, _i, _p, _p, _p]),
@@ -141,6 +143,11 @@ def check(rc):
 
 
 DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+# codes of ocnn_conv_gather_choose / ocnn_conv_wgrad_choose (include/ocnn_hip.h)
+(GATHER_PLAIN, GATHER_DENSE_RW, GATHER_DENSE, GATHER_RW, GATHER_SPARSE, GATHER_WIDE, GATHER_PLANNED,
+ GATHER_ZERO_PADDED) = range(8)
+WGRAD_PLAIN, WGRAD_DENSE_RW, WGRAD_SPARSE, WGRAD_PLANNED, WGRAD_ZERO_PADDED = range(5)
 
 
 def dtype_code(t):

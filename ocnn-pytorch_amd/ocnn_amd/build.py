@@ -30,6 +30,7 @@ SOURCES = {
     'wgrad_planned.hip': [],
     'plan.hip': [],
     'misc.hip': [],
+    'select.hip': [],
     'interp.hip': ['-ffp-contract=off'],
     'norm.hip': ['-ffp-contract=off'],
 }

@@ -52,6 +52,65 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(const u32x4* __restri
   if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
 }
 
+// The MFMA loop again, now with what a wave of the register-resident gather-GEMM kernel issues
+// around its MFMAs, in that kernel's proportions per 8 MFMAs: NV independent VALU operations
+// per MFMA, NR 16-byte LDS reads, NW 16-byte LDS writes, NU 2-byte LDS reads (all conflict-free,
+// results awaited half an iteration later).  Two accumulator chains, as in that kernel.
+template <int NV, int NR, int NW, int NU>
+__global__ __launch_bounds__(256, 1) void mfma_mix_kernel(const u32x4* __restrict__ src, float* __restrict__ out,
+                                                          int iters, long long* __restrict__ ticks) {
+  __shared__ __attribute__((aligned(16))) char lds[65536];
+  for (int i = threadIdx.x * 16; i < 65536; i += 256 * 16) *(u32x4*)(lds + i) = u32x4{1u, 2u, 3u, 4u};
+  __syncthreads();
+  u32x4 a[4], b[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = src[i * 256 + threadIdx.x];
+  b[0] = src[7 * 256 + threadIdx.x];
+  b[1] = src[8 * 256 + threadIdx.x];
+  f32x16 c[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) c[i][j] = 0.f;
+  unsigned v[8] = {1, 2, 3, 4, 5, 6, 7, 8}, u[4] = {0, 0, 0, 0};
+  u32x4 r[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = u32x4{0u, 0u, 0u, 0u};
+  const unsigned wave = threadIdx.x >> 6;
+  const unsigned off = (threadIdx.x & 63) * 16 + wave * 8192, offw = off + 32768;
+  constexpr int kWait = (NR + NW + NU) / 2 > 15 ? 15 : (NR + NW + NU) / 2;
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      c[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[i & 3]),
+                                                         __builtin_bit_cast(bf16x8, b[(i >> 1) & 1]), c[i & 1], 0, 0, 0);
+#pragma unroll
+      for (int k = 0; k < NV; ++k)
+        asm volatile("v_xor_b32 %0, %0, %1" : "+v"(v[(i + k) & 7]) : "v"(v[(i + k + 3) & 7]));
+#pragma unroll
+      for (int k = (i * NR) / 8; k < ((i + 1) * NR) / 8; ++k)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r[k & 7]) : "v"(off), "n"(1024 * (k & 7)) : "memory");
+#pragma unroll
+      for (int k = (i * NW) / 8; k < ((i + 1) * NW) / 8; ++k)
+        asm volatile("ds_write_b128 %0, %1 offset:%2" :: "v"(offw), "v"(r[0]), "n"(1024 * (k & 7)) : "memory");
+#pragma unroll
+      for (int k = (i * NU) / 8; k < ((i + 1) * NU) / 8; ++k)
+        asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(u[k & 3]) : "v"(off), "n"(64 * (k & 7)) : "memory");
+      if (i == 3 || i == 7) asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(kWait) : "memory");
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  const long long t1 = clock64();
+  float s = c[0][0] + c[0][9] + c[1][0] + c[1][9];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += (float)(v[i] ^ r[i][0]);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) s += (float)u[i];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+  if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
+}
+
 // Every lane reads (WRITE: writes) 16 bytes at its 8 byte offsets `addr[j * threads + tid]`,
 // `iters` times.  The caller chooses the offsets, i.e. the bank pattern: consecutive lanes on
 // consecutive 16-byte chunks, rows gathered through a swizzle, a deliberate conflict ...
@@ -162,6 +221,26 @@ extern "C" int ocnn_probe_lds_rate(int write, int threads, const void* addr, voi
                          (float*)out, iters, (long long*)ticks);
     else
       hipLaunchKernelGGL(lds_rate_kernel<false>, dim3(n_cu), dim3(threads), 64 * 1024, st, (const uint32_t*)addr,
+                         (float*)out, iters, (long long*)ticks);
+  }, ms);
+}
+
+// The same count of MFMAs as ocnn_probe_mfma_rate per iteration would be 14; here an iteration
+// is 8 MFMAs (bf16) with the gather-GEMM kernel's side work when mix != 0 (per 8 MFMAs: 16
+// VALU operations, six 16-byte LDS reads, one 16-byte LDS write, two 2-byte LDS reads), none
+// when mix == 0.  flops = CUs x 4 waves x iters x 8 x 32768.
+extern "C" int ocnn_probe_mfma_mix(int mix, const void* operands, void* out, void* ticks, int iters, void* stream,
+                                   double* ms, double* flops) {
+  const int n_cu = cu_count();
+  if (n_cu <= 0 || iters <= 0 || iters > (1 << 22)) return -1;
+  hipStream_t st = (hipStream_t)stream;
+  *flops = (double)n_cu * 4.0 * iters * 8.0 * 32768.0;
+  return timed(st, [&]() {
+    if (mix)
+      hipLaunchKernelGGL((mfma_mix_kernel<2, 6, 1, 2>), dim3(n_cu), dim3(256), 0, st, (const u32x4*)operands,
+                         (float*)out, iters, (long long*)ticks);
+    else
+      hipLaunchKernelGGL((mfma_mix_kernel<0, 0, 0, 0>), dim3(n_cu), dim3(256), 0, st, (const u32x4*)operands,
                          (float*)out, iters, (long long*)ticks);
   }, ms);
 }

@@ -25,9 +25,12 @@ from .octree2col import col2octree, octree2col
 from .octree_pad import octree_depad, octree_pad
 
 
-PAD_MIN_ROWS = 16384     # from this many table rows on, odd channel counts are zero-padded
-SPARSE_MAX_OCCUPANCY = 0.3   # share of table entries that hold a row, up to which it is used
-SPARSE_MIN_ROWS = 32768      # (a workgroup loads its weights once and needs many tiles to pay for it)
+# (thresholds of the kernel selection live in the library, csrc/select.hip; these are the ones
+# the layer level needs: when odd channel counts run zero-padded, and from how many rows on the
+# pair-plan kernels pay for loading their weights)
+PAD_MIN_ROWS = 16384
+SPARSE_MAX_OCCUPANCY = 0.3
+SPARSE_MIN_ROWS = 32768
 
 
 def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False):
@@ -42,9 +45,17 @@ def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, p
   return out
 
 
+def _plan_args(plan):
+  """(has_plan, max distinct rows, entries of the row lists, occupancy, reuse) for the
+  selection functions of the library."""
+  if plan is None:
+    return 0, 0, 0, 1.0, 0.0
+  return 1, plan.umax, plan.total, float(plan.occupancy), float(plan.reuse)
+
+
 def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense):
   """conv_gather without the overflow rows of the plan; also returns whether a kernel on
-  the plan ran."""
+  the plan ran.  The library picks the kernel (ocnn_conv_gather_choose)."""
   _lib.require_gpu(data, table, W)
   L = _lib.lib()
   data, W, table = data.contiguous(), W.contiguous(), table.contiguous()
@@ -54,9 +65,9 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
   assert W.numel() == K * cin * cout, 'weights do not match the table and channels'
   if bias is not None:
     bias = bias.to(data.dtype).contiguous()
-  # channel counts the MFMA kernels do not take (cin % 32, cout % 16) are padded with zeros
-  # when the layer is large enough for that to beat the plain kernel
-  if rows >= PAD_MIN_ROWS and (cin % 32 or cout % 16) and data.dtype in _lib.DTYPE_CODE:
+  code = _lib.dtype_code(data)
+  kernel = L.ocnn_conv_gather_choose(code, rows_in, rows, K, cin, cout, int(bool(dense)), *_plan_args(plan))
+  if kernel == _lib.GATHER_ZERO_PADDED:
     cin_p, cout_p = -(-cin // 32) * 32, -(-cout // 16) * 16
     Wk = W.view(K, cout, cin) if transposed else W.view(K, cin, cout)
     pad_w = (0, cin_p - cin, 0, cout_p - cout) if transposed else (0, cout_p - cout, 0, cin_p - cin)
@@ -64,28 +75,18 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
                       transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), plan)
     return out[:, :cout].contiguous(), False
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
-  code = _lib.dtype_code(data)
-  nbytes = L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout)
-  ws = _lib.workspace(nbytes, data.device)
-  if dense and K == 1 and rows == rows_in and L.ocnn_conv_dense_rw_supported(code, rows, cin, cout):
-    _lib.check(L.ocnn_conv_dense_rw(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed),
-                                    _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  ws = _lib.workspace(L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout), data.device)
+  tail = (_lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream())
+  if kernel in (_lib.GATHER_DENSE_RW, _lib.GATHER_DENSE):
+    fn = L.ocnn_conv_dense_rw if kernel == _lib.GATHER_DENSE_RW else L.ocnn_conv_dense
+    _lib.check(fn(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed), *tail))
     return out, False
-  # (many input channels into few output channels: the row tile that fits LDS is small and
-  # the weights are streamed once per tile; the plan-free kernel is no slower there)
-  if (dense and K == 1 and rows == rows_in and not (cin >= 512 and cout < 256) and
-      L.ocnn_conv_dense_supported(code, rows, cin, cout)):
-    _lib.check(L.ocnn_conv_dense(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed),
-                                 _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out, False
-  if plan is not None and L.ocnn_conv_gather_rw_supported(code, rows_in, K, cin, cout, plan.umax):
-    _lib.check(L.ocnn_conv_gather_rw(
-        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
-        _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
-        int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+  if kernel in (_lib.GATHER_RW, _lib.GATHER_WIDE):
+    fn = L.ocnn_conv_gather_rw if kernel == _lib.GATHER_RW else L.ocnn_conv_gather_wide
+    _lib.check(fn(code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
+                  plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse), *tail))
     return out, True
-  if (plan is not None and plan.occupancy <= SPARSE_MAX_OCCUPANCY and
-      rows >= SPARSE_MIN_ROWS and L.ocnn_conv_gather_sparse_supported(code, rows_in, K, cin, cout, plan.umax)):
+  if kernel == _lib.GATHER_SPARSE:
     pp = plan.pairs()
     ws = _lib.workspace(L.ocnn_conv_gather_sparse_workspace_bytes(cin, cout), data.device)
     _lib.check(L.ocnn_conv_gather_sparse(
@@ -94,24 +95,14 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
         ctypes.addressof(pp.group_bounds_host), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
         _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return out, True
-  if plan is not None and plan.reuse >= 2.0 and L.ocnn_conv_gather_wide_supported(
-      code, rows_in, K, cin, cout, plan.umax):
-    _lib.check(L.ocnn_conv_gather_wide(
-        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
-        _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed),
-        int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
-    return out, True
-  if plan is not None and plan.reuse >= 2.0 and L.ocnn_conv_gather_planned_supported(
-      code, rows_in, cin, cout):
+  if kernel == _lib.GATHER_PLANNED:
     _lib.check(L.ocnn_conv_gather_planned(
         code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
-        _lib.ptr(plan.urows), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse),
-        _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
+        _lib.ptr(plan.urows), rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse), *tail))
     return out, True
   _lib.check(L.ocnn_conv_gather(
       code, _lib.ptr(data), rows_in, _lib.ptr(table), rows, K, _lib.ptr(W),
-      cin, cout, int(transposed), int(reverse), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws),
-      ws.numel(), _lib.stream()))
+      cin, cout, int(transposed), int(reverse), *tail))
   return out, False
 
 
@@ -130,35 +121,27 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
 
 def _conv_wgrad(x, g, table, out_transposed, plan, dense):
   """conv_wgrad without the overflow rows of the plan; also returns whether a kernel on the
-  plan ran."""
+  plan ran.  The library picks the kernel (ocnn_conv_wgrad_choose)."""
   _lib.require_gpu(x, g, table)
   L = _lib.lib()
   x, g, table = x.contiguous(), g.contiguous(), table.contiguous()
   rows, K = table.shape
   ca, cb = x.shape[1], g.shape[1]
   assert g.shape[0] == rows and x.dtype == g.dtype and table.dtype == torch.int32
-  if rows >= PAD_MIN_ROWS and (ca % 32 or cb % 32) and x.dtype in _lib.DTYPE_CODE:
+  code = _lib.dtype_code(x)
+  kernel = L.ocnn_conv_wgrad_choose(code, x.shape[0], rows, K, ca, cb, int(bool(dense)), *_plan_args(plan)[:4])
+  if kernel == _lib.WGRAD_ZERO_PADDED:
     ca_p, cb_p = -(-ca // 32) * 32, -(-cb // 32) * 32
     gw = conv_wgrad(F.pad(x, (0, ca_p - ca)), F.pad(g, (0, cb_p - cb)), table, out_transposed, plan)
     return (gw[:, :cb, :ca] if out_transposed else gw[:, :ca, :cb]).contiguous(), False
   shape = (K, cb, ca) if out_transposed else (K, ca, cb)
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
-  code = _lib.DTYPE_CODE.get(x.dtype, -1)
-  # (below some 8 k channel pairs a workgroup's 128 k-pair block is mostly zeros and the
-  # plan-free kernel is as fast: 96 x 64 on 1.2 M rows 0.19 against 0.22 ms)
-  if (dense and K == 1 and x.shape[0] == rows and ca * cb >= 8192 and
-      L.ocnn_conv_dense_wgrad_rw_supported(code, rows, ca, cb)):
+  if kernel == _lib.WGRAD_DENSE_RW:
     ws = _lib.workspace(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(ca, cb), x.device)
     _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x), _lib.ptr(g), rows, ca, cb, int(out_transposed),
                                           _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw, False
-  # (32 x 32 and 64 x 64 have kernels of their own on the tile plan that are faster still; with
-  # channel counts that are not multiples of 64 on the table-row side the pair-plan kernel, which
-  # sums exactly ca x cb and only over the pairs, beats the planned kernel's zero-padded 64 x 64
-  # blocks on dense tables too: 96 -> 96 on 5.0 M rows 2.3 against 3.3 ms)
-  if (plan is not None and (plan.occupancy <= SPARSE_MAX_OCCUPANCY or cb % 64 != 0) and
-      rows >= SPARSE_MIN_ROWS and not (ca == cb and ca in (32, 64)) and
-      L.ocnn_conv_wgrad_sparse_supported(code, x.shape[0], rows, K, ca, cb, plan.umax)):
+  if kernel == _lib.WGRAD_SPARSE:
     pp = plan.pairs()
     ws = _lib.workspace(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, ca, cb), x.device)
     _lib.check(L.ocnn_conv_wgrad_sparse(
@@ -167,18 +150,16 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense):
         ctypes.addressof(pp.lists_host), ctypes.addressof(pp.list_count_host), pp.n_lists, K,
         int(not out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw, True
-  if plan is not None and L.ocnn_conv_wgrad_planned_supported(code, x.shape[0], rows, K, ca, cb,
-                                                              plan.umax):
+  if kernel == _lib.WGRAD_PLANNED:
     ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K, ca, cb), x.device)
     _lib.check(L.ocnn_conv_wgrad_planned(
         code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, ca, cb, int(out_transposed),
         _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw, True
-  ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes_for(_lib.dtype_code(x), x.shape[0], rows, K,
-                                                            ca, cb), x.device)
+  ws = _lib.workspace(L.ocnn_conv_wgrad_workspace_bytes_for(code, x.shape[0], rows, K, ca, cb), x.device)
   _lib.check(L.ocnn_conv_wgrad(
-      _lib.dtype_code(x), _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
+      code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(table), rows, K, ca, cb,
       int(out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
   return gw, False
 
@@ -369,18 +350,20 @@ class _OctreeDeconv(OctreeConvBase):
 
 
 class OctreeConvFunction(Function):
-  """Autograd wiring of the convolution (ocnn/nn/octree_conv.py:219-254)."""
+  """Autograd wiring of the convolution (ocnn/nn/octree_conv.py:219-254).  `bias` (optional,
+  last argument) is added in the epilogue of the gather-GEMM kernel instead of by a pass of
+  its own; its gradient is the fixed-order column sum of the output gradient."""
 
   @staticmethod
   def forward(ctx, data, weights, octree, depth: int, in_channels: int, out_channels: int,
               kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
-              max_buffer: int = int(2e8)):
+              max_buffer: int = int(2e8), bias=None):
     eng = _OctreeConv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
     eng.check_and_init(data)
     data = data.contiguous()
     weights = weights.to(data.dtype).contiguous()
-    out = eng.forward_gemm(data, weights)
+    out = eng.forward_gemm(data, weights, bias)
     ctx.save_for_backward(data, weights)
     ctx.eng = eng
     return out
@@ -392,7 +375,8 @@ class OctreeConvFunction(Function):
     grad = grad.contiguous()
     grad_out = eng.backward_gemm(grad, weights) if ctx.needs_input_grad[0] else None
     grad_w = eng.weight_gemm(data, grad) if ctx.needs_input_grad[1] else None
-    return (grad_out, grad_w) + (None,) * 8
+    grad_b = column_sum(grad) if ctx.needs_input_grad[10] else None
+    return (grad_out, grad_w) + (None,) * 8 + (grad_b,)
 
 
 class OctreeDeconvFunction(Function):
@@ -401,13 +385,13 @@ class OctreeDeconvFunction(Function):
   @staticmethod
   def forward(ctx, data, weights, octree, depth: int, in_channels: int, out_channels: int,
               kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
-              max_buffer: int = int(2e8)):
+              max_buffer: int = int(2e8), bias=None):
     eng = _OctreeDeconv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
     eng.check_and_init(data)
     data = data.contiguous()
     weights = weights.to(data.dtype).contiguous()
-    out = eng.backward_gemm(data, weights)
+    out = eng.backward_gemm(data, weights, bias)
     ctx.save_for_backward(data, weights)
     ctx.eng = eng
     return out
@@ -420,11 +404,24 @@ class OctreeDeconvFunction(Function):
     grad_out = eng.forward_gemm(grad, weights) if ctx.needs_input_grad[0] else None
     # weights are (K, out_channels, in_channels): x = grad (fine side), g = data
     grad_w = eng.weight_gemm(grad, data) if ctx.needs_input_grad[1] else None
-    return (grad_out, grad_w) + (None,) * 8
+    grad_b = column_sum(grad) if ctx.needs_input_grad[10] else None
+    return (grad_out, grad_w) + (None,) * 8 + (grad_b,)
 
 
-octree_conv = OctreeConvFunction.apply
-octree_deconv = OctreeDeconvFunction.apply
+def octree_conv(data, weights, octree, depth: int, in_channels: int, out_channels: int,
+                kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
+                max_buffer: int = int(2e8), bias=None):
+  """Functional form (ocnn/nn/octree_conv.py:296), with an optional bias that the kernel adds."""
+  return OctreeConvFunction.apply(data, weights, octree, depth, in_channels, out_channels, kernel_size, stride,
+                                  nempty, max_buffer, bias)
+
+
+def octree_deconv(data, weights, octree, depth: int, in_channels: int, out_channels: int,
+                  kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
+                  max_buffer: int = int(2e8), bias=None):
+  """Functional form (ocnn/nn/octree_conv.py:297), with an optional bias that the kernel adds."""
+  return OctreeDeconvFunction.apply(data, weights, octree, depth, in_channels, out_channels, kernel_size, stride,
+                                    nempty, max_buffer, bias)
 
 
 class OctreeConv(OctreeConvBase, torch.nn.Module):
@@ -467,8 +464,9 @@ class OctreeConv(OctreeConvBase, torch.nn.Module):
       out = self.explicit_gemm(data, octree, depth)
     else:
       out = octree_conv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
-                        self.kernel_size, self.stride, self.nempty, self.max_buffer)
-    if self.use_bias:
+                        self.kernel_size, self.stride, self.nempty, self.max_buffer,
+                        self.bias if self.use_bias else None)              # bias: in the kernel's epilogue
+    if self.use_bias and self.method == 'explicit_gemm':
       out = out + self.bias.to(out.dtype)
     if self.stride == 2 and not self.nempty:
       out = octree_pad(out, octree, depth - 1)
@@ -497,7 +495,8 @@ class OctreeDeconv(OctreeConv):
                        self.stride, self.nempty)
     else:
       out = octree_deconv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
-                          self.kernel_size, self.stride, self.nempty, self.max_buffer)
-    if self.use_bias:
+                          self.kernel_size, self.stride, self.nempty, self.max_buffer,
+                          self.bias if self.use_bias else None)
+    if self.use_bias and self.method == 'explicit_gemm':
       out = out + self.bias.to(out.dtype)
     return out

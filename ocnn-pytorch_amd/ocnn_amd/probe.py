@@ -25,6 +25,8 @@ def lib():
     h.ocnn_probe_lds_rate.restype = c_int
     h.ocnn_probe_lds_rate.argtypes = [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                       POINTER(c_double), POINTER(c_double)]
+    h.ocnn_probe_mfma_mix.restype = c_int
+    h.ocnn_probe_mfma_mix.argtypes = h.ocnn_probe_mfma_rate.argtypes
     _lib = h
   return _lib
 
@@ -52,6 +54,29 @@ def mfma_rate(dtype=torch.bfloat16, operands='normal', iters=20000, device='cuda
   per = iters * 14
   return {'tflops': flops.value / ms.value / 1e9, 'ms': ms.value,
           'ticks_per_mfma': float(ticks.double().mean()) / per, 'ns_per_mfma': ms.value * 1e6 / per}
+
+
+def mfma_mix(mix=True, operands='normal', iters=30000, device='cuda'):
+  """The bf16 MFMA loop with two accumulator chains, alone (mix=False) or with the side work of
+  the register-resident gather-GEMM kernel in its proportions (per 8 MFMAs: 16 VALU operations,
+  six 16-byte LDS reads, one 16-byte write, two 2-byte reads).  Returns dict(tflops, ms,
+  ticks_per_mfma, ns_per_mfma, ghz)."""
+  g = torch.Generator().manual_seed(1)
+  n = 9 * 256 * 8
+  src = {'zero': torch.zeros(n), 'constant': torch.full((n,), 0.5),
+         'uniform': torch.rand(n, generator=g) * 2 - 1, 'normal': torch.randn(n, generator=g)}[operands]
+  src = src.to(torch.bfloat16).to(device)
+  out = torch.empty(_cus(device) * 256, dtype=torch.float32, device=device)
+  ticks = torch.zeros(_cus(device), dtype=torch.int64, device=device)
+  ms, flops = c_double(), c_double()
+  rc = lib().ocnn_probe_mfma_mix(int(bool(mix)), src.data_ptr(), out.data_ptr(), ticks.data_ptr(), iters,
+                                 torch.cuda.current_stream().cuda_stream, byref(ms), byref(flops))
+  if rc != 0:
+    raise RuntimeError('ocnn_probe_mfma_mix failed')
+  per = iters * 8
+  t, ns = float(ticks.double().mean()) / per, ms.value * 1e6 / per
+  return {'tflops': flops.value / ms.value / 1e9, 'ms': ms.value, 'ticks_per_mfma': t, 'ns_per_mfma': ns,
+          'ghz': t / ns}
 
 
 def lds_rate(offsets, write=False, iters=4000, device='cuda'):

@@ -167,3 +167,51 @@ def test_plan_history_is_bounded_and_clearable():
   assert h.requests((PlanHistory.MAX_KINDS + 4, 2))[key] is True
   h.clear()
   assert h.requests((PlanHistory.MAX_KINDS + 4, 2)) == {}
+
+
+def test_kernel_selection_is_consistent_with_the_predicates():
+  """ocnn_conv_gather_choose / ocnn_conv_wgrad_choose (host arithmetic only): every choice is
+  a kernel whose *_supported() predicate takes the shape and whose entry point's row ranges
+  hold; shapes past those ranges fall through to the plan-free kernels instead of failing."""
+  from ocnn_amd import _lib
+  L = _lib.lib()
+  BF = 2
+  lim = 0xfff00000
+  for rows in (1000, 40000, 1 << 21, 17_000_000, 70_000_000):
+    for K in (27, 8, 3, 1):
+      for cin, cout in ((64, 64), (32, 32), (96, 96), (128, 128), (256, 256), (64, 128), (4, 32), (32, 10)):
+        for occ, reuse in ((0.6, 9.0), (0.15, 4.0), (0.6, 1.2)):
+          for umax in (200, 416, 500, 2000):
+            k = L.ocnn_conv_gather_choose(BF, rows, rows, K, cin, cout, 0, 1, umax, rows * 2, occ, reuse)
+            if k == _lib.GATHER_RW:
+              assert L.ocnn_conv_gather_rw_supported(BF, rows, K, cin, cout, umax) and rows * K * 2 < lim
+            elif k == _lib.GATHER_SPARSE:
+              assert L.ocnn_conv_gather_sparse_supported(BF, rows, K, cin, cout, umax)
+              assert rows * cout * 2 <= lim and occ <= 0.3 and rows >= 32768
+            elif k == _lib.GATHER_WIDE:
+              assert L.ocnn_conv_gather_wide_supported(BF, rows, K, cin, cout, umax) and reuse >= 2
+            elif k == _lib.GATHER_PLANNED:
+              assert L.ocnn_conv_gather_planned_supported(BF, rows, cin, cout) and reuse >= 2
+            elif k == _lib.GATHER_ZERO_PADDED:
+              assert rows >= 16384 and (cin % 32 or cout % 16)
+            else:
+              assert k == _lib.GATHER_PLAIN
+            w = L.ocnn_conv_wgrad_choose(BF, rows, rows, K, cin, cout, 0, 1, umax, rows * 2, occ)
+            if w == _lib.WGRAD_SPARSE:
+              assert L.ocnn_conv_wgrad_sparse_supported(BF, rows, rows, K, cin, cout, umax) and rows * K * 2 < lim
+            elif w == _lib.WGRAD_PLANNED:
+              assert L.ocnn_conv_wgrad_planned_supported(BF, rows, rows, K, cin, cout, umax) and rows * K * 2 < lim
+            elif w == _lib.WGRAD_ZERO_PADDED:
+              assert rows >= 16384 and (cin % 32 or cout % 32)
+            else:
+              assert w == _lib.WGRAD_PLAIN
+  # the benchmark layer and its neighbours take the kernels built for them
+  assert L.ocnn_conv_gather_choose(BF, 1885272, 1885272, 27, 64, 64, 0, 1, 366, 3400000, 0.61, 9.0) == _lib.GATHER_RW
+  assert L.ocnn_conv_wgrad_choose(BF, 1885272, 1885272, 27, 64, 64, 0, 1, 366, 3400000, 0.61) == _lib.WGRAD_PLANNED
+  assert L.ocnn_conv_gather_choose(BF, 925113, 925113, 27, 96, 96, 0, 1, 300, 2000000, 0.145, 4.0) == _lib.GATHER_SPARSE
+  assert L.ocnn_conv_gather_choose(BF, 211136, 211136, 27, 256, 256, 0, 1, 400, 500000, 0.74, 9.0) == _lib.GATHER_WIDE
+  assert L.ocnn_conv_gather_choose(BF, 235659, 235659, 1, 512, 128, 1, 0, 0, 0, 1.0, 0.0) == _lib.GATHER_DENSE_RW
+  assert L.ocnn_conv_gather_choose(BF, 1000, 1000, 27, 64, 64, 0, 0, 0, 0, 1.0, 0.0) == _lib.GATHER_PLAIN
+  # 128 output channels on more rows than 32-bit offsets of the output reach: not the pair-plan kernel
+  big = 17_000_000
+  assert L.ocnn_conv_gather_choose(BF, big, big, 27, 128, 128, 0, 1, 300, big * 2, 0.15, 4.0) != _lib.GATHER_SPARSE
