@@ -38,6 +38,38 @@ static __device__ __forceinline__ void dp_unpack(u32x4 v, float (&f)[8]) {
   for (int e = 0; e < 8; ++e) f[e] = (float)t[e];
 }
 
+// acc += a.lo * b.lo + a.hi * b.hi in fp32 (v_dot2c_f32_{f16,bf16}), a and b pairs of 16-bit
+// values.  With one half of b zero this is a multiply-add of ONE channel of the pair straight
+// out of the packed register: no unpacking of the 16-bit operand, one instruction per product.
+template <typename T> static __device__ __forceinline__ float dp_dot2(unsigned a, unsigned b, float acc);
+template <> __device__ __forceinline__ float dp_dot2<bf16>(unsigned a, unsigned b, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 v2;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), acc, false);
+}
+template <> __device__ __forceinline__ float dp_dot2<f16>(unsigned a, unsigned b, float acc) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 v2;
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), acc, false);
+}
+
+// 8 channels of one operand as (value, 0) and (0, value) pairs: lo[e] multiplies channel 2 e of a
+// packed register, hi[e] channel 2 e + 1.
+static __device__ __forceinline__ void dp_split(u32x4 v, unsigned (&lo)[4], unsigned (&hi)[4]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    lo[e] = v[e] & 0x0000ffffu;
+    hi[e] = v[e] & 0xffff0000u;
+  }
+}
+
+// Table positions (16 bits each, two per dword, at most 511) -> byte offsets of the LDS rows with
+// the swizzle bits in place: (p << 7) | (((p >> 1) & 7) << 4); a thread's 16-byte chunk c of that
+// row is then at offset ^ (c << 4).  Position 0 (empty entry) stays 0: the zero row.
+static __device__ __forceinline__ u32x4 dp_loc_offsets(u32x4 v) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = (v[e] << 7) | ((v[e] & 0x000e000eu) << 3);
+  return v;
+}
+
 // Stages the 64-channel chunk `chunk` of the rows in the list s_u (LDS row p = list entry
 // p - 1, row 0 and everything past the list = zeros) into s_rows.  A lane's 16-byte chunk c
 // of LDS row p lands at chunk c ^ ((p >> 1) & 7) (bank swizzle).
@@ -84,7 +116,7 @@ __global__ __launch_bounds__(256, 2) void dw_gather_planned_kernel(
   for (int i = tid; i < kDpRowsAlloc; i += 256) s_u[i] = (i >= 1 && i <= U) ? urows[p0 + i - 1] : -1;
   {
     const u32x4* src = (const u32x4*)(loc + tile * (int64_t)(kDpRows * K));
-    for (int i = tid; i < K * 16; i += 256) ((u32x4*)s_loc)[i] = src[i];
+    for (int i = tid; i < K * 16; i += 256) ((u32x4*)s_loc)[i] = dp_loc_offsets(src[i]);
     if (tid < K * 8) {
       const int k = tid >> 3, kk = reverse ? K - 1 - k : k;
       ((u32x4*)s_w)[tid] = *(const u32x4*)(w + (int64_t)kk * C + 64 * chunk + 8 * (tid & 7));
@@ -103,23 +135,24 @@ __global__ __launch_bounds__(256, 2) void dw_gather_planned_kernel(
     for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
   const char* rows_c = (const char*)s_rows;
   const uint16_t* lcw = s_loc + r0;
+  const uint32_t cx = (uint32_t)c << 4;
 #pragma unroll 3
   for (int k = 0; k < K; ++k) {
-    float wf[8];
-    dp_unpack<T>(((const u32x4*)s_w)[k * 8 + c], wf);
+    unsigned wlo[4], whi[4];
+    dp_split(((const u32x4*)s_w)[k * 8 + c], wlo, whi);
     uint32_t p[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) p[j] = lcw[k * kDpRows + 32 * j];
     u32x4 xv[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      xv[j] = *(const u32x4*)(rows_c + ((p[j] << 7) | ((((p[j] >> 1) ^ (uint32_t)c) & 7u) << 4)));
+    for (int j = 0; j < 4; ++j) xv[j] = *(const u32x4*)(rows_c + (p[j] ^ cx));
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float xf[8];
-      dp_unpack<T>(xv[j], xf);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(xf[e], wf[e], acc[j][e]);
+      for (int e = 0; e < 4; ++e) {
+        acc[j][2 * e] = dp_dot2<T>(xv[j][e], wlo[e], acc[j][2 * e]);
+        acc[j][2 * e + 1] = dp_dot2<T>(xv[j][e], whi[e], acc[j][2 * e + 1]);
+      }
     }
   }
   float bv[8];
@@ -183,7 +216,7 @@ __global__ __launch_bounds__(256, 2) void dw_wgrad_planned_kernel(
     dp_stage_rows(rs_x, (char*)s_rows, s_u[b], (U + 8) >> 3, (uint32_t)C * 2u, (uint32_t)chunk * 128u, wave, lane);
     {
       const u32x4* src = (const u32x4*)(loc + (tile * K + k0) * (int64_t)kDpRows);
-      for (int i = tid; i < KG * 16; i += 256) ((u32x4*)s_loc)[i] = src[i];
+      for (int i = tid; i < KG * 16; i += 256) ((u32x4*)s_loc)[i] = dp_loc_offsets(src[i]);
     }
     u32x4 gv[4];
 #pragma unroll
@@ -194,9 +227,10 @@ __global__ __launch_bounds__(256, 2) void dw_wgrad_planned_kernel(
     if (tile + 1 < t_end) U = load_list(tile + 1, s_u[b ^ 1]);       // the next list, under this tile's loads
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    float gf[4][8];
+    unsigned glo[4][4], ghi[4][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dp_unpack<T>(gv[j], gf[j]);
+    for (int j = 0; j < 4; ++j) dp_split(gv[j], glo[j], ghi[j]);
+    const uint32_t cx = (uint32_t)c << 4;
 #pragma unroll
     for (int k = 0; k < KG; ++k) {
       uint32_t p[4];
@@ -204,14 +238,14 @@ __global__ __launch_bounds__(256, 2) void dw_wgrad_planned_kernel(
       for (int j = 0; j < 4; ++j) p[j] = lcw[k * kDpRows + 32 * j];
       u32x4 xv[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        xv[j] = *(const u32x4*)(rows_c + ((p[j] << 7) | ((((p[j] >> 1) ^ (uint32_t)c) & 7u) << 4)));
+      for (int j = 0; j < 4; ++j) xv[j] = *(const u32x4*)(rows_c + (p[j] ^ cx));
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        float xf[8];
-        dp_unpack<T>(xv[j], xf);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[k][e] = fmaf(xf[e], gf[j][e], acc[k][e]);
+        for (int e = 0; e < 4; ++e) {
+          acc[k][2 * e] = dp_dot2<T>(xv[j][e], glo[j][e], acc[k][2 * e]);
+          acc[k][2 * e + 1] = dp_dot2<T>(xv[j][e], ghi[j][e], acc[k][2 * e + 1]);
+        }
       }
     }
   }
