@@ -30,8 +30,8 @@ from bench_common import PEAK_HBM_GBS, PEAK_MFMA_16BIT_TFLOPS, build_octree, tim
 # HBM bytes per launch of the gather-GEMM kernel at the default workload, from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes summarised in this file under profiles/ (not measured by this
 # run: counters need the profiler); None for any other workload.
-TRAFFIC_SOURCE = 'profiles/conv_gather_rw_hbm_traffic_depth8_c64_fp16.txt'
-TRAFFIC_GATHER_DEFAULT = int((209100 * 2.0 + 235970 * 1.0) * 1024)
+TRAFFIC_SOURCE = 'profiles/conv_kernels_counters_depth8_c64_bf16.txt'
+TRAFFIC_GATHER_DEFAULT = int((208782 * 2.0 + 235796 * 1.0) * 1024)
 
 
 def parse():
@@ -279,8 +279,9 @@ def main():
           'unit': 'TFLOP/s',
           'frac': achieved / PEAK_MFMA_16BIT_TFLOPS,
           'traffic': TRAFFIC_GATHER_DEFAULT if default_workload else None,
-          'traffic_source': (TRAFFIC_SOURCE + ' (rocprofv3 counters of an earlier run of this command, fp16; '
-                             'not measured by this run)') if default_workload else None,
+          'traffic_source': (TRAFFIC_SOURCE + ' (rocprofv3 FETCH_SIZE / WRITE_SIZE of an earlier run of this '
+                             'command with --no-extras --calib, bf16; not measured by this run)')
+          if default_workload else None,
           'launches': n_gather,
           'avg_launch_ms': gather_ms,
           'algorithmic_flops_per_launch': flops_launch,

@@ -116,12 +116,14 @@ _lib = None
 
 
 def lib():
-  """Loads the library once.  Builds it first only when no built file exists."""
+  """Loads the library once.  A library that is missing, or that was built from other sources
+  than the ones in csrc/ and include/ now (their hash is stored beside it), is built first: a
+  stale binary is never loaded."""
   global _lib
   if _lib is not None:
     return _lib
   path = _build.LIB_PATH
-  if not os.path.exists(path):
+  if not _build.is_current():
     _build.build_library()
   handle = ctypes.CDLL(path)
   for name, (res, args) in SIGNATURES.items():

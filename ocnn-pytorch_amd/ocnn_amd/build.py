@@ -1,5 +1,6 @@
 """Builds libocnn_hip.so (gfx950) from csrc/ with hipcc, in-tree."""
 
+import hashlib
 import os
 import subprocess
 from concurrent.futures import ThreadPoolExecutor
@@ -39,6 +40,32 @@ COMMON = ['-O3', '--offload-arch=gfx950', '-fPIC', '-std=c++17', '-I', INCLUDE, 
           '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']
 
 
+STAMP_PATH = os.path.join(LIB_DIR, 'sources.sha256')
+
+
+def source_hash():
+  """Hash of everything the libraries are built from (sources, headers, flags)."""
+  h = hashlib.sha256()
+  names = sorted(os.listdir(CSRC))
+  for path in [os.path.join(CSRC, n) for n in names] + [os.path.join(INCLUDE, n) for n in sorted(os.listdir(INCLUDE))]:
+    if os.path.isfile(path):
+      h.update(os.path.basename(path).encode())
+      with open(path, 'rb') as f:
+        h.update(f.read())
+  h.update(repr((COMMON[:4] + COMMON[8:], sorted(SOURCES.items()))).encode())
+  return h.hexdigest()
+
+
+def is_current():
+  """True when both libraries exist and were built from the sources as they are now."""
+  try:
+    with open(STAMP_PATH) as f:
+      stamp = f.read().strip()
+  except OSError:
+    return False
+  return os.path.exists(LIB_PATH) and os.path.exists(PROBE_LIB_PATH) and stamp == source_hash()
+
+
 def _hipcc():
   for cand in (os.environ.get('HIPCC'), '/opt/rocm/bin/hipcc', 'hipcc'):
     if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -70,6 +97,8 @@ def build_library(verbose=False):
     objs = list(pool.map(compile_one, SOURCES.items()))
   _run([hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-o', LIB_PATH] + objs)
   _run([hipcc] + COMMON + ['-shared', os.path.join(CSRC, 'probe.hip'), '-o', PROBE_LIB_PATH])
+  with open(STAMP_PATH, 'w') as f:
+    f.write(source_hash() + '\n')
   if verbose:
     print('built', LIB_PATH)
   return LIB_PATH

@@ -26,8 +26,10 @@ constexpr int kRwCap = 416;    // staged rows; plans with a larger tile use anot
 // v_mfma_f32_32x32x16 A operand: lane l holds A[l % 32][8 * (l / 32) + j];
 // D: lane l, register r holds D[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32].
 //   input channel  = 32 half + 16 s + 8 (lane / 32) + j
-//   output channel = 32 tM + perm(lane % 32), perm(8a + 4q + b) = 16 q + 4 a + b,
-// so that a lane ends with 16 consecutive output channels per M tile.
+//   output channel = 32 tM + perm(lane % 32), perm(8a + 4q + b) = 16 (a / 2) + 8 q + 4 (a % 2) + b,
+// so that registers 8 R .. 8 R + 7 of a lane are the 8 consecutive output channels
+// 16 R + 8 q ..: a 16-byte store per lane, and the two lanes (q = 0, 1) of a row write 32
+// contiguous bytes.
 template <typename T>
 __global__ void pack_weights_rw_kernel(const T* __restrict__ w, T* __restrict__ out, int K,
                                        int transposed, int reverse) {
@@ -41,7 +43,7 @@ __global__ void pack_weights_rw_kernel(const T* __restrict__ w, T* __restrict__ 
   int k = gid >> 1, half = gid & 1;
   int q = lane >> 5, m = lane & 31;
   int chan = 32 * half + 16 * s + 8 * q + j;
-  int co = 32 * tM + 16 * ((m >> 2) & 1) + 4 * (m >> 3) + (m & 3);
+  int co = 32 * tM + 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
   int kk = reverse ? K - 1 - k : k;
   out[e] = transposed ? w[((int64_t)kk * 64 + co) * 64 + chan] : w[((int64_t)kk * 64 + chan) * 64 + co];
 }
@@ -100,11 +102,11 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
         wreg[u][s][tM] = v;
       }
   }
-  // bias as fp32 in LDS (zeros without one); a lane finishes the 16 output channels
-  // 32 (wave % 2) + 16 q .. of a row
+  // bias as fp32 in LDS (zeros without one); a lane finishes the output channels
+  // 32 (wave % 2) + 16 round + 8 q .. + 7 of a row
   if (tid < 64) s_bias[tid] = bias ? to_f32(bias[tid]) : 0.f;
   if (tid == 0) s_u0[3] = s_u1[3] = -1;
-  const f32x4* bias4 = (const f32x4*)(&s_bias[32 * (wave & 1) + 16 * q]);
+  const f32x4* bias4 = (const f32x4*)(&s_bias[32 * (wave & 1) + 8 * q]);
 
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
   const __amdgpu_buffer_rsrc_t rs_loc = make_rsrc(loc, loc_bytes);
@@ -201,12 +203,12 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw_kernel(
         const int h = f - 8;
 #pragma unroll
         for (int src = 0; src < 4; ++src) red[src] = s_red[((src * 4 + wave) * 2 + h) * 64 + lane];
-        rb = bias4[2 * rnd + h];
+        rb = bias4[4 * rnd + h];
       }
       if (f == 11) {                                          // 8 channels = 16 bytes per lane
         const int64_t row = row0 + 32 * (wave >> 1) + r32;
         if (row < rows_out)
-          *(u32x4*)(out + row * 64 + 32 * (wave & 1) + 16 * q + 8 * rnd) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+          *(u32x4*)(out + row * 64 + 32 * (wave & 1) + 16 * rnd + 8 * q) = u32x4{pk[0], pk[1], pk[2], pk[3]};
       }
     } else if (f == 12) {
       barrier();                                              // the round has been read: s_red is free again

@@ -16,7 +16,7 @@ _lib = None
 def lib():
   global _lib
   if _lib is None:
-    if not os.path.exists(_build.PROBE_LIB_PATH):
+    if not _build.is_current():
       _build.build_library()
     h = ctypes.CDLL(_build.PROBE_LIB_PATH)
     h.ocnn_probe_mfma_rate.restype = c_int
@@ -94,3 +94,57 @@ def lds_rate(offsets, write=False, iters=4000, device='cuda'):
     raise RuntimeError('ocnn_probe_lds_rate failed')
   return {'tbytes_per_s': nbytes.value / ms.value / 1e9, 'ms': ms.value,
           'bytes_per_tick_per_cu': nbytes.value / n_cu / float(ticks.double().mean())}
+
+
+def _gather_pattern(threads, rows_of_lane, seed=0):
+  """Offsets of the gather-GEMM kernel's B-operand reads: lane (r32, q) of wave w reads the
+  16-byte chunk 4 (w % 2) + q of LDS row p = rows_of_lane(j, r32, generator), stored at chunk
+  c ^ ((p >> 1) & 7) of the 128-byte row."""
+  g = torch.Generator().manual_seed(seed)
+  out = torch.zeros(8, threads, dtype=torch.long)
+  for t in range(threads):
+    w, lane = t // 64, t % 64
+    c0 = 4 * (w & 1) + (lane >> 5)
+    for j in range(8):
+      p = rows_of_lane(j, lane & 31, g)
+      out[j, t] = p * 128 + ((c0 ^ (p >> 1)) & 7) * 16
+  return out % 65536
+
+
+def main():
+  """Prints the tables kept under profiles/: MFMA rates by operand statistics, the MFMA loop
+  with the gather-GEMM kernel's side work, LDS rates by address pattern."""
+  torch.cuda.set_device(0)
+  print('device:', torch.cuda.get_device_name(0), ' CUs:', _cus('cuda'))
+  print('\nv_mfma_f32_32x32x16, one wave per SIMD, 14 accumulators per wave, all CUs:')
+  for dt in (torch.bfloat16, torch.float16):
+    for ops in ('zero', 'constant', 'uniform', 'normal'):
+      r = mfma_rate(dt, ops, 20000)
+      print('  %-9s operands %-9s %7.1f TFLOP/s  %5.2f ticks/MFMA  %5.2f ns/MFMA  (%.2f GHz)' % (
+          str(dt)[6:], ops, r['tflops'], r['ticks_per_mfma'], r['ns_per_mfma'], r['ticks_per_mfma'] / r['ns_per_mfma']))
+  print('\nbf16 MFMA loop, two accumulator chains, N(0,1) operands:')
+  for mix, name in ((False, 'alone'), (True, 'with the gather-GEMM kernel\'s side work (per 8 MFMAs: 16 VALU, 6 ds_read_b128, '
+                                            '1 ds_write_b128, 2 ds_read_u16)')):
+    r = mfma_mix(mix)
+    print('  %-8s %7.1f TFLOP/s  %5.2f ticks/MFMA  %5.2f ns/MFMA  (%.2f GHz)  %s' % (
+        'alone' if not mix else 'mixed', r['tflops'], r['ticks_per_mfma'], r['ns_per_mfma'], r['ghz'], '' if not mix else name))
+  print('\nLDS, 16 bytes per lane and access, one workgroup of 256 threads per CU (B / tick / CU):')
+  lanes = torch.arange(256)
+  patterns = [
+      ('consecutive 16-byte chunks', torch.stack([(lanes % 64) * 16 + j * 1024 + (lanes // 64) * 8192 for j in range(8)])),
+      ('stride 32 B (2 lanes per 16-bank group)', torch.stack([((lanes % 64) * 32 + j * 2048) % 65536 for j in range(8)])),
+      ('stride 64 B', torch.stack([((lanes % 64) * 64 + j * 4096) % 65536 for j in range(8)])),
+      ('stride 128 B (same chunk of consecutive rows, no swizzle)', torch.stack([((lanes % 64) * 128 + j * 8192) % 65536 for j in range(8)])),
+      ('stride 256 B (all lanes on one bank group)', torch.stack([((lanes % 64) * 256) % 65536 for j in range(8)])),
+      ('gathered rows: 32 consecutive rows per access, swizzled', _gather_pattern(256, lambda j, r, g: 1 + r + 32 * j)),
+      ('gathered rows: two sibling groups 16 rows apart, swizzled', _gather_pattern(256, lambda j, r, g: 1 + (r % 8) + 16 * (r // 8) + 64 * j)),
+      ('gathered rows: random rows 0..416, swizzled', _gather_pattern(256, lambda j, r, g: int(torch.randint(0, 417, (1,), generator=g)))),
+  ]
+  for name, off in patterns:
+    rd, wr = lds_rate(off, False, 4000), lds_rate(off, True, 4000)
+    print('  %-60s read %6.1f   write %6.1f   (read %.1f TB/s whole GPU)' % (
+        name, rd['bytes_per_tick_per_cu'], wr['bytes_per_tick_per_cu'], rd['tbytes_per_s']))
+
+
+if __name__ == '__main__':
+  main()

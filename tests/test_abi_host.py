@@ -215,3 +215,17 @@ def test_kernel_selection_is_consistent_with_the_predicates():
   # 128 output channels on more rows than 32-bit offsets of the output reach: not the pair-plan kernel
   big = 17_000_000
   assert L.ocnn_conv_gather_choose(BF, big, big, 27, 128, 128, 0, 1, 300, big * 2, 0.15, 4.0) != _lib.GATHER_SPARSE
+
+
+def test_a_stale_library_is_not_loaded(monkeypatch):
+  """The built libraries carry the hash of their sources; when a source changes, the loader
+  builds again instead of loading the old binary."""
+  from ocnn_amd import _lib, build
+  assert build.is_current()                       # the tree's libraries match the tree's sources
+  calls = []
+  monkeypatch.setattr(build, 'source_hash', lambda: 'something else')
+  monkeypatch.setattr(build, 'build_library', lambda verbose=False: calls.append(1))
+  monkeypatch.setattr(_lib, '_lib', None)
+  assert not build.is_current()
+  _lib.lib()
+  assert calls == [1]
