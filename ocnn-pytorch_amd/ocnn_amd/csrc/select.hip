@@ -36,7 +36,7 @@ extern "C" int ocnn_conv_gather_choose(int dtype, int64_t rows_in, int64_t rows_
   }
   if (has_plan && rows_ok(rows_out, plan_total)) {
     if (ocnn_conv_gather_rw_supported(dtype, rows_in, K, cin, cout, plan_max_distinct) &&
-        rows_out * K * 2 < kOffsetLimit)
+        rows_out * K * 2 < kOffsetLimit && (rows_out + 128) * cout * 2 < kOffsetLimit)
       return OCNN_GATHER_RW;
     if (plan_occupancy <= kSparseMaxOccupancy && rows_out >= kSparseMinRows &&
         rows_out * cout * 2 <= kOffsetLimit &&
