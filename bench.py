@@ -173,22 +173,22 @@ def main():
   with torch.no_grad():
     bound = 1.0 / (27 * C) ** 0.5                      # Kaiming-uniform bound
     conv.weights.copy_((torch.rand(conv.weights.shape, generator=g) * 2 - 1) * bound)
-  x32 = torch.randn(rows, C, generator=g)
-  gout32 = torch.randn(rows, C, generator=g)
+  x_dev = torch.randn(rows, C, generator=g).to(dev)
+  gout_dev = torch.randn(rows, C, generator=g).to(dev)
 
   t_gather = KernelTimer(torch, conv_mod, 'conv_gather')
   t_wgrad = KernelTimer(torch, conv_mod, 'conv_wgrad')
   eng = conv_mod._OctreeConv(C, C, [3], 1, nempty)
   eng.setup(octree, depth)
 
-  def timed_steps(dt, steps, warmup, oct=octree, only='all'):
-    """ms per step of the layer in dtype `dt` on octree `oct` (kernel timers enabled)."""
+  def make_step(dt, oct=octree, only='all'):
+    """The step closure of the layer in dtype `dt` on octree `oct`; all its tensors on the device."""
     m = OctreeConv(C, C, [3], 1, nempty=nempty)
     with torch.no_grad():
       m.weights.copy_(conv.weights)
     m = m.to(dev).to(dt)
-    x = x32.to(dt).to(dev).requires_grad_()
-    gout = gout32.to(dt).to(dev)
+    x = x_dev.to(dt).requires_grad_()
+    gout = gout_dev.to(dt)
     w_cast = m.weights.detach()
 
     def step():
@@ -202,7 +202,11 @@ def main():
         x.grad = None
         m.weights.grad = None
         m(x, oct, depth).backward(gout)
+    return step
 
+  def run_steps(step, steps, warmup):
+    """`warmup` untimed steps, then `steps` timed ones between synchronisations: ms per step,
+    and the mean launch times of the two kernel families (events around every launch)."""
     for _ in range(warmup):
       step()
     torch.cuda.synchronize()
@@ -216,6 +220,9 @@ def main():
     dt_s = time.perf_counter() - t0
     t_gather.enabled = t_wgrad.enabled = False
     return dt_s * 1e3 / steps, t_gather.mean_ms(), t_wgrad.mean_ms(), t_gather.count()
+
+  def timed_steps(dt, steps, warmup, oct=octree, only='all'):
+    return run_steps(make_step(dt, oct, only), steps, warmup)
 
   if args.calib:
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -231,13 +238,23 @@ def main():
   # its layers with triton.testing.do_bench, 25 ms of warm-up before 100 ms of repetitions
   # (test/benchmark_conv.py:115,131).  This section shows the ramp and leaves the chip where
   # such a warm-up would; the W warm-up steps and the K timed steps of the contract follow.
+  headline = make_step(dtype, only=args.only)
   cold = []
   if extras:
-    for _ in range(8):
-      cold.append(timed_steps(dtype, 5, 0)[0])
+    headline()                                         # first call: module load, allocations, the plan
+    torch.cuda.synchronize()
+    time.sleep(1.0)                                    # from idle
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(9)]
+    marks[0].record()
+    for b in range(8):
+      for _ in range(5):
+        headline()
+      marks[b + 1].record()
+    torch.cuda.synchronize()
+    cold = [marks[b].elapsed_time(marks[b + 1]) / 5 for b in range(8)]
 
-  # ---- the headline step ------------------------------------------------------
-  ms, gather_ms, wgrad_ms, n_gather = timed_steps(dtype, args.steps, args.warmup, only=args.only)
+  # ---- the headline step: W warm-up steps, K timed steps ---------------------------
+  ms, gather_ms, wgrad_ms, n_gather = run_steps(headline, args.steps, args.warmup)
   gather_ms = gather_ms or float('nan')
   wgrad_ms = wgrad_ms or float('nan')
   flops_step = 6.0 * nnz * C * C
@@ -308,8 +325,8 @@ def main():
 
   if extras:
     result['cold_start'] = {'ms_per_step_blocks_of_5': [round(v, 4) for v in cold],
-                            'note': 'the first 40 steps of the process, run before the W warm-up steps: the step '
-                                    'time falls for about 30 ms of sustained work before it settles'}
+                            'note': '40 steps from an idle GPU (events every 5 steps), run right before the W warm-up '
+                                    'steps: the step time falls for about 30 ms of sustained work before it settles'}
     # ---- the same step in the other 16-bit type ------------------------------
     other = 'fp16' if args.dtype == 'bf16' else 'bf16'
     oms, ogm, owm, _ = timed_steps(DT[other], args.steps, args.warmup)
