@@ -13,6 +13,9 @@ MI355X (the headline number is bench.py's; these lines are supporting data).
   config 4: the U-Net's octree (batch of 8, 150k points each, depth 9), bf16: 3x3x3 and
             2x2x2 stride-2 layers of 96 / 128 channels on the non-empty nodes of depths 9 and
             8 (the tables the pair-plan kernels are for).
+  config f4: the rest of the kernel-shape x stride grid on the depth-8 batch of config 2, bf16,
+            64 channels: 3x3x3 stride 2 (conv and deconv), the axis kernels 3x1x1 and 3x3x1 at
+            stride 1 and 2, 2x2x2 at stride 1, on all nodes and on non-empty nodes.
 
 Every layer runs forward + backward through the module (autograd included); one JSON
 line per layer: ms per fwd+bwd, effective TFLOP/s over non-empty neighbours, and the
@@ -35,7 +38,7 @@ def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--steps', type=int, default=30)
   ap.add_argument('--warmup', type=int, default=5)
-  ap.add_argument('--configs', default='2,3,4')
+  ap.add_argument('--configs', default='2,3,4,f4')
   args = ap.parse_args()
   import torch
   from ocnn_amd import synthetic
@@ -173,6 +176,23 @@ def main():
         o._table(9, '333', 1, False), bf)
     run('conv 3x3x3 s1 256->256 d6', OctreeConv(256, 256, [3], 1), o, 6, int(o.nnum[6]), 256, 256,
         o._table(6, '333', 1, False), bf)
+  if 'f4' in args.configs.split(','):
+    o, b_ms, n_ms, npts = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
+    print(json.dumps({'octree': 'config f4 (batch 8, depth 8)', 'points': npts, 'build_octree_ms': b_ms,
+                      'construct_all_neigh_ms': n_ms}), flush=True)
+    C = 64
+    for ks, stride in (([3, 3, 3], 2), ([3, 1, 1], 1), ([3, 1, 1], 2), ([3, 3, 1], 1), ([3, 3, 1], 2), ([2, 2, 2], 1)):
+      kern = ''.join(str(k) for k in ks)
+      for ne in (False, True):
+        for kind, Mod in (('conv', OctreeConv), ('deconv', OctreeDeconv)):
+          if kind == 'deconv' and stride == 1:
+            continue
+          d = 8 if kind == 'conv' else 7
+          rows_in = int(o.nnum_nempty[d] if ne else o.nnum[d])
+          run('%s %s s%d %d->%d d%d%s' % (kind, 'x'.join(kern), stride, C, C, d, ' nempty' if ne else ''),
+              Mod(C, C, ks, stride, nempty=ne), o, d, rows_in, C, C,
+              o._table(d if kind == 'conv' else d + 1, kern, stride, ne), bf)
+    del o
   if '4' in args.configs.split(','):
     # the U-Net's octree (config 4: batch 8, 150k points each, depth 9), layers on the non-empty
     # nodes of depths 9 and 8, where 14 % / 25 % of the table entries hold a neighbour
