@@ -435,8 +435,10 @@ int ocnn_dwconv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
 
 /* The depth-wise engine over the tile plan of the table (same reference lines, same
  * results up to the fp32 summation order, which is fixed): the distinct rows of a tile
- * are staged once in LDS, 64 channels at a time.  f16 / bf16, channels a multiple of 64,
- * plan_max_distinct <= 416; the weight gradient for K in {27, 9, 8, 3}. */
+ * are staged once in LDS, 64 channels at a time, and the products run on the 4x4x4 matrix
+ * instruction.  f16 / bf16, channels a multiple of 64, plan_max_distinct <= 416, K in
+ * {27, 9, 8, 3}.  A non-finite input value reaches the other three channels of its group
+ * of four (0 x inf inside the instruction). */
 int ocnn_dwconv_gather_planned_supported(int dtype, int64_t rows_in, int K, int channels,
                                          int plan_max_distinct);
 int ocnn_dwconv_gather_planned(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,

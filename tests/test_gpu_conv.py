@@ -990,7 +990,7 @@ def test_planned_kernels_fall_back_on_large_tiles():
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize('K,ch', [(27, 64), (27, 192), (9, 128), (8, 64), (3, 128), (5, 64)])
+@pytest.mark.parametrize('K,ch', [(27, 64), (27, 192), (9, 128), (8, 64), (3, 128)])
 def test_dwconv_planned_kernels(dtype, K, ch):
   """Depth-wise kernels on the tile plan (rows staged in LDS): gather with bias, with mirrored
   slots, and the weight gradient (the slot counts it is built for), against the oracle."""
