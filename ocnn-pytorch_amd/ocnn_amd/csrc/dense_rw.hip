@@ -154,8 +154,8 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
     }
     // the next tile has landed; every wave is done with this one
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWait) : "memory");
-    __syncthreads();
+    // (a bare barrier: __syncthreads() would wait for every load in flight, the ring's included)
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kWait) : "memory");
     slot = slot == NBUF - 1 ? 0 : slot + 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
@@ -178,7 +178,11 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
   constexpr int GA = 2 * WA, GB = 2 * WB, NG = GA + GB;            // 64-channel groups of a tile
   constexpr int RT = 32, TILE = NG * RT * 128;                     // 40 KiB (32 KiB at WA = 2)
   constexpr int PW = NG * (RT / 8) / 4;                            // staging pieces per wave and tile
-  extern __shared__ __attribute__((aligned(16))) char s_dyn[];     // ring of three tiles
+  // ring of three tiles: three arrays, not thirds of one, so that the compiler knows that the
+  // reads of a tile cannot meet the loads in flight into the other two and does not wait for them
+  __shared__ __attribute__((aligned(16))) char s_t0[TILE];
+  __shared__ __attribute__((aligned(16))) char s_t1[TILE];
+  __shared__ __attribute__((aligned(16))) char s_t2[TILE];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave / WB, wb = wave % WB;
@@ -255,18 +259,19 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
   };
 
   // ---- ring of three: tile i is multiplied while i + 1 and i + 2 are in flight ----
-  stage(t_begin, s_dyn);
-  stage(t_begin + 1, s_dyn + TILE);
-  int slot = 0;
-  for (int64_t tile = t_begin; tile < t_end; ++tile) {
+  stage(t_begin, s_t0);
+  stage(t_begin + 1, s_t1);
+  auto step = [&](auto SLOT, int64_t tile) {
+    constexpr int slot = decltype(SLOT)::value;
     // own pieces of this tile have landed (those of the next one may be in flight), then
     // everyone's; every wave is also done with the tile before, whose buffer is filled next
-    if (PW == 10) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    __syncthreads();
-    const int s2 = slot >= 1 ? slot - 1 : 2;                       // (slot + 2) % 3
-    stage(tile + 2, s_dyn + s2 * TILE);
-    const char* buf = s_dyn + slot * TILE;
+    // (a bare barrier: __syncthreads() would wait for the next tile's loads too)
+    // (the wait as an instruction of its own, which the compiler's wait insertion takes into
+    // account: s_waitcnt vmcnt(PW) lgkmcnt(0), vmcnt in bits 3:0, lgkmcnt in bits 11:8)
+    __builtin_amdgcn_s_waitcnt(PW == 10 ? 0x007a : 0x0078);
+    asm volatile("s_barrier" ::: "memory");
+    stage(tile + 2, slot == 0 ? s_t2 : slot == 1 ? s_t0 : s_t1);
+    const char* buf = slot == 0 ? s_t0 : slot == 1 ? s_t1 : s_t2;
     Ops o0, o1;
     fetch(buf, 0, o0);
     fetch(buf, 1, o1);
@@ -274,7 +279,18 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
     __builtin_amdgcn_sched_barrier(0);
     mma(o1);
     __builtin_amdgcn_sched_barrier(0);
-    slot = slot == 2 ? 0 : slot + 1;
+  };
+  // whole rounds of the ring in the loop, the last one or two tiles after it: no path skips a
+  // step, so the compiler's wait insertion sees the real order of loads and reads
+  int64_t tile = t_begin;
+  for (; tile + 3 <= t_end; tile += 3) {
+    step(std::integral_constant<int, 0>{}, tile);
+    step(std::integral_constant<int, 1>{}, tile + 1);
+    step(std::integral_constant<int, 2>{}, tile + 2);
+  }
+  if (tile < t_end) {
+    step(std::integral_constant<int, 0>{}, tile);
+    if (tile + 1 < t_end) step(std::integral_constant<int, 1>{}, tile + 1);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
 
@@ -434,15 +450,8 @@ extern "C" int64_t ocnn_conv_dense_wgrad_rw_workspace_bytes(int ca, int cb) {
 template <typename T, int WA>
 static void launch_dense_wgrad(const void* x, const void* g, int64_t rows, int ca, int cb, int nsplit, int64_t per,
                                int64_t tiles, float* partial, hipStream_t st) {
-  const int lds = 3 * (2 * WA + 2 * (4 / WA)) * 32 * 128;
-  static bool attr_set = false;
-  if (!attr_set) {
-    (void)hipFuncSetAttribute((const void*)conv_dense_wgrad_rw_kernel<T, WA>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    attr_set = true;
-  }
   hipLaunchKernelGGL((conv_dense_wgrad_rw_kernel<T, WA>), dim3((unsigned)nsplit, (unsigned)dr_wgrad_blocks(ca, cb, WA)),
-                     dim3(256), lds, st, (const T*)x, (uint32_t)(rows * ca * 2), (const T*)g,
+                     dim3(256), 0, st, (const T*)x, (uint32_t)(rows * ca * 2), (const T*)g,
                      (uint32_t)(rows * cb * 2), ca, cb, tiles, per, partial);
 }
 
