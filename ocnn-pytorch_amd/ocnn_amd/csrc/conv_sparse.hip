@@ -170,12 +170,25 @@ __global__ __launch_bounds__(128 * NG, WPC) void conv_gather_sparse_kernel(
   // global->LDS loads of a tile's rows and entries (asynchronous)
   auto dma = [&](const Meta& m, int buf) {
     const int chunks = (m.U + 1) * CPR;
-    for (int piece = wave; piece * 64 < chunks; piece += 2 * NG) {
-      const int L = piece * 64 + lane;
-      const int p = L / CPR, c = L - p * CPR;
-      const int32_t id = s_u[buf * su + min(p, su - 1)];
-      const uint32_t off = (id >= 0 && c < CPR - 1) ? (uint32_t)id * pitch_g + (uint32_t)c * 16u : 0xffffff00u;
-      sp_dma16(rs_in, s_rows + piece * 1024, off);
+    // four pieces at a time: their list entries first (one LDS wait for the four), then the loads
+    for (int piece0 = wave; piece0 * 64 < chunks; piece0 += 8 * NG) {
+      int32_t id[4];
+      uint32_t cb16[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int L = (piece0 + 2 * NG * e) * 64 + lane;
+        const int p = L / CPR, c = L - p * CPR;
+        id[e] = s_u[buf * su + min(p, su - 1)];
+        cb16[e] = c < CPR - 1 ? (uint32_t)c * 16u : 0xffffffffu;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int piece = piece0 + 2 * NG * e;
+        if (piece * 64 < chunks) {
+          const uint32_t off = (id[e] >= 0 && cb16[e] != 0xffffffffu) ? (uint32_t)id[e] * pitch_g + cb16[e] : 0xffffff00u;
+          sp_dma16(rs_in, s_rows + piece * 1024, off);
+        }
+      }
     }
     for (int piece = wave; piece * 16 < m.nb; piece += 2 * NG)           // 16 blocks (1 KiB) per load
       sp_dma16(rs_ent, (char*)s_ent + piece * 1024, (uint32_t)m.cb * 64u + (uint32_t)(piece * 1024 + lane * 16));

@@ -138,14 +138,19 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   };
 
   // the distinct rows' channels 64 cc .. of the tile -> LDS
+  // the list entries of this lane's pieces, read once for all chunks (one LDS wait, not one per piece)
+  __syncthreads();
+  int32_t ids[kRowPieces];
+#pragma unroll
+  for (int i = 0; i < kRowPieces; ++i) ids[i] = s_u[min(st_p + 32 * i, kWdRowsAlloc - 1)];   // -1: out of range, loads zeros
   auto stage_chunk = [&](int cc) {
-    // every wave is done with the chunk before (and, the first time, s_u is complete)
+    // every wave is done with the chunk before
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < kRowPieces; ++i) {
       const int g = wave + 4 * i;
       if (g < groups) {
-        const int32_t id = s_u[st_p + 32 * i];               // -1: out of range, loads zeros
+        const int32_t id = ids[i];
         uint32_t off = (uint32_t)id * pitch + ((uint32_t)cc * 128u + st_c);
         if (cc == ncc - 1 && half_oob) off = 0xffffff00u;    // past the row's channels: zeros, not the next row
         wd_dma16(rs_in, (char*)s_rows + g * 1024, off);

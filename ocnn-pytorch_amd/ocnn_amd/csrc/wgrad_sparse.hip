@@ -58,9 +58,16 @@ static __device__ __forceinline__ void ws_stage(char* __restrict__ sa, char* __r
   const int row = lane >> 2;
   const uint32_t chunk = (uint32_t)(lane & 3) * 16u;
   const int na = (t.U + 16) >> 4;                                         // positions 0 .. U
-  for (int p = wave; p < na; p += 8) {
-    const int32_t id = u[p * 16 + row];
-    ws_dma16(rs_a, sa + p * 1024, id >= 0 ? (uint32_t)id * a_pitch + a_col + chunk : 0xffffff00u);
+  // four pieces at a time: their list entries first (one LDS wait for the four), then the loads
+  for (int p0 = wave; p0 < na; p0 += 32) {
+    int32_t id[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) id[e] = u[min(p0 + 8 * e, na - 1) * 16 + row];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int p = p0 + 8 * e;
+      if (p < na) ws_dma16(rs_a, sa + p * 1024, id[e] >= 0 ? (uint32_t)id[e] * a_pitch + a_col + chunk : 0xffffff00u);
+    }
   }
 #pragma unroll
   for (int half = 0; half < HB; ++half)                                   // 8 HB pieces, HB per wave
