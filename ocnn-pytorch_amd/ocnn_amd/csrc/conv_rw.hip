@@ -411,20 +411,34 @@ __global__ void pack_weights_rw32_kernel(const T* __restrict__ w, T* __restrict_
   out[e] = transposed ? w[((int64_t)kk * 32 + co) * 32 + chan] : w[((int64_t)kk * 32 + chan) * 32 + co];
 }
 
+// 32 -> 32 channels: per tile half the bytes of the 64-channel kernel and a quarter of its
+// matrix work, so what bounds this kernel is how much a CU has in flight.  A ring of THREE
+// tiles in LDS: while tile i is multiplied, the rows and positions of tiles i + 1 and i + 2
+// are in flight.  Vector memory operations complete in issue order, so "tile i + 1 has landed"
+// is a count: every wave issues exactly kOps operations per tile (pieces that a tile does not
+// need go to a dump area out of range, rows past the end are stored out of range), the first
+// of them the list boundary six tiles ahead, and the wait at the end of a tile leaves the
+// kOps - 1 after that one in flight.  What an operation of tile i loads may therefore be used
+// from tile i + 2 on: list boundary (six tiles ahead) -> the lane's entries of the list of
+// distinct rows (four ahead, straight into registers, no list in LDS) -> rows and positions
+// (two ahead) -> products.
 template <typename T, int KK>
 __global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const uint16_t* __restrict__ loc,
     uint32_t loc_bytes, const int32_t* __restrict__ uptr, const int32_t* __restrict__ urows,
     uint32_t urows_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
-    T* __restrict__ out, int64_t rows_out, int64_t tiles, int64_t tiles_per_wg) {
+    T* __restrict__ out, uint32_t out_bytes, int64_t rows_out, int64_t tiles, int64_t tiles_per_wg) {
   constexpr int kLocElems = (kRwRows * 27 * 2 + 1023) / 1024 * 512;
   constexpr int kRowsAlloc = (kRwCap + 16) / 16 * 16;            // rows 0..kRwCap, whole 16-row groups
+  // one array per buffer of the ring: the compiler then knows that the reads of one cannot meet
+  // the loads in flight into the others and does not wait for them
   __shared__ __attribute__((aligned(16))) T s_rows0[kRowsAlloc * 32];
   __shared__ __attribute__((aligned(16))) T s_rows1[kRowsAlloc * 32];
+  __shared__ __attribute__((aligned(16))) T s_rows2[kRowsAlloc * 32];
   __shared__ __attribute__((aligned(16))) uint16_t s_loc0[kLocElems];
   __shared__ __attribute__((aligned(16))) uint16_t s_loc1[kLocElems];
-  __shared__ __attribute__((aligned(16))) int32_t s_u0[4 + 512];
-  __shared__ __attribute__((aligned(16))) int32_t s_u1[4 + 512];
+  __shared__ __attribute__((aligned(16))) uint16_t s_loc2[kLocElems];
+  __shared__ __attribute__((aligned(16))) char s_dump[1024];     // where the pieces a tile does not need go
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -441,80 +455,84 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
   float bq[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) bq[i] = bias ? to_f32(bias[16 * q + i]) : 0.f;
-  if (tid == 0) s_u0[3] = s_u1[3] = -1;
 
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
   const __amdgpu_buffer_rsrc_t rs_loc = make_rsrc(loc, loc_bytes);
   const __amdgpu_buffer_rsrc_t rs_u = make_rsrc(urows, urows_bytes);
   const __amdgpu_buffer_rsrc_t rs_p = make_rsrc(uptr, (uint32_t)(tiles + 1) * 4u);
+  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(out, out_bytes);
 
-  // staging pieces per wave: 0, 1 table positions; 2 list of the tile after; 3 + i LDS rows
+  // Staging pieces of a tile per wave: kLocPieces of table positions, then kRowPieces of LDS rows
   // 16 (wave + 4 i) .. + 15 (row p >= 1 = distinct row p - 1, row 0 = zero row).  The 16-byte
   // chunk c of row p lands at chunk c ^ ((p >> 2) & 3), a per-lane constant here.
   constexpr int kRowPieces = (kRwCap + 1 + 63) / 64;
-  constexpr int kPieces = 3 + kRowPieces;
+  constexpr int kLocChunks = (kRwRows * KK * 2 + 1023) >> 10;
+  constexpr int kLocPieces = (kLocChunks + 3) / 4;
+  constexpr int kPieces = kLocPieces + kRowPieces;
+  constexpr int kOps = 1 + kRowPieces + kPieces + 2;             // boundary, list entries, pieces, stores
+  static_assert(kOps - 1 <= 63, "vmcnt is a 6-bit counter");
   const uint32_t st_c = (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
-  const int st_p = 16 * wave + (lane >> 2);
-  auto make_stage = [&](int64_t tile, int U, int32_t list_first, int32_t list_len, const int32_t* su,
-                        int32_t* su_out, T* rows, uint16_t* locs) {
-    RwStage st;
-    const int64_t tc = min(tile, tiles - 1);
-    st.loc_off = (uint32_t)(tc * kRwRows * KK * 2);
-    const int e = wave * 256 + lane * 4;
-    st.list_off = e < list_len ? (uint32_t)(list_first + e) * 4u : 0xffffff00u;
-    st.groups = (U + 16) >> 4;
-    st.su = su; st.su_out = su_out; st.rows = (char*)rows; st.locs = (char*)locs;
-    return st;
+  const int st_p = 16 * wave + (lane >> 2);                       // LDS row of row piece 0; piece i: + 64 i
+  // the lane's entry of the list that starts at `first` for row piece i (position 0: the zero row)
+  auto load_id = [&](int i, int32_t first) -> int32_t {
+    return (int32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_u, (uint32_t)(first + st_p + 64 * i - 1) * 4u, 0, 0);
   };
-  auto stage_id = [&](int t, const RwStage& st) -> int32_t {
-    return t >= 3 ? st.su[st_p + 64 * (t - 3) - 1] : 0;
-  };
-  auto stage_piece = [&](int t, const RwStage& st, int32_t id) {
-    if (t < 2) {
-      constexpr int nchunk = (kRwRows * KK * 2 + 1023) >> 10;
-      if (4 * t < nchunk) {
-        const int c = min(wave + 4 * t, nchunk - 1);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_loc, (lds_ptr_t)(st.locs + c * 1024), 16,
-                                                 st.loc_off + (uint32_t)c * 1024u + lane * 16u, 0, 0, 0);
-      }
-    } else if (t == 2) {
-      if (wave < 2)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_u, (lds_ptr_t)(st.su_out + wave * 256), 16, st.list_off,
-                                                 0, 0, 0);
+  auto stage_piece = [&](int t, int64_t tile, int groups, const int32_t (&ids)[kRowPieces], char* rows, char* locs) {
+    if (t < kLocPieces) {
+      const int c = min(wave + 4 * t, kLocChunks - 1);            // a spare wave repeats the last chunk
+      const uint32_t loc_off = (uint32_t)(min(tile, tiles - 1) * kRwRows * KK * 2);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_loc, (lds_ptr_t)(locs + c * 1024), 16,
+                                               loc_off + (uint32_t)c * 1024u + lane * 16u, 0, 0, 0);
     } else {
-      if (wave + 4 * (t - 3) < st.groups)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(st.rows + (wave + 4 * (t - 3)) * 1024), 16,
-                                                 ((uint32_t)id << 6) | st_c, 0, 0, 0);
+      const int i = t - kLocPieces;
+      const int g = wave + 4 * i;
+      const bool need = g < groups;
+      const int32_t id = (st_p + 64 * i == 0) ? -1 : ids[i];     // -1: out of range, zeros
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (lds_ptr_t)(need ? rows + g * 1024 : s_dump), 16,
+                                               need ? (((uint32_t)id << 6) | st_c) : 0xffffff00u, 0, 0, 0);
     }
   };
 
-  int32_t p_nxt = uptr[t_begin + 1];
-  int32_t p_nx2 = uptr[min(t_begin + 2, tiles)];
-  int32_t p_nx3 = uptr[min(t_begin + 3, tiles)];
+  // ---- prologue: tiles 0 and 1 staged, list entries of tiles 2 and 3 in registers ----
+  // p_a .. p_d: list boundaries of the tiles i + 2 .. i + 5 while tile i is multiplied
+  int32_t ids[3][kRowPieces];
+  int32_t p_a, p_b, p_c, p_d;
   {
-    const int32_t p_cur = uptr[t_begin];
-    RwStage st = make_stage(t_begin, 0, p_cur, p_nxt - p_cur, s_u0 + 4, s_u0 + 4, s_rows0, s_loc0);
-    stage_piece(2, st, 0);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    st = make_stage(t_begin, p_nxt - p_cur, p_nxt, p_nx2 - p_nxt, s_u0 + 4, s_u1 + 4, s_rows0, s_loc0);
+    const int32_t p0 = uptr[t_begin], p1 = uptr[min(t_begin + 1, tiles)];
+    p_a = uptr[min(t_begin + 2, tiles)];
+    p_b = uptr[min(t_begin + 3, tiles)];
+    p_c = uptr[min(t_begin + 4, tiles)];
+    p_d = uptr[min(t_begin + 5, tiles)];
 #pragma unroll
-    for (int t = 0; t < kPieces; ++t) stage_piece(t, st, stage_id(t, st));
+    for (int i = 0; i < kRowPieces; ++i) {
+      ids[0][i] = load_id(i, p0);
+      ids[1][i] = load_id(i, p1);
+    }
+#pragma unroll
+    for (int t = 0; t < kPieces; ++t) stage_piece(t, t_begin, (p1 - p0 + 16) >> 4, ids[0], (char*)s_rows0, (char*)s_loc0);
+#pragma unroll
+    for (int t = 0; t < kPieces; ++t) stage_piece(t, t_begin + 1, (p_a - p1 + 16) >> 4, ids[1], (char*)s_rows1, (char*)s_loc1);
+#pragma unroll
+    for (int i = 0; i < kRowPieces; ++i) {
+      ids[2][i] = load_id(i, p_a);
+      ids[0][i] = load_id(i, p_b);
+    }
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+    asm volatile("s_barrier" ::: "memory");
   }
 
   constexpr int PD = 8;      // table positions are read PD slots ahead of their MFMAs ...
   constexpr int BD = 4;      // ... and the neighbour rows BD slots ahead
   auto tile_body = [&](auto BC, int64_t tile) {
-    constexpr int B = decltype(BC)::value;
-    const T* rows = B ? s_rows1 : s_rows0;
-    const uint16_t* lc = B ? s_loc1 : s_loc0;
-    const RwStage st = make_stage(tile + 1, p_nx2 - p_nxt, p_nx2, p_nx3 - p_nx2, B ? s_u0 + 4 : s_u1 + 4,
-                                  B ? s_u1 + 4 : s_u0 + 4, B ? s_rows0 : s_rows1, B ? s_loc0 : s_loc1);
-    const uint32_t p_raw = __builtin_amdgcn_raw_buffer_load_b32(rs_p, (uint32_t)min(tile + 4, tiles) * 4u, 0, 0);
-    p_nxt = p_nx2;
-    p_nx2 = p_nx3;
+    constexpr int B = decltype(BC)::value;                       // this tile's buffer of the ring
+    constexpr int B1 = (B + 1) % 3, B2 = (B + 2) % 3;
+    const T* rows = B == 0 ? s_rows0 : B == 1 ? s_rows1 : s_rows2;
+    const uint16_t* lc = B == 0 ? s_loc0 : B == 1 ? s_loc1 : s_loc2;
+    char* rows_st = (char*)(B2 == 0 ? s_rows0 : B2 == 1 ? s_rows1 : s_rows2);
+    char* locs_st = (char*)(B2 == 0 ? s_loc0 : B2 == 1 ? s_loc1 : s_loc2);
+    const int groups_st = (p_b - p_a + 16) >> 4;                 // tile + 2 fills this many 16-row groups
+    // the first operation of the tile: list boundary six tiles ahead
+    const uint32_t p_raw = __builtin_amdgcn_raw_buffer_load_b32(rs_p, (uint32_t)min(tile + 6, tiles) * 4u, 0, 0);
 
     const uint16_t* lcw = lc + 32 * wave + r32;                 // this lane's row, slot k at + 128 k
     uint32_t pos[PD];
@@ -533,7 +551,6 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
 #pragma unroll
     for (int k = 0; k < BD && k < KK; ++k) issue_b(k);
     __builtin_amdgcn_sched_barrier(0);
-    int32_t id_next = 0;
 #pragma unroll
     for (int k = 0; k < KK; ++k) {
       acc = Mma32<T>::run(wreg[k][0], ring[k % PD][0], acc);
@@ -541,38 +558,55 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
       acc = Mma32<T>::run(wreg[k][1], ring[k % PD][1], acc);
       if (k + PD < KK) pos[k % PD] = lcw[kRwRows * (k + PD)];
       __builtin_amdgcn_sched_barrier(0);
-      // staging of the next tile: list entry on an even slot, its load on the odd one after
+      // staging: the list entries of tile + 4 on the even slots, the pieces of tile + 2 on the odd ones
       {
         const int t = k >> 1;
-        if (t < kPieces) {
-          if ((k & 1) == 0) id_next = stage_id(t, st);
-          else stage_piece(t, st, id_next);
+        if ((k & 1) == 0) {
+          if (t < kRowPieces) ids[B1][t] = load_id(t, p_c);
+        } else {
+          if (t < kPieces) stage_piece(t, tile + 2, groups_st, ids[B2], rows_st, locs_st);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (KK < 2 * kPieces) {                                      // few slots: the rest of the pieces
+    // few slots: the rest of the staging
 #pragma unroll
-      for (int t = KK / 2; t < kPieces; ++t) stage_piece(t, st, stage_id(t, st));
-    }
+    for (int t = (KK + 1) / 2; t < kRowPieces; ++t) ids[B1][t] = load_id(t, p_c);
+#pragma unroll
+    for (int t = KK / 2; t < kPieces; ++t) stage_piece(t, tile + 2, groups_st, ids[B2], rows_st, locs_st);
     // bias, pack, two 16-byte stores: 16 consecutive output channels of one row per lane
-    const int64_t row = tile * kRwRows + 32 * wave + r32;
-    if (row < rows_out) {
+    // (every lane issues both: the wait below counts on it; rows past the end are dropped)
+    {
+      const int64_t row = tile * kRwRows + 32 * wave + r32;
       unsigned pk[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) pk[i] = pack2<T>(acc[2 * i] + bq[2 * i], acc[2 * i + 1] + bq[2 * i + 1]);
-      T* dst = out + row * 32 + 16 * q;
-      *(u32x4*)(dst) = u32x4{pk[0], pk[1], pk[2], pk[3]};
-      *(u32x4*)(dst + 8) = u32x4{pk[4], pk[5], pk[6], pk[7]};
+      const uint32_t off = row < rows_out ? (uint32_t)row * 64u + 32u * q : 0xffffff00u;
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{pk[0], pk[1], pk[2], pk[3]}, rs_out, off, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{pk[4], pk[5], pk[6], pk[7]}, rs_out, off + 16u, 0, 0);
     }
-    // the next tile has landed; every wave is past its last read of this tile's buffers
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    p_nx3 = __builtin_amdgcn_readfirstlane((int32_t)p_raw);
+    // tile + 1 has landed (everything up to this tile's first operation has); every wave is past
+    // its last read of this tile's buffers.  vmcnt in bits 3:0 and 15:14, LDS counter (bits 11:8) 0.
+    __builtin_amdgcn_s_waitcnt(0x0070 | ((kOps - 1) & 15) | (((kOps - 1) >> 4) << 14));
+    asm volatile("s_barrier" ::: "memory");
+    p_a = p_b;
+    p_b = p_c;
+    p_c = p_d;
+    p_d = __builtin_amdgcn_readfirstlane((int32_t)p_raw);
   };
-  for (int64_t tile = t_begin; tile < t_end; tile += 2) {
+  // whole rounds of the ring in the loop, the last one or two tiles after it: no path skips a
+  // tile, so the compiler's own wait insertion sees the real order of loads and uses
+  int64_t tile = t_begin;
+  for (; tile + 3 <= t_end; tile += 3) {
+    tile_body(std::integral_constant<int, 0>{}, tile);
+    tile_body(std::integral_constant<int, 1>{}, tile + 1);
+    tile_body(std::integral_constant<int, 2>{}, tile + 2);
+  }
+  if (tile < t_end) {
     tile_body(std::integral_constant<int, 0>{}, tile);
     if (tile + 1 < t_end) tile_body(std::integral_constant<int, 1>{}, tile + 1);
   }
+  __builtin_amdgcn_s_waitcnt(0x0070);                            // loads past the range still write LDS
 }
 
 }  // namespace ocnn
@@ -613,7 +647,8 @@ static void launch_rw32(const void* in, int64_t rows_in, const uint16_t* loc, co
   wgs = cdiv(tiles, per);
   hipLaunchKernelGGL((conv_gather_rw32_kernel<T, KK>), dim3((unsigned)wgs), dim3(256), 0, st, (const T*)in,
                      (uint32_t)(rows_in * 64), loc, (uint32_t)(tiles * kRwRows * KK * 2), uptr, urows,
-                     urows_bytes, (const T*)ws, (const T*)bias, (T*)out, rows_out, tiles, per);
+                     urows_bytes, (const T*)ws, (const T*)bias, (T*)out, (uint32_t)(rows_out * 64), rows_out, tiles,
+                     per);
 }
 
 template <typename T>
