@@ -385,6 +385,21 @@ int ocnn_conv_dense_wgrad_rw(int dtype, const void* x, const void* g, int64_t ro
                              int out_transposed, void* gw, void* workspace,
                              int64_t workspace_bytes, void* stream);
 
+/* The two of them with the rows of an operand taken through an index: row i of the GEMM's
+ * input (of x, of g) is row index[i] of a tensor with rows_in (rows_x, rows_g) rows; a NULL
+ * index means the operand's own rows 0 .. rows - 1, as above.  This is how the stride-2 layers
+ * over all nodes read the rows of the non-empty nodes out of a tensor padded to all nodes
+ * without a depad pass (the reference depads first: ocnn/nn/octree_conv.py:419-420, 450-451,
+ * ocnn/nn/octree_pad.py:32-39). */
+int ocnn_conv_dense_rw_indexed(int dtype, const void* in, int64_t rows_in, const int32_t* row_index,
+                               int64_t rows, const void* w, int cin, int cout, int w_transposed,
+                               const void* bias, void* out, void* workspace,
+                               int64_t workspace_bytes, void* stream);
+int ocnn_conv_dense_wgrad_rw_indexed(int dtype, const void* x, int64_t rows_x, const int32_t* x_index,
+                                     const void* g, int64_t rows_g, const int32_t* g_index,
+                                     int64_t rows, int ca, int cb, int out_transposed, void* gw,
+                                     void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Weight gradient, ocnn/nn/octree_conv.py:170-202 (weight_gemm) and
  * ocnn/nn/kernels/conv_bwd_implicit_gemm_splitk.py:94-184,294-306:
  * gw[k][a][b] = sum_i [t[i][k] >= 0] x[t[i][k]][a] * g[i][b], computed as

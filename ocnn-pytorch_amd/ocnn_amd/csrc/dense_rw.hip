@@ -33,8 +33,8 @@ static __device__ __forceinline__ void dr_dma16(__amdgpu_buffer_rsrc_t rs, char*
 // ---------------------------------------------------------------------------------------
 template <typename T, int NKS, int MB>
 __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
-    const T* __restrict__ in, uint32_t in_bytes, const T* __restrict__ wpk, const T* __restrict__ bias,
-    T* __restrict__ out, int64_t rows, int cout, int64_t tiles, int64_t tiles_per_wg) {
+    const T* __restrict__ in, uint32_t in_bytes, const int32_t* __restrict__ row_index, const T* __restrict__ wpk,
+    const T* __restrict__ bias, T* __restrict__ out, int64_t rows, int cout, int64_t tiles, int64_t tiles_per_wg) {
   constexpr int RB = 2, RT = 32 * RB, NCC = NKS / 4, CIN = 16 * NKS;
   constexpr int BUF = NCC * RT * 128;
   constexpr int NBUF = NCC >= 8 ? 2 : 4;                           // tiles resident in LDS
@@ -60,15 +60,33 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
   const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(out, (uint32_t)(rows * cout * 2));
   const int rl = lane >> 3;
-  auto stage = [&](int64_t tile, char* buf) {
+  // Row r of the operand is row row_index[r] of `in` when an index is given (the compact rows of
+  // the non-empty nodes read straight from the tensor over all nodes).  A lane stages the rows
+  // 8 wave + rl and 8 (wave + 4) + rl of a tile: two index entries per tile, loaded IDXD tiles
+  // before the tile is staged (without an index the loads point out of range and cost nothing;
+  // they are issued all the same, the waits below count operations).
+  const bool indexed = row_index != nullptr;
+  const __amdgpu_buffer_rsrc_t rs_idx = make_rsrc(row_index, indexed ? (uint32_t)(rows * 4) : 0u);
+  struct Idx { int32_t r[2]; };
+  auto load_index = [&](int64_t tile) {
+    Idx x;
+    const uint32_t row0 = (uint32_t)min(tile, tiles) * RT;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      x.r[h] = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_idx, (row0 + 8 * (wave + 4 * h) + rl) * 4u, 0, 0);
+    return x;
+  };
+  auto stage = [&](int64_t tile, char* buf, const Idx& x) {
     const uint32_t row0 = (uint32_t)min(tile, tiles) * RT;        // past the table: out of range, zeros
 #pragma unroll
     for (int j = 0; j < NCC * 2; ++j) {                           // NCC * 8 pieces of 1 KiB, 4 waves
       const int i = wave + 4 * j;
       const int cc = i >> 3, g = i & 7;
       const uint32_t swz = (uint32_t)((4 * g + (lane >> 4)) & 7);
+      // (with an index, rows past the end read entry 0 = some row: their results are dropped)
+      const uint32_t src = indexed ? (uint32_t)x.r[j & 1] : row0 + 8 * g + rl;
       dr_dma16(rs_in, buf + (cc * RT + 8 * g) * 128,
-               (row0 + 8 * g + rl) * (uint32_t)(CIN * 2) + (uint32_t)cc * 128u + (((uint32_t)(lane & 7) ^ swz) << 4));
+               src * (uint32_t)(CIN * 2) + (uint32_t)cc * 128u + (((uint32_t)(lane & 7) ^ swz) << 4));
     }
   };
   // B operand of k-step ks, row block rb: 16 bytes of row 32 rb + r32
@@ -87,27 +105,41 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
   // (tiles past the range load zeros or rows of another range; rows past the end are stored
   // out of range and dropped).  NST dropped stores per prologue tile make the count right from
   // the first tile on.
-  constexpr int P = NCC * 2, NST = RB * MB * 2;
+  constexpr int P = NCC * 2 + 2, NST = RB * MB * 2;                 // a tile's loads: its pieces and two index entries
   constexpr int kWait = (NBUF - 2) * P + (NBUF - 1) * NST;
   static_assert(kWait <= 63, "vmcnt is a 6-bit counter");
+  // s_waitcnt vmcnt(kWait) lgkmcnt(0) as an instruction of its own (vmcnt in bits 3:0 and 15:14,
+  // lgkmcnt in bits 11:8), which the compiler's wait insertion takes into account
+  constexpr int kWaitImm = 0x0070 | (kWait & 15) | ((kWait >> 4) << 14);
+  // Index entries loaded with the operations of tile i have landed when tile i + NBUF - 2 ends:
+  // they are loaded IDXD = 2 NBUF - 2 tiles ahead of their tile and used NBUF - 1 tiles later
+  constexpr int IDXD = 2 * NBUF - 2;
+  Idx iq[NBUF - 1];                                                // iq[0]: of the tile staged next
 #pragma unroll
   for (int v = 0; v < NBUF - 1; ++v) {
-    stage(t_begin + v, s_dyn + v * BUF);
+    const Idx x = load_index(t_begin + v);
+    stage(t_begin + v, s_dyn + v * BUF, x);
 #pragma unroll
     for (int j = 0; j < NST; ++j)
       __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, rs_out, 0xfffffff0u, 0, 0);
   }
+#pragma unroll
+  for (int v = 0; v < NBUF - 1; ++v) iq[v] = load_index(t_begin + NBUF - 1 + v);
   for (int i = tid; i < 128 * MB; i += 256)
     s_bias[i] = bias ? to_f32(bias[(int)blockIdx.y * 128 * MB + i]) : 0.f;
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWait) : "memory");
+  __builtin_amdgcn_s_waitcnt(0x0070);
   __syncthreads();
 
   int slot = 0;
-  for (int64_t tile = t_begin; tile < t_end; ++tile) {
+  // one tile; U: which of the NBUF - 1 index registers it consumes and refills (the registers are
+  // taken in turn and never copied: a copy would wait for the load of the tile before)
+  auto tile_step = [&](auto UC, int64_t tile) {
+    constexpr int U = decltype(UC)::value;
     const char* cur = s_dyn + slot * BUF;
     {
       const int sn = slot == 0 ? NBUF - 1 : slot - 1;              // the buffer of the tile before
-      stage(tile + NBUF - 1, s_dyn + sn * BUF);
+      stage(tile + NBUF - 1, s_dyn + sn * BUF, iq[U]);
+      iq[U] = load_index(tile + IDXD);
     }
     f32x16 acc[RB][MB];
 #pragma unroll
@@ -155,8 +187,26 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
     // the next tile has landed; every wave is done with this one
     __builtin_amdgcn_sched_barrier(0);
     // (a bare barrier: __syncthreads() would wait for every load in flight, the ring's included)
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kWait) : "memory");
+    __builtin_amdgcn_s_waitcnt(kWaitImm);
+    asm volatile("s_barrier" ::: "memory");
     slot = slot == NBUF - 1 ? 0 : slot + 1;
+  };
+  // whole rounds of the index registers in the loop, the rest after it (no path skips a tile, so
+  // the compiler's wait insertion sees the real order of loads and uses)
+  int64_t tile = t_begin;
+  if constexpr (NBUF == 4) {
+    for (; tile + 3 <= t_end; tile += 3) {
+      tile_step(std::integral_constant<int, 0>{}, tile);
+      tile_step(std::integral_constant<int, 1>{}, tile + 1);
+      tile_step(std::integral_constant<int, 2>{}, tile + 2);
+    }
+    if (tile < t_end) {
+      tile_step(std::integral_constant<int, 0>{}, tile);
+      if (tile + 1 < t_end) tile_step(std::integral_constant<int, 1>{}, tile + 1);
+    }
+  } else {
+    static_assert(NBUF == 2 || NBUF == 4, "index registers are taken in turn");
+    for (; tile < t_end; ++tile) tile_step(std::integral_constant<int, 0>{}, tile);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
 }
@@ -172,8 +222,9 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
 // skipping those 32 x 32 pieces with wave-uniform branches made the kernel slower.)
 template <typename T, int WA>
 __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
-    const T* __restrict__ x, uint32_t x_bytes, const T* __restrict__ g, uint32_t g_bytes, int ca, int cb,
-    int64_t tiles, int64_t tiles_per_split, float* __restrict__ partial) {
+    const T* __restrict__ x, uint32_t x_bytes, const int32_t* __restrict__ x_index, const T* __restrict__ g,
+    uint32_t g_bytes, const int32_t* __restrict__ g_index, int64_t rows, int ca, int cb, int64_t tiles,
+    int64_t tiles_per_split, float* __restrict__ partial) {
   constexpr int WB = 4 / WA;
   constexpr int GA = 2 * WA, GB = 2 * WB, NG = GA + GB;            // 64-channel groups of a tile
   constexpr int RT = 32, TILE = NG * RT * 128;                     // 40 KiB (32 KiB at WA = 2)
@@ -198,21 +249,39 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
   const int rl = lane >> 3;
   // source chunk of the lane: its LDS chunk, with the halves swapped for rows 2, 3 (mod 4)
   const uint32_t sc = (((uint32_t)(lane & 7) ^ (uint32_t)(4 * ((rl >> 1) & 1))) << 4);
-  auto stage = [&](int64_t tile, char* buf) {                      // every wave issues exactly PW loads
+  // Row r of an operand is row index[r] of its tensor when an index is given (the compact rows
+  // of the non-empty nodes read straight from a tensor over all nodes).  A lane stages row
+  // 8 wave + rl of a tile for every channel group: one index entry per operand and tile, loaded
+  // four tiles ahead (without an index the loads point out of range and cost nothing; they are
+  // issued all the same, the waits count operations).
+  const bool x_indexed = x_index != nullptr, g_indexed = g_index != nullptr;
+  const __amdgpu_buffer_rsrc_t rs_xi = make_rsrc(x_index, x_indexed ? (uint32_t)(rows * 4) : 0u);
+  const __amdgpu_buffer_rsrc_t rs_gi = make_rsrc(g_index, g_indexed ? (uint32_t)(rows * 4) : 0u);
+  struct Idx { int32_t x, g; };
+  auto load_index = [&](int64_t tile) {
+    const uint32_t row = (uint32_t)min(tile, tiles) * RT + 8 * wave + rl;
+    Idx r;
+    r.x = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_xi, row * 4u, 0, 0);
+    r.g = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_gi, row * 4u, 0, 0);
+    return r;
+  };
+  auto stage = [&](int64_t tile, char* buf, const Idx& ix) {       // every wave issues exactly PW loads
     const uint32_t row0 = (uint32_t)min(tile, tiles) * RT;        // past the range: past the rows, zeros
+    const uint32_t row = row0 + 8 * wave + rl;                    // (piece i = wave + 4 j: row group i % 4 = wave)
+    const bool live = (int64_t)row < rows;                        // an indexed row past the end must read zeros too
+    const uint32_t xrow = x_indexed ? (uint32_t)ix.x : row, grow = g_indexed ? (uint32_t)ix.g : row;
 #pragma unroll
     for (int j = 0; j < PW; ++j) {
       const int i = wave + 4 * j;
       const int grp = i >> 2, rg = i & 3;
       char* dst = buf + (grp * RT + 8 * rg) * 128;
-      const uint32_t row = row0 + 8 * rg + rl;
       // channels past the end of a row: an offset past the buffer, which reads as zeros
       if (grp < GA) {
         const uint32_t cbyte = (uint32_t)((blk_a * GA + grp) * 128) + sc;
-        dr_dma16(rs_x, dst, cbyte < xp ? row * xp + cbyte : 0xffffff00u);
+        dr_dma16(rs_x, dst, cbyte < xp && live ? xrow * xp + cbyte : 0xffffff00u);
       } else {
         const uint32_t cbyte = (uint32_t)((blk_b * GB + grp - GA) * 128) + sc;
-        dr_dma16(rs_g, dst, cbyte < gp ? row * gp + cbyte : 0xffffff00u);
+        dr_dma16(rs_g, dst, cbyte < gp && live ? grow * gp + cbyte : 0xffffff00u);
       }
     }
   };
@@ -259,18 +328,23 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
   };
 
   // ---- ring of three: tile i is multiplied while i + 1 and i + 2 are in flight ----
-  stage(t_begin, s_t0);
-  stage(t_begin + 1, s_t1);
+  Idx iq[3];                                                     // iq[t % 3]: index entries of tile t_begin + t
+  stage(t_begin, s_t0, load_index(t_begin));
+  stage(t_begin + 1, s_t1, load_index(t_begin + 1));
+  iq[2] = load_index(t_begin + 2);
+  iq[0] = load_index(t_begin + 3);
   auto step = [&](auto SLOT, int64_t tile) {
     constexpr int slot = decltype(SLOT)::value;
-    // own pieces of this tile have landed (those of the next one may be in flight), then
-    // everyone's; every wave is also done with the tile before, whose buffer is filled next
-    // (a bare barrier: __syncthreads() would wait for the next tile's loads too)
-    // (the wait as an instruction of its own, which the compiler's wait insertion takes into
-    // account: s_waitcnt vmcnt(PW) lgkmcnt(0), vmcnt in bits 3:0, lgkmcnt in bits 11:8)
-    __builtin_amdgcn_s_waitcnt(PW == 10 ? 0x007a : 0x0078);
+    // own pieces of this tile have landed (those of the next one and its two index entries may be
+    // in flight), then everyone's; every wave is also done with the tile before, whose buffer is
+    // filled next
+    // (a bare barrier: __syncthreads() would wait for the next tile's loads too; the wait as an
+    // instruction of its own, which the compiler's wait insertion takes into account:
+    // s_waitcnt vmcnt(PW + 2) lgkmcnt(0), vmcnt in bits 3:0, lgkmcnt in bits 11:8)
+    __builtin_amdgcn_s_waitcnt(0x0070 | (PW + 2));
     asm volatile("s_barrier" ::: "memory");
-    stage(tile + 2, slot == 0 ? s_t2 : slot == 1 ? s_t0 : s_t1);
+    stage(tile + 2, slot == 0 ? s_t2 : slot == 1 ? s_t0 : s_t1, iq[(slot + 2) % 3]);
+    iq[(slot + 1) % 3] = load_index(tile + 4);
     const char* buf = slot == 0 ? s_t0 : slot == 1 ? s_t1 : s_t2;
     Ops o0, o1;
     fetch(buf, 0, o0);
@@ -341,8 +415,8 @@ extern "C" int ocnn_conv_dense_rw_supported(int dtype, int64_t rows, int cin, in
 }
 
 template <typename T, int NKS, int MB>
-static void launch_dense_rw(const void* in, int64_t rows, int cout, const void* ws, const void* bias, void* out,
-                            int n_cu, hipStream_t st) {
+static void launch_dense_rw(const void* in, int64_t rows_in, const int32_t* row_index, int64_t rows, int cout,
+                            const void* ws, const void* bias, void* out, int n_cu, hipStream_t st) {
   const int lds = ((NKS / 4) >= 8 ? 2 : 4) * (NKS / 4) * 64 * 128;
   static bool attr_set = false;
   if (!attr_set) {
@@ -356,8 +430,8 @@ static void launch_dense_rw(const void* in, int64_t rows, int cout, const void* 
   const int64_t per = cdiv(tiles, wgs);
   wgs = cdiv(tiles, per);
   hipLaunchKernelGGL((conv_dense_rw_kernel<T, NKS, MB>), dim3((unsigned)wgs, (unsigned)ny), dim3(256), lds, st,
-                     (const T*)in, (uint32_t)(rows * NKS * 32), (const T*)ws, (const T*)bias, (T*)out, rows, cout,
-                     tiles, per);
+                     (const T*)in, (uint32_t)(rows_in * NKS * 32), row_index, (const T*)ws, (const T*)bias, (T*)out,
+                     rows, cout, tiles, per);
 }
 
 template <typename T>
@@ -381,8 +455,8 @@ __global__ void pack_weights_dense_kernel(const T* __restrict__ w, T* __restrict
 }
 
 template <typename T>
-static int run_dense_rw(const void* in, int64_t rows, const void* w, int cin, int cout, int w_transposed,
-                        const void* bias, void* out, void* ws, hipStream_t st) {
+static int run_dense_rw(const void* in, int64_t rows_in, const int32_t* row_index, int64_t rows, const void* w,
+                        int cin, int cout, int w_transposed, const void* bias, void* out, void* ws, hipStream_t st) {
   const int n_cu = dr_cu_count();
   if (n_cu <= 0) {
     set_error("conv_dense_rw: cannot query the device");
@@ -392,7 +466,7 @@ static int run_dense_rw(const void* in, int64_t rows, const void* w, int cin, in
                      (const T*)w, (T*)ws, cin, cout, w_transposed);
   const int mb = dr_mb(cin, cout);
 #define OCNN_DRW(CIN_, MB_) \
-  if (cin == CIN_ && mb == MB_) { launch_dense_rw<T, CIN_ / 16, MB_>(in, rows, cout, ws, bias, out, n_cu, st); return check_launch("conv_dense_rw"); }
+  if (cin == CIN_ && mb == MB_) { launch_dense_rw<T, CIN_ / 16, MB_>(in, rows_in, row_index, rows, cout, ws, bias, out, n_cu, st); return check_launch("conv_dense_rw"); }
   OCNN_DRW(512, 1) OCNN_DRW(256, 1) OCNN_DRW(256, 2) OCNN_DRW(128, 1) OCNN_DRW(128, 2) OCNN_DRW(128, 4)
   OCNN_DRW(64, 1) OCNN_DRW(64, 2) OCNN_DRW(64, 4)
 #undef OCNN_DRW
@@ -400,18 +474,29 @@ static int run_dense_rw(const void* in, int64_t rows, const void* w, int cin, in
   return OCNN_ERR_ARG;
 }
 
-extern "C" int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
-                                  int w_transposed, const void* bias, void* out, void* workspace,
-                                  int64_t workspace_bytes, void* stream) {
+extern "C" int ocnn_conv_dense_rw_indexed(int dtype, const void* in, int64_t rows_in, const int32_t* row_index,
+                                          int64_t rows, const void* w, int cin, int cout, int w_transposed,
+                                          const void* bias, void* out, void* workspace, int64_t workspace_bytes,
+                                          void* stream) {
   OCNN_REQUIRE(ocnn_conv_dense_rw_supported(dtype, rows, cin, cout), "conv_dense_rw: shape not supported");
+  OCNN_REQUIRE(row_index != nullptr || rows_in == rows, "conv_dense_rw: without an index the operand has `rows` rows");
+  OCNN_REQUIRE(rows_in >= 0 && ((int64_t)rows_in + 128) * cin * 2 <= 0xfff00000ll, "conv_dense_rw: operand too large");
   if (rows <= 0) return OCNN_OK;
   if (workspace_bytes < (int64_t)cin * cout * 2) {
     set_error("conv_dense_rw: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == OCNN_F16) return run_dense_rw<f16>(in, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
-  return run_dense_rw<bf16>(in, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+  if (dtype == OCNN_F16)
+    return run_dense_rw<f16>(in, rows_in, row_index, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+  return run_dense_rw<bf16>(in, rows_in, row_index, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+}
+
+extern "C" int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
+                                  int w_transposed, const void* bias, void* out, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+  return ocnn_conv_dense_rw_indexed(dtype, in, rows, nullptr, rows, w, cin, cout, w_transposed, bias, out, workspace,
+                                    workspace_bytes, stream);
 }
 
 // ---- weight gradient ----
@@ -447,17 +532,23 @@ extern "C" int64_t ocnn_conv_dense_wgrad_rw_workspace_bytes(int ca, int cb) {
   return align_up((int64_t)dr_wgrad_splits(ca, cb, n_cu > 0 ? n_cu : 1024) * ca * cb * 4, 256);
 }
 
+struct DrOperand {            // a (rows x channels) operand, its rows taken through an index if there is one
+  const void* data;
+  int64_t rows_total;         // rows of the tensor `data` points to (= rows without an index)
+  const int32_t* index;
+};
+
 template <typename T, int WA>
-static void launch_dense_wgrad(const void* x, const void* g, int64_t rows, int ca, int cb, int nsplit, int64_t per,
-                               int64_t tiles, float* partial, hipStream_t st) {
+static void launch_dense_wgrad(const DrOperand& x, const DrOperand& g, int64_t rows, int ca, int cb, int nsplit,
+                               int64_t per, int64_t tiles, float* partial, hipStream_t st) {
   hipLaunchKernelGGL((conv_dense_wgrad_rw_kernel<T, WA>), dim3((unsigned)nsplit, (unsigned)dr_wgrad_blocks(ca, cb, WA)),
-                     dim3(256), 0, st, (const T*)x, (uint32_t)(rows * ca * 2), (const T*)g,
-                     (uint32_t)(rows * cb * 2), ca, cb, tiles, per, partial);
+                     dim3(256), 0, st, (const T*)x.data, (uint32_t)(x.rows_total * ca * 2), x.index, (const T*)g.data,
+                     (uint32_t)(g.rows_total * cb * 2), g.index, rows, ca, cb, tiles, per, partial);
 }
 
 template <typename T>
-static int run_dense_wgrad(const void* x, const void* g, int64_t rows, int ca, int cb, int out_transposed, void* gw,
-                           void* ws, int64_t ws_bytes, hipStream_t st) {
+static int run_dense_wgrad(const DrOperand& x, const DrOperand& g, int64_t rows, int ca, int cb, int out_transposed,
+                           void* gw, void* ws, int64_t ws_bytes, hipStream_t st) {
   const int n_cu = dr_cu_count();
   if (n_cu <= 0) {
     set_error("conv_dense_wgrad_rw: cannot query the device");
@@ -482,12 +573,26 @@ static int run_dense_wgrad(const void* x, const void* g, int64_t rows, int ca, i
   return check_launch("conv_dense_wgrad_rw");
 }
 
+extern "C" int ocnn_conv_dense_wgrad_rw_indexed(int dtype, const void* x, int64_t rows_x, const int32_t* x_index,
+                                                const void* g, int64_t rows_g, const int32_t* g_index, int64_t rows,
+                                                int ca, int cb, int out_transposed, void* gw, void* workspace,
+                                                int64_t workspace_bytes, void* stream) {
+  OCNN_REQUIRE(ocnn_conv_dense_wgrad_rw_supported(dtype, rows, ca, cb), "conv_dense_wgrad_rw: shape not supported");
+  OCNN_REQUIRE((x_index != nullptr || rows_x == rows) && (g_index != nullptr || rows_g == rows),
+               "conv_dense_wgrad_rw: without an index an operand has `rows` rows");
+  OCNN_REQUIRE(rows_x >= 0 && rows_g >= 0 && ((int64_t)rows_x + 128) * ca * 2 <= 0xfff00000ll &&
+                   ((int64_t)rows_g + 128) * cb * 2 <= 0xfff00000ll,
+               "conv_dense_wgrad_rw: operand too large");
+  hipStream_t st = (hipStream_t)stream;
+  const DrOperand xo{x, rows_x, x_index}, go{g, rows_g, g_index};
+  if (dtype == OCNN_F16)
+    return run_dense_wgrad<f16>(xo, go, rows, ca, cb, out_transposed, gw, workspace, workspace_bytes, st);
+  return run_dense_wgrad<bf16>(xo, go, rows, ca, cb, out_transposed, gw, workspace, workspace_bytes, st);
+}
+
 extern "C" int ocnn_conv_dense_wgrad_rw(int dtype, const void* x, const void* g, int64_t rows, int ca, int cb,
                                         int out_transposed, void* gw, void* workspace, int64_t workspace_bytes,
                                         void* stream) {
-  OCNN_REQUIRE(ocnn_conv_dense_wgrad_rw_supported(dtype, rows, ca, cb), "conv_dense_wgrad_rw: shape not supported");
-  hipStream_t st = (hipStream_t)stream;
-  if (dtype == OCNN_F16)
-    return run_dense_wgrad<f16>(x, g, rows, ca, cb, out_transposed, gw, workspace, workspace_bytes, st);
-  return run_dense_wgrad<bf16>(x, g, rows, ca, cb, out_transposed, gw, workspace, workspace_bytes, st);
+  return ocnn_conv_dense_wgrad_rw_indexed(dtype, x, rows, nullptr, g, rows, nullptr, rows, ca, cb, out_transposed, gw,
+                                          workspace, workspace_bytes, stream);
 }

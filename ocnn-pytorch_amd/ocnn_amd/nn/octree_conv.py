@@ -22,7 +22,7 @@ from torch.autograd import Function
 from .. import _lib
 from ..utils import list2str, resize_with_last_val, xavier_uniform_
 from .octree2col import col2octree, octree2col
-from .octree_pad import octree_depad, octree_pad
+from .octree_pad import _pad_raw, octree_depad, octree_pad
 
 
 # (thresholds of the kernel selection live in the library, csrc/select.hip; these are the ones
@@ -33,11 +33,15 @@ SPARSE_MAX_OCCUPANCY = 0.3
 SPARSE_MIN_ROWS = 32768
 
 
-def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False):
+def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False,
+                in_index=None):
   """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K)).  With a
   tile plan of the same table (and a supported shape) the staged kernel runs.
-  dense: the table is the one-slot identity (row i reads row i)."""
-  out, planned = _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense)
+  dense: the table is the one-slot identity (row i reads row i).
+  in_index (int32, with dense only): row i reads row in_index[i] of `data`, which may then have
+  more rows than the table (the compact rows of the non-empty nodes, read from a tensor over
+  all nodes without a depad pass)."""
+  out, planned = _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index)
   if planned and plan is not None and plan.overflow_rows is not None:
     # the few tiles that are too dense for the plan: plan-free kernel, results put in place
     sub, _ = _conv_gather(data, rows_in, plan.overflow_table, W, cout, transposed, reverse, bias, None, False)
@@ -53,7 +57,7 @@ def _plan_args(plan):
   return 1, plan.umax, plan.total, float(plan.occupancy), float(plan.reuse)
 
 
-def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense):
+def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index=None):
   """conv_gather without the overflow rows of the plan; also returns whether a kernel on
   the plan ran.  The library picks the kernel (ocnn_conv_gather_choose)."""
   _lib.require_gpu(data, table, W)
@@ -67,6 +71,8 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
     bias = bias.to(data.dtype).contiguous()
   code = _lib.dtype_code(data)
   kernel = L.ocnn_conv_gather_choose(code, rows_in, rows, K, cin, cout, int(bool(dense)), *_plan_args(plan))
+  if in_index is not None and kernel != _lib.GATHER_DENSE_RW:
+    data, in_index = data.index_select(0, in_index.long()), None       # the other kernels take compact rows
   if kernel == _lib.GATHER_ZERO_PADDED:
     cin_p, cout_p = -(-cin // 32) * 32, -(-cout // 16) * 16
     Wk = W.view(K, cout, cin) if transposed else W.view(K, cin, cout)
@@ -77,9 +83,12 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
   out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
   ws = _lib.workspace(L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout), data.device)
   tail = (_lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream())
-  if kernel in (_lib.GATHER_DENSE_RW, _lib.GATHER_DENSE):
-    fn = L.ocnn_conv_dense_rw if kernel == _lib.GATHER_DENSE_RW else L.ocnn_conv_dense
-    _lib.check(fn(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed), *tail))
+  if kernel == _lib.GATHER_DENSE_RW:
+    _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(data), data.shape[0], _lib.ptr(in_index), rows,
+                                            _lib.ptr(W), cin, cout, int(transposed), *tail))
+    return out, False
+  if kernel == _lib.GATHER_DENSE:
+    _lib.check(L.ocnn_conv_dense(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed), *tail))
     return out, False
   if kernel in (_lib.GATHER_RW, _lib.GATHER_WIDE):
     fn = L.ocnn_conv_gather_rw if kernel == _lib.GATHER_RW else L.ocnn_conv_gather_wide
@@ -106,11 +115,13 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
   return out, False
 
 
-def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
+def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False, g_index=None):
   """gW (K, ca, cb) [or (K, cb, ca)] = sum_i x[T[i,k]]^T (x) g[i].  With a tile
   plan of the same table (and a supported shape) the staged kernel runs.
-  dense: the table is the one-slot identity (row i reads row i)."""
-  gw, planned = _conv_wgrad(x, g, table, out_transposed, plan, dense)
+  dense: the table is the one-slot identity (row i reads row i).
+  g_index (int32, with dense only): row i of the sum takes row g_index[i] of `g`, which may then
+  have more rows than the table (see conv_gather)."""
+  gw, planned = _conv_wgrad(x, g, table, out_transposed, plan, dense, g_index)
   if planned and plan is not None and plan.overflow_rows is not None:
     # the few tiles that are too dense for the plan: their share of the sums, plan-free kernel
     more, _ = _conv_wgrad(x, g.index_select(0, plan.overflow_rows), plan.overflow_table, out_transposed, None,
@@ -119,7 +130,7 @@ def conv_wgrad(x, g, table, out_transposed=False, plan=None, dense=False):
   return gw
 
 
-def _conv_wgrad(x, g, table, out_transposed, plan, dense):
+def _conv_wgrad(x, g, table, out_transposed, plan, dense, g_index=None):
   """conv_wgrad without the overflow rows of the plan; also returns whether a kernel on the
   plan ran.  The library picks the kernel (ocnn_conv_wgrad_choose)."""
   _lib.require_gpu(x, g, table)
@@ -127,9 +138,11 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense):
   x, g, table = x.contiguous(), g.contiguous(), table.contiguous()
   rows, K = table.shape
   ca, cb = x.shape[1], g.shape[1]
-  assert g.shape[0] == rows and x.dtype == g.dtype and table.dtype == torch.int32
   code = _lib.dtype_code(x)
   kernel = L.ocnn_conv_wgrad_choose(code, x.shape[0], rows, K, ca, cb, int(bool(dense)), *_plan_args(plan)[:4])
+  if g_index is not None and kernel != _lib.WGRAD_DENSE_RW:
+    g, g_index = g.index_select(0, g_index.long()), None                # the other kernels take compact rows
+  assert (g_index is not None or g.shape[0] == rows) and x.dtype == g.dtype and table.dtype == torch.int32
   if kernel == _lib.WGRAD_ZERO_PADDED:
     ca_p, cb_p = -(-ca // 32) * 32, -(-cb // 32) * 32
     gw = conv_wgrad(F.pad(x, (0, ca_p - ca)), F.pad(g, (0, cb_p - cb)), table, out_transposed, plan)
@@ -138,8 +151,9 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense):
   gw = torch.empty(shape, dtype=x.dtype, device=x.device)
   if kernel == _lib.WGRAD_DENSE_RW:
     ws = _lib.workspace(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(ca, cb), x.device)
-    _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x), _lib.ptr(g), rows, ca, cb, int(out_transposed),
-                                          _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    _lib.check(L.ocnn_conv_dense_wgrad_rw_indexed(code, _lib.ptr(x), x.shape[0], None, _lib.ptr(g), g.shape[0],
+                                                  _lib.ptr(g_index), rows, ca, cb, int(out_transposed),
+                                                  _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw, False
   if kernel == _lib.WGRAD_SPARSE:
     pp = plan.pairs()
@@ -305,16 +319,20 @@ class OctreeConvBase:
     return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias,
                        plan)
 
-  def backward_gemm(self, grad, weights, bias=None):
-    """(table rows, out_conv) -> (fine rows, in_conv)."""
+  def backward_gemm(self, grad, weights, bias=None, coarse_index=None):
+    """(table rows, out_conv) -> (fine rows, in_conv).  coarse_index (int32): `grad` holds the
+    table's rows at these rows of a larger tensor (all nodes of the depth, not only the
+    non-empty ones the table has rows for)."""
     if self.dense_children:
       # gin.view(P, 8 * in_conv) = grad @ W'^T with W' = weights.view(8 * in_conv, out_conv)
       P = self.neigh.shape[0]
       b8 = None if bias is None else bias.repeat(8)
       out = conv_gather(grad, P, self._identity(P, grad.device),
                         weights.view(1, 8 * self.in_conv, self.out_conv), 8 * self.in_conv, True,
-                        False, b8, None, dense=True)
+                        False, b8, None, dense=True, in_index=coarse_index)
       return out.view(8 * P, self.in_conv)
+    if coarse_index is not None:
+      grad = grad.index_select(0, coarse_index.long())
     if self.symmetric:
       plan = self._plan(grad, self.out_conv, self.in_conv)
       return conv_gather(grad, grad.shape[0], self.neigh, weights, self.in_conv, True, True, bias,
@@ -323,13 +341,16 @@ class OctreeConvBase:
     return conv_gather(grad, grad.shape[0], self._inverse_table(), weights, self.in_conv, True,
                        False, bias, plan)
 
-  def weight_gemm(self, data, grad, out_transposed=False):
-    """data: fine rows; grad: table rows -> (K, in_conv, out_conv)."""
+  def weight_gemm(self, data, grad, out_transposed=False, coarse_index=None):
+    """data: fine rows; grad: table rows -> (K, in_conv, out_conv).  coarse_index: as in
+    backward_gemm."""
     if self.dense_children:
       P = self.neigh.shape[0]
       gw = conv_wgrad(data.view(P, 8 * self.in_conv), grad, self._identity(P, data.device), False,
-                      None, dense=True).view(8, self.in_conv, self.out_conv)
+                      None, dense=True, g_index=coarse_index).view(8, self.in_conv, self.out_conv)
       return gw.transpose(1, 2).contiguous() if out_transposed else gw
+    if coarse_index is not None:
+      grad = grad.index_select(0, coarse_index.long())
     if self.stride == 2 and self.kernel == '222' and self.neigh.shape[0] >= SPARSE_MIN_ROWS // 8 and \
         _lib.lib().ocnn_conv_wgrad_sparse_supported(_lib.DTYPE_CODE.get(data.dtype, -1), grad.shape[0],
                                                     data.shape[0], self.kdim, grad.shape[1], data.shape[1], 0):
@@ -350,14 +371,17 @@ class _OctreeDeconv(OctreeConvBase):
 
 
 class OctreeConvFunction(Function):
-  """Autograd wiring of the convolution (ocnn/nn/octree_conv.py:219-254).  `bias` (optional,
-  last argument) is added in the epilogue of the gather-GEMM kernel instead of by a pass of
-  its own; its gradient is the fixed-order column sum of the output gradient."""
+  """Autograd wiring of the convolution (ocnn/nn/octree_conv.py:219-254).  `bias` (optional)
+  is added in the epilogue of the gather-GEMM kernel instead of by a pass of its own; its
+  gradient is the fixed-order column sum of the output gradient.  `padded` (stride 2 over all
+  nodes): the result comes back padded to all nodes of depth - 1 (what the module's octree_pad
+  does, ocnn/nn/octree_conv.py:388-389), and the backward pass reads the rows of the non-empty
+  nodes straight from the padded gradient through the octree's index of them: no depad pass."""
 
   @staticmethod
   def forward(ctx, data, weights, octree, depth: int, in_channels: int, out_channels: int,
               kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
-              max_buffer: int = int(2e8), bias=None):
+              max_buffer: int = int(2e8), bias=None, padded: bool = False):
     eng = _OctreeConv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
     eng.check_and_init(data)
@@ -366,34 +390,47 @@ class OctreeConvFunction(Function):
     out = eng.forward_gemm(data, weights, bias)
     ctx.save_for_backward(data, weights)
     ctx.eng = eng
-    return out
+    ctx.pad_depth = depth - 1 if padded else None
+    return _pad_raw(out, octree, depth - 1) if padded else out
 
   @staticmethod
   def backward(ctx, grad):
     data, weights = ctx.saved_tensors
     eng = ctx.eng
     grad = grad.contiguous()
-    grad_out = eng.backward_gemm(grad, weights) if ctx.needs_input_grad[0] else None
-    grad_w = eng.weight_gemm(data, grad) if ctx.needs_input_grad[1] else None
-    grad_b = column_sum(grad) if ctx.needs_input_grad[10] else None
-    return (grad_out, grad_w) + (None,) * 8 + (grad_b,)
+    index = None if ctx.pad_depth is None else eng.octree._nempty_index32(ctx.pad_depth)
+    grad_out = eng.backward_gemm(grad, weights, coarse_index=index) if ctx.needs_input_grad[0] else None
+    grad_w = eng.weight_gemm(data, grad, coarse_index=index) if ctx.needs_input_grad[1] else None
+    grad_b = None
+    if ctx.needs_input_grad[10]:
+      grad_b = column_sum(grad if index is None else grad.index_select(0, index.long()))
+    return (grad_out, grad_w) + (None,) * 8 + (grad_b, None)
 
 
 class OctreeDeconvFunction(Function):
-  """Autograd wiring of the deconvolution (ocnn/nn/octree_conv.py:257-292)."""
+  """Autograd wiring of the deconvolution (ocnn/nn/octree_conv.py:257-292).  `padded` (stride 2
+  over all nodes): `data` has a row for every node of `depth` and the rows of the non-empty
+  ones are read through the octree's index of them (what the module's octree_depad would copy
+  out first, ocnn/nn/octree_conv.py:450-451); the data gradient comes back padded."""
 
   @staticmethod
   def forward(ctx, data, weights, octree, depth: int, in_channels: int, out_channels: int,
               kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
-              max_buffer: int = int(2e8), bias=None):
+              max_buffer: int = int(2e8), bias=None, padded: bool = False):
     eng = _OctreeDeconv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
-    eng.check_and_init(data)
+    index = None
+    if padded:
+      assert tuple(data.shape) == (int(octree.nnum[depth]), in_channels), 'The shape of input data is wrong'
+      index = octree._nempty_index32(depth)
+    else:
+      eng.check_and_init(data)
     data = data.contiguous()
     weights = weights.to(data.dtype).contiguous()
-    out = eng.backward_gemm(data, weights, bias)
+    out = eng.backward_gemm(data, weights, bias, coarse_index=index)
     ctx.save_for_backward(data, weights)
     ctx.eng = eng
+    ctx.pad_depth = depth if padded else None
     return out
 
   @staticmethod
@@ -401,27 +438,34 @@ class OctreeDeconvFunction(Function):
     data, weights = ctx.saved_tensors
     eng = ctx.eng
     grad = grad.contiguous()
-    grad_out = eng.forward_gemm(grad, weights) if ctx.needs_input_grad[0] else None
+    index = None if ctx.pad_depth is None else eng.octree._nempty_index32(ctx.pad_depth)
+    grad_out = None
+    if ctx.needs_input_grad[0]:
+      grad_out = eng.forward_gemm(grad, weights)
+      if index is not None:
+        grad_out = _pad_raw(grad_out, eng.octree, ctx.pad_depth)
     # weights are (K, out_channels, in_channels): x = grad (fine side), g = data
-    grad_w = eng.weight_gemm(grad, data) if ctx.needs_input_grad[1] else None
+    grad_w = eng.weight_gemm(grad, data, coarse_index=index) if ctx.needs_input_grad[1] else None
     grad_b = column_sum(grad) if ctx.needs_input_grad[10] else None
-    return (grad_out, grad_w) + (None,) * 8 + (grad_b,)
+    return (grad_out, grad_w) + (None,) * 8 + (grad_b, None)
 
 
 def octree_conv(data, weights, octree, depth: int, in_channels: int, out_channels: int,
                 kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
-                max_buffer: int = int(2e8), bias=None):
-  """Functional form (ocnn/nn/octree_conv.py:296), with an optional bias that the kernel adds."""
+                max_buffer: int = int(2e8), bias=None, padded: bool = False):
+  """Functional form (ocnn/nn/octree_conv.py:296), with an optional bias that the kernel adds
+  and, for stride 2 over all nodes, the octree_pad of the result folded in (`padded`)."""
   return OctreeConvFunction.apply(data, weights, octree, depth, in_channels, out_channels, kernel_size, stride,
-                                  nempty, max_buffer, bias)
+                                  nempty, max_buffer, bias, padded)
 
 
 def octree_deconv(data, weights, octree, depth: int, in_channels: int, out_channels: int,
                   kernel_size: List[int] = [3, 3, 3], stride: int = 1, nempty: bool = False,
-                  max_buffer: int = int(2e8), bias=None):
-  """Functional form (ocnn/nn/octree_conv.py:297), with an optional bias that the kernel adds."""
+                  max_buffer: int = int(2e8), bias=None, padded: bool = False):
+  """Functional form (ocnn/nn/octree_conv.py:297), with an optional bias that the kernel adds
+  and, for stride 2 over all nodes, the octree_depad of the input folded in (`padded`)."""
   return OctreeDeconvFunction.apply(data, weights, octree, depth, in_channels, out_channels, kernel_size, stride,
-                                    nempty, max_buffer, bias)
+                                    nempty, max_buffer, bias, padded)
 
 
 class OctreeConv(OctreeConvBase, torch.nn.Module):
@@ -460,15 +504,18 @@ class OctreeConv(OctreeConvBase, torch.nn.Module):
   def is_conv_layer(self): return True
 
   def forward(self, data: torch.Tensor, octree, depth: int):
+    pad = self.stride == 2 and not self.nempty
     if self.method == 'explicit_gemm':
       out = self.explicit_gemm(data, octree, depth)
     else:
-      out = octree_conv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
-                        self.kernel_size, self.stride, self.nempty, self.max_buffer,
-                        self.bias if self.use_bias else None)              # bias: in the kernel's epilogue
-    if self.use_bias and self.method == 'explicit_gemm':
+      # bias: in the kernel's epilogue; the pad: inside the function, whose backward pass then
+      # needs no depad
+      return octree_conv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
+                         self.kernel_size, self.stride, self.nempty, self.max_buffer,
+                         self.bias if self.use_bias else None, pad)
+    if self.use_bias:
       out = out + self.bias.to(out.dtype)
-    if self.stride == 2 and not self.nempty:
+    if pad:
       out = octree_pad(out, octree, depth - 1)
     return out
 
@@ -486,7 +533,13 @@ class OctreeDeconv(OctreeConv):
   def is_conv_layer(self): return False
 
   def forward(self, data: torch.Tensor, octree, depth: int):
-    if self.stride == 2 and not self.nempty:
+    depad = self.stride == 2 and not self.nempty
+    if self.method != 'explicit_gemm':
+      # the depad: inside the function, which reads the rows of the non-empty nodes through an index
+      return octree_deconv(data, self.weights, octree, depth, self.in_channels, self.out_channels,
+                           self.kernel_size, self.stride, self.nempty, self.max_buffer,
+                           self.bias if self.use_bias else None, depad)
+    if depad:
       data = octree_depad(data, octree, depth)
     if self.method == 'explicit_gemm':
       # one product for all slots, then the adjoint of im2col (ocnn/nn/octree_conv.py:453-457)

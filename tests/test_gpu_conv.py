@@ -548,6 +548,56 @@ def test_dense_rows_kernel(dtype, cin, cout):
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('cin,cout', [(128, 512), (512, 128), (64, 128), (256, 256), (96, 64)])
+def test_dense_rows_register_kernels_indexed(dtype, cin, cout):
+  """The same kernels with the rows of an operand taken through an index (the rows of the
+  non-empty nodes read out of a tensor over all nodes): bit-identical to the kernels run on the
+  rows copied out first, for ragged row counts, fewer tiles than the rings hold, an index that
+  is the identity and one with gaps, and guard rows around the output."""
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(5 * cin + cout)
+  code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+  for rows, total in ((1, 9), (130, 130), (4133, 9000), (64 * 300 + 5, 64 * 800)):
+    say('dense rows rw indexed', dtype, cin, cout, rows, total)
+    index = torch.sort(torch.randperm(total, generator=g)[:rows]).values.to(torch.int32)
+    x_all = torch.randn(total, cin, generator=g).to(dtype).to(DEV)
+    g_all = torch.randn(total, cout, generator=g).to(dtype).to(DEV)
+    x_own = torch.randn(rows, cin, generator=g).to(dtype).to(DEV)
+    idx = index.to(DEV)
+    x_sel, g_sel = x_all.index_select(0, idx.long()), g_all.index_select(0, idx.long())
+    if L.ocnn_conv_dense_rw_supported(code, rows, cin, cout):
+      w = (torch.randn(cin, cout, generator=g) / cin ** 0.5).to(dtype).to(DEV)
+      b = torch.randn(cout, generator=g).to(dtype).to(DEV)
+      ws = torch.empty(cin * cout * 2, dtype=torch.uint8, device=DEV)
+      want = torch.empty((rows, cout), dtype=dtype, device=DEV)
+      _lib.check(L.ocnn_conv_dense_rw(code, _lib.ptr(x_sel), rows, _lib.ptr(w), cin, cout, 0, _lib.ptr(b),
+                                      _lib.ptr(want), _lib.ptr(ws), ws.numel(), _lib.stream()))
+      out = torch.full((rows + 1, cout), 7.0, dtype=dtype, device=DEV)
+      _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(x_all), total, _lib.ptr(idx), rows, _lib.ptr(w), cin,
+                                              cout, 0, _lib.ptr(b), _lib.ptr(out), _lib.ptr(ws), ws.numel(),
+                                              _lib.stream()))
+      assert torch.equal(out[:rows], want) and bool((out[rows] == 7.0).all())
+      assert rel_err(out[:rows], f64(x_sel) @ f64(w) + f64(b)) < TOL[dtype]
+    ws = torch.empty(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(cin, cout), dtype=torch.uint8, device=DEV)
+    want = torch.empty((cin, cout), dtype=dtype, device=DEV)
+    _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x_own), _lib.ptr(g_sel), rows, cin, cout, 0,
+                                          _lib.ptr(want), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    gw = torch.empty((cin, cout), dtype=dtype, device=DEV)
+    _lib.check(L.ocnn_conv_dense_wgrad_rw_indexed(code, _lib.ptr(x_own), rows, None, _lib.ptr(g_all), total,
+                                                  _lib.ptr(idx), rows, cin, cout, 0, _lib.ptr(gw), _lib.ptr(ws),
+                                                  ws.numel(), _lib.stream()))
+    assert torch.equal(gw, want)
+    assert rel_err(gw, f64(x_own).T @ f64(g_sel)) < TOL[dtype]
+    # both operands through the index
+    _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x_sel), _lib.ptr(g_sel), rows, cin, cout, 0,
+                                          _lib.ptr(want), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    _lib.check(L.ocnn_conv_dense_wgrad_rw_indexed(code, _lib.ptr(x_all), total, _lib.ptr(idx), _lib.ptr(g_all), total,
+                                                  _lib.ptr(idx), rows, cin, cout, 0, _lib.ptr(gw), _lib.ptr(ws),
+                                                  ws.numel(), _lib.stream()))
+    assert torch.equal(gw, want)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('cin,cout', [(64, 128), (64, 512), (128, 128), (128, 256), (128, 512), (256, 128), (256, 256),
                                       (512, 128), (512, 384), (1024, 128), (128, 1024), (96, 64), (768, 96),
                                       (64, 16), (128, 96), (384, 256), (72, 40), (256, 32), (8, 8)])
