@@ -29,7 +29,7 @@ constexpr int kDpCap = 416;    // staged rows; plans with a larger tile use anot
 constexpr int kDpRowsAlloc = (kDpCap + 8) / 8 * 8;
 constexpr int kDpThreads = 512;   // eight waves a workgroup, two a SIMD: one computes while the other waits
 constexpr int kDpWaves = kDpThreads / 64;
-constexpr int kDpListAlloc = 448;   // entries of a list array in LDS (read in whole pieces of 32)
+constexpr int kDpListAlloc = 448;   // entries of a list array in LDS (read in whole pieces of 8 rows a wave)
 
 // (Not in the kernel templates: the arguments of the global->LDS load builtin must not be
 // type-dependent expressions.)
