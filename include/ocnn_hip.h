@@ -209,6 +209,18 @@ int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile_nnz, int64
                            int32_t* uptr, int64_t* stats, void* stream);
 int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
                         int32_t* urows, uint16_t* loc, void* stream);
+/* The same plan with ONE pass over the table instead of two: ocnn_tile_plan_build counts
+ * (as ocnn_tile_plan_count) and writes the positions and, at the fixed place
+ * ulist[tile * pad + u], the lists of the tiles with at most `pad` distinct rows;
+ * ocnn_tile_plan_offsets as above; ocnn_tile_plan_compact moves the lists to their offsets
+ * and clears the positions of the tiles the offsets dropped (stats: the device vector that
+ * ocnn_tile_plan_offsets wrote; cap <= pad).  A plan whose largest count (stats[3]) exceeds
+ * `pad` is filled with ocnn_tile_plan_fill instead. */
+int ocnn_tile_plan_build(const int32_t* table, int64_t rows, int K, int pad, int32_t* ucount,
+                         int32_t* tile_nnz, int32_t* ulist, uint16_t* loc, void* stream);
+int ocnn_tile_plan_compact(const int32_t* ucount, const int32_t* uptr, const int64_t* stats, int cap,
+                           int pad, const int32_t* ulist, int32_t* urows, uint16_t* loc, int K,
+                           int64_t tiles, void* stream);
 
 /* ---- kernel selection ----------------------------------------------------
  * Which entry point runs a gather-GEMM (forward_gemm / backward_gemm in gather form,

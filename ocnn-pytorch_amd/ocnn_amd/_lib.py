@@ -47,6 +47,8 @@ SIGNATURES = {
     'ocnn_tile_plan_count': (_i, [_p, _l, _i, _p, _p, _p]),
     'ocnn_tile_plan_offsets': (_i, [_p, _p, _l, _i, _p, _p, _p]),
     'ocnn_tile_plan_fill': (_i, [_p, _l, _i, _p, _p, _p, _p]),
+    'ocnn_tile_plan_build': (_i, [_p, _l, _i, _i, _p, _p, _p, _p, _p]),
+    'ocnn_tile_plan_compact': (_i, [_p, _p, _p, _i, _i, _p, _p, _p, _i, _l, _p]),
     'ocnn_conv_gather_planned_supported': (_i, [_i, _l, _i, _i]),
     'ocnn_conv_gather_planned': (_i, [_i, _p, _l, _p, _p, _p, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                       _p, _l, _p]),

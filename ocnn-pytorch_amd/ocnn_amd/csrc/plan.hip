@@ -11,100 +11,107 @@ namespace ocnn {
 
 constexpr int kPlanRows = 128;          // table rows per tile
 constexpr int kPlanMaxEntries = 4096;   // >= kPlanRows * 27, power of two
-constexpr int kPlanHash = 8192;         // open-addressing slots (load <= 42 %)
+constexpr int kPlanHash = 4096;         // open-addressing slots (an octree table fills a tenth; at most 84 %)
 constexpr int kPlanRankMax = 1024;      // up to here the distinct rows are ordered by counting
+constexpr int kPlanThreads = 512;       // threads a tile: the kernel waits on LDS round trips, more waves hide them
 
 __device__ __forceinline__ int plan_hash(int32_t v) {
-  return (int)(((uint32_t)v * 2654435761u) >> 19);      // 13 bits
+  return (int)(((uint32_t)v * 2654435761u) >> 20);      // 12 bits
 }
 
 // mode 0: ucount[tile] = number of distinct valid entries, tile_nnz[tile] = valid entries
 // mode 1: urows[uptr[tile] + u] = u-th distinct row; loc[tile][k][row in tile] = u + 1, or
 //         0 for an empty entry (also for the rows of the last tile that lie past the table)
+// mode 2: both in one pass over the table: counts as mode 0, positions as mode 1, and the
+//         list at the fixed place urows[tile * pad + u] (only when it has at most `pad`
+//         rows); tile_plan_compact_kernel moves the lists to their offsets afterwards
 //
 // The distinct rows are found with a hash set in LDS (a tile of an octree table has a few
 // hundred distinct rows among its 3456 entries), ordered by counting (no barriers) or, for
 // tables without locality, by a bitonic sort; positions come back out of the hash set.
-__global__ __launch_bounds__(256) void tile_plan_kernel(
+__global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     const int32_t* __restrict__ table, int64_t rows, int K, int mode,
     int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, int32_t* __restrict__ urows,
-    uint16_t* __restrict__ loc, int32_t* __restrict__ tile_nnz) {
+    uint16_t* __restrict__ loc, int32_t* __restrict__ tile_nnz, int pad) {
   __shared__ int32_t s_key[kPlanHash];
   __shared__ int32_t s_nnz;
   __shared__ uint16_t s_val[kPlanHash];
-  __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];
-  __shared__ int32_t s_scan[256];
-  __shared__ int32_t s_tab[kPlanRows * 27];
+  __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];   // later: the positions, [slot][row]
+  __shared__ int32_t s_scan[kPlanThreads];
   const int tid = threadIdx.x;
   const int64_t tile = blockIdx.x;
   const int64_t e0 = tile * kPlanRows * K;
   const int64_t lim = rows * (int64_t)K;
   const int n = kPlanRows * K;
-  // the tile's entries -> LDS: all loads in flight at once, then used twice
-  constexpr int kPer = (kPlanRows * 27 + 255) / 256;      // entries per thread, at most
+  // the tile's entries: all loads in flight at once; a thread keeps its entries and the hash
+  // slots it finds them in
+  constexpr int kPer = (kPlanRows * 27 + kPlanThreads - 1) / kPlanThreads;      // entries per thread, at most
   int32_t ent[kPer];
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    const int e = tid + 256 * i;
+    const int e = tid + kPlanThreads * i;
     ent[i] = (e < n && e0 + e < lim) ? table[e0 + e] : -1;
   }
-  for (int i = tid; i < kPlanHash; i += 256) s_key[i] = -1;
+  for (int i = tid; i < kPlanHash; i += kPlanThreads) s_key[i] = -1;
   if (tid == 0) s_nnz = 0;
-#pragma unroll
-  for (int i = 0; i < kPer; ++i)
-    if (tid + 256 * i < n) s_tab[tid + 256 * i] = ent[i];
   __syncthreads();
-  if (mode == 0 && tile_nnz != nullptr) {
+  if (mode != 1 && tile_nnz != nullptr) {
     int set = 0;
 #pragma unroll
     for (int i = 0; i < kPer; ++i) set += ent[i] >= 0 ? 1 : 0;
     atomicAdd(&s_nnz, set);
   }
+  int slot[kPer];
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
     const int32_t v = ent[i];
+    slot[i] = -1;
     if (v >= 0) {
+      // a row is read by a dozen entries of the tile: look before the atomic, most find it there
       int h = plan_hash(v);
       while (true) {
-        const int32_t old = atomicCAS(&s_key[h], -1, v);
+        int32_t old = ((volatile int32_t*)s_key)[h];
+        if (old == -1) old = atomicCAS(&s_key[h], -1, v);
         if (old == -1 || old == v) break;
         h = (h + 1) & (kPlanHash - 1);
       }
+      slot[i] = h;
     }
   }
   __syncthreads();
-  // occupied slots: per-thread counts (slots tid, tid + 256, ..: the order of the distinct
+  // occupied slots: per-thread counts (slots tid, tid + kPlanThreads, ..: the order of the distinct
   // rows does not matter before they are ranked), block scan
-  constexpr int per = kPlanHash / 256;
+  constexpr int per = kPlanHash / kPlanThreads;
   int32_t held[per];
   int cnt = 0;
 #pragma unroll
   for (int i = 0; i < per; ++i) {
-    held[i] = s_key[tid + 256 * i];
+    held[i] = s_key[tid + kPlanThreads * i];
     cnt += held[i] >= 0 ? 1 : 0;
   }
   s_scan[tid] = cnt;
   __syncthreads();
-  for (int off = 1; off < 256; off <<= 1) {
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
     int v = tid >= off ? s_scan[tid - off] : 0;
     __syncthreads();
     s_scan[tid] += v;
     __syncthreads();
   }
-  const int total = s_scan[255];
-  if (mode == 0) {
+  const int total = s_scan[kPlanThreads - 1];
+  if (mode != 1) {
     if (tid == 0) {
       ucount[tile] = total;
       if (tile_nnz != nullptr) tile_nnz[tile] = s_nnz;
     }
-    return;
+    if (mode == 0) return;
   }
+  const bool keep_list = mode == 1 || total <= pad;
   int pos = s_scan[tid] - cnt;
 #pragma unroll
   for (int i = 0; i < per; ++i)
     if (held[i] >= 0) s_uq[pos++] = held[i];
   __syncthreads();
-  const int32_t ub = uptr[tile];
+  const int64_t ub = mode == 1 ? (int64_t)uptr[tile] : tile * (int64_t)pad;
   auto slot_of = [&](int32_t v) {
     int h = plan_hash(v);
     while (s_key[h] != v) h = (h + 1) & (kPlanHash - 1);
@@ -113,10 +120,10 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
   if (total <= kPlanRankMax) {
     // rank of a value = number of smaller distinct values
     const int tpad = (total + 15) & ~15;                  // whole groups of 16; the padding ranks last
-    for (int e = total + tid; e < tpad; e += 256) s_uq[e] = 0x7fffffff;
+    for (int e = total + tid; e < tpad; e += kPlanThreads) s_uq[e] = 0x7fffffff;
     __syncthreads();
     typedef __attribute__((ext_vector_type(4))) int i32x4;
-    for (int j = tid; j < total; j += 256) {
+    for (int j = tid; j < total; j += kPlanThreads) {
       const int32_t v = s_uq[j];
       int r = 0;
       for (int i = 0; i < tpad; i += 16) {                // 4 x 16-byte broadcast reads in flight
@@ -128,16 +135,16 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
           r += (q[u][0] < v ? 1 : 0) + (q[u][1] < v ? 1 : 0) + (q[u][2] < v ? 1 : 0) + (q[u][3] < v ? 1 : 0);
       }
       s_val[slot_of(v)] = (uint16_t)(r + 1);
-      urows[ub + r] = v;
+      if (keep_list) urows[ub + r] = v;
     }
   } else {
     int npad = kPlanRankMax * 2;
     while (npad < total) npad <<= 1;
-    for (int e = total + tid; e < npad; e += 256) s_uq[e] = 0x7fffffff;
+    for (int e = total + tid; e < npad; e += kPlanThreads) s_uq[e] = 0x7fffffff;
     __syncthreads();
     for (int k = 2; k <= npad; k <<= 1) {          // bitonic sort, ascending
       for (int j = k >> 1; j > 0; j >>= 1) {
-        for (int t = tid; t < (npad >> 1); t += 256) {
+        for (int t = tid; t < (npad >> 1); t += kPlanThreads) {
           int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
           int p = i | j;
           int32_t a = s_uq[i], b = s_uq[p];
@@ -147,43 +154,31 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(
         __syncthreads();
       }
     }
-    for (int j = tid; j < total; j += 256) {
+    for (int j = tid; j < total; j += kPlanThreads) {
       const int32_t v = s_uq[j];
       s_val[slot_of(v)] = (uint16_t)(j + 1);
-      urows[ub + j] = v;
+      if (keep_list) urows[ub + j] = v;
     }
   }
   __syncthreads();
-  // positions, written in the order they are stored ([slot][row]: coalesced); the first
-  // probes of all entries of a thread are in flight together
-  int32_t vv[kPer], kk[kPer];
-  int hh[kPer];
-#pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    const int o = tid + 256 * i;
-    vv[i] = o < n ? s_tab[(o % kPlanRows) * K + o / kPlanRows] : -1;
-  }
-#pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    hh[i] = plan_hash(vv[i] < 0 ? 0 : vv[i]);
-    kk[i] = s_key[hh[i]];
-  }
-#pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    if (vv[i] >= 0)
-      while (kk[i] != vv[i]) {
-        hh[i] = (hh[i] + 1) & (kPlanHash - 1);
-        kk[i] = s_key[hh[i]];
-      }
-  }
+  // positions: every entry knows its slot of the hash set; through LDS into the order they are
+  // stored in ([slot][row]), then out in 16-byte pieces
+  uint16_t* s_pos = (uint16_t*)s_uq;                      // (the list of distinct rows is done with)
   uint16_t pp[kPer];
 #pragma unroll
-  for (int i = 0; i < kPer; ++i) pp[i] = s_val[hh[i]];
+  for (int i = 0; i < kPer; ++i) pp[i] = slot[i] >= 0 ? s_val[slot[i]] : (uint16_t)0;
+  __syncthreads();
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    const int o = tid + 256 * i;
-    if (o < n) loc[e0 + o] = vv[i] >= 0 ? pp[i] : (uint16_t)0;
+    const int e = tid + kPlanThreads * i;
+    if (e < n) {
+      const int row = e / K, k = e - row * K;
+      s_pos[k * kPlanRows + row] = pp[i];
+    }
   }
+  __syncthreads();
+  u32x4* dst = (u32x4*)(loc + e0);
+  for (int i = tid; i < K * (kPlanRows / 8); i += kPlanThreads) dst[i] = ((const u32x4*)s_pos)[i];
 }
 
 // Pair plan of a table, on top of its tile plan: per tile and LIST the rows that have a
@@ -227,19 +222,26 @@ __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles
 __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     const int32_t* __restrict__ ucount, const int32_t* __restrict__ tile_nnz, int64_t tiles, int cap,
     int32_t* __restrict__ uptr, int64_t* __restrict__ stats) {
-  __shared__ long long s_sum[1024];
-  __shared__ int s_big, s_max;
-  __shared__ long long s_nnz;
-  const int tid = threadIdx.x;
+  __shared__ long long s_wsum[16], s_wnnz[16];
+  __shared__ int s_wbig[16], s_wmax[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t per = (tiles + 1023) / 1024;
   const int64_t t0 = min(tiles, tid * per), t1 = min(tiles, t0 + per);
-  if (tid == 0) { s_big = 0; s_max = 0; s_nnz = 0; }
-  __syncthreads();
+  // sums over a wave with lane exchanges, one LDS slot per wave: 1024 threads adding to one LDS
+  // word take longer than everything else here
+  auto wave_sum = [&](long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+  };
   int big = 0;
   for (int64_t t = t0; t < t1; ++t) big += ucount[t] > cap ? 1 : 0;
-  if (big) atomicAdd(&s_big, big);
+  big = (int)wave_sum(big);
+  if (lane == 0) s_wbig[wave] = big;
   __syncthreads();
-  const int n_big = s_big;
+  int n_big = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) n_big += s_wbig[w];
   const bool drop = n_big > 0 && n_big <= max((int64_t)1, tiles / 10);
   long long sum = 0, nnz = 0;
   int mx = 0;
@@ -250,30 +252,65 @@ __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     mx = max(mx, c);
     nnz += tile_nnz[t];
   }
-  s_sum[tid] = sum;
-  atomicMax(&s_max, mx);
-  atomicAdd((unsigned long long*)&s_nnz, (unsigned long long)nnz);
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    const long long v = tid >= off ? s_sum[tid - off] : 0;
-    __syncthreads();
-    s_sum[tid] += v;
-    __syncthreads();
+  // inclusive scan of `sum` over the wave, then over the 16 waves
+  long long incl = sum;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const long long v = __shfl_up(incl, o);
+    if (lane >= o) incl += v;
   }
-  long long at = s_sum[tid] - sum;
+  const long long wnnz = wave_sum(nnz);
+  int wmx = mx;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) wmx = max(wmx, __shfl_xor(wmx, o));
+  if (lane == 63) s_wsum[wave] = incl;
+  if (lane == 0) { s_wnnz[wave] = wnnz; s_wmax[wave] = wmx; }
+  __syncthreads();
+  long long before = 0, total = 0, nnz_all = 0;
+  int max_all = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    if (w < wave) before += s_wsum[w];
+    total += s_wsum[w];
+    nnz_all += s_wnnz[w];
+    max_all = max(max_all, s_wmax[w]);
+  }
+  long long at = before + incl - sum;
   for (int64_t t = t0; t < t1; ++t) {
     uptr[t] = (int32_t)at;
     const int c = ucount[t];
     at += (drop && c > cap) ? 0 : c;
   }
   if (tid == 1023) {
-    uptr[tiles] = (int32_t)s_sum[1023];
+    uptr[tiles] = (int32_t)total;
     stats[0] = n_big;
     stats[1] = drop ? 1 : 0;
-    stats[2] = s_sum[1023];
-    stats[3] = s_max;
-    stats[4] = s_nnz;
+    stats[2] = total;
+    stats[3] = max_all;
+    stats[4] = nnz_all;
   }
+}
+
+// After a one-pass build (mode 2 above): a wave per tile moves the tile's list from its fixed
+// place to its offset; a tile that the offsets dropped (more than `cap` distinct rows, few such
+// tiles) becomes empty: its positions are cleared.
+__global__ __launch_bounds__(256) void tile_plan_compact_kernel(
+    const int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, const int64_t* __restrict__ stats,
+    int cap, int pad, const int32_t* __restrict__ ulist, int32_t* __restrict__ urows, uint16_t* __restrict__ loc,
+    int K, int64_t tiles) {
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= tiles) return;
+  const int U = ucount[tile];
+  if (stats[1] != 0 && U > cap) {
+    u32x4* p = (u32x4*)(loc + tile * (int64_t)(K * kPlanRows));
+    for (int i = lane; i < K * (kPlanRows / 8); i += 64) p[i] = u32x4{0u, 0u, 0u, 0u};
+    return;
+  }
+  if (U > pad) return;                                    // (the caller fills such a plan in two passes)
+  const int32_t* src = ulist + tile * (int64_t)pad;
+  int32_t* dst = urows + uptr[tile];
+  for (int i = lane; i < U; i += 64) dst[i] = src[i];
 }
 
 __global__ void pair_plan_zero_kernel(unsigned long long* __restrict__ slot_count, int K) {
@@ -311,18 +348,36 @@ using namespace ocnn;
 extern "C" int ocnn_tile_plan_rows(void) { return kPlanRows; }
 
 static int plan_launch(const int32_t* table, int64_t rows, int K, int mode, int32_t* ucount,
-                       const int32_t* uptr, int32_t* urows, uint16_t* loc, int32_t* tile_nnz, void* stream) {
+                       const int32_t* uptr, int32_t* urows, uint16_t* loc, int32_t* tile_nnz, int pad,
+                       void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows >= 0 && rows < (1ll << 31), "tile_plan: bad shape");
   if (rows == 0) return OCNN_OK;
   int64_t tiles = cdiv(rows, kPlanRows);
-  hipLaunchKernelGGL(tile_plan_kernel, dim3((unsigned)tiles), dim3(256), 0, (hipStream_t)stream,
-                     table, rows, K, mode, ucount, uptr, urows, loc, tile_nnz);
+  hipLaunchKernelGGL(tile_plan_kernel, dim3((unsigned)tiles), dim3(kPlanThreads), 0, (hipStream_t)stream,
+                     table, rows, K, mode, ucount, uptr, urows, loc, tile_nnz, pad);
   return check_launch("tile_plan");
+}
+
+extern "C" int ocnn_tile_plan_build(const int32_t* table, int64_t rows, int K, int pad, int32_t* ucount,
+                                    int32_t* tile_nnz, int32_t* ulist, uint16_t* loc, void* stream) {
+  OCNN_REQUIRE(pad >= 1 && pad <= 4096, "tile_plan_build: bad list size");
+  return plan_launch(table, rows, K, 2, ucount, nullptr, ulist, loc, tile_nnz, pad, stream);
+}
+
+extern "C" int ocnn_tile_plan_compact(const int32_t* ucount, const int32_t* uptr, const int64_t* stats, int cap,
+                                      int pad, const int32_t* ulist, int32_t* urows, uint16_t* loc, int K,
+                                      int64_t tiles, void* stream) {
+  OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 31) && cap >= 0 && cap <= pad,
+               "tile_plan_compact: bad shape");
+  if (tiles == 0) return OCNN_OK;
+  hipLaunchKernelGGL(tile_plan_compact_kernel, dim3((unsigned)cdiv(tiles, 4)), dim3(256), 0, (hipStream_t)stream,
+                     ucount, uptr, stats, cap, pad, ulist, urows, loc, K, tiles);
+  return check_launch("tile_plan_compact");
 }
 
 extern "C" int ocnn_tile_plan_count(const int32_t* table, int64_t rows, int K, int32_t* ucount,
                                     int32_t* tile_nnz, void* stream) {
-  return plan_launch(table, rows, K, 0, ucount, nullptr, nullptr, nullptr, tile_nnz, stream);
+  return plan_launch(table, rows, K, 0, ucount, nullptr, nullptr, nullptr, tile_nnz, 0, stream);
 }
 
 extern "C" int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile_nnz, int64_t tiles, int cap,
@@ -335,7 +390,7 @@ extern "C" int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile
 
 extern "C" int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t* uptr,
                                    int32_t* urows, uint16_t* loc, void* stream) {
-  return plan_launch(table, rows, K, 1, nullptr, uptr, urows, loc, nullptr, stream);
+  return plan_launch(table, rows, K, 1, nullptr, uptr, urows, loc, nullptr, 0, stream);
 }
 
 extern "C" int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,

@@ -120,6 +120,7 @@ class TilePlan:
   before it and leaves the device idle while the host catches up."""
 
   CAP = 415      # the smallest limit of the kernels on the plan
+  LIST_PAD = 416  # rows a tile's list may have in the one-pass build
 
   def __init__(self, table: torch.Tensor, cap: int = None):
     self._count(table, cap)
@@ -156,7 +157,18 @@ class TilePlan:
     tile_nnz = torch.empty(tiles, dtype=torch.int32, device=dev)
     self.uptr = torch.empty(tiles + 1, dtype=torch.int32, device=dev)
     self._stats = torch.empty(5, dtype=torch.int64, device=dev)
-    _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(self._ucount), _lib.ptr(tile_nnz), st))
+    # One pass over the table: counts, positions and the lists at fixed places (LIST_PAD rows a
+    # tile); the second half only moves the lists to their offsets.  (A limit above LIST_PAD, or
+    # a table whose tiles do not fit it, takes the two passes of count and fill.)
+    self._lists = None
+    if self._cap <= self.LIST_PAD:
+      self._lists = torch.empty(max(tiles, 1) * self.LIST_PAD, dtype=torch.int32, device=dev)
+      # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"
+      self.loc = torch.empty((tiles, K, self._tile_rows), dtype=torch.int16, device=dev)
+      _lib.check(L.ocnn_tile_plan_build(_lib.ptr(table), rows, K, self.LIST_PAD, _lib.ptr(self._ucount),
+                                        _lib.ptr(tile_nnz), _lib.ptr(self._lists), _lib.ptr(self.loc), st))
+    else:
+      _lib.check(L.ocnn_tile_plan_count(_lib.ptr(table), rows, K, _lib.ptr(self._ucount), _lib.ptr(tile_nnz), st))
     _lib.check(L.ocnn_tile_plan_offsets(_lib.ptr(self._ucount), _lib.ptr(tile_nnz), tiles, self._cap,
                                         _lib.ptr(self.uptr), _lib.ptr(self._stats), st))
 
@@ -168,23 +180,30 @@ class TilePlan:
     tiles = self._ucount.numel()
     dev = table.device
     _, dropped, total, umax, nnz = stats
+    one_pass = self._lists is not None and umax <= self.LIST_PAD
     if dropped:
       big = self._ucount > self._cap
       idx = (big.nonzero().view(-1, 1) * tile_rows + torch.arange(tile_rows, device=dev).view(1, -1)).view(-1)
       idx = idx[idx < rows]
       self.overflow_rows = idx
       self.overflow_table = table.index_select(0, idx).contiguous()
-      table = table.clone()
-      table[idx] = -1
+      if not one_pass:
+        table = table.clone()
+        table[idx] = -1
     # how often a staged row is used by its tile: near 1 there is nothing to gain from staging
     self.reuse = nnz / max(total, 1)
     self.urows = torch.empty(max(total, 1), dtype=torch.int32, device=dev)
-    # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"
-    self.loc = torch.empty((tiles, K, tile_rows), dtype=torch.int16, device=dev)
-    _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(self.uptr),
-                                     _lib.ptr(self.urows), _lib.ptr(self.loc), _lib.stream()))
+    if one_pass:
+      _lib.check(L.ocnn_tile_plan_compact(_lib.ptr(self._ucount), _lib.ptr(self.uptr), _lib.ptr(self._stats),
+                                          self._cap, self.LIST_PAD, _lib.ptr(self._lists), _lib.ptr(self.urows),
+                                          _lib.ptr(self.loc), K, tiles, _lib.stream()))
+    else:
+      # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"
+      self.loc = torch.empty((tiles, K, tile_rows), dtype=torch.int16, device=dev)
+      _lib.check(L.ocnn_tile_plan_fill(_lib.ptr(table), rows, K, _lib.ptr(self.uptr),
+                                       _lib.ptr(self.urows), _lib.ptr(self.loc), _lib.stream()))
     self.total, self.umax, self.nnz = total, umax, nnz
-    self._table = self._ucount = self._stats = None
+    self._table = self._ucount = self._stats = self._lists = None
 
   @property
   def occupancy(self):
