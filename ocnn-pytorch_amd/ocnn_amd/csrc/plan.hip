@@ -26,25 +26,30 @@ __device__ __forceinline__ int plan_hash(int32_t v) {
 //         list at the fixed place urows[tile * pad + u] (only when it has at most `pad`
 //         rows); tile_plan_compact_kernel moves the lists to their offsets afterwards
 //
-// The distinct rows are found with a hash set in LDS (a tile of an octree table has a few
-// hundred distinct rows among its 3456 entries), ordered by counting (no barriers) or, for
-// tables without locality, by a bitonic sort; positions come back out of the hash set.
+// The distinct rows of a tile (a few hundred among its 3456 entries in an octree table) come
+// in runs of consecutive row numbers, so the set is kept by BLOCKS of 32 row numbers: a hash
+// set of block numbers in LDS, each with a 32-bit mask of the rows present.  Ordering the rows
+// then means ordering the blocks (a tenth as many: by counting, no barriers; tables without
+// locality: by a bitonic sort) and counting bits: the position of a row is the number of rows
+// in smaller blocks plus the bits below its own in its block's mask.
 __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     const int32_t* __restrict__ table, int64_t rows, int K, int mode,
     int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, int32_t* __restrict__ urows,
     uint16_t* __restrict__ loc, int32_t* __restrict__ tile_nnz, int pad) {
-  __shared__ int32_t s_key[kPlanHash];
+  __shared__ int32_t s_key[kPlanHash];                    // block number, -1 = free
+  __shared__ uint32_t s_mask[kPlanHash];                  // its rows
+  __shared__ uint16_t s_base[kPlanHash];                  // rows in smaller blocks
+  __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];   // the blocks; later: the positions, [slot][row]
+  __shared__ __attribute__((aligned(16))) int32_t s_w[kPlanMaxEntries];    // rows of each of them
+  __shared__ int32_t s_scan[2][kPlanThreads / 64];
   __shared__ int32_t s_nnz;
-  __shared__ uint16_t s_val[kPlanHash];
-  __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];   // later: the positions, [slot][row]
-  __shared__ int32_t s_scan[kPlanThreads];
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t tile = blockIdx.x;
   const int64_t e0 = tile * kPlanRows * K;
   const int64_t lim = rows * (int64_t)K;
   const int n = kPlanRows * K;
   // the tile's entries: all loads in flight at once; a thread keeps its entries and the hash
-  // slots it finds them in
+  // slots of their blocks
   constexpr int kPer = (kPlanRows * 27 + kPlanThreads - 1) / kPlanThreads;      // entries per thread, at most
   int32_t ent[kPer];
 #pragma unroll
@@ -52,14 +57,19 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     const int e = tid + kPlanThreads * i;
     ent[i] = (e < n && e0 + e < lim) ? table[e0 + e] : -1;
   }
-  for (int i = tid; i < kPlanHash; i += kPlanThreads) s_key[i] = -1;
+  for (int i = tid; i < kPlanHash; i += kPlanThreads) {
+    s_key[i] = -1;
+    s_mask[i] = 0u;
+  }
   if (tid == 0) s_nnz = 0;
   __syncthreads();
   if (mode != 1 && tile_nnz != nullptr) {
     int set = 0;
 #pragma unroll
     for (int i = 0; i < kPer; ++i) set += ent[i] >= 0 ? 1 : 0;
-    atomicAdd(&s_nnz, set);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) set += __shfl_xor(set, o);
+    if (lane == 0) atomicAdd(&s_nnz, set);
   }
   int slot[kPer];
 #pragma unroll
@@ -67,37 +77,55 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     const int32_t v = ent[i];
     slot[i] = -1;
     if (v >= 0) {
-      // a row is read by a dozen entries of the tile: look before the atomic, most find it there
-      int h = plan_hash(v);
+      // a block is met by dozens of entries of the tile: look before the atomics, most find
+      // block and bit in place
+      const int32_t blk = v >> 5;
+      const uint32_t bit = 1u << (v & 31);
+      int h = plan_hash(blk);
       while (true) {
         int32_t old = ((volatile int32_t*)s_key)[h];
-        if (old == -1) old = atomicCAS(&s_key[h], -1, v);
-        if (old == -1 || old == v) break;
+        if (old == -1) old = atomicCAS(&s_key[h], -1, blk);
+        if (old == -1 || old == blk) break;
         h = (h + 1) & (kPlanHash - 1);
       }
+      if ((((volatile uint32_t*)s_mask)[h] & bit) == 0u) atomicOr(&s_mask[h], bit);
       slot[i] = h;
     }
   }
   __syncthreads();
-  // occupied slots: per-thread counts (slots tid, tid + kPlanThreads, ..: the order of the distinct
-  // rows does not matter before they are ranked), block scan
+  // occupied slots: per-thread counts of blocks and rows (slots tid, tid + kPlanThreads, ..: the
+  // order of the blocks does not matter before they are ranked), scanned within a wave by lane
+  // exchanges, across the waves through LDS
   constexpr int per = kPlanHash / kPlanThreads;
   int32_t held[per];
-  int cnt = 0;
+  uint32_t hmask[per];
+  int cnt = 0, nrows = 0;
 #pragma unroll
   for (int i = 0; i < per; ++i) {
     held[i] = s_key[tid + kPlanThreads * i];
+    hmask[i] = s_mask[tid + kPlanThreads * i];
     cnt += held[i] >= 0 ? 1 : 0;
+    nrows += __popc(hmask[i]);
   }
-  s_scan[tid] = cnt;
+  int incl = cnt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(incl, o);
+    if (lane >= o) incl += v;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) nrows += __shfl_xor(nrows, o);
+  if (lane == 63) s_scan[0][wave] = incl;
+  if (lane == 0) s_scan[1][wave] = nrows;
   __syncthreads();
-  for (int off = 1; off < kPlanThreads; off <<= 1) {
-    int v = tid >= off ? s_scan[tid - off] : 0;
-    __syncthreads();
-    s_scan[tid] += v;
-    __syncthreads();
+  int before = 0, nblk = 0, total = 0;                    // blocks in the waves before, blocks, distinct rows
+#pragma unroll
+  for (int w = 0; w < kPlanThreads / 64; ++w) {
+    const int v = s_scan[0][w];
+    if (w < wave) before += v;
+    nblk += v;
+    total += s_scan[1][w];
   }
-  const int total = s_scan[kPlanThreads - 1];
   if (mode != 1) {
     if (tid == 0) {
       ucount[tile] = total;
@@ -106,41 +134,63 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     if (mode == 0) return;
   }
   const bool keep_list = mode == 1 || total <= pad;
-  int pos = s_scan[tid] - cnt;
+  int pos = before + incl - cnt;
 #pragma unroll
   for (int i = 0; i < per; ++i)
-    if (held[i] >= 0) s_uq[pos++] = held[i];
+    if (held[i] >= 0) {
+      s_uq[pos] = held[i];
+      s_w[pos] = __popc(hmask[i]);
+      ++pos;
+    }
   __syncthreads();
   const int64_t ub = mode == 1 ? (int64_t)uptr[tile] : tile * (int64_t)pad;
-  auto slot_of = [&](int32_t v) {
-    int h = plan_hash(v);
-    while (s_key[h] != v) h = (h + 1) & (kPlanHash - 1);
+  auto slot_of = [&](int32_t blk) {
+    int h = plan_hash(blk);
+    while (s_key[h] != blk) h = (h + 1) & (kPlanHash - 1);
     return h;
   };
-  if (total <= kPlanRankMax) {
-    // rank of a value = number of smaller distinct values
-    const int tpad = (total + 15) & ~15;                  // whole groups of 16; the padding ranks last
-    for (int e = total + tid; e < tpad; e += kPlanThreads) s_uq[e] = 0x7fffffff;
+  // a block's rows go to the list from `base` on, in the order of their bits
+  auto put_block = [&](int32_t blk, int h, int base) {
+    s_base[h] = (uint16_t)base;
+    if (keep_list) {
+      uint32_t m = s_mask[h];
+      int32_t* dst = urows + ub + base;
+      while (m != 0u) {
+        *dst++ = blk * 32 + (__ffs(m) - 1);
+        m &= m - 1u;
+      }
+    }
+  };
+  if (nblk <= kPlanRankMax) {
+    // rows before a block = rows of the smaller blocks
+    const int tpad = (nblk + 15) & ~15;                   // whole groups of 16; the padding ranks last and weighs nothing
+    for (int e = nblk + tid; e < tpad; e += kPlanThreads) {
+      s_uq[e] = 0x7fffffff;
+      s_w[e] = 0;
+    }
     __syncthreads();
     typedef __attribute__((ext_vector_type(4))) int i32x4;
-    for (int j = tid; j < total; j += kPlanThreads) {
+    for (int j = tid; j < nblk; j += kPlanThreads) {
       const int32_t v = s_uq[j];
       int r = 0;
-      for (int i = 0; i < tpad; i += 16) {                // 4 x 16-byte broadcast reads in flight
-        i32x4 q[4];
+      for (int i = 0; i < tpad; i += 16) {                // 8 x 16-byte broadcast reads in flight
+        i32x4 q[4], w[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) q[u] = *(const i32x4*)(&s_uq[i + 4 * u]);
+        for (int u = 0; u < 4; ++u) {
+          q[u] = *(const i32x4*)(&s_uq[i + 4 * u]);
+          w[u] = *(const i32x4*)(&s_w[i + 4 * u]);
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-          r += (q[u][0] < v ? 1 : 0) + (q[u][1] < v ? 1 : 0) + (q[u][2] < v ? 1 : 0) + (q[u][3] < v ? 1 : 0);
+          r += (q[u][0] < v ? w[u][0] : 0) + (q[u][1] < v ? w[u][1] : 0) + (q[u][2] < v ? w[u][2] : 0) +
+               (q[u][3] < v ? w[u][3] : 0);
       }
-      s_val[slot_of(v)] = (uint16_t)(r + 1);
-      if (keep_list) urows[ub + r] = v;
+      put_block(v, slot_of(v), r);
     }
   } else {
     int npad = kPlanRankMax * 2;
-    while (npad < total) npad <<= 1;
-    for (int e = total + tid; e < npad; e += kPlanThreads) s_uq[e] = 0x7fffffff;
+    while (npad < nblk) npad <<= 1;
+    for (int e = nblk + tid; e < npad; e += kPlanThreads) s_uq[e] = 0x7fffffff;
     __syncthreads();
     for (int k = 2; k <= npad; k <<= 1) {          // bitonic sort, ascending
       for (int j = k >> 1; j > 0; j >>= 1) {
@@ -154,31 +204,66 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
         __syncthreads();
       }
     }
-    for (int j = tid; j < total; j += kPlanThreads) {
-      const int32_t v = s_uq[j];
-      s_val[slot_of(v)] = (uint16_t)(j + 1);
-      if (keep_list) urows[ub + j] = v;
+    // rows before each block of the sorted list: a thread takes 8 consecutive blocks, their row
+    // counts are scanned like the block counts above
+    constexpr int kSeq = kPlanMaxEntries / kPlanThreads;
+    int hs[kSeq], ws[kSeq], sum = 0;
+#pragma unroll
+    for (int i = 0; i < kSeq; ++i) {
+      const int j = tid * kSeq + i;
+      hs[i] = j < nblk ? slot_of(s_uq[j]) : -1;
+      ws[i] = hs[i] >= 0 ? __popc(s_mask[hs[i]]) : 0;
+      sum += ws[i];
+    }
+    int inc2 = sum;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int v = __shfl_up(inc2, o);
+      if (lane >= o) inc2 += v;
+    }
+    __syncthreads();                                      // (s_scan is read above by every thread)
+    if (lane == 63) s_scan[0][wave] = inc2;
+    __syncthreads();
+    int base = inc2 - sum;
+#pragma unroll
+    for (int w = 0; w < kPlanThreads / 64; ++w)
+      if (w < wave) base += s_scan[0][w];
+#pragma unroll
+    for (int i = 0; i < kSeq; ++i) {
+      if (hs[i] >= 0) put_block(s_uq[tid * kSeq + i], hs[i], base);
+      base += ws[i];
     }
   }
   __syncthreads();
-  // positions: every entry knows its slot of the hash set; through LDS into the order they are
+  // positions: every entry knows the slot of its block; through LDS into the order they are
   // stored in ([slot][row]), then out in 16-byte pieces
-  uint16_t* s_pos = (uint16_t*)s_uq;                      // (the list of distinct rows is done with)
+  uint16_t* s_pos = (uint16_t*)s_uq;                      // (the list of blocks is done with)
   uint16_t pp[kPer];
 #pragma unroll
-  for (int i = 0; i < kPer; ++i) pp[i] = slot[i] >= 0 ? s_val[slot[i]] : (uint16_t)0;
+  for (int i = 0; i < kPer; ++i) {
+    pp[i] = 0;
+    if (slot[i] >= 0) {
+      const uint32_t below = (1u << (ent[i] & 31)) - 1u;
+      pp[i] = (uint16_t)(s_base[slot[i]] + __popc(s_mask[slot[i]] & below) + 1);
+    }
+  }
   __syncthreads();
+  // (e / K by a multiplication: exact for e < 4096 and K <= 27; a slot's positions 136 apart in
+  // LDS, so that the entries of a row, which neighbouring lanes hold, fall on different banks)
+  constexpr int kPitch = kPlanRows + 8;
+  const uint32_t inv_k = ((1u << 20) + (uint32_t)K - 1u) / (uint32_t)K;
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
     const int e = tid + kPlanThreads * i;
     if (e < n) {
-      const int row = e / K, k = e - row * K;
-      s_pos[k * kPlanRows + row] = pp[i];
+      const int row = (int)(((uint32_t)e * inv_k) >> 20), k = e - row * K;
+      s_pos[k * kPitch + row] = pp[i];
     }
   }
   __syncthreads();
   u32x4* dst = (u32x4*)(loc + e0);
-  for (int i = tid; i < K * (kPlanRows / 8); i += kPlanThreads) dst[i] = ((const u32x4*)s_pos)[i];
+  for (int i = tid; i < K * (kPlanRows / 8); i += kPlanThreads)
+    dst[i] = *(const u32x4*)(s_pos + (i >> 4) * kPitch + (i & 15) * 8);
 }
 
 // Pair plan of a table, on top of its tile plan: per tile and LIST the rows that have a
