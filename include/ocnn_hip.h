@@ -87,6 +87,14 @@ int ocnn_sort_unique(const int64_t* key, int64_t n, int key_bits,
  *        [n_parent] = parent key with the batch id moved back to bit 48 when
  *        batched != 0. */
 int64_t ocnn_build_level_workspace_bytes(int64_t n);
+/* The node counts of every sparse level at once (the reference learns them one
+ * level at a time from torch.unique, octree.py:244), so that a build reads
+ * sizes back once: sizes[0] += number of leaf keys (*n_unique, at most n_max),
+ * sizes[l] += distinct (key >> 3 l, batch id) for l = 1 .. levels.  sizes
+ * [levels + 1] must hold zeros on entry. */
+int ocnn_build_level_sizes(const int64_t* node_key, int64_t n_max,
+                           const int64_t* n_unique, int levels, int64_t* sizes,
+                           void* stream);
 int ocnn_build_level_count(const int64_t* node_key, int64_t n, void* workspace,
                            int64_t workspace_bytes, int32_t* pidx,
                            int64_t* n_parent, void* stream);
@@ -94,6 +102,43 @@ int ocnn_build_level_fill(const int64_t* node_key, const int32_t* pidx,
                           int64_t n, int64_t n_parent, int batched,
                           int64_t* keys, int32_t* children, int64_t* next_key,
                           void* stream);
+
+/* The whole of ocnn/octree/octree.py:227-270 above the point keys in two
+ * calls with one read-back between them (the reference and the level_count /
+ * level_fill pair read one count back per level).
+ * scan: sorts the n keys (batch id packed above the 3 * depth Morton bits;
+ *       batch_bits = bits of the largest batch id), perm[n] = the stable
+ *       sorting order, and numbers the nodes of every layer in one scan.
+ *       sizes (device, depth - full_depth + 1 values): sizes[0] = leaves,
+ *       sizes[l] = non-empty nodes l layers above them.
+ * fill: h_sizes = sizes read back (host).  h_keys / h_children: host arrays of
+ *       depth + 1 device pointers, layer d holding batch_size * 8^d nodes for
+ *       d <= full_depth and 8 * h_sizes[depth - d + 1] below.  Writes every
+ *       layer's keys and children, inverse[n] (point -> leaf, the reference's
+ *       idx) and seg_start[sizes[0] + 1] (leaf -> its run in perm).  Same
+ *       workspace as given to scan, untouched in between. */
+int64_t ocnn_octree_build_workspace_bytes(int64_t n, int depth, int full_depth,
+                                          int batch_bits);
+int ocnn_octree_build_scan(const int64_t* key, int64_t n, int depth,
+                           int full_depth, int batch_bits, void* workspace,
+                           int64_t workspace_bytes, int32_t* perm,
+                           int64_t* sizes, void* stream);
+int ocnn_octree_build_fill(const void* workspace, int64_t n, int depth,
+                           int full_depth, int batch_size, int batch_bits,
+                           const int64_t* h_sizes, const int32_t* perm,
+                           int64_t* const* h_keys, int32_t* const* h_children,
+                           int64_t* inverse, int32_t* seg_start, void* stream);
+
+/* A full layer (ocnn/octree/octree.py:289-321): keys[i] = (i mod 8^depth) |
+ * (i div 8^depth) << 48 for the batch_size * 8^depth nodes; children[i] = i
+ * when with_children != 0, else -1 (the deepest full layer, whose children
+ * build_full_layer_children sets: children[key position of node_key[j]] = j,
+ * octree.py:262-268). */
+int ocnn_build_full_layer(int depth, int batch_size, int with_children,
+                          int64_t* keys, int32_t* children, void* stream);
+int ocnn_build_full_layer_children(const int64_t* node_key, int64_t n,
+                                   int depth, int batch_size,
+                                   int32_t* children, void* stream);
 
 /* Regrowing an octree from split decisions, ocnn/octree/octree.py:323-351 (octree_split) and
  * :353-402 (octree_grow).

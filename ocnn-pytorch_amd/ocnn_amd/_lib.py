@@ -25,6 +25,12 @@ SIGNATURES = {
     'ocnn_sort_unique_workspace_bytes': (_l, [_l]),
     'ocnn_sort_unique': (_i, [_p, _l, _i, _i, _p, _l, _p, _p, _p, _p, _p, _p, _p]),
     'ocnn_build_level_workspace_bytes': (_l, [_l]),
+    'ocnn_octree_build_workspace_bytes': (_l, [_l, _i, _i, _i]),
+    'ocnn_octree_build_scan': (_i, [_p, _l, _i, _i, _i, _p, _l, _p, _p, _p]),
+    'ocnn_octree_build_fill': (_i, [_p, _l, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p]),
+    'ocnn_build_level_sizes': (_i, [_p, _l, _p, _i, _p, _p]),
+    'ocnn_build_full_layer': (_i, [_i, _i, _i, _p, _p, _p]),
+    'ocnn_build_full_layer_children': (_i, [_p, _l, _i, _i, _p, _p]),
     'ocnn_build_level_count': (_i, [_p, _l, _p, _l, _p, _p, _p]),
     'ocnn_build_level_fill': (_i, [_p, _p, _l, _l, _i, _p, _p, _p, _p]),
     'ocnn_split_children': (_i, [_p, _l, _p, _l, _p, _p, _p]),

@@ -60,6 +60,34 @@ __global__ void level_count_finish_kernel(const int32_t* uid, int64_t n, int32_t
   if (i == n - 1) *n_parent = (int64_t)u;
 }
 
+// Node counts of ALL the sparse layers from the sorted leaf keys in one pass, so that the host
+// reads sizes back once for the whole build: sizes[0] = leaves, sizes[l] = distinct nodes l
+// layers up.  Two neighbouring keys part ways l layers up iff their highest differing bit is at
+// least 3 l (any bit of the batch index, bits 48 and up: at every layer).
+__global__ void level_sizes_kernel(const int64_t* __restrict__ node_key, const int64_t* __restrict__ n_ptr,
+                                   int levels, unsigned long long* __restrict__ sizes) {
+  __shared__ unsigned int s_hist[32];
+  const int64_t n = *n_ptr;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (threadIdx.x < 32) s_hist[threadIdx.x] = 0u;
+  __syncthreads();
+  if (i < n) {
+    int lv = levels;                                        // the first key starts a node at every layer
+    if (i > 0) {
+      const unsigned long long x = (unsigned long long)(node_key[i] ^ node_key[i - 1]);
+      const int hb = 63 - __clzll((long long)x);
+      lv = hb >= 48 ? levels : min(levels, hb / 3);
+    }
+    atomicAdd(&s_hist[lv], 1u);
+  }
+  __syncthreads();
+  if ((int)threadIdx.x <= levels) {
+    unsigned int c = 0;
+    for (int v = threadIdx.x; v <= levels; ++v) c += s_hist[v];
+    if (c != 0u) atomicAdd(&sizes[threadIdx.x], (unsigned long long)c);
+  }
+}
+
 __global__ void level_fill_parent_kernel(const int64_t* node_key, const int32_t* pidx, int64_t n,
                                          int batched, int64_t* keys, int32_t* children,
                                          int64_t* next_key) {
@@ -143,6 +171,209 @@ __global__ void grow_layer_kernel(const int64_t* key_above, const int32_t* nempt
   keys[i] = (k - low) | (low << 3) | (i & 7);
   children[i] = (int32_t)i;
 }
+
+// ---- the whole tree above the sorted point keys in one scan and one scatter ---------------
+// A sorted point starts a new node l layers above the leaves (l = 0: a new leaf) iff its key
+// differs from its predecessor's in a bit at or above 3 l, or in the batch id.  Counting those
+// starts for all layers together numbers the nodes of every layer in one scan over the points.
+constexpr int kBuildMaxDepth = 16;
+
+template <int N>
+struct LevelCount {
+  uint32_t v[N];
+};
+
+template <int N>
+struct LevelCountPlus {
+  __host__ __device__ LevelCount<N> operator()(const LevelCount<N>& a, const LevelCount<N>& b) const {
+    LevelCount<N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = a.v[i] + b.v[i];
+    return r;
+  }
+};
+
+// number of layers at which sorted point i starts a node, minus one (-1: same leaf as i - 1)
+template <typename K>
+__host__ __device__ inline int start_level(const K* sorted, int64_t i, int key_bits, int levels) {
+  if (i == 0) return levels;
+  const K x = sorted[i] ^ sorted[i - 1];
+  if (x == 0) return -1;
+  const int hb = 63 - __builtin_clzll((unsigned long long)x);
+  if (hb >= key_bits) return levels;
+  const int l = hb / 3;
+  return l < levels ? l : levels;
+}
+
+template <typename K, int N>
+struct LevelFlags {
+  const K* sorted;
+  int key_bits, levels;
+  __host__ __device__ LevelCount<N> operator()(int64_t i) const {
+    const int lv = start_level(sorted, i, key_bits, levels);
+    LevelCount<N> r;
+#pragma unroll
+    for (int l = 0; l < N; ++l) r.v[l] = l <= lv ? 1u : 0u;
+    return r;
+  }
+};
+
+template <typename K>
+__global__ void build_prep_kernel(const int64_t* __restrict__ key, int64_t n, int key_bits, K* __restrict__ ckey,
+                                  int32_t* __restrict__ iota) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint64_t k = (uint64_t)key[i];
+  ckey[i] = (K)(((k >> 48) << key_bits) | (k & ((1ull << key_bits) - 1)));
+  iota[i] = (int32_t)i;
+}
+
+template <int N>
+__global__ void build_sizes_kernel(const LevelCount<N>* __restrict__ scan, int64_t n, int levels,
+                                   int64_t* __restrict__ sizes) {
+  const int l = threadIdx.x;
+  if (l <= levels) sizes[l] = (int64_t)scan[n - 1].v[l];
+}
+
+struct BuildTree {
+  int64_t* keys[kBuildMaxDepth + 1];
+  int32_t* children[kBuildMaxDepth + 1];
+  int64_t begin[kBuildMaxDepth + 2];   // running total of the node counts, by depth
+};
+
+// full layers, and -1 in the children of every other layer
+__global__ void build_init_kernel(BuildTree t, int depth, int full_depth) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= t.begin[depth + 1]) return;
+  int d = 0;
+  while (i >= t.begin[d + 1]) ++d;
+  const int64_t j = i - t.begin[d];
+  if (d <= full_depth) {
+    t.keys[d][j] = (j & ((1ll << (3 * d)) - 1)) | ((j >> (3 * d)) << 48);
+    t.children[d][j] = d < full_depth ? (int32_t)j : -1;
+  } else {
+    t.children[d][j] = -1;
+  }
+}
+
+template <typename K, int N>
+__global__ void build_scatter_kernel(const K* __restrict__ sorted, const LevelCount<N>* __restrict__ scan,
+                                     const int32_t* __restrict__ perm, int64_t n, int key_bits, int depth,
+                                     int full_depth, BuildTree t, int64_t* __restrict__ inverse,
+                                     int32_t* __restrict__ seg_start) {
+  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= n) return;
+  const int levels = depth - full_depth;
+  const LevelCount<N> s = scan[q];
+  const int32_t leaf = (int32_t)s.v[0] - 1;
+  inverse[perm[q]] = leaf;
+  if (q == n - 1) seg_start[leaf + 1] = (int32_t)n;
+  const int lv = start_level(sorted, q, key_bits, levels);
+  if (lv < 0) return;
+  seg_start[leaf] = (int32_t)q;
+  const uint64_t c = (uint64_t)sorted[q];
+  const int64_t b = (int64_t)(c >> key_bits);
+  const int64_t m = (int64_t)(c & ((1ull << key_bits) - 1));
+#pragma unroll
+  for (int l = 0; l < N - 1; ++l) {
+    if (l < levels && l <= lv) {
+      const int d = depth - l;
+      const int64_t kl = m >> (3 * l);
+      const int64_t p = (int64_t)s.v[l + 1] - 1;
+      t.children[d][(p << 3) | (kl & 7)] = (int32_t)s.v[l] - 1;
+      if (l + 1 <= lv) {
+        const int64_t base = (b << 48) | ((kl >> 3) << 3);
+        int64_t* dst = t.keys[d] + (p << 3);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = base + j;
+      }
+    }
+  }
+  if (lv >= levels) {
+    const int64_t at = (b << (3 * full_depth)) | (m >> (3 * levels));
+    if (at < t.begin[full_depth + 1] - t.begin[full_depth])      // a batch id beyond batch_size has no node
+      t.children[full_depth][at] = (int32_t)s.v[levels] - 1;
+  }
+}
+
+using ForceOnesweep = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                                 rocprim::default_config, 0>;
+
+struct BuildLayout {
+  int64_t ckey, csorted, iota, scan, temp, temp_bytes, total;
+};
+
+template <typename K, int N>
+static int build_layout_t(int64_t n, BuildLayout* L) {
+  size_t sort_bytes = 0, scan_bytes = 0;
+  hipError_t e = rocprim::radix_sort_pairs<ForceOnesweep>(nullptr, sort_bytes, (K*)nullptr, (K*)nullptr,
+                                                          (int32_t*)nullptr, (int32_t*)nullptr, (size_t)n, 0,
+                                                          8 * sizeof(K));
+  if (e != hipSuccess) return OCNN_ERR_HIP;
+  auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<int64_t>(0),
+                                             LevelFlags<K, N>{nullptr, 0, 0});
+  e = rocprim::inclusive_scan(nullptr, scan_bytes, in, (LevelCount<N>*)nullptr, (size_t)n, LevelCountPlus<N>());
+  if (e != hipSuccess) return OCNN_ERR_HIP;
+  int64_t off = 0;
+  L->ckey = off;    off += align_up(n * (int64_t)sizeof(K), 256);
+  L->csorted = off; off += align_up(n * (int64_t)sizeof(K), 256);
+  L->iota = off;    off += align_up(n * 4, 256);
+  L->scan = off;    off += align_up(n * (int64_t)sizeof(LevelCount<N>), 256);
+  L->temp = off;
+  L->temp_bytes = align_up((int64_t)(sort_bytes > scan_bytes ? sort_bytes : scan_bytes) + 256, 256);
+  L->total = off + L->temp_bytes;
+  return OCNN_OK;
+}
+
+template <typename K, int N>
+static int build_scan_t(const int64_t* key, int64_t n, int key_bits, int batch_bits, int levels, char* ws,
+                        int64_t ws_bytes, int32_t* perm, int64_t* sizes, hipStream_t st) {
+  BuildLayout L;
+  if (build_layout_t<K, N>(n, &L) != OCNN_OK) { set_error("octree_build_scan: rocprim size query failed"); return OCNN_ERR_HIP; }
+  if (ws_bytes < L.total) { set_error("octree_build_scan: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
+  K* ckey = (K*)(ws + L.ckey);
+  K* csorted = (K*)(ws + L.csorted);
+  int32_t* iota = (int32_t*)(ws + L.iota);
+  LevelCount<N>* scan = (LevelCount<N>*)(ws + L.scan);
+  dim3 grid((unsigned)cdiv(n, 256)), block(256);
+  hipLaunchKernelGGL(build_prep_kernel<K>, grid, block, 0, st, key, n, key_bits, ckey, iota);
+  size_t tb = (size_t)L.temp_bytes;
+  hipError_t e = rocprim::radix_sort_pairs<ForceOnesweep>(ws + L.temp, tb, ckey, csorted, iota, perm, (size_t)n, 0u,
+                                                          (unsigned)(key_bits + batch_bits), st);
+  if (e != hipSuccess) { set_error("octree_build_scan: radix sort: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
+  auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<int64_t>(0),
+                                             LevelFlags<K, N>{csorted, key_bits, levels});
+  tb = (size_t)L.temp_bytes;
+  e = rocprim::inclusive_scan(ws + L.temp, tb, in, scan, (size_t)n, LevelCountPlus<N>(), st);
+  if (e != hipSuccess) { set_error("octree_build_scan: scan: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
+  hipLaunchKernelGGL(build_sizes_kernel<N>, dim3(1), dim3(64), 0, st, scan, n, levels, sizes);
+  return check_launch("octree_build_scan");
+}
+
+template <typename K, int N>
+static int build_fill_t(const char* ws, int64_t n, int key_bits, int depth, int full_depth, const BuildTree& t,
+                        const int32_t* perm, int64_t* inverse, int32_t* seg_start, hipStream_t st) {
+  BuildLayout L;
+  if (build_layout_t<K, N>(n, &L) != OCNN_OK) { set_error("octree_build_fill: rocprim size query failed"); return OCNN_ERR_HIP; }
+  const K* csorted = (const K*)(ws + L.csorted);
+  const LevelCount<N>* scan = (const LevelCount<N>*)(ws + L.scan);
+  hipLaunchKernelGGL(build_init_kernel, dim3((unsigned)cdiv(t.begin[depth + 1], 256)), dim3(256), 0, st, t, depth,
+                     full_depth);
+  hipLaunchKernelGGL((build_scatter_kernel<K, N>), dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, csorted, scan, perm,
+                     n, key_bits, depth, full_depth, t, inverse, seg_start);
+  return check_launch("octree_build_fill");
+}
+
+// key type and counter count of a build: 32-bit sort keys when batch id and Morton bits fit
+#define OCNN_BUILD_DISPATCH(CALL)                                   \
+  do {                                                               \
+    const bool narrow = key_bits + batch_bits <= 32;                 \
+    if (levels + 1 <= 8) {                                           \
+      if (narrow) return CALL(uint32_t, 8); else return CALL(uint64_t, 8);   \
+    } else {                                                         \
+      if (narrow) return CALL(uint32_t, 16); else return CALL(uint64_t, 16); \
+    }                                                                \
+  } while (0)
 
 struct SortLayout {
   int64_t ckey, csorted, iota, flag, uid, temp, temp_bytes, total;
@@ -238,6 +469,57 @@ extern "C" int64_t ocnn_build_level_workspace_bytes(int64_t n) {
   return L.total;
 }
 
+// A full layer: every node of every octree of the batch exists, in key order.
+__global__ void full_layer_kernel(int depth, int64_t total, int32_t child_fill, int64_t* __restrict__ keys,
+                                  int32_t* __restrict__ children) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t b = i >> (3 * depth);
+  keys[i] = (i & ((1ll << (3 * depth)) - 1)) | (b << 48);
+  children[i] = child_fill < 0 ? child_fill : (int32_t)i;
+}
+
+// children of the deepest full layer: node j of the layer below's parents sits at its key.
+__global__ void full_layer_children_kernel(const int64_t* __restrict__ node_key, int64_t n, int depth,
+                                           int64_t total, int32_t* __restrict__ children) {
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= n) return;
+  const int64_t k = node_key[j];
+  const int64_t at = ((k >> 48) << (3 * depth)) | (k & ((1ll << 48) - 1));
+  if (at >= 0 && at < total) children[at] = (int32_t)j;
+}
+
+extern "C" int ocnn_build_full_layer(int depth, int batch_size, int with_children, int64_t* keys,
+                                     int32_t* children, void* stream) {
+  OCNN_REQUIRE(depth >= 0 && depth <= 8 && batch_size >= 1 && ((int64_t)batch_size << (3 * depth)) < (1ll << 31),
+               "build_full_layer: depth=%d batch_size=%d out of range", depth, batch_size);
+  const int64_t total = (int64_t)batch_size << (3 * depth);
+  hipLaunchKernelGGL(full_layer_kernel, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, (hipStream_t)stream, depth,
+                     total, with_children ? 0 : -1, keys, children);
+  return check_launch("build_full_layer");
+}
+
+extern "C" int ocnn_build_full_layer_children(const int64_t* node_key, int64_t n, int depth, int batch_size,
+                                              int32_t* children, void* stream) {
+  OCNN_REQUIRE(depth >= 0 && depth <= 8 && batch_size >= 1 && n >= 0 && n < (1ll << 31),
+               "build_full_layer_children: depth=%d batch_size=%d n=%lld out of range", depth, batch_size,
+               (long long)n);
+  if (n == 0) return 0;
+  const int64_t total = (int64_t)batch_size << (3 * depth);
+  hipLaunchKernelGGL(full_layer_children_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream,
+                     node_key, n, depth, total, children);
+  return check_launch("build_full_layer_children");
+}
+
+extern "C" int ocnn_build_level_sizes(const int64_t* node_key, int64_t n_max, const int64_t* n_unique, int levels,
+                                      int64_t* sizes, void* stream) {
+  OCNN_REQUIRE(n_max > 0 && n_max < (1ll << 28) && levels >= 0 && levels <= 16,
+               "build_level_sizes: n_max=%lld levels=%d out of range", (long long)n_max, levels);
+  hipLaunchKernelGGL(level_sizes_kernel, dim3((unsigned)cdiv(n_max, 256)), dim3(256), 0, (hipStream_t)stream,
+                     node_key, n_unique, levels, (unsigned long long*)sizes);
+  return check_launch("build_level_sizes");
+}
+
 extern "C" int ocnn_build_level_count(const int64_t* node_key, int64_t n, void* workspace,
                                       int64_t workspace_bytes, int32_t* pidx, int64_t* n_parent,
                                       void* stream) {
@@ -315,4 +597,61 @@ extern "C" int ocnn_leaf_average(const float* src, int channels, const int32_t* 
                        channels, perm, seg_start, n_leaf, out);
   }
   return check_launch("leaf_average");
+}
+
+// ---- fused build ---------------------------------------------------------------------------
+static int build_args_ok(int64_t n, int depth, int full_depth, int batch_bits) {
+  OCNN_REQUIRE(n > 0 && n < (1ll << 31), "octree_build: n=%lld out of range", (long long)n);
+  OCNN_REQUIRE(depth >= 1 && depth <= kBuildMaxDepth && full_depth >= 0 && full_depth <= depth && full_depth <= 8,
+               "octree_build: depth=%d full_depth=%d out of range", depth, full_depth);
+  OCNN_REQUIRE(batch_bits >= 0 && batch_bits <= 15, "octree_build: batch_bits=%d out of range", batch_bits);
+  return OCNN_OK;
+}
+
+extern "C" int64_t ocnn_octree_build_workspace_bytes(int64_t n, int depth, int full_depth, int batch_bits) {
+  if (n <= 0 || depth < 1 || depth > kBuildMaxDepth || full_depth < 0 || full_depth > depth) return -1;
+  const int key_bits = 3 * depth, levels = depth - full_depth;
+  BuildLayout L;
+#define OCNN_BUILD_BYTES(K, N) (build_layout_t<K, N>(n, &L) == OCNN_OK ? L.total : (int64_t)-1)
+  OCNN_BUILD_DISPATCH(OCNN_BUILD_BYTES);
+#undef OCNN_BUILD_BYTES
+}
+
+extern "C" int ocnn_octree_build_scan(const int64_t* key, int64_t n, int depth, int full_depth, int batch_bits,
+                                      void* workspace, int64_t workspace_bytes, int32_t* perm, int64_t* sizes,
+                                      void* stream) {
+  if (int rc = build_args_ok(n, depth, full_depth, batch_bits)) return rc;
+  const int key_bits = 3 * depth, levels = depth - full_depth;
+#define OCNN_BUILD_SCAN(K, N) \
+  build_scan_t<K, N>(key, n, key_bits, batch_bits, levels, (char*)workspace, workspace_bytes, perm, sizes, (hipStream_t)stream)
+  OCNN_BUILD_DISPATCH(OCNN_BUILD_SCAN);
+#undef OCNN_BUILD_SCAN
+}
+
+extern "C" int ocnn_octree_build_fill(const void* workspace, int64_t n, int depth, int full_depth, int batch_size,
+                                      int batch_bits, const int64_t* h_sizes, const int32_t* perm,
+                                      int64_t* const* h_keys, int32_t* const* h_children, int64_t* inverse,
+                                      int32_t* seg_start, void* stream) {
+  if (int rc = build_args_ok(n, depth, full_depth, batch_bits)) return rc;
+  OCNN_REQUIRE(batch_size >= 1 && batch_size <= (1 << batch_bits) && ((int64_t)batch_size << (3 * full_depth)) < (1ll << 31),
+               "octree_build_fill: batch_size=%d does not fit batch_bits=%d / full_depth=%d", batch_size, batch_bits,
+               full_depth);
+  const int key_bits = 3 * depth, levels = depth - full_depth;
+  BuildTree t;
+  t.begin[0] = 0;
+  for (int d = 0; d <= depth; ++d) {
+    const int64_t nnum = d <= full_depth ? ((int64_t)batch_size << (3 * d)) : 8 * h_sizes[depth - d + 1];
+    OCNN_REQUIRE(nnum > 0 && nnum < (1ll << 31) && h_keys[d] && h_children[d],
+                 "octree_build_fill: depth %d: %lld nodes or a missing array", d, (long long)nnum);
+    t.keys[d] = h_keys[d];
+    t.children[d] = h_children[d];
+    t.begin[d + 1] = t.begin[d] + nnum;
+  }
+  OCNN_REQUIRE(h_sizes[levels] <= ((int64_t)batch_size << (3 * full_depth)),
+               "octree_build_fill: %lld nodes at the deepest full layer of %d octrees", (long long)h_sizes[levels],
+               batch_size);
+#define OCNN_BUILD_FILL(K, N) \
+  build_fill_t<K, N>((const char*)workspace, n, key_bits, depth, full_depth, t, perm, inverse, seg_start, (hipStream_t)stream)
+  OCNN_BUILD_DISPATCH(OCNN_BUILD_FILL);
+#undef OCNN_BUILD_FILL
 }

@@ -474,54 +474,35 @@ class Octree:
     _lib.check(L.ocnn_points2key(_lib.ptr(pts), npt, h_lo, factor, _lib.ptr(batch),
                                  batch_is_float, depth, _lib.ptr(pts_norm), _lib.ptr(key), st))
 
-    # sorted unique keys + inverse map + counts
-    ws = _lib.workspace(L.ocnn_sort_unique_workspace_bytes(npt), dev)
-    node_key = torch.empty(npt, dtype=torch.long, device=dev)
-    idx = torch.empty(npt, dtype=torch.long, device=dev)
-    counts = torch.empty(npt, dtype=torch.long, device=dev)
-    seg_start = torch.empty(npt + 1, dtype=torch.int32, device=dev)
-    perm = torch.empty(npt, dtype=torch.int32, device=dev)
-    n_dev = torch.zeros(1, dtype=torch.long, device=dev)
+    # sort, then every layer's node numbering in one scan: one read-back for the whole build
+    full_depth = self.full_depth
+    levels = depth - full_depth
     batch_bits = max(0, (self.batch_size - 1).bit_length())
-    _lib.check(L.ocnn_sort_unique(_lib.ptr(key), npt, 3 * depth, batch_bits, _lib.ptr(ws),
-                                  ws.numel(), _lib.ptr(node_key), _lib.ptr(idx),
-                                  _lib.ptr(counts), _lib.ptr(seg_start), _lib.ptr(perm),
-                                  _lib.ptr(n_dev), st))
-    n = int(n_dev.item())
-    nleaf = n
-    node_key = node_key[:n]
+    ws = _lib.workspace(L.ocnn_octree_build_workspace_bytes(npt, depth, full_depth, batch_bits), dev)
+    perm = torch.empty(npt, dtype=torch.int32, device=dev)
+    sizes = torch.empty(levels + 1, dtype=torch.long, device=dev)
+    _lib.check(L.ocnn_octree_build_scan(_lib.ptr(key), npt, depth, full_depth, batch_bits,
+                                        _lib.ptr(ws), ws.numel(), _lib.ptr(perm), _lib.ptr(sizes),
+                                        st))
+    sizes = sizes.tolist()
+    nleaf = sizes[0]
 
-    for d in range(self.full_depth + 1):
-      self.octree_grow_full(d, update_neigh=False)
-
-    # sparse levels, finest first
-    for d in range(depth, self.full_depth, -1):
-      n = node_key.numel()
-      ws = _lib.workspace(L.ocnn_build_level_workspace_bytes(n), dev)
-      pidx = torch.empty(n, dtype=torch.int32, device=dev)
-      _lib.check(L.ocnn_build_level_count(_lib.ptr(node_key), n, _lib.ptr(ws), ws.numel(),
-                                          _lib.ptr(pidx), _lib.ptr(n_dev), st))
-      n_parent = int(n_dev.item())
-      keys = torch.empty(8 * n_parent, dtype=torch.long, device=dev)
-      children = torch.empty(8 * n_parent, dtype=torch.int32, device=dev)
-      next_key = torch.empty(n_parent, dtype=torch.long, device=dev)
-      _lib.check(L.ocnn_build_level_fill(_lib.ptr(node_key), _lib.ptr(pidx), n, n_parent,
-                                         int(self.batch_size > 1), _lib.ptr(keys),
-                                         _lib.ptr(children), _lib.ptr(next_key), st))
-      self.keys[d] = keys
-      self.children[d] = children
-      self.nnum[d] = 8 * n_parent
-      self.nnum_nempty[d] = n
-      node_key = next_key
-
-    # children of the deepest full layer
-    d = self.full_depth
-    children = -torch.ones_like(self.children[d])
-    at = node_key if self.batch_size == 1 else \
-        ((node_key >> 48) << (3 * d)) | (node_key & ((1 << 48) - 1))
-    children[at] = torch.arange(node_key.numel(), dtype=torch.int32, device=dev)
-    self.children[d] = children
-    self.nnum_nempty[d] = node_key.numel()
+    full = [self.batch_size << (3 * d) for d in range(full_depth + 1)]
+    nnum = full + [8 * sizes[depth - d + 1] for d in range(full_depth + 1, depth + 1)]
+    self.nnum[:depth + 1] = torch.tensor(nnum, dtype=torch.long)
+    self.nnum_nempty[:depth + 1] = torch.tensor(
+        full[:-1] + [sizes[depth - d] for d in range(full_depth, depth + 1)], dtype=torch.long)
+    for d in range(depth + 1):
+      self.keys[d] = torch.empty(nnum[d], dtype=torch.long, device=dev)
+      self.children[d] = torch.empty(nnum[d], dtype=torch.int32, device=dev)
+    idx = torch.empty(npt, dtype=torch.long, device=dev)
+    seg_start = torch.empty(nleaf + 1, dtype=torch.int32, device=dev)
+    h_sizes = (ctypes.c_int64 * (levels + 1))(*sizes)
+    h_keys = (ctypes.c_void_p * (depth + 1))(*[t.data_ptr() for t in self.keys[:depth + 1]])
+    h_children = (ctypes.c_void_p * (depth + 1))(*[t.data_ptr() for t in self.children[:depth + 1]])
+    _lib.check(L.ocnn_octree_build_fill(_lib.ptr(ws), npt, depth, full_depth, self.batch_size,
+                                        batch_bits, h_sizes, _lib.ptr(perm), h_keys, h_children,
+                                        _lib.ptr(idx), _lib.ptr(seg_start), st))
 
     # per-leaf signals
     def leaf(src, mode):
@@ -546,17 +527,26 @@ class Octree:
     self._plans_prebuilt = False
     return idx
 
+  def _grow_full(self, depth: int, with_children: bool = True):
+    num = self.batch_size << (3 * depth)
+    self.nnum[depth] = num
+    self.nnum_nempty[depth] = num
+    dev = torch.device(self.device)
+    if dev.type != 'cuda':
+      raise RuntimeError('ocnn_amd builds octrees on the GPU only (device=%s)' % (dev,))
+    keys = torch.empty(num, dtype=torch.long, device=dev)
+    children = torch.empty(num, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+      _lib.check(_lib.lib().ocnn_build_full_layer(depth, self.batch_size, int(with_children),
+                                                  _lib.ptr(keys), _lib.ptr(children),
+                                                  _lib.stream()))
+    self.keys[depth] = keys
+    self.children[depth] = children
+
   def octree_grow_full(self, depth: int, update_neigh: bool = True):
     """Dense layer (ocnn/octree/octree.py:289-321)."""
     assert depth <= self.full_depth, 'error'
-    num = 1 << (3 * depth)
-    bs = self.batch_size
-    self.nnum[depth] = num * bs
-    self.nnum_nempty[depth] = num * bs
-    key = torch.arange(num, dtype=torch.long, device=self.device)
-    b = torch.arange(bs, dtype=torch.long, device=self.device)
-    self.keys[depth] = (key.unsqueeze(0) | (b.unsqueeze(1) << 48)).view(-1)
-    self.children[depth] = torch.arange(num * bs, dtype=torch.int32, device=self.device)
+    self._grow_full(depth)
     self._drop_nempty(depth)
     if update_neigh:
       self.construct_neigh(depth)

@@ -371,6 +371,37 @@ def test_random_octrees_vs_oracle():
       assert np.array_equal(np_(o._table(depth, kern, stride, ne)), w.get_neigh(depth, kern, stride, ne))
 
 
+@pytest.mark.parametrize('depth,full,batch,n', [(11, 2, 1, 3000), (11, 1, 5, 4000), (12, 3, 3, 2500),
+                                                (10, 1, 2, 6000), (10, 2, 8, 6000), (16, 6, 1, 300)])
+def test_deep_octrees_vs_oracle(depth, full, batch, n):
+  """Depths at which batch id and Morton code pass 32 bits (the build then sorts 64-bit keys) and
+  more than seven sparse layers (the wider scan element): every layer's keys and children, the
+  counts, the point -> leaf map and the leaf signals bit exact against the oracle."""
+  say('deep octree: depth', depth, 'full', full, 'batch', batch, 'points', n)
+  rng = np.random.default_rng(depth * 100 + batch)
+  c = rng.uniform(-0.8, 0.8, (7, 3))
+  pts = c[rng.integers(0, 7, n)] + rng.normal(0, 0.02, (n, 3)) * (rng.random((n, 1)) < 0.8)
+  pts = np.clip(pts, -1.0, 0.999999).astype(np.float32)
+  nrm = rng.standard_normal((n, 3)).astype(np.float32)
+  bid = None
+  if batch > 1:
+    bid = rng.integers(0, batch, n)
+    bid[:batch] = np.arange(batch)
+    bid = np.sort(bid).astype(np.int64)
+  pc = Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV),
+              batch_id=None if bid is None else torch.from_numpy(bid).view(-1, 1).to(DEV), batch_size=batch)
+  o = Octree(depth, full, batch_size=batch)
+  idx = o.build_octree(pc)
+  w, widx = R.build_octree(pts, nrm, None, bid, depth, full, batch)
+  assert np.array_equal(o.nnum.numpy(), w.nnum) and np.array_equal(o.nnum_nempty.numpy(), w.nnum_nempty)
+  assert np.array_equal(np_(idx), widx)
+  for d in range(depth + 1):
+    assert np.array_equal(np_(o.keys[d]), w.keys[d]), d
+    assert np.array_equal(np_(o.children[d]), w.children[d]), d
+  assert np.array_equal(np_(o.points[depth]), w.points[depth])
+  assert np.allclose(np_(o.normals[depth]), w.normals[depth], atol=1e-6)
+
+
 def test_input_feature_vs_oracle():
   """Octree.get_input_feature (ocnn/octree/octree.py:525-568) and modules.InputFeature: every
   letter and combinations, all nodes (zero rows for empty leaves) and non-empty nodes; the
