@@ -178,24 +178,12 @@ __global__ void grow_layer_kernel(const int64_t* key_above, const int32_t* nempt
 // starts for all layers together numbers the nodes of every layer in one scan over the points.
 constexpr int kBuildMaxDepth = 16;
 
-template <int N>
-struct LevelCount {
-  uint32_t v[N];
-};
-
-template <int N>
-struct LevelCountPlus {
-  __host__ __device__ LevelCount<N> operator()(const LevelCount<N>& a, const LevelCount<N>& b) const {
-    LevelCount<N> r;
-#pragma unroll
-    for (int i = 0; i < N; ++i) r.v[i] = a.v[i] + b.v[i];
-    return r;
-  }
-};
+constexpr int kBuildSpan = 1024;     // sorted points per workgroup of the counting and the scatter kernel
+constexpr int kBuildThreads = 256;   // four waves, each on a run of 256 consecutive points
 
 // number of layers at which sorted point i starts a node, minus one (-1: same leaf as i - 1)
 template <typename K>
-__host__ __device__ inline int start_level(const K* sorted, int64_t i, int key_bits, int levels) {
+__device__ inline int start_level(const K* __restrict__ sorted, int64_t i, int key_bits, int levels) {
   if (i == 0) return levels;
   const K x = sorted[i] ^ sorted[i - 1];
   if (x == 0) return -1;
@@ -205,34 +193,62 @@ __host__ __device__ inline int start_level(const K* sorted, int64_t i, int key_b
   return l < levels ? l : levels;
 }
 
-template <typename K, int N>
-struct LevelFlags {
-  const K* sorted;
-  int key_bits, levels;
-  __host__ __device__ LevelCount<N> operator()(int64_t i) const {
-    const int lv = start_level(sorted, i, key_bits, levels);
-    LevelCount<N> r;
-#pragma unroll
-    for (int l = 0; l < N; ++l) r.v[l] = l <= lv ? 1u : 0u;
-    return r;
-  }
-};
-
-template <typename K>
-__global__ void build_prep_kernel(const int64_t* __restrict__ key, int64_t n, int key_bits, K* __restrict__ ckey,
-                                  int32_t* __restrict__ iota) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const uint64_t k = (uint64_t)key[i];
-  ckey[i] = (K)(((k >> 48) << key_bits) | (k & ((1ull << key_bits) - 1)));
-  iota[i] = (int32_t)i;
+__device__ inline uint32_t lanes_below(unsigned long long mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
+// starts of nodes, by layer, among the points of each workgroup's span: sums[span][N]
+template <typename K, int N>
+__global__ __launch_bounds__(kBuildThreads) void build_count_kernel(const K* __restrict__ sorted, int64_t n,
+                                                                    int key_bits, int levels,
+                                                                    uint32_t* __restrict__ sums) {
+  __shared__ uint32_t s_cnt[kBuildThreads / 64][N];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t base = (int64_t)blockIdx.x * kBuildSpan + wave * (kBuildSpan / 4);
+  uint32_t cnt[N];
+#pragma unroll
+  for (int l = 0; l < N; ++l) cnt[l] = 0u;
+#pragma unroll
+  for (int it = 0; it < kBuildSpan / kBuildThreads; ++it) {
+    const int64_t q = base + it * 64 + lane;
+    const int lv = q < n ? start_level(sorted, q, key_bits, levels) : -1;
+#pragma unroll
+    for (int l = 0; l < N; ++l) cnt[l] += (uint32_t)__popcll(__ballot(lv >= l));
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int l = 0; l < N; ++l) s_cnt[wave][l] = cnt[l];
+  }
+  __syncthreads();
+  if (threadIdx.x < N) {
+    uint32_t c = 0u;
+    for (int w = 0; w < kBuildThreads / 64; ++w) c += s_cnt[w][threadIdx.x];
+    sums[(int64_t)blockIdx.x * N + threadIdx.x] = c;
+  }
+}
+
+// offs[span][l] = starts at layer l before the span; sizes[l] = their total.  One workgroup: thread
+// (chunk, l) walks a chunk of spans twice, the chunks' totals meet in LDS in between.
 template <int N>
-__global__ void build_sizes_kernel(const LevelCount<N>* __restrict__ scan, int64_t n, int levels,
-                                   int64_t* __restrict__ sizes) {
-  const int l = threadIdx.x;
-  if (l <= levels) sizes[l] = (int64_t)scan[n - 1].v[l];
+__global__ __launch_bounds__(1024) void build_offsets_kernel(const uint32_t* __restrict__ sums, int64_t spans,
+                                                             int levels, uint32_t* __restrict__ offs,
+                                                             int64_t* __restrict__ sizes) {
+  constexpr int kChunks = 1024 / N;
+  __shared__ uint32_t s_tot[kChunks][N];
+  const int l = threadIdx.x % N, c = threadIdx.x / N;
+  const int64_t per = (spans + kChunks - 1) / kChunks;
+  const int64_t lo = c * per < spans ? c * per : spans, hi = lo + per < spans ? lo + per : spans;
+  uint32_t tot = 0u;
+  for (int64_t b = lo; b < hi; ++b) tot += sums[b * N + l];
+  s_tot[c][l] = tot;
+  __syncthreads();
+  uint32_t run = 0u;
+  for (int cc = 0; cc < c; ++cc) run += s_tot[cc][l];
+  if (c == kChunks - 1 && l <= levels) sizes[l] = (int64_t)(run + tot);
+  for (int64_t b = lo; b < hi; ++b) {
+    offs[b * N + l] = run;
+    run += sums[b * N + l];
+  }
 }
 
 struct BuildTree {
@@ -256,43 +272,82 @@ __global__ void build_init_kernel(BuildTree t, int depth, int full_depth) {
   }
 }
 
+// Numbers every point's nodes (its span's offsets + the starts before it inside the span, counted
+// with wave ballots) and writes what the point starts: a leaf's entry in its parent's children, a
+// parent's eight keys, and so on up to the deepest full layer.
 template <typename K, int N>
-__global__ void build_scatter_kernel(const K* __restrict__ sorted, const LevelCount<N>* __restrict__ scan,
-                                     const int32_t* __restrict__ perm, int64_t n, int key_bits, int depth,
-                                     int full_depth, BuildTree t, int64_t* __restrict__ inverse,
-                                     int32_t* __restrict__ seg_start) {
-  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (q >= n) return;
+__global__ __launch_bounds__(kBuildThreads) void build_scatter_kernel(
+    const K* __restrict__ sorted, const uint32_t* __restrict__ offs, const int32_t* __restrict__ perm, int64_t n,
+    int key_bits, int depth, int full_depth, BuildTree t, int64_t* __restrict__ inverse,
+    int32_t* __restrict__ seg_start) {
+  __shared__ uint32_t s_cnt[kBuildThreads / 64][N];
+  constexpr int kIt = kBuildSpan / kBuildThreads;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t base = (int64_t)blockIdx.x * kBuildSpan + wave * (kBuildSpan / 4);
   const int levels = depth - full_depth;
-  const LevelCount<N> s = scan[q];
-  const int32_t leaf = (int32_t)s.v[0] - 1;
-  inverse[perm[q]] = leaf;
-  if (q == n - 1) seg_start[leaf + 1] = (int32_t)n;
-  const int lv = start_level(sorted, q, key_bits, levels);
-  if (lv < 0) return;
-  seg_start[leaf] = (int32_t)q;
-  const uint64_t c = (uint64_t)sorted[q];
-  const int64_t b = (int64_t)(c >> key_bits);
-  const int64_t m = (int64_t)(c & ((1ull << key_bits) - 1));
+  int lv[kIt];
+  uint32_t run[N];
 #pragma unroll
-  for (int l = 0; l < N - 1; ++l) {
-    if (l < levels && l <= lv) {
-      const int d = depth - l;
-      const int64_t kl = m >> (3 * l);
-      const int64_t p = (int64_t)s.v[l + 1] - 1;
-      t.children[d][(p << 3) | (kl & 7)] = (int32_t)s.v[l] - 1;
-      if (l + 1 <= lv) {
-        const int64_t base = (b << 48) | ((kl >> 3) << 3);
-        int64_t* dst = t.keys[d] + (p << 3);
+  for (int l = 0; l < N; ++l) run[l] = 0u;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dst[j] = base + j;
+  for (int it = 0; it < kIt; ++it) {
+    const int64_t q = base + it * 64 + lane;
+    lv[it] = q < n ? start_level(sorted, q, key_bits, levels) : -1;
+#pragma unroll
+    for (int l = 0; l < N; ++l) run[l] += (uint32_t)__popcll(__ballot(lv[it] >= l));
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int l = 0; l < N; ++l) s_cnt[wave][l] = run[l];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int l = 0; l < N; ++l) {
+    uint32_t r = offs[(int64_t)blockIdx.x * N + l];
+    for (int w = 0; w < wave; ++w) r += s_cnt[w][l];
+    run[l] = r;
+  }
+#pragma unroll
+  for (int it = 0; it < kIt; ++it) {
+    const int64_t q = base + it * 64 + lane;
+    uint32_t s[N];                      // inclusive: nodes of layer l started up to and with this point
+#pragma unroll
+    for (int l = 0; l < N; ++l) {
+      const unsigned long long mask = __ballot(lv[it] >= l);
+      s[l] = run[l] + lanes_below(mask) + (lv[it] >= l ? 1u : 0u);
+      run[l] += (uint32_t)__popcll(mask);
+    }
+    if (q >= n) continue;
+    const int32_t leaf = (int32_t)s[0] - 1;
+    inverse[perm[q]] = leaf;
+    if (q == n - 1) seg_start[leaf + 1] = (int32_t)n;
+    if (lv[it] < 0) continue;
+    seg_start[leaf] = (int32_t)q;
+    const uint64_t c = (uint64_t)sorted[q];
+    const int64_t b = (int64_t)(c >> key_bits);
+    const int64_t m = (int64_t)(c & ((1ull << key_bits) - 1));
+    uint32_t top = 0u;
+#pragma unroll
+    for (int l = 0; l < N; ++l) {
+      if (l == levels) top = s[l];
+      if (l < N - 1 && l < levels && l <= lv[it]) {
+        const int d = depth - l;
+        const int64_t kl = m >> (3 * l);
+        const int64_t p = (int64_t)s[l + 1 < N ? l + 1 : l] - 1;
+        t.children[d][(p << 3) | (kl & 7)] = (int32_t)s[l] - 1;
+        if (l + 1 <= lv[it]) {
+          const int64_t first = (b << 48) | ((kl >> 3) << 3);
+          int64_t* dst = t.keys[d] + (p << 3);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) dst[j] = first + j;
+        }
       }
     }
-  }
-  if (lv >= levels) {
-    const int64_t at = (b << (3 * full_depth)) | (m >> (3 * levels));
-    if (at < t.begin[full_depth + 1] - t.begin[full_depth])      // a batch id beyond batch_size has no node
-      t.children[full_depth][at] = (int32_t)s.v[levels] - 1;
+    if (lv[it] >= levels) {
+      const int64_t at = (b << (3 * full_depth)) | (m >> (3 * levels));
+      if (at < t.begin[full_depth + 1] - t.begin[full_depth])      // a batch id beyond batch_size has no node
+        t.children[full_depth][at] = (int32_t)top - 1;
+    }
   }
 }
 
@@ -300,27 +355,34 @@ using ForceOnesweep = rocprim::radix_sort_config<rocprim::default_config, rocpri
                                                  rocprim::default_config, 0>;
 
 struct BuildLayout {
-  int64_t ckey, csorted, iota, scan, temp, temp_bytes, total;
+  int64_t csorted, sums, offs, temp, temp_bytes, total, spans;
+};
+
+// batch id packed right above the Morton bits, read straight from the 64-bit keys by the sort
+template <typename K>
+struct PackKey {
+  int key_bits;
+  __host__ __device__ K operator()(int64_t key) const {
+    const uint64_t k = (uint64_t)key;
+    return (K)(((k >> 48) << key_bits) | (k & ((1ull << key_bits) - 1)));
+  }
 };
 
 template <typename K, int N>
 static int build_layout_t(int64_t n, BuildLayout* L) {
-  size_t sort_bytes = 0, scan_bytes = 0;
-  hipError_t e = rocprim::radix_sort_pairs<ForceOnesweep>(nullptr, sort_bytes, (K*)nullptr, (K*)nullptr,
-                                                          (int32_t*)nullptr, (int32_t*)nullptr, (size_t)n, 0,
-                                                          8 * sizeof(K));
+  size_t sort_bytes = 0;
+  auto kin = rocprim::make_transform_iterator((const int64_t*)nullptr, PackKey<K>{0});
+  auto vin = rocprim::make_counting_iterator<int32_t>(0);
+  hipError_t e = rocprim::radix_sort_pairs<ForceOnesweep>(nullptr, sort_bytes, kin, (K*)nullptr, vin,
+                                                          (int32_t*)nullptr, (size_t)n, 0, 8 * sizeof(K));
   if (e != hipSuccess) return OCNN_ERR_HIP;
-  auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<int64_t>(0),
-                                             LevelFlags<K, N>{nullptr, 0, 0});
-  e = rocprim::inclusive_scan(nullptr, scan_bytes, in, (LevelCount<N>*)nullptr, (size_t)n, LevelCountPlus<N>());
-  if (e != hipSuccess) return OCNN_ERR_HIP;
+  L->spans = cdiv(n, kBuildSpan);
   int64_t off = 0;
-  L->ckey = off;    off += align_up(n * (int64_t)sizeof(K), 256);
   L->csorted = off; off += align_up(n * (int64_t)sizeof(K), 256);
-  L->iota = off;    off += align_up(n * 4, 256);
-  L->scan = off;    off += align_up(n * (int64_t)sizeof(LevelCount<N>), 256);
+  L->sums = off;    off += align_up(L->spans * N * 4, 256);
+  L->offs = off;    off += align_up(L->spans * N * 4, 256);
   L->temp = off;
-  L->temp_bytes = align_up((int64_t)(sort_bytes > scan_bytes ? sort_bytes : scan_bytes) + 256, 256);
+  L->temp_bytes = align_up((int64_t)sort_bytes + 256, 256);
   L->total = off + L->temp_bytes;
   return OCNN_OK;
 }
@@ -331,22 +393,18 @@ static int build_scan_t(const int64_t* key, int64_t n, int key_bits, int batch_b
   BuildLayout L;
   if (build_layout_t<K, N>(n, &L) != OCNN_OK) { set_error("octree_build_scan: rocprim size query failed"); return OCNN_ERR_HIP; }
   if (ws_bytes < L.total) { set_error("octree_build_scan: workspace %lld < %lld", (long long)ws_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
-  K* ckey = (K*)(ws + L.ckey);
   K* csorted = (K*)(ws + L.csorted);
-  int32_t* iota = (int32_t*)(ws + L.iota);
-  LevelCount<N>* scan = (LevelCount<N>*)(ws + L.scan);
-  dim3 grid((unsigned)cdiv(n, 256)), block(256);
-  hipLaunchKernelGGL(build_prep_kernel<K>, grid, block, 0, st, key, n, key_bits, ckey, iota);
+  uint32_t* sums = (uint32_t*)(ws + L.sums);
+  uint32_t* offs = (uint32_t*)(ws + L.offs);
   size_t tb = (size_t)L.temp_bytes;
-  hipError_t e = rocprim::radix_sort_pairs<ForceOnesweep>(ws + L.temp, tb, ckey, csorted, iota, perm, (size_t)n, 0u,
+  auto kin = rocprim::make_transform_iterator(key, PackKey<K>{key_bits});
+  auto vin = rocprim::make_counting_iterator<int32_t>(0);
+  hipError_t e = rocprim::radix_sort_pairs<ForceOnesweep>(ws + L.temp, tb, kin, csorted, vin, perm, (size_t)n, 0u,
                                                           (unsigned)(key_bits + batch_bits), st);
   if (e != hipSuccess) { set_error("octree_build_scan: radix sort: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
-  auto in = rocprim::make_transform_iterator(rocprim::make_counting_iterator<int64_t>(0),
-                                             LevelFlags<K, N>{csorted, key_bits, levels});
-  tb = (size_t)L.temp_bytes;
-  e = rocprim::inclusive_scan(ws + L.temp, tb, in, scan, (size_t)n, LevelCountPlus<N>(), st);
-  if (e != hipSuccess) { set_error("octree_build_scan: scan: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
-  hipLaunchKernelGGL(build_sizes_kernel<N>, dim3(1), dim3(64), 0, st, scan, n, levels, sizes);
+  hipLaunchKernelGGL((build_count_kernel<K, N>), dim3((unsigned)L.spans), dim3(kBuildThreads), 0, st, csorted, n,
+                     key_bits, levels, sums);
+  hipLaunchKernelGGL(build_offsets_kernel<N>, dim3(1), dim3(1024), 0, st, sums, L.spans, levels, offs, sizes);
   return check_launch("octree_build_scan");
 }
 
@@ -356,11 +414,11 @@ static int build_fill_t(const char* ws, int64_t n, int key_bits, int depth, int 
   BuildLayout L;
   if (build_layout_t<K, N>(n, &L) != OCNN_OK) { set_error("octree_build_fill: rocprim size query failed"); return OCNN_ERR_HIP; }
   const K* csorted = (const K*)(ws + L.csorted);
-  const LevelCount<N>* scan = (const LevelCount<N>*)(ws + L.scan);
+  const uint32_t* offs = (const uint32_t*)(ws + L.offs);
   hipLaunchKernelGGL(build_init_kernel, dim3((unsigned)cdiv(t.begin[depth + 1], 256)), dim3(256), 0, st, t, depth,
                      full_depth);
-  hipLaunchKernelGGL((build_scatter_kernel<K, N>), dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, csorted, scan, perm,
-                     n, key_bits, depth, full_depth, t, inverse, seg_start);
+  hipLaunchKernelGGL((build_scatter_kernel<K, N>), dim3((unsigned)L.spans), dim3(kBuildThreads), 0, st, csorted, offs,
+                     perm, n, key_bits, depth, full_depth, t, inverse, seg_start);
   return check_launch("octree_build_fill");
 }
 
