@@ -484,19 +484,20 @@ class Octree:
     _lib.check(L.ocnn_octree_build_scan(_lib.ptr(key), npt, depth, full_depth, batch_bits,
                                         _lib.ptr(ws), ws.numel(), _lib.ptr(perm), _lib.ptr(sizes),
                                         st))
+    # what does not wait for the sizes is allocated while the sort runs
+    full = [self.batch_size << (3 * d) for d in range(full_depth + 1)]
+    for d in range(full_depth + 1):
+      self.keys[d] = torch.empty(full[d], dtype=torch.long, device=dev)
+      self.children[d] = torch.empty(full[d], dtype=torch.int32, device=dev)
+    idx = torch.empty(npt, dtype=torch.long, device=dev)
+    seg_start = torch.empty(npt + 1, dtype=torch.int32, device=dev)
     sizes = sizes.tolist()
     nleaf = sizes[0]
 
-    full = [self.batch_size << (3 * d) for d in range(full_depth + 1)]
     nnum = full + [8 * sizes[depth - d + 1] for d in range(full_depth + 1, depth + 1)]
-    self.nnum[:depth + 1] = torch.tensor(nnum, dtype=torch.long)
-    self.nnum_nempty[:depth + 1] = torch.tensor(
-        full[:-1] + [sizes[depth - d] for d in range(full_depth, depth + 1)], dtype=torch.long)
-    for d in range(depth + 1):
+    for d in range(full_depth + 1, depth + 1):
       self.keys[d] = torch.empty(nnum[d], dtype=torch.long, device=dev)
       self.children[d] = torch.empty(nnum[d], dtype=torch.int32, device=dev)
-    idx = torch.empty(npt, dtype=torch.long, device=dev)
-    seg_start = torch.empty(nleaf + 1, dtype=torch.int32, device=dev)
     h_sizes = (ctypes.c_int64 * (levels + 1))(*sizes)
     h_keys = (ctypes.c_void_p * (depth + 1))(*[t.data_ptr() for t in self.keys[:depth + 1]])
     h_children = (ctypes.c_void_p * (depth + 1))(*[t.data_ptr() for t in self.children[:depth + 1]])
@@ -512,6 +513,9 @@ class Octree:
                                      _lib.ptr(seg_start), nleaf, mode, _lib.ptr(out), st))
       return out
 
+    self.nnum[:depth + 1] = torch.tensor(nnum, dtype=torch.long)
+    self.nnum_nempty[:depth + 1] = torch.tensor(
+        full[:-1] + [sizes[depth - d] for d in range(full_depth, depth + 1)], dtype=torch.long)
     self.points[depth] = leaf(pts_norm, 0)
     if point_cloud.normals is not None:
       self.normals[depth] = leaf(point_cloud.normals, 1)

@@ -402,6 +402,40 @@ def test_deep_octrees_vs_oracle(depth, full, batch, n):
   assert np.allclose(np_(o.normals[depth]), w.normals[depth], atol=1e-6)
 
 
+@pytest.mark.parametrize('depth,batch', [(8, 1), (9, 4), (6, 2)])
+def test_uneven_clouds_vs_oracle(depth, batch):
+  """Nine points in ten of a cloud inside one small cell (thousands of points to a leaf, a few
+  leaves holding most of the cloud), next to an even cloud of the same size: both bit exact
+  against the oracle."""
+  n = 40000
+  rng = np.random.default_rng(depth)
+  for uneven in (True, False):
+    say('uneven cloud' if uneven else 'even cloud', 'depth', depth, 'batch', batch)
+    pts = rng.uniform(-0.95, 0.95, (n, 3))
+    if uneven:
+      pts[: 9 * n // 10] = np.array([0.3, -0.2, 0.6]) + rng.normal(0, 2e-4, (9 * n // 10, 3))
+      pts = pts[rng.permutation(n)]
+    pts = pts.astype(np.float32)
+    nrm = rng.standard_normal((n, 3)).astype(np.float32)
+    bid = None
+    if batch > 1:
+      bid = np.sort(rng.integers(0, batch, n)).astype(np.int64)
+      bid[:batch] = np.arange(batch)
+      bid = np.sort(bid)
+    pc = Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV),
+                batch_id=None if bid is None else torch.from_numpy(bid).view(-1, 1).to(DEV), batch_size=batch)
+    o = Octree(depth, 2, batch_size=batch)
+    idx = o.build_octree(pc)
+    w, widx = R.build_octree(pts, nrm, None, bid, depth, 2, batch)
+    assert np.array_equal(o.nnum.numpy(), w.nnum) and np.array_equal(o.nnum_nempty.numpy(), w.nnum_nempty)
+    assert np.array_equal(np_(idx), widx)
+    for d in range(depth + 1):
+      assert np.array_equal(np_(o.keys[d]), w.keys[d]), d
+      assert np.array_equal(np_(o.children[d]), w.children[d]), d
+    assert np.array_equal(np_(o.points[depth]), w.points[depth])
+    assert np.allclose(np_(o.normals[depth]), w.normals[depth], atol=1e-6)
+
+
 def test_input_feature_vs_oracle():
   """Octree.get_input_feature (ocnn/octree/octree.py:525-568) and modules.InputFeature: every
   letter and combinations, all nodes (zero rows for empty leaves) and non-empty nodes; the
