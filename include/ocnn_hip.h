@@ -63,49 +63,10 @@ void ocnn_host_decode_key(int64_t key, int depth, int64_t* h_xyzb);
 
 /* ---- octree build ------------------------------------------------------ */
 
-/* torch.unique(key, sorted, return_inverse, return_counts) as used by
- * ocnn/octree/octree.py:227-228, plus the segment layout the leaf averaging
- * needs.  key_bits = number of significant low bits of the Morton part
- * (3*depth); batch ids live at bit 48 and up (batch_bits of them).
- * Outputs (capacity n each unless noted): node_key, inverse (int64, per
- * point), counts (int64), seg_start (int32, capacity n+1: first sorted
- * position of each unique key, closed by n), perm (int32: sorted position ->
- * point index, stable).  n_unique: one int64 on the device. */
-int64_t ocnn_sort_unique_workspace_bytes(int64_t n);
-int ocnn_sort_unique(const int64_t* key, int64_t n, int key_bits,
-                     int batch_bits, void* workspace, int64_t workspace_bytes,
-                     int64_t* node_key, int64_t* inverse, int64_t* counts,
-                     int32_t* seg_start, int32_t* perm, int64_t* n_unique,
-                     void* stream);
-
-/* One level of ocnn/octree/octree.py:235-259, in two steps because the node
- * count of the level is data dependent.
- * count: pidx[i] = ordinal of the parent of node_key[i] among the distinct
- *        (node_key >> 3); n_parent (device int64) = their number.
- * fill : keys[8*n_parent] = (parent_key << 3) + 0..7; children[8*n_parent] =
- *        -1 except children[(pidx << 3) | (node_key & 7)] = i; next_key
- *        [n_parent] = parent key with the batch id moved back to bit 48 when
- *        batched != 0. */
-int64_t ocnn_build_level_workspace_bytes(int64_t n);
-/* The node counts of every sparse level at once (the reference learns them one
- * level at a time from torch.unique, octree.py:244), so that a build reads
- * sizes back once: sizes[0] += number of leaf keys (*n_unique, at most n_max),
- * sizes[l] += distinct (key >> 3 l, batch id) for l = 1 .. levels.  sizes
- * [levels + 1] must hold zeros on entry. */
-int ocnn_build_level_sizes(const int64_t* node_key, int64_t n_max,
-                           const int64_t* n_unique, int levels, int64_t* sizes,
-                           void* stream);
-int ocnn_build_level_count(const int64_t* node_key, int64_t n, void* workspace,
-                           int64_t workspace_bytes, int32_t* pidx,
-                           int64_t* n_parent, void* stream);
-int ocnn_build_level_fill(const int64_t* node_key, const int32_t* pidx,
-                          int64_t n, int64_t n_parent, int batched,
-                          int64_t* keys, int32_t* children, int64_t* next_key,
-                          void* stream);
-
-/* The whole of ocnn/octree/octree.py:227-270 above the point keys in two
- * calls with one read-back between them (the reference and the level_count /
- * level_fill pair read one count back per level).
+/* The whole of ocnn/octree/octree.py:227-270 above the point keys
+ * (torch.unique with inverse, then one unique_consecutive per layer) in two
+ * calls with ONE read-back between them (the reference reads a count back per
+ * layer).
  * scan: sorts the n keys (batch id packed above the 3 * depth Morton bits;
  *       batch_bits = bits of the largest batch id), perm[n] = the stable
  *       sorting order, and numbers the nodes of every layer in one scan.
@@ -131,24 +92,21 @@ int ocnn_octree_build_fill(const void* workspace, int64_t n, int depth,
 
 /* A full layer (ocnn/octree/octree.py:289-321): keys[i] = (i mod 8^depth) |
  * (i div 8^depth) << 48 for the batch_size * 8^depth nodes; children[i] = i
- * when with_children != 0, else -1 (the deepest full layer, whose children
- * build_full_layer_children sets: children[key position of node_key[j]] = j,
- * octree.py:262-268). */
+ * when with_children != 0, else -1. */
 int ocnn_build_full_layer(int depth, int batch_size, int with_children,
                           int64_t* keys, int32_t* children, void* stream);
-int ocnn_build_full_layer_children(const int64_t* node_key, int64_t n,
-                                   int depth, int batch_size,
-                                   int32_t* children, void* stream);
+
 
 /* Regrowing an octree from split decisions, ocnn/octree/octree.py:323-351 (octree_split) and
  * :353-402 (octree_grow).
  * split_children: children[i] = ordinal of node i among the nodes with split[i] != 0, or -1;
  *        *count (device) = their number.  A layer without any split node keeps node 0
- *        (children[0] = 0, count 1), as the reference does.  Workspace as for
- *        ocnn_build_level_count.
+ *        (children[0] = 0, count 1), as the reference does.  Workspace:
+ *        ocnn_build_level_workspace_bytes(n) bytes.
  * grow_layer: the layer below `n_nempty` non-empty nodes (nempty_index = their rows, keys of
  *        their layer in key_above): keys[8 p + j] = key of the p-th of them with j appended
  *        below the batch bits, children[8 p + j] = 8 p + j. */
+int64_t ocnn_build_level_workspace_bytes(int64_t n);
 int ocnn_split_children(const int32_t* split, int64_t n, void* workspace, int64_t workspace_bytes,
                         int32_t* children, int64_t* count, void* stream);
 int ocnn_grow_layer(const int64_t* key_above, const int32_t* nempty_index, int64_t n_nempty,

@@ -22,17 +22,11 @@ SIGNATURES = {
     'ocnn_points2key': (_i, [_p, _l, POINTER(_f), _f, _p, _i, _i, _p, _p, _p]),
     'ocnn_host_encode_key': (_l, [_l, _l, _l, _l, _i]),
     'ocnn_host_decode_key': (None, [_l, _i, POINTER(_l)]),
-    'ocnn_sort_unique_workspace_bytes': (_l, [_l]),
-    'ocnn_sort_unique': (_i, [_p, _l, _i, _i, _p, _l, _p, _p, _p, _p, _p, _p, _p]),
     'ocnn_build_level_workspace_bytes': (_l, [_l]),
     'ocnn_octree_build_workspace_bytes': (_l, [_l, _i, _i, _i]),
     'ocnn_octree_build_scan': (_i, [_p, _l, _i, _i, _i, _p, _l, _p, _p, _p]),
     'ocnn_octree_build_fill': (_i, [_p, _l, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p]),
-    'ocnn_build_level_sizes': (_i, [_p, _l, _p, _i, _p, _p]),
     'ocnn_build_full_layer': (_i, [_i, _i, _i, _p, _p, _p]),
-    'ocnn_build_full_layer_children': (_i, [_p, _l, _i, _i, _p, _p]),
-    'ocnn_build_level_count': (_i, [_p, _l, _p, _l, _p, _p, _p]),
-    'ocnn_build_level_fill': (_i, [_p, _p, _l, _l, _i, _p, _p, _p, _p]),
     'ocnn_split_children': (_i, [_p, _l, _p, _l, _p, _p, _p]),
     'ocnn_grow_layer': (_i, [_p, _p, _l, _p, _p, _p]),
     'ocnn_leaf_average': (_i, [_p, _i, _p, _p, _l, _i, _p, _p]),

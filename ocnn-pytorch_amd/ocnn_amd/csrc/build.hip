@@ -1,5 +1,6 @@
-// Octree construction: sorted-unique of the point keys, the per-level parent
-// pass, and the per-leaf signal averages.
+// Octree construction: the sort of the point keys, the numbering of every layer's nodes in one
+// pass over the sorted points, keys and children of all layers, the per-leaf signal averages, and
+// the regrowing of an octree from split decisions.
 #include <cstring>
 
 #include <rocprim/rocprim.hpp>
@@ -7,108 +8,6 @@
 #include "common.hpp"
 
 namespace ocnn {
-
-__global__ void sort_prep_kernel(const int64_t* key, int64_t n, int key_bits, uint64_t* ckey,
-                                 int32_t* iota) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  uint64_t k = (uint64_t)key[i];
-  // pack the batch id right above the Morton bits: fewer radix passes
-  ckey[i] = ((k >> 48) << key_bits) | (k & ((1ull << key_bits) - 1));
-  iota[i] = (int32_t)i;
-}
-
-template <typename K>
-__global__ void head_flag_kernel(const K* sorted, int64_t n, int shift, int32_t* flag) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  flag[i] = (i == 0 || (sorted[i] >> shift) != (sorted[i - 1] >> shift)) ? 1 : 0;
-}
-
-__global__ void unique_finish_kernel(const uint64_t* ckey, const int32_t* uid,
-                                     const int32_t* perm, int64_t n, int key_bits,
-                                     int64_t* node_key, int64_t* inverse, int32_t* seg_start,
-                                     int64_t* n_unique) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int32_t u = uid[i] - 1;
-  inverse[perm[i]] = u;
-  if (i == 0 || uid[i - 1] != uid[i]) {
-    uint64_t c = ckey[i];
-    node_key[u] = (int64_t)(((c >> key_bits) << 48) | (c & ((1ull << key_bits) - 1)));
-    seg_start[u] = (int32_t)i;
-  }
-  if (i == n - 1) {
-    seg_start[u + 1] = (int32_t)n;
-    *n_unique = (int64_t)u + 1;
-  }
-}
-
-__global__ void counts_kernel(const int32_t* seg_start, const int64_t* n_unique, int64_t n,
-                              int64_t* counts) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n || i >= *n_unique) return;
-  counts[i] = (int64_t)(seg_start[i + 1] - seg_start[i]);
-}
-
-__global__ void level_count_finish_kernel(const int32_t* uid, int64_t n, int32_t* pidx,
-                                          int64_t* n_parent) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int32_t u = uid[i];
-  pidx[i] = u - 1;
-  if (i == n - 1) *n_parent = (int64_t)u;
-}
-
-// Node counts of ALL the sparse layers from the sorted leaf keys in one pass, so that the host
-// reads sizes back once for the whole build: sizes[0] = leaves, sizes[l] = distinct nodes l
-// layers up.  Two neighbouring keys part ways l layers up iff their highest differing bit is at
-// least 3 l (any bit of the batch index, bits 48 and up: at every layer).
-__global__ void level_sizes_kernel(const int64_t* __restrict__ node_key, const int64_t* __restrict__ n_ptr,
-                                   int levels, unsigned long long* __restrict__ sizes) {
-  __shared__ unsigned int s_hist[32];
-  const int64_t n = *n_ptr;
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (threadIdx.x < 32) s_hist[threadIdx.x] = 0u;
-  __syncthreads();
-  if (i < n) {
-    int lv = levels;                                        // the first key starts a node at every layer
-    if (i > 0) {
-      const unsigned long long x = (unsigned long long)(node_key[i] ^ node_key[i - 1]);
-      const int hb = 63 - __clzll((long long)x);
-      lv = hb >= 48 ? levels : min(levels, hb / 3);
-    }
-    atomicAdd(&s_hist[lv], 1u);
-  }
-  __syncthreads();
-  if ((int)threadIdx.x <= levels) {
-    unsigned int c = 0;
-    for (int v = threadIdx.x; v <= levels; ++v) c += s_hist[v];
-    if (c != 0u) atomicAdd(&sizes[threadIdx.x], (unsigned long long)c);
-  }
-}
-
-__global__ void level_fill_parent_kernel(const int64_t* node_key, const int32_t* pidx, int64_t n,
-                                         int batched, int64_t* keys, int32_t* children,
-                                         int64_t* next_key) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  int32_t p = pidx[i];
-  if (i != 0 && pidx[i - 1] == p) return;   // only the first child of a parent writes
-  int64_t pk = node_key[i] >> 3;
-  for (int j = 0; j < 8; ++j) {
-    keys[8 * (int64_t)p + j] = (pk << 3) + j;
-    children[8 * (int64_t)p + j] = -1;
-  }
-  next_key[p] = batched ? (((pk >> 45) << 48) | (pk & ((1ll << 45) - 1))) : pk;
-}
-
-__global__ void level_fill_child_kernel(const int64_t* node_key, const int32_t* pidx, int64_t n,
-                                        int32_t* children) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  children[((int64_t)pidx[i] << 3) | (node_key[i] & 7)] = (int32_t)i;
-}
 
 __global__ void leaf_mean_kernel(const float* src, int C, const int32_t* perm,
                                  const int32_t* seg_start, int64_t n_leaf, float* out) {
@@ -433,31 +332,6 @@ static int build_fill_t(const char* ws, int64_t n, int key_bits, int depth, int 
     }                                                                \
   } while (0)
 
-struct SortLayout {
-  int64_t ckey, csorted, iota, flag, uid, temp, temp_bytes, total;
-};
-
-static int sort_layout(int64_t n, SortLayout* L) {
-  size_t sort_bytes = 0, scan_bytes = 0;
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, (uint64_t*)nullptr,
-                                           (uint64_t*)nullptr, (int32_t*)nullptr,
-                                           (int32_t*)nullptr, (size_t)n, 0, 64);
-  if (e != hipSuccess) return OCNN_ERR_HIP;
-  e = rocprim::inclusive_scan(nullptr, scan_bytes, (int32_t*)nullptr, (int32_t*)nullptr,
-                              (size_t)n, rocprim::plus<int32_t>());
-  if (e != hipSuccess) return OCNN_ERR_HIP;
-  int64_t off = 0;
-  L->ckey = off;    off += align_up(n * 8, 256);
-  L->csorted = off; off += align_up(n * 8, 256);
-  L->iota = off;    off += align_up(n * 4, 256);
-  L->flag = off;    off += align_up(n * 4, 256);
-  L->uid = off;     off += align_up(n * 4, 256);
-  L->temp = off;
-  L->temp_bytes = (int64_t)align_up((int64_t)(sort_bytes > scan_bytes ? sort_bytes : scan_bytes) + 256, 256);
-  L->total = off + L->temp_bytes;
-  return OCNN_OK;
-}
-
 struct LevelLayout {
   int64_t flag, uid, temp, temp_bytes, total;
 };
@@ -480,46 +354,6 @@ static int level_layout(int64_t n, LevelLayout* L) {
 
 using namespace ocnn;
 
-extern "C" int64_t ocnn_sort_unique_workspace_bytes(int64_t n) {
-  if (n <= 0) return 256;
-  SortLayout L;
-  if (sort_layout(n, &L) != OCNN_OK) return -1;
-  return L.total;
-}
-
-extern "C" int ocnn_sort_unique(const int64_t* key, int64_t n, int key_bits, int batch_bits,
-                                void* workspace, int64_t workspace_bytes, int64_t* node_key,
-                                int64_t* inverse, int64_t* counts, int32_t* seg_start,
-                                int32_t* perm, int64_t* n_unique, void* stream) {
-  OCNN_REQUIRE(n > 0 && n < (1ll << 31), "sort_unique: n=%lld out of range", (long long)n);
-  OCNN_REQUIRE(key_bits >= 3 && key_bits <= 48 && batch_bits >= 0 && batch_bits <= 15,
-               "sort_unique: key_bits=%d batch_bits=%d", key_bits, batch_bits);
-  SortLayout L;
-  if (sort_layout(n, &L) != OCNN_OK) { set_error("sort_unique: rocprim size query failed"); return OCNN_ERR_HIP; }
-  if (workspace_bytes < L.total) { set_error("sort_unique: workspace %lld < %lld", (long long)workspace_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
-  hipStream_t st = (hipStream_t)stream;
-  char* ws = (char*)workspace;
-  uint64_t* ckey = (uint64_t*)(ws + L.ckey);
-  uint64_t* csorted = (uint64_t*)(ws + L.csorted);
-  int32_t* iota = (int32_t*)(ws + L.iota);
-  int32_t* flag = (int32_t*)(ws + L.flag);
-  int32_t* uid = (int32_t*)(ws + L.uid);
-  dim3 grid(cdiv(n, 256)), block(256);
-  hipLaunchKernelGGL(sort_prep_kernel, grid, block, 0, st, key, n, key_bits, ckey, iota);
-  size_t tb = (size_t)L.temp_bytes;
-  hipError_t e = rocprim::radix_sort_pairs(ws + L.temp, tb, ckey, csorted, iota, perm, (size_t)n,
-                                           0u, (unsigned)(key_bits + batch_bits), st);
-  if (e != hipSuccess) { set_error("sort_unique: radix sort: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
-  hipLaunchKernelGGL(head_flag_kernel<uint64_t>, grid, block, 0, st, csorted, n, 0, flag);
-  tb = (size_t)L.temp_bytes;
-  e = rocprim::inclusive_scan(ws + L.temp, tb, flag, uid, (size_t)n, rocprim::plus<int32_t>(), st);
-  if (e != hipSuccess) { set_error("sort_unique: scan: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
-  hipLaunchKernelGGL(unique_finish_kernel, grid, block, 0, st, csorted, uid, perm, n, key_bits,
-                     node_key, inverse, seg_start, n_unique);
-  hipLaunchKernelGGL(counts_kernel, grid, block, 0, st, seg_start, n_unique, n, counts);
-  return check_launch("sort_unique");
-}
-
 extern "C" int64_t ocnn_build_level_workspace_bytes(int64_t n) {
   if (n <= 0) return 256;
   LevelLayout L;
@@ -537,16 +371,6 @@ __global__ void full_layer_kernel(int depth, int64_t total, int32_t child_fill, 
   children[i] = child_fill < 0 ? child_fill : (int32_t)i;
 }
 
-// children of the deepest full layer: node j of the layer below's parents sits at its key.
-__global__ void full_layer_children_kernel(const int64_t* __restrict__ node_key, int64_t n, int depth,
-                                           int64_t total, int32_t* __restrict__ children) {
-  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= n) return;
-  const int64_t k = node_key[j];
-  const int64_t at = ((k >> 48) << (3 * depth)) | (k & ((1ll << 48) - 1));
-  if (at >= 0 && at < total) children[at] = (int32_t)j;
-}
-
 extern "C" int ocnn_build_full_layer(int depth, int batch_size, int with_children, int64_t* keys,
                                      int32_t* children, void* stream) {
   OCNN_REQUIRE(depth >= 0 && depth <= 8 && batch_size >= 1 && ((int64_t)batch_size << (3 * depth)) < (1ll << 31),
@@ -555,61 +379,6 @@ extern "C" int ocnn_build_full_layer(int depth, int batch_size, int with_childre
   hipLaunchKernelGGL(full_layer_kernel, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, (hipStream_t)stream, depth,
                      total, with_children ? 0 : -1, keys, children);
   return check_launch("build_full_layer");
-}
-
-extern "C" int ocnn_build_full_layer_children(const int64_t* node_key, int64_t n, int depth, int batch_size,
-                                              int32_t* children, void* stream) {
-  OCNN_REQUIRE(depth >= 0 && depth <= 8 && batch_size >= 1 && n >= 0 && n < (1ll << 31),
-               "build_full_layer_children: depth=%d batch_size=%d n=%lld out of range", depth, batch_size,
-               (long long)n);
-  if (n == 0) return 0;
-  const int64_t total = (int64_t)batch_size << (3 * depth);
-  hipLaunchKernelGGL(full_layer_children_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream,
-                     node_key, n, depth, total, children);
-  return check_launch("build_full_layer_children");
-}
-
-extern "C" int ocnn_build_level_sizes(const int64_t* node_key, int64_t n_max, const int64_t* n_unique, int levels,
-                                      int64_t* sizes, void* stream) {
-  OCNN_REQUIRE(n_max > 0 && n_max < (1ll << 28) && levels >= 0 && levels <= 16,
-               "build_level_sizes: n_max=%lld levels=%d out of range", (long long)n_max, levels);
-  hipLaunchKernelGGL(level_sizes_kernel, dim3((unsigned)cdiv(n_max, 256)), dim3(256), 0, (hipStream_t)stream,
-                     node_key, n_unique, levels, (unsigned long long*)sizes);
-  return check_launch("build_level_sizes");
-}
-
-extern "C" int ocnn_build_level_count(const int64_t* node_key, int64_t n, void* workspace,
-                                      int64_t workspace_bytes, int32_t* pidx, int64_t* n_parent,
-                                      void* stream) {
-  OCNN_REQUIRE(n > 0 && n < (1ll << 28), "build_level_count: n=%lld out of range", (long long)n);
-  LevelLayout L;
-  if (level_layout(n, &L) != OCNN_OK) { set_error("build_level: rocprim size query failed"); return OCNN_ERR_HIP; }
-  if (workspace_bytes < L.total) { set_error("build_level: workspace %lld < %lld", (long long)workspace_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
-  hipStream_t st = (hipStream_t)stream;
-  char* ws = (char*)workspace;
-  int32_t* flag = (int32_t*)(ws + L.flag);
-  int32_t* uid = (int32_t*)(ws + L.uid);
-  dim3 grid(cdiv(n, 256)), block(256);
-  hipLaunchKernelGGL(head_flag_kernel<int64_t>, grid, block, 0, st, node_key, n, 3, flag);
-  size_t tb = (size_t)L.temp_bytes;
-  hipError_t e = rocprim::inclusive_scan(ws + L.temp, tb, flag, uid, (size_t)n,
-                                         rocprim::plus<int32_t>(), st);
-  if (e != hipSuccess) { set_error("build_level: scan: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
-  hipLaunchKernelGGL(level_count_finish_kernel, grid, block, 0, st, uid, n, pidx, n_parent);
-  return check_launch("build_level_count");
-}
-
-extern "C" int ocnn_build_level_fill(const int64_t* node_key, const int32_t* pidx, int64_t n,
-                                     int64_t n_parent, int batched, int64_t* keys,
-                                     int32_t* children, int64_t* next_key, void* stream) {
-  OCNN_REQUIRE(n > 0 && n_parent > 0 && n_parent <= n, "build_level_fill: n=%lld n_parent=%lld",
-               (long long)n, (long long)n_parent);
-  hipStream_t st = (hipStream_t)stream;
-  dim3 grid(cdiv(n, 256)), block(256);
-  hipLaunchKernelGGL(level_fill_parent_kernel, grid, block, 0, st, node_key, pidx, n, batched, keys,
-                     children, next_key);
-  hipLaunchKernelGGL(level_fill_child_kernel, grid, block, 0, st, node_key, pidx, n, children);
-  return check_launch("build_level_fill");
 }
 
 extern "C" int ocnn_split_children(const int32_t* split, int64_t n, void* workspace, int64_t workspace_bytes,

@@ -37,12 +37,21 @@ __host__ __device__ __forceinline__ void child_slot_lut(int j, int k, int* lp, i
 
 constexpr int kParentsPerBlock = 32;
 
+// The 8 x 27 entries below one parent repeat the same (parent slot, child number) pattern, so
+// the pattern sits in LDS once a workgroup, and a thread writes four entries at a time: they
+// never straddle two parents (216 = 4 * 54).
 __global__ __launch_bounds__(256) void neigh_from_parent_kernel(
     const int32_t* __restrict__ child_p, const int32_t* __restrict__ neigh_p,
     const int32_t* __restrict__ nempty_p, int64_t n_ne, int64_t* __restrict__ out64,
     int32_t* __restrict__ out32) {
   __shared__ int32_t cp[kParentsPerBlock * 27];
+  __shared__ uint16_t lut[216];
   const int64_t c0 = (int64_t)blockIdx.x * kParentsPerBlock;
+  if (threadIdx.x < 216) {
+    int lp, lc;
+    child_slot_lut(threadIdx.x / 27, threadIdx.x % 27, &lp, &lc);
+    lut[threadIdx.x] = (uint16_t)(lp | (lc << 8));
+  }
   for (int e = threadIdx.x; e < kParentsPerBlock * 27; e += 256) {
     int p = e / 27, s = e % 27;
     int32_t v = -1;
@@ -54,17 +63,23 @@ __global__ __launch_bounds__(256) void neigh_from_parent_kernel(
     cp[e] = v;
   }
   __syncthreads();
-  const int64_t base = c0 * 8 * 27;
-  const int64_t limit = (n_ne - c0) * 8 * 27;   // entries this block owns
-  for (int o = threadIdx.x; o < kParentsPerBlock * 8 * 27; o += 256) {
-    if (o >= limit) break;
-    int row = o / 27, k = o % 27;
-    int lp, lc;
-    child_slot_lut(row & 7, k, &lp, &lc);
-    int32_t v = cp[(row >> 3) * 27 + lp];
-    int32_t r = v < 0 ? -1 : v * 8 + lc;
-    if (out64) out64[base + o] = (int64_t)r;
-    if (out32) out32[base + o] = r;
+  const int64_t base = c0 * 216;
+  const int parents = (int)(n_ne - c0 < kParentsPerBlock ? n_ne - c0 : kParentsPerBlock);
+  for (int c = threadIdx.x; c < parents * 54; c += 256) {
+    const int p = c / 54, w = (c - p * 54) * 4;
+    int32_t r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int l = lut[w + e];
+      const int32_t v = cp[p * 27 + (l & 255)];
+      r[e] = v < 0 ? -1 : v * 8 + (l >> 8);
+    }
+    const int64_t o = base + 4 * (int64_t)c;
+    if (out32) *reinterpret_cast<int4*>(out32 + o) = make_int4(r[0], r[1], r[2], r[3]);
+    if (out64) {
+      *reinterpret_cast<longlong2*>(out64 + o) = make_longlong2((int64_t)r[0], (int64_t)r[1]);
+      *reinterpret_cast<longlong2*>(out64 + o + 2) = make_longlong2((int64_t)r[2], (int64_t)r[3]);
+    }
   }
 }
 
