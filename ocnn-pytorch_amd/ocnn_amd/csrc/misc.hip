@@ -285,6 +285,81 @@ __global__ __launch_bounds__(256) void colsum_kernel(const T* __restrict__ g, in
   }
 }
 
+// The same with 16-byte pieces: a thread keeps one piece of the row (8 or 4 channels) and walks
+// every (256 / pieces)-th row of the split, four loads in flight; the row lanes meet in LDS and
+// are added in lane order.  C % (16 / sizeof(T)) == 0.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_rows_kernel(const T* __restrict__ g, int64_t rows, int C,
+                                                          int64_t rows_per_split, float* __restrict__ partial) {
+  constexpr int VEC = 16 / sizeof(T);
+  struct alignas(16) Piece { T v[VEC]; };
+  __shared__ float s_acc[256][VEC + 1];
+  const int cpr = C / VEC;
+  const int lanes_c = cpr < 256 ? cpr : 256, rpi = 256 / lanes_c;
+  const int pc = threadIdx.x % lanes_c, rl = threadIdx.x / lanes_c;
+  const int64_t r_begin = (int64_t)blockIdx.x * rows_per_split;
+  const int64_t r_end = min(rows, r_begin + rows_per_split);
+  for (int p0 = 0; p0 < cpr; p0 += lanes_c) {
+    const int piece = p0 + pc;
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    if (rl < rpi && piece < cpr) {
+      const Piece* src = reinterpret_cast<const Piece*>(g) + piece;
+      int64_t i = r_begin + rl;
+      for (; i + 3 * rpi < r_end; i += 4 * rpi) {
+        Piece q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) q[u] = src[(i + u * rpi) * cpr];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) acc[v] += to_f32(q[u].v[v]);
+      }
+      for (; i < r_end; i += rpi) {
+        const Piece q = src[i * cpr];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] += to_f32(q.v[v]);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) s_acc[threadIdx.x][v] = acc[v];
+    __syncthreads();
+    if (rl == 0 && piece < cpr) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        float sum = 0.f;
+        for (int r = 0; r < rpi; ++r) sum += s_acc[r * lanes_c + pc][v];
+        partial[(int64_t)blockIdx.x * C + piece * VEC + v] = sum;
+      }
+    }
+  }
+}
+
+// out[c] = sum over the splits, 16 split lanes a channel, each adding every 16th split in order,
+// the lanes then in lane order
+template <typename T>
+__global__ __launch_bounds__(1024) void colsum_finish_kernel(const float* __restrict__ partial, int splits, int C,
+                                                             T* __restrict__ out) {
+  __shared__ float s_acc[16][64];
+  const int cl = threadIdx.x & 63, sl = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + cl;
+  float acc = 0.f;
+  if (c < C) {
+#pragma unroll 4
+    for (int s = sl; s < splits; s += 16) acc += partial[(int64_t)s * C + c];
+  }
+  s_acc[sl][cl] = acc;
+  __syncthreads();
+  if (sl == 0 && c < C) {
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sum += s_acc[r][cl];
+    out[c] = from_f32<T>(sum);
+  }
+}
+
 static void split_rows(int64_t rows, int64_t cols, int64_t* splits, int64_t* rps) {
   int64_t s = std::max<int64_t>(1, std::min<int64_t>(cdiv(2048, std::max<int64_t>(1, cols)),
                                                      cdiv(rows, 256)));
@@ -460,11 +535,17 @@ extern "C" int ocnn_colsum(int dtype, const void* g, int64_t rows, int channels,
   }
   float* partial = (float*)workspace;
   OCNN_DISPATCH_DTYPE(dtype, {
-    if (rows > 0)
-      hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)splits), dim3(256), 0, st, (const T*)g,
-                         rows, channels, rps, partial);
-    hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3(cdiv((int64_t)channels, 256)), dim3(256), 0, st,
-                       partial, (int)splits, 1, 1, channels, 0, (T*)out);
+    constexpr int VEC = 16 / sizeof(T);
+    if (rows > 0) {
+      if (channels % VEC == 0 && ((uintptr_t)g % 16) == 0)
+        hipLaunchKernelGGL(colsum_rows_kernel<T>, dim3((unsigned)splits), dim3(256), 0, st, (const T*)g, rows,
+                           channels, rps, partial);
+      else
+        hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)splits), dim3(256), 0, st, (const T*)g,
+                           rows, channels, rps, partial);
+    }
+    hipLaunchKernelGGL(colsum_finish_kernel<T>, dim3((unsigned)cdiv((int64_t)channels, 64)), dim3(1024), 0, st,
+                       partial, (int)splits, channels, (T*)out);
   });
   return check_launch("colsum");
 }

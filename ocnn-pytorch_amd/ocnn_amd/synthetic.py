@@ -102,6 +102,31 @@ def planes_cloud(n=250000, seed=1003, n_planes=4, n_spheres=3):
   return torch.cat(pts), torch.cat(nrm)
 
 
+def shell_voxels(depth, device='cpu', thickness=1.25):
+  """Integer coordinates of the cells of the 2^depth grid whose centre lies within `thickness` cells
+  inside the sphere inscribed in the grid: the octree of the reference's layer benchmark
+  (test/utils.py:43-70; 3 840 / 15 192 / 64 160 / 252 392 / 1 026 536 / 4 113 056 cells at depths
+  5 .. 10, test/benchmark_conv.py:23-31).  Deterministic; x-major order."""
+  res = 1 << depth
+  half = res / 2.0
+  axis = torch.arange(res, device=device, dtype=torch.float32) - half + 0.5
+  yz2 = (axis * axis).view(-1, 1) + (axis * axis).view(1, -1)                # (res, res)
+  lo2 = max(half - thickness, 0.0)
+  cells = []
+  for x0 in range(0, res, 32):                                                # slabs of 32 planes
+    d = (yz2.unsqueeze(0) + (axis[x0:x0 + 32] ** 2).view(-1, 1, 1)).sqrt()
+    at = torch.nonzero((d <= half) & (d >= lo2))
+    at[:, 0] += x0
+    cells.append(at)
+  return torch.cat(cells).int()
+
+
+def shell_points(depth, device='cpu'):
+  """The cells of shell_voxels as points in [-1, 1)^3 (each at its cell's lower corner, so that an
+  octree of the same depth has exactly these cells as leaves)."""
+  return shell_voxels(depth, device).float() / float(1 << depth) * 2.0 - 1.0
+
+
 def batch_clouds(maker, batch, seed, **kw):
   """`batch` clouds -> (points, normals, batch_id as float32 (N,1))."""
   pts, nrm, bid = [], [], []
