@@ -22,7 +22,7 @@ from torch.autograd import Function
 from .. import _lib
 from ..utils import list2str, resize_with_last_val, xavier_uniform_
 from .octree2col import col2octree, octree2col
-from .octree_pad import _pad_raw, octree_depad, octree_pad
+from .octree_pad import _depad_raw, _pad_raw, octree_depad, octree_pad
 
 
 # (thresholds of the kernel selection live in the library, csrc/select.hip; these are the ones
@@ -398,12 +398,15 @@ class OctreeConvFunction(Function):
     data, weights = ctx.saved_tensors
     eng = ctx.eng
     grad = grad.contiguous()
-    index = None if ctx.pad_depth is None else eng.octree._nempty_index32(ctx.pad_depth)
+    index = None
+    if ctx.pad_depth is not None:
+      if eng.dense_children and not ctx.needs_input_grad[10]:
+        index = eng.octree._nempty_index32(ctx.pad_depth)       # the dense kernels read through it
+      else:
+        grad = _depad_raw(grad, eng.octree, ctx.pad_depth)      # one copy for all three gradients
     grad_out = eng.backward_gemm(grad, weights, coarse_index=index) if ctx.needs_input_grad[0] else None
     grad_w = eng.weight_gemm(data, grad, coarse_index=index) if ctx.needs_input_grad[1] else None
-    grad_b = None
-    if ctx.needs_input_grad[10]:
-      grad_b = column_sum(grad if index is None else grad.index_select(0, index.long()))
+    grad_b = column_sum(grad) if ctx.needs_input_grad[10] else None
     return (grad_out, grad_w) + (None,) * 8 + (grad_b, None)
 
 
@@ -420,17 +423,21 @@ class OctreeDeconvFunction(Function):
     eng = _OctreeDeconv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
     index = None
+    data = data.contiguous()
     if padded:
       assert tuple(data.shape) == (int(octree.nnum[depth]), in_channels), 'The shape of input data is wrong'
-      index = octree._nempty_index32(depth)
+      if eng.dense_children:
+        index = octree._nempty_index32(depth)                   # the dense kernels read through it
+      else:
+        data = _depad_raw(data, octree, depth)                  # one copy for forward and weight gradient
     else:
       eng.check_and_init(data)
-    data = data.contiguous()
     weights = weights.to(data.dtype).contiguous()
     out = eng.backward_gemm(data, weights, bias, coarse_index=index)
     ctx.save_for_backward(data, weights)
     ctx.eng = eng
     ctx.pad_depth = depth if padded else None
+    ctx.indexed = index is not None
     return out
 
   @staticmethod
@@ -438,11 +445,11 @@ class OctreeDeconvFunction(Function):
     data, weights = ctx.saved_tensors
     eng = ctx.eng
     grad = grad.contiguous()
-    index = None if ctx.pad_depth is None else eng.octree._nempty_index32(ctx.pad_depth)
+    index = eng.octree._nempty_index32(ctx.pad_depth) if ctx.indexed else None
     grad_out = None
     if ctx.needs_input_grad[0]:
       grad_out = eng.forward_gemm(grad, weights)
-      if index is not None:
+      if ctx.pad_depth is not None:
         grad_out = _pad_raw(grad_out, eng.octree, ctx.pad_depth)
     # weights are (K, out_channels, in_channels): x = grad (fine side), g = data
     grad_w = eng.weight_gemm(grad, data, coarse_index=index) if ctx.needs_input_grad[1] else None
