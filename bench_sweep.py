@@ -1,6 +1,7 @@
 """The reference's own layer benchmark (test/benchmark_conv.py) on this library: one 3x3x3 stride-1
 OctreeConv with bias on the non-empty nodes of a thin spherical shell, depth 5 .. 10 with 256, 128,
-128, 64, 32, 32 channels, forward and backward timed apart, fp32 / fp16 / bf16.  Prints one table
+128, 64, 32, 32 channels, forward and backward timed apart (and both together replayed from a HIP
+graph), fp32 / fp16 / bf16.  Prints one table
 with the figures the reference publishes for its Triton kernels on an RTX 4090 beside ours
 (test/benchmark/results.csv; other hardware, for orientation only) and one JSON line.
 
@@ -51,6 +52,31 @@ def timed(torch, fn, min_ms=25.0, reps=20):
   return s.elapsed_time(e) / reps
 
 
+def graph_replay_ms(torch, conv, x, octree, depth, gout):
+  """Forward + backward of the layer captured once in a HIP graph (the library only launches
+  kernels on the caller's stream), ms per replay: what is left when the host-side launch path
+  is taken out.  No autograd graph of an earlier eager run may be alive: its gradient
+  accumulation nodes belong to the stream they were made on, and a capture cannot wait for it."""
+  params = [x] + list(conv.parameters())
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    for _ in range(2):
+      for p in params:
+        p.grad = None
+      conv(x, octree, depth).backward(gout)
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  for p in params:
+    p.grad = None
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    conv(x, octree, depth).backward(gout)
+  ms = timed(torch, graph.replay)
+  del graph
+  return ms
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument('--depths', default='5,6,7,8,9,10')
@@ -83,21 +109,23 @@ def main():
       gout = torch.randn(out.shape, generator=g).to(dtype).to(dev)
       fwd = timed(torch, lambda: conv(x, octree, depth))
       bwd = timed(torch, lambda: out.backward(gout, retain_graph=True))
+      del out                 # with it the autograd graph of the eager runs and its nodes on this stream
+      replay = graph_replay_ms(torch, conv, x.detach().clone().requires_grad_(), octree, depth, gout)
       i = depth - 5
       records.append({'depth': depth, 'channels': c, 'rows': rows, 'nnz': nnz, 'dtype': name,
-                      'fwd_ms': fwd, 'bwd_ms': bwd,
+                      'fwd_ms': fwd, 'bwd_ms': bwd, 'fwd_bwd_hip_graph_ms': replay,
                       'eff_tflops_fwd_bwd': 6.0 * nnz * c * c / (fwd + bwd) / 1e9,
                       'published_rtx4090_triton_fwd_ms': PUBLISHED['fwd'][name][i],
                       'published_rtx4090_triton_bwd_ms': PUBLISHED['bwd'][name][i]})
-      del conv, x, out, gout
+      del conv, x, gout
     del octree
     torch.cuda.empty_cache()
-  print('%5s %4s %9s %-9s %8s %8s %10s   %s' % ('depth', 'C', 'rows', 'dtype', 'fwd ms', 'bwd ms', 'TFLOP/s',
-                                              'reference (Triton, RTX 4090) fwd / bwd ms'))
+  print('%5s %4s %9s %-9s %8s %8s %10s %10s   %s' % ('depth', 'C', 'rows', 'dtype', 'fwd ms', 'bwd ms', 'TFLOP/s',
+                                                   'graph ms', 'reference (Triton, RTX 4090) fwd / bwd ms'))
   for r in records:
-    print('%5d %4d %9d %-9s %8.3f %8.3f %10.1f   %.3f / %.3f' % (
+    print('%5d %4d %9d %-9s %8.3f %8.3f %10.1f %10.3f   %.3f / %.3f' % (
         r['depth'], r['channels'], r['rows'], r['dtype'], r['fwd_ms'], r['bwd_ms'], r['eff_tflops_fwd_bwd'],
-        r['published_rtx4090_triton_fwd_ms'], r['published_rtx4090_triton_bwd_ms']))
+        r['fwd_bwd_hip_graph_ms'], r['published_rtx4090_triton_fwd_ms'], r['published_rtx4090_triton_bwd_ms']))
   print(json.dumps({'benchmark': 'test/benchmark_conv.py sweep, 3x3x3 stride 1, non-empty nodes, bias',
                     'data': 'synthetic (spherical shell of the reference benchmark)', 'n_gpus': 1,
                     'records': records}))

@@ -1232,3 +1232,62 @@ def test_empty_inputs(dtype):
       assert torch.equal(out, b.view(1, -1).expand(300, cout))
       gw = ocnn_amd.nn.conv_wgrad(x0, g1, t1, True, plan1)
       assert tuple(gw.shape) == (K, cout, cin) and not gw.any()
+
+
+@pytest.mark.parametrize('kind,ks,stride,nempty,cin,cout', [
+    ('conv', [3], 1, False, 64, 64), ('conv', [3], 1, True, 96, 96), ('conv', [2], 2, False, 64, 128),
+    ('deconv', [2], 2, False, 128, 64), ('dwconv', [3], 1, False, 64, 64)])
+def test_layers_replay_from_a_hip_graph(medium, kind, ks, stride, nempty, cin, cout):
+  """The library only launches kernels on the caller's stream (no allocation, memset, copy or
+  synchronisation of its own), so forward + backward of a layer can be captured in a HIP graph once
+  its plans exist: three replays, with eager work and synchronisations in between, give the bits
+  of the eager run."""
+  depth, dtype = 7, torch.bfloat16
+  o = medium.gpu
+  say('hip graph', kind, ks, stride, nempty, cin, cout)
+  g = torch.Generator().manual_seed(5)
+  if kind == 'conv':
+    mod = OctreeConv(cin, cout, ks, stride, nempty, use_bias=True)
+  elif kind == 'deconv':
+    mod = OctreeDeconv(cin, cout, ks, stride, nempty, use_bias=True)
+  else:
+    mod = OctreeDWConv(cin, ks, stride, nempty, use_bias=True)
+  mod = mod.to(DEV).to(dtype)
+  d_in = depth - 1 if kind == 'deconv' else depth
+  rows = int(o.nnum_nempty[d_in] if nempty else o.nnum[d_in])
+  x = torch.randn(rows, cin, generator=g).to(dtype).to(DEV).requires_grad_()
+  params = [x] + list(mod.parameters())
+
+  def step():
+    for p in params:
+      p.grad = None
+    out = mod(x, o, d_in)
+    out.backward(gout)
+    return out
+
+  gout = torch.randn(mod(x, o, d_in).shape, generator=g).to(dtype).to(DEV)
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    for _ in range(2):
+      out = step()                                    # plans, tables and workspaces exist from here on
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  want = [out.clone()] + [p.grad.clone() for p in params]
+  graph = torch.cuda.CUDAGraph()
+  for p in params:
+    p.grad = None
+  with torch.cuda.graph(graph):
+    out_g = mod(x, o, d_in)
+    out_g.backward(gout)
+  for replay in range(3):
+    out_g.detach().zero_()
+    for p in params:
+      p.grad.zero_()
+    (torch.randn(1000, 64, device=DEV) @ torch.randn(64, 64, device=DEV)).sum().item()     # eager work in between
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    got = [out_g] + [p.grad for p in params]
+    for a, b in zip(want, got):
+      assert torch.equal(a, b), (replay, kind)
