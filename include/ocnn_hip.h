@@ -542,6 +542,17 @@ int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const int32_t* c
                   const float* val, const void* data, int channels, const float* rowdiv,
                   void* out, int64_t rows, void* stream);
 
+/* The transposed matrix in that row form (what torch.sparse.mm's backward needs,
+ * ocnn/nn/octree_interp.py:98-102, here without atomics): entry (p, j) of idx (points, k) with
+ * idx >= 0 becomes an entry of data row idx[p, j] with column p and value w[p, j] /
+ * (norm[p] + 1e-12) (norm NULL: no division; w NULL: ones; both NULL: val NULL, nothing stored).  The entries
+ * of a row keep the order of the points.  rowptr: rows + 1 values; col, val: capacity points * k,
+ * the first rowptr[rows] of them used. */
+int64_t ocnn_csr_transpose_workspace_bytes(int64_t entries);
+int ocnn_csr_transpose(const int32_t* idx, const float* w, const float* norm, int64_t points,
+                       int k, int64_t rows, void* workspace, int64_t workspace_bytes,
+                       int32_t* rowptr, int32_t* col, float* val, void* stream);
+
 /* 2x2x2 max pooling, ocnn/nn/octree_pool.py:16-65.
  * ocnn_max_pool: maximum over the children 8p .. 8p+7 of the p-th non-empty node (first on
  * ties) and its index (indices (parents, c) int64).  fine_child = children of the fine

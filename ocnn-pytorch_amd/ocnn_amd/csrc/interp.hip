@@ -4,6 +4,9 @@
 // element is produced by exactly one thread from a fixed list of inputs (gather form), so
 // nothing here needs atomics and every result is reproducible bit for bit.
 #include <algorithm>
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
 
 #include "common.hpp"
 #include "morton.hpp"
@@ -89,10 +92,13 @@ __global__ void interp_linear_prepare_kernel(const float* __restrict__ pts, int6
 // out[r][c] = (sum_e val[e] * data[col[e]][c]) / (rowdiv[r] + 1e-12), e over the entries of
 // row r: rowptr[r] .. rowptr[r + 1] - 1, or kfixed entries per row.  col < 0 = no entry.
 // fp32 sums in entry order.
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PoolVec { T v[VEC]; };
+
 template <typename T, int VEC>
 __global__ void csr_rows_kernel(const int32_t* __restrict__ rowptr, int kfixed, const int32_t* __restrict__ col,
                                 const float* __restrict__ val, const T* __restrict__ data, int C,
                                 const float* __restrict__ rowdiv, T* __restrict__ out, int64_t rows) {
+  typedef PoolVec<T, VEC> V;
   const int lpr = C / VEC;
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= rows * lpr) return;
@@ -103,20 +109,81 @@ __global__ void csr_rows_kernel(const int32_t* __restrict__ rowptr, int kfixed, 
   float acc[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
-  for (int64_t e = e0; e < e1; ++e) {
+  int64_t e = e0;
+  for (; e + 4 <= e1; e += 4) {                // four rows in flight, added in entry order
+    int32_t cidx[4];
+    float we[4];
+    V q[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      cidx[u] = col[e + u];
+      we[u] = val ? val[e + u] : 1.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (cidx[u] >= 0) q[u] = *(const V*)(data + (int64_t)cidx[u] * C + c0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (cidx[u] >= 0) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] += we[u] * to_f32(q[u].v[v]);
+      }
+  }
+  for (; e < e1; ++e) {
     const int32_t cidx = col[e];
     if (cidx < 0) continue;
     const float we = val ? val[e] : 1.0f;
-    const T* src = data + (int64_t)cidx * C + c0;
+    const V q = *(const V*)(data + (int64_t)cidx * C + c0);
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[v] += we * to_f32(src[v]);
+    for (int v = 0; v < VEC; ++v) acc[v] += we * to_f32(q.v[v]);
   }
   const float div = rowdiv ? rowdiv[r] + 1e-12f : 1.0f;
+  V o;
 #pragma unroll
-  for (int v = 0; v < VEC; ++v) out[r * C + c0 + v] = from_f32<T>(rowdiv ? acc[v] / div : acc[v]);
+  for (int v = 0; v < VEC; ++v) o.v[v] = from_f32<T>(rowdiv ? acc[v] / div : acc[v]);
+  *(V*)(out + r * C + c0) = o;
 }
 
-template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PoolVec { T v[VEC]; };
+// ---- row form of the transposed matrix ------------------------------------------------------
+// Entry e = (point e / k, slot e % k) of idx names data row idx[e] (< 0: none).  Sorted by data
+// row (stable: the points of a row ascend), the entries of row r are rowptr[r] .. rowptr[r + 1].
+struct RowKey {
+  const int32_t* idx;
+  uint32_t rows;
+  __host__ __device__ uint32_t operator()(int64_t e) const {
+    const int32_t v = idx[e];
+    return v < 0 ? rows : (uint32_t)v;
+  }
+};
+
+__global__ void csr_transpose_finish_kernel(const uint32_t* __restrict__ sorted, const int32_t* __restrict__ order,
+                                            int64_t n, int k, uint32_t rows, const float* __restrict__ w,
+                                            const float* __restrict__ norm, int32_t* __restrict__ col,
+                                            float* __restrict__ val) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n || sorted[i] >= rows) return;
+  const int32_t e = order[i];
+  const int32_t p = e / k;
+  col[i] = p;
+  if (val) {
+    const float we = w ? w[e] : 1.0f;
+    val[i] = norm ? we / (norm[p] + 1e-12f) : we;
+  }
+}
+
+__global__ void csr_transpose_rowptr_kernel(const uint32_t* __restrict__ sorted, int64_t n, uint32_t rows,
+                                            int32_t* __restrict__ rowptr) {
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r > rows) return;
+  int64_t lo = 0, hi = n;                       // first entry whose row is at least r
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (sorted[mid] < (uint32_t)r) lo = mid + 1; else hi = mid;
+  }
+  rowptr[r] = (int32_t)lo;
+}
+
+
 
 // Max over the 8 children of a node (first one on ties) and which child it was.
 //   out row r: node r of the coarse level when `coarse_child` is given (rows of empty
@@ -258,14 +325,73 @@ extern "C" int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const
   if (rows == 0) return OCNN_OK;
   hipStream_t st = (hipStream_t)stream;
   OCNN_DISPATCH_DTYPE(dtype, {
-    if (channels % 4 == 0)
-      hipLaunchKernelGGL((csr_rows_kernel<T, 4>), dim3((unsigned)cdiv(rows * (channels / 4), 256)), dim3(256), 0, st,
-                         rowptr, kfixed, col, val, (const T*)data, channels, rowdiv, (T*)out, rows);
+    constexpr int VEC = 16 / sizeof(T);
+    if (channels % VEC == 0 && ((uintptr_t)data % 16) == 0 && ((uintptr_t)out % 16) == 0)
+      hipLaunchKernelGGL((csr_rows_kernel<T, VEC>), dim3((unsigned)cdiv(rows * (channels / VEC), 256)), dim3(256), 0,
+                         st, rowptr, kfixed, col, val, (const T*)data, channels, rowdiv, (T*)out, rows);
     else
       hipLaunchKernelGGL((csr_rows_kernel<T, 1>), dim3((unsigned)cdiv(rows * channels, 256)), dim3(256), 0, st,
                          rowptr, kfixed, col, val, (const T*)data, channels, rowdiv, (T*)out, rows);
   });
   return check_launch("csr_rows");
+}
+
+struct TransposeLayout {
+  int64_t sorted, order, temp, temp_bytes, total;
+};
+
+static int transpose_layout(int64_t n, TransposeLayout* L) {
+  size_t sort_bytes = 0;
+  auto kin = rocprim::make_transform_iterator(rocprim::make_counting_iterator<int64_t>(0), RowKey{nullptr, 0u});
+  auto vin = rocprim::make_counting_iterator<int32_t>(0);
+  if (rocprim::radix_sort_pairs(nullptr, sort_bytes, kin, (uint32_t*)nullptr, vin, (int32_t*)nullptr, (size_t)n, 0,
+                                32) != hipSuccess)
+    return OCNN_ERR_HIP;
+  int64_t off = 0;
+  L->sorted = off; off += align_up(n * 4, 256);
+  L->order = off;  off += align_up(n * 4, 256);
+  L->temp = off;
+  L->temp_bytes = align_up((int64_t)sort_bytes + 256, 256);
+  L->total = off + L->temp_bytes;
+  return OCNN_OK;
+}
+
+extern "C" int64_t ocnn_csr_transpose_workspace_bytes(int64_t entries) {
+  if (entries <= 0) return 256;
+  TransposeLayout L;
+  return transpose_layout(entries, &L) == OCNN_OK ? L.total : (int64_t)-1;
+}
+
+extern "C" int ocnn_csr_transpose(const int32_t* idx, const float* w, const float* norm, int64_t points, int k,
+                                  int64_t rows, void* workspace, int64_t workspace_bytes, int32_t* rowptr,
+                                  int32_t* col, float* val, void* stream) {
+  const int64_t n = points * k;
+  OCNN_REQUIRE(points >= 0 && k >= 1 && rows >= 0 && rows < (1ll << 31) - 1 && n < (1ll << 31),
+               "csr_transpose: points=%lld k=%d rows=%lld out of range", (long long)points, k, (long long)rows);
+  OCNN_REQUIRE((w != nullptr || norm != nullptr) == (val != nullptr),
+               "csr_transpose: values are written exactly when weights or a norm are given");
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  TransposeLayout L;
+  L.sorted = L.order = 0;
+  if (n > 0) {
+    if (transpose_layout(n, &L) != OCNN_OK) { set_error("csr_transpose: rocprim size query failed"); return OCNN_ERR_HIP; }
+    if (workspace_bytes < L.total) { set_error("csr_transpose: workspace %lld < %lld", (long long)workspace_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
+    uint32_t* sorted = (uint32_t*)(ws + L.sorted);
+    int32_t* order = (int32_t*)(ws + L.order);
+    int bits = 1;
+    while ((1ll << bits) <= rows) ++bits;                  // the key `rows` of an empty entry included
+    size_t tb = (size_t)L.temp_bytes;
+    auto kin = rocprim::make_transform_iterator(rocprim::make_counting_iterator<int64_t>(0), RowKey{idx, (uint32_t)rows});
+    auto vin = rocprim::make_counting_iterator<int32_t>(0);
+    hipError_t e = rocprim::radix_sort_pairs(ws + L.temp, tb, kin, sorted, vin, order, (size_t)n, 0u, (unsigned)bits, st);
+    if (e != hipSuccess) { set_error("csr_transpose: radix sort: %s", hipGetErrorString(e)); return OCNN_ERR_HIP; }
+    hipLaunchKernelGGL(csr_transpose_finish_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, sorted, order, n, k,
+                       (uint32_t)rows, w, norm, col, val);
+  }
+  hipLaunchKernelGGL(csr_transpose_rowptr_kernel, dim3((unsigned)cdiv(rows + 1, 256)), dim3(256), 0, st,
+                     (const uint32_t*)(ws + L.sorted), n, (uint32_t)rows, rowptr);
+  return check_launch("csr_transpose");
 }
 
 extern "C" int ocnn_max_pool(int dtype, const void* data, const int32_t* fine_child, const int32_t* coarse_child,

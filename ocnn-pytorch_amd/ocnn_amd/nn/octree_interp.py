@@ -20,21 +20,18 @@ def _csr_rows(data, col, val, rowptr, kfixed, rowdiv, rows):
   return out
 
 
-def _transpose(idx, w, rows):
+def _transpose(idx, w, norm, rows):
   """Row form of the transposed matrix of (point, neighbour) entries: for every data row the
-  points that read it (ascending) and their weights."""
-  flat = idx.reshape(-1)
-  k = idx.shape[1]
-  valid = flat >= 0
-  order = torch.argsort(torch.where(valid, flat, torch.full_like(flat, rows)), stable=True)
-  n = int(valid.sum())
-  order = order[:n]
-  col = torch.div(order, k, rounding_mode='floor').to(torch.int32)
-  val = None if w is None else w.reshape(-1)[order].contiguous()
-  counts = torch.bincount(flat[order].long(), minlength=rows)
-  rowptr = torch.zeros(rows + 1, dtype=torch.int32, device=idx.device)
-  rowptr[1:] = counts.cumsum(0)
-  return rowptr, col.contiguous(), val
+  points that read it (ascending) and their weights, divided by the points' weight sums."""
+  L = _lib.lib()
+  m, k = idx.shape
+  ws = _lib.workspace(L.ocnn_csr_transpose_workspace_bytes(m * k), idx.device)
+  rowptr = torch.empty(rows + 1, dtype=torch.int32, device=idx.device)
+  col = torch.empty(m * k, dtype=torch.int32, device=idx.device)
+  val = None if w is None and norm is None else torch.empty(m * k, dtype=torch.float32, device=idx.device)
+  _lib.check(L.ocnn_csr_transpose(_lib.ptr(idx), _lib.ptr(w), _lib.ptr(norm), m, k, rows, _lib.ptr(ws),
+                                  ws.numel(), _lib.ptr(rowptr), _lib.ptr(col), _lib.ptr(val), _lib.stream()))
+  return rowptr, col, val
 
 
 class _Interp(torch.autograd.Function):
@@ -50,11 +47,8 @@ class _Interp(torch.autograd.Function):
   @staticmethod
   def backward(ctx, grad):
     idx, w, norm = ctx.saved_tensors
-    grad = grad.contiguous()
-    if norm is not None:
-      grad = (grad / (norm.unsqueeze(1) + 1e-12).to(grad.dtype)).contiguous()
-    rowptr, col, val = _transpose(idx, w, ctx.rows)
-    return _csr_rows(grad, col, val, rowptr, 0, None, ctx.rows), None, None, None
+    rowptr, col, val = _transpose(idx, w, norm, ctx.rows)
+    return _csr_rows(grad.contiguous(), col, val, rowptr, 0, None, ctx.rows), None, None, None
 
 
 def _keys(octree, depth, nempty):
