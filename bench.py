@@ -128,6 +128,20 @@ def cpu_baseline(torch, table32, rows_in, cin, cout, sample_rows):
   }
 
 
+def cpu_baseline_octree(pts, nrm, bid, depth, batch):
+  """The octree construction and the neighbour search of the same clouds on the host: the oracle's
+  numpy restatement of ocnn/octree/octree.py:201-287 and :404-446 (one thread), one run each."""
+  from oracle import octree_ref
+  t0 = time.perf_counter()
+  o, _ = octree_ref.build_octree(pts.numpy(), nrm.numpy(), None, None if bid is None else bid.numpy(), depth, 2,
+                                 batch)
+  t1 = time.perf_counter()
+  octree_ref.construct_all_neigh(o)
+  t2 = time.perf_counter()
+  return {'build_octree_ms': (t1 - t0) * 1e3, 'construct_all_neigh_ms': (t2 - t1) * 1e3, 'cores': 1, 'kind': 'port',
+          'sample': 'all {} points, depth {}, batch {}; numpy, one run'.format(pts.shape[0], depth, batch)}
+
+
 def main():
   args = parse()
   if args.gpus != 1:
@@ -155,8 +169,11 @@ def main():
 
   # ---- inputs: synthetic clouds -> octree (timed separately) ----------------
   build_octree(torch, synthetic, Octree, Points, synthetic.mixed_cloud, args.batch, 1001, args.points, depth, dev, 1)
-  octree, build_ms, neigh_ms, pts, _, pc = build_octree(torch, synthetic, Octree, Points, synthetic.mixed_cloud,
-                                                        args.batch, 1001, args.points, depth, dev)
+  octree, build_ms, neigh_ms, pts, bid, pc = build_octree(torch, synthetic, Octree, Points, synthetic.mixed_cloud,
+                                                          args.batch, 1001, args.points, depth, dev)
+  # every table written once, the parents' rows and the children read once
+  neigh_bytes = sum(int(octree.nnum[d]) * 27 * 4 + int(octree.nnum_nempty[d - 1]) * 27 * 4 + int(octree.nnum[d - 1]) * 4
+                    for d in range(1, depth + 1))
   table = octree._table(depth, '333', 1, nempty)
   rows = table.shape[0]
   nnz = int((table >= 0).sum())
@@ -315,6 +332,8 @@ def main():
           'points': int(pts.shape[0]),
           'build_octree_ms': build_ms,
           'construct_all_neigh_ms': neigh_ms,
+          'construct_all_neigh_algorithmic_bytes': neigh_bytes,
+          'construct_all_neigh_hbm_frac': neigh_bytes / (neigh_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
           'tile_plan_ms_per_table': min(plan_ms),
           'nnum': octree.nnum.tolist(),
           'nnum_nempty': octree.nnum_nempty.tolist(),
@@ -404,6 +423,8 @@ def main():
 
   if not args.no_cpu:
     result['cpu_baseline'] = cpu_baseline(torch, table, rows, C, C, args.cpu_rows)
+    result['cpu_baseline']['octree'] = cpu_baseline_octree(pts, pc.normals.cpu(), bid if args.batch > 1 else None,
+                                                           depth, args.batch)
   print(json.dumps(result))
 
 
