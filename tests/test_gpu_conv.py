@@ -1273,7 +1273,8 @@ def test_layers_replay_from_a_hip_graph(medium, kind, ks, stride, nempty, cin, c
       out = step()                                    # plans, tables and workspaces exist from here on
   torch.cuda.current_stream().wait_stream(side)
   torch.cuda.synchronize()
-  want = [out.clone()] + [p.grad.clone() for p in params]
+  want = [out.detach().clone()] + [p.grad.clone() for p in params]
+  del out                              # no autograd graph of the eager runs (and its stream) stays alive
   graph = torch.cuda.CUDAGraph()
   for p in params:
     p.grad = None
