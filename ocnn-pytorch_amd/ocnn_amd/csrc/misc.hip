@@ -337,6 +337,38 @@ __global__ __launch_bounds__(256) void colsum_rows_kernel(const T* __restrict__ 
   }
 }
 
+// Few channels that do not fill 16-byte pieces (C <= 256): the split's elements as one flat run,
+// (256 / C) C threads walk it with that stride, so that a thread stays on one channel and a wave
+// reads consecutive elements; eight loads in flight; threads of a channel meet in LDS, in thread order.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_flat_kernel(const T* __restrict__ g, int64_t rows, int C,
+                                                          int64_t rows_per_split, float* __restrict__ partial) {
+  __shared__ float s_acc[256];
+  const int active = (256 / C) * C;
+  const int64_t r_begin = (int64_t)blockIdx.x * rows_per_split;
+  const int64_t r_end = min(rows, r_begin + rows_per_split);
+  const int64_t f_end = r_end * C;
+  float acc = 0.f;
+  if ((int)threadIdx.x < active) {
+    int64_t f = r_begin * C + threadIdx.x;
+    for (; f + 7 * (int64_t)active < f_end; f += 8 * (int64_t)active) {
+      T q[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) q[u] = g[f + u * (int64_t)active];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += to_f32(q[u]);
+    }
+    for (; f < f_end; f += active) acc += to_f32(g[f]);
+  }
+  s_acc[threadIdx.x] = acc;
+  __syncthreads();
+  if ((int)threadIdx.x < C) {
+    float sum = 0.f;
+    for (int t = threadIdx.x; t < active; t += C) sum += s_acc[t];
+    partial[(int64_t)blockIdx.x * C + threadIdx.x] = sum;
+  }
+}
+
 // out[c] = sum over the splits, 16 split lanes a channel, each adding every 16th split in order,
 // the lanes then in lane order
 template <typename T>
@@ -539,6 +571,9 @@ extern "C" int ocnn_colsum(int dtype, const void* g, int64_t rows, int channels,
     if (rows > 0) {
       if (channels % VEC == 0 && ((uintptr_t)g % 16) == 0)
         hipLaunchKernelGGL(colsum_rows_kernel<T>, dim3((unsigned)splits), dim3(256), 0, st, (const T*)g, rows,
+                           channels, rps, partial);
+      else if (channels <= 256)
+        hipLaunchKernelGGL(colsum_flat_kernel<T>, dim3((unsigned)splits), dim3(256), 0, st, (const T*)g, rows,
                            channels, rps, partial);
       else
         hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)splits), dim3(256), 0, st, (const T*)g,

@@ -1292,3 +1292,21 @@ def test_layers_replay_from_a_hip_graph(medium, kind, ks, stride, nempty, cin, c
     got = [out_g] + [p.grad for p in params]
     for a, b in zip(want, got):
       assert torch.equal(a, b), (replay, kind)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_column_sums(dtype):
+  """The bias gradient's column sums on each of its three kernels (16-byte pieces, the flat run
+  for few channels, one channel per lane) against an fp64 sum, and the same bits on a second run."""
+  from ocnn_amd.nn.octree_conv import column_sum
+  g = torch.Generator().manual_seed(3)
+  for rows, C in [(1, 1), (7, 3), (1000, 4), (30011, 5), (4097, 7), (50000, 12), (2500, 40), (999, 100),
+                  (70000, 64), (1234, 96), (300, 257), (513, 300), (100000, 8)]:
+    say('column sums', dtype, rows, C)
+    x = torch.randn(rows, C, generator=g).to(dtype).to(DEV)
+    got = column_sum(x)
+    want = x.double().sum(0)
+    tol = 1e-5 if dtype == torch.float32 else 4e-3
+    assert got.dtype == dtype and tuple(got.shape) == (C,)
+    assert float((got.double() - want).abs().max()) <= tol * max(1.0, float(want.abs().max())) + tol * rows ** 0.5
+    assert torch.equal(got, column_sum(x))
