@@ -194,11 +194,11 @@ int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in,
  *   count: ucount[tile] = number of distinct rows        (tiles = ceil(rows / R));
  *          tile_nnz[tile] (may be NULL) = entries of the tile that hold a row;
  *   offsets: uptr (tiles + 1) = exclusive prefix sum of ucount, and what the host needs to
- *          size the lists, stats (device, 5 x int64) = [tiles with more than cap distinct
- *          rows, dropped (0 | 1), total, largest count, entries set].  When the tiles over
- *          cap are few (at most a tenth of the tiles, at least one) they are dropped: they
- *          count as empty in uptr and in the last three figures, and the caller runs their
- *          rows without the plan;
+ *          size the lists, stats (device, 6 x int64) = [tiles with more than cap distinct
+ *          rows, dropped (0 | 1), total, largest count, entries set, tiles the one-pass
+ *          build gave up on].  When the tiles over cap are few (at most a tenth of the
+ *          tiles, at least one) they are dropped: they count as empty in uptr and in the
+ *          third to fifth figure, and the caller runs their rows without the plan;
  *   fill : uptr as made by offsets (or by the caller);
  *          urows[uptr[tile] + u] = u-th distinct row; loc (tiles, K, R) uint16:
  *          loc[tile][k][r] = 1 + position of table[tile * R + r][k], or 0 for -1 and
@@ -218,7 +218,10 @@ int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, const int32_t
  * ocnn_tile_plan_offsets as above; ocnn_tile_plan_compact moves the lists to their offsets
  * and clears the positions of the tiles the offsets dropped (stats: the device vector that
  * ocnn_tile_plan_offsets wrote; cap <= pad).  A plan whose largest count (stats[3]) exceeds
- * `pad` is filled with ocnn_tile_plan_fill instead. */
+ * `pad` is filled with ocnn_tile_plan_fill instead.  The build keeps a tile's distinct rows
+ * in a small set (1024 blocks of 32 row numbers; the tiles of an octree table use a tenth),
+ * so that four tiles share a CU: a tile that does not fit gets the count 2^20 and is counted
+ * in stats[5]; such a table (one without locality) is planned with count, offsets and fill. */
 int ocnn_tile_plan_build(const int32_t* table, int64_t rows, int K, int pad, int32_t* ucount,
                          int32_t* tile_nnz, int32_t* ulist, uint16_t* loc, void* stream);
 int ocnn_tile_plan_compact(const int32_t* ucount, const int32_t* uptr, const int64_t* stats, int cap,

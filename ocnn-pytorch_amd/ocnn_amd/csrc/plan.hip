@@ -11,12 +11,18 @@ namespace ocnn {
 
 constexpr int kPlanRows = 128;          // table rows per tile
 constexpr int kPlanMaxEntries = 4096;   // >= kPlanRows * 27, power of two
-constexpr int kPlanHash = 4096;         // open-addressing slots (an octree table fills a tenth; at most 84 %)
+constexpr int kPlanHash = 4096;         // open-addressing slots that hold any tile (at most 84 % full)
+constexpr int kPlanHashQuick = 1024;    // slots of the one-pass build: an octree table fills a tenth of them, and
+                                        // with 20 KiB of LDS instead of 72 four tiles share a CU instead of two
 constexpr int kPlanRankMax = 1024;      // up to here the distinct rows are ordered by counting
 constexpr int kPlanThreads = 512;       // threads a tile: the kernel waits on LDS round trips, more waves hide them
+constexpr int kPlanOverflow = 1 << 20;  // count of a tile whose blocks did not fit the quick build's slots
+constexpr int kPlanPosWords = (27 * (kPlanRows + 8) + 1) / 2;   // the staged positions, in 32-bit words
 
+template <int HASH>
 __device__ __forceinline__ int plan_hash(int32_t v) {
-  return (int)(((uint32_t)v * 2654435761u) >> 20);      // 12 bits
+  static_assert(HASH == 4096 || HASH == 1024, "12 or 10 bits");
+  return (int)(((uint32_t)v * 2654435761u) >> (HASH == 4096 ? 20 : 22));
 }
 
 // mode 0: ucount[tile] = number of distinct valid entries, tile_nnz[tile] = valid entries
@@ -32,17 +38,22 @@ __device__ __forceinline__ int plan_hash(int32_t v) {
 // then means ordering the blocks (a tenth as many: by counting, no barriers; tables without
 // locality: by a bitonic sort) and counting bits: the position of a row is the number of rows
 // in smaller blocks plus the bits below its own in its block's mask.
+//
+// HASH = kPlanHashQuick (mode 2 only): a tile whose blocks do not fit gives up, ucount[tile] =
+// kPlanOverflow; the caller then plans the table in two passes with HASH = kPlanHash.
+template <int HASH>
 __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     const int32_t* __restrict__ table, int64_t rows, int K, int mode,
     int32_t* __restrict__ ucount, const int32_t* __restrict__ uptr, int32_t* __restrict__ urows,
     uint16_t* __restrict__ loc, int32_t* __restrict__ tile_nnz, int pad) {
-  __shared__ int32_t s_key[kPlanHash];                    // block number, -1 = free
-  __shared__ uint32_t s_mask[kPlanHash];                  // its rows
-  __shared__ uint16_t s_base[kPlanHash];                  // rows in smaller blocks
-  __shared__ __attribute__((aligned(16))) int32_t s_uq[kPlanMaxEntries];   // the blocks; later: the positions, [slot][row]
-  __shared__ __attribute__((aligned(16))) int32_t s_w[kPlanMaxEntries];    // rows of each of them
+  constexpr int kList = HASH == kPlanHash ? kPlanMaxEntries : (HASH + 16 > kPlanPosWords ? HASH + 16 : kPlanPosWords);
+  __shared__ int32_t s_key[HASH];                         // block number, -1 = free
+  __shared__ uint32_t s_mask[HASH];                       // its rows
+  __shared__ uint16_t s_base[HASH];                       // rows in smaller blocks
+  __shared__ __attribute__((aligned(16))) int32_t s_uq[(kList + 15) & ~15];   // the blocks; later: the positions, [slot][row]
+  __shared__ __attribute__((aligned(16))) int32_t s_w[HASH == kPlanHash ? kPlanMaxEntries : HASH + 16];   // rows of each of them
   __shared__ int32_t s_scan[2][kPlanThreads / 64];
-  __shared__ int32_t s_nnz;
+  __shared__ int32_t s_nnz, s_over;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t tile = blockIdx.x;
   const int64_t e0 = tile * kPlanRows * K;
@@ -57,11 +68,14 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
     const int e = tid + kPlanThreads * i;
     ent[i] = (e < n && e0 + e < lim) ? table[e0 + e] : -1;
   }
-  for (int i = tid; i < kPlanHash; i += kPlanThreads) {
+  for (int i = tid; i < HASH; i += kPlanThreads) {
     s_key[i] = -1;
     s_mask[i] = 0u;
   }
-  if (tid == 0) s_nnz = 0;
+  if (tid == 0) {
+    s_nnz = 0;
+    s_over = 0;
+  }
   __syncthreads();
   if (mode != 1 && tile_nnz != nullptr) {
     int set = 0;
@@ -81,22 +95,37 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
       // block and bit in place
       const int32_t blk = v >> 5;
       const uint32_t bit = 1u << (v & 31);
-      int h = plan_hash(blk);
-      while (true) {
+      int h = plan_hash<HASH>(blk);
+      bool found = true;
+      for (int probes = 0;; ++probes) {
         int32_t old = ((volatile int32_t*)s_key)[h];
         if (old == -1) old = atomicCAS(&s_key[h], -1, blk);
         if (old == -1 || old == blk) break;
-        h = (h + 1) & (kPlanHash - 1);
+        if (HASH != kPlanHash && probes >= HASH - 1) {     // every slot holds another block
+          found = false;
+          s_over = 1;
+          break;
+        }
+        h = (h + 1) & (HASH - 1);
       }
-      if ((((volatile uint32_t*)s_mask)[h] & bit) == 0u) atomicOr(&s_mask[h], bit);
-      slot[i] = h;
+      if (found) {
+        if ((((volatile uint32_t*)s_mask)[h] & bit) == 0u) atomicOr(&s_mask[h], bit);
+        slot[i] = h;
+      }
     }
   }
   __syncthreads();
+  if (HASH != kPlanHash && s_over != 0) {
+    if (tid == 0) {
+      ucount[tile] = kPlanOverflow;
+      if (tile_nnz != nullptr) tile_nnz[tile] = s_nnz;
+    }
+    return;
+  }
   // occupied slots: per-thread counts of blocks and rows (slots tid, tid + kPlanThreads, ..: the
   // order of the blocks does not matter before they are ranked), scanned within a wave by lane
   // exchanges, across the waves through LDS
-  constexpr int per = kPlanHash / kPlanThreads;
+  constexpr int per = HASH / kPlanThreads;
   int32_t held[per];
   uint32_t hmask[per];
   int cnt = 0, nrows = 0;
@@ -145,8 +174,8 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
   __syncthreads();
   const int64_t ub = mode == 1 ? (int64_t)uptr[tile] : tile * (int64_t)pad;
   auto slot_of = [&](int32_t blk) {
-    int h = plan_hash(blk);
-    while (s_key[h] != blk) h = (h + 1) & (kPlanHash - 1);
+    int h = plan_hash<HASH>(blk);
+    while (s_key[h] != blk) h = (h + 1) & (HASH - 1);
     return h;
   };
   // a block's rows go to the list from `base` on, in the order of their bits
@@ -161,7 +190,7 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
       }
     }
   };
-  if (nblk <= kPlanRankMax) {
+  if (HASH <= kPlanRankMax || nblk <= kPlanRankMax) {
     // rows before a block = rows of the smaller blocks
     const int tpad = (nblk + 15) & ~15;                   // whole groups of 16; the padding ranks last and weighs nothing
     for (int e = nblk + tid; e < tpad; e += kPlanThreads) {
@@ -187,7 +216,7 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
       }
       put_block(v, slot_of(v), r);
     }
-  } else {
+  } else if constexpr (HASH > kPlanRankMax) {
     int npad = kPlanRankMax * 2;
     while (npad < nblk) npad <<= 1;
     for (int e = nblk + tid; e < npad; e += kPlanThreads) s_uq[e] = 0x7fffffff;
@@ -302,13 +331,14 @@ __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles
 // What the host needs to know of the counts, and the offsets of the row lists, in one
 // workgroup (a table has tens of thousands of tiles at most).  Tiles with more than `cap`
 // distinct rows are dropped (counted as empty) when they are few: at most a tenth of the
-// tiles.  stats: [tiles over cap, dropped (0 | 1), total, largest count, entries set], the
-// last three without the dropped tiles.
+// tiles.  stats: [tiles over cap, dropped (0 | 1), total, largest count, entries set, tiles the
+// quick one-pass build gave up on (then nothing else here means anything)], the third to fifth
+// without the dropped tiles.
 __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     const int32_t* __restrict__ ucount, const int32_t* __restrict__ tile_nnz, int64_t tiles, int cap,
     int32_t* __restrict__ uptr, int64_t* __restrict__ stats) {
   __shared__ long long s_wsum[16], s_wnnz[16];
-  __shared__ int s_wbig[16], s_wmax[16];
+  __shared__ int s_wbig[16], s_wover[16], s_wmax[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t per = (tiles + 1023) / 1024;
   const int64_t t0 = min(tiles, tid * per), t1 = min(tiles, t0 + per);
@@ -319,20 +349,31 @@ __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     return v;
   };
-  int big = 0;
-  for (int64_t t = t0; t < t1; ++t) big += ucount[t] > cap ? 1 : 0;
+  int big = 0, over = 0;
+  for (int64_t t = t0; t < t1; ++t) {
+    const int c = ucount[t];
+    big += c > cap && c < kPlanOverflow ? 1 : 0;
+    over += c >= kPlanOverflow ? 1 : 0;
+  }
   big = (int)wave_sum(big);
-  if (lane == 0) s_wbig[wave] = big;
+  over = (int)wave_sum(over);
+  if (lane == 0) {
+    s_wbig[wave] = big;
+    s_wover[wave] = over;
+  }
   __syncthreads();
-  int n_big = 0;
+  int n_big = 0, n_over = 0;
 #pragma unroll
-  for (int w = 0; w < 16; ++w) n_big += s_wbig[w];
+  for (int w = 0; w < 16; ++w) {
+    n_big += s_wbig[w];
+    n_over += s_wover[w];
+  }
   const bool drop = n_big > 0 && n_big <= max((int64_t)1, tiles / 10);
   long long sum = 0, nnz = 0;
   int mx = 0;
   for (int64_t t = t0; t < t1; ++t) {
     const int c = ucount[t];
-    if (drop && c > cap) continue;
+    if ((drop && c > cap) || c >= kPlanOverflow) continue;
     sum += c;
     mx = max(mx, c);
     nnz += tile_nnz[t];
@@ -364,7 +405,7 @@ __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
   for (int64_t t = t0; t < t1; ++t) {
     uptr[t] = (int32_t)at;
     const int c = ucount[t];
-    at += (drop && c > cap) ? 0 : c;
+    at += ((drop && c > cap) || c >= kPlanOverflow) ? 0 : c;
   }
   if (tid == 1023) {
     uptr[tiles] = (int32_t)total;
@@ -373,6 +414,7 @@ __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     stats[2] = total;
     stats[3] = max_all;
     stats[4] = nnz_all;
+    stats[5] = n_over;
   }
 }
 
@@ -438,8 +480,12 @@ static int plan_launch(const int32_t* table, int64_t rows, int K, int mode, int3
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows >= 0 && rows < (1ll << 31), "tile_plan: bad shape");
   if (rows == 0) return OCNN_OK;
   int64_t tiles = cdiv(rows, kPlanRows);
-  hipLaunchKernelGGL(tile_plan_kernel, dim3((unsigned)tiles), dim3(kPlanThreads), 0, (hipStream_t)stream,
-                     table, rows, K, mode, ucount, uptr, urows, loc, tile_nnz, pad);
+  if (mode == 2)
+    hipLaunchKernelGGL(tile_plan_kernel<kPlanHashQuick>, dim3((unsigned)tiles), dim3(kPlanThreads), 0,
+                       (hipStream_t)stream, table, rows, K, mode, ucount, uptr, urows, loc, tile_nnz, pad);
+  else
+    hipLaunchKernelGGL(tile_plan_kernel<kPlanHash>, dim3((unsigned)tiles), dim3(kPlanThreads), 0,
+                       (hipStream_t)stream, table, rows, K, mode, ucount, uptr, urows, loc, tile_nnz, pad);
   return check_launch("tile_plan");
 }
 

@@ -124,7 +124,15 @@ class TilePlan:
 
   def __init__(self, table: torch.Tensor, cap: int = None):
     self._count(table, cap)
-    self._finish([int(v) for v in self._stats.tolist()])
+    self._finish(self._host_stats(self._stats.tolist(), table, cap))
+
+  def _host_stats(self, stats, table, cap):
+    """The sizes on the host; a table the one-pass build gave up on (tiles with more distinct
+    blocks of rows than its set holds: no locality) is counted again the long way first."""
+    if stats[5]:
+      self._count(table, cap, one_pass=False)
+      stats = self._stats.tolist()
+    return [int(v) for v in stats]
 
   @classmethod
   def build_many(cls, tables, cap: int = None):
@@ -133,11 +141,11 @@ class TilePlan:
     for p, t in zip(plans, tables):
       p._count(t, cap)
     host = torch.stack([p._stats for p in plans]).tolist() if plans else []
-    for p, st in zip(plans, host):
-      p._finish([int(v) for v in st])
+    for p, t, st in zip(plans, tables, host):
+      p._finish(p._host_stats(st, t, cap))
     return plans
 
-  def _count(self, table, cap):
+  def _count(self, table, cap, one_pass=True):
     """First half: distinct rows per tile, their offsets, and the sizes the second half
     needs on the host as one device vector."""
     _lib.require_gpu(table)
@@ -156,12 +164,12 @@ class TilePlan:
     self._ucount = torch.empty(tiles, dtype=torch.int32, device=dev)
     tile_nnz = torch.empty(tiles, dtype=torch.int32, device=dev)
     self.uptr = torch.empty(tiles + 1, dtype=torch.int32, device=dev)
-    self._stats = torch.empty(5, dtype=torch.int64, device=dev)
+    self._stats = torch.empty(6, dtype=torch.int64, device=dev)
     # One pass over the table: counts, positions and the lists at fixed places (LIST_PAD rows a
     # tile); the second half only moves the lists to their offsets.  (A limit above LIST_PAD, or
     # a table whose tiles do not fit it, takes the two passes of count and fill.)
     self._lists = None
-    if self._cap <= self.LIST_PAD:
+    if one_pass and self._cap <= self.LIST_PAD:
       self._lists = torch.empty(max(tiles, 1) * self.LIST_PAD, dtype=torch.int32, device=dev)
       # uint16 payload, [tile][slot][row in tile]: whole tiles, the tail reads "empty"
       self.loc = torch.empty((tiles, K, self._tile_rows), dtype=torch.int16, device=dev)
@@ -179,7 +187,7 @@ class TilePlan:
     rows, K = self.rows, self.K
     tiles = self._ucount.numel()
     dev = table.device
-    _, dropped, total, umax, nnz = stats
+    _, dropped, total, umax, nnz = stats[:5]
     one_pass = self._lists is not None and umax <= self.LIST_PAD
     if dropped:
       big = self._ucount > self._cap

@@ -362,6 +362,47 @@ def test_tile_plan_reconstructs_table(medium):
       assert np.array_equal(u[lb[blk >= 0] - 1], blk[blk >= 0])
 
 
+def test_tile_plan_of_tables_without_locality():
+  """Tiles whose entries name thousands of scattered rows do not fit the small set of the
+  one-pass build: the plan is then built the long way and still reproduces the table, whether
+  all tiles are like that or a few among local ones (those few are dropped from the plan and
+  listed as overflow rows)."""
+  from ocnn_amd.octree.octree import TilePlan
+  R = _lib.lib().ocnn_tile_plan_rows()
+  g = torch.Generator().manual_seed(17)
+  rows, K = 40 * R + 37, 27
+  scattered = torch.randint(0, 1 << 20, (rows, K), generator=g, dtype=torch.int32)
+  scattered[torch.rand(rows, K, generator=g) < 0.2] = -1
+  local = (torch.arange(rows, dtype=torch.int32).view(-1, 1) + torch.randint(-60, 60, (rows, K), generator=g,
+                                                                              dtype=torch.int32)).clamp_(0, rows - 1)
+  mixed = local.clone()
+  mixed[3 * R:4 * R] = scattered[3 * R:4 * R]
+  mixed[17 * R:18 * R] = scattered[17 * R:18 * R]
+  for name, t in (('scattered', scattered), ('mixed', mixed), ('local', local)):
+    say('tile plan without locality:', name)
+    plan = TilePlan(t.to(DEV))
+    tab = t.numpy().copy()
+    if name == 'mixed':
+      want = np.concatenate([np.arange(3 * R, 4 * R), np.arange(17 * R, 18 * R)])
+      assert np.array_equal(plan.overflow_rows.cpu().numpy(), want)
+      assert np.array_equal(plan.overflow_table.cpu().numpy(), tab[want])
+      tab[want] = -1                                         # those tiles are empty in the plan
+    else:
+      assert plan.overflow_rows is None
+    assert (plan.umax > TilePlan.CAP) == (name == 'scattered')
+    loc = plan.loc.cpu().numpy().view(np.uint16)
+    uptr = plan.uptr.cpu().numpy()
+    urows = plan.urows.cpu().numpy()
+    assert uptr[0] == 0 and uptr[-1] == plan.total
+    for tile in range((rows + R - 1) // R):
+      blk = tab[tile * R:(tile + 1) * R]
+      u = urows[uptr[tile]:uptr[tile + 1]]
+      assert np.array_equal(u, np.unique(blk[blk >= 0])), (name, tile)
+      lb = loc[tile].T[:blk.shape[0]]
+      assert np.array_equal(lb == 0, blk < 0)
+      assert np.array_equal(u[lb[blk >= 0] - 1], blk[blk >= 0])
+
+
 def _same_plan(a, b):
   assert (a.rows, a.K, a.total, a.umax, a.nnz) == (b.rows, b.K, b.total, b.umax, b.nnz)
   assert torch.equal(a.uptr, b.uptr) and torch.equal(a.urows[:a.total], b.urows[:b.total]) and torch.equal(a.loc, b.loc)
