@@ -134,6 +134,14 @@ int ocnn_neigh_from_parent(const int32_t* child_p, const int32_t* neigh_p,
                            const int32_t* nempty_p, int64_t n_ne,
                            int64_t* out64, int32_t* out32, void* stream);
 
+/* construct_all_neigh (ocnn/octree/octree.py:443-446) as one call: layers 1 .. depth in turn,
+ * ocnn_neigh_full up to full_depth, then ocnn_nempty_index of the layer above (written to
+ * h_nempty_index[d - 1], int32) and ocnn_neigh_from_parent.  h_*: host arrays indexed by depth
+ * (depth + 1 entries; node counts, children, outputs); tables int32 (nnum[d], 27). */
+int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_t* h_nnum,
+                   const int64_t* h_nnum_nempty, const int32_t* const* h_children,
+                   int32_t* const* h_nempty_index, int32_t* const* h_neigh, void* stream);
+
 /* Host evaluation of the arithmetic that replaces the reference's lut_parent /
  * lut_child tables (ocnn/octree/octree.py:87-95) inside the kernel above. */
 void ocnn_host_child_slot_lut(int j, int k, int* lut_parent, int* lut_child);

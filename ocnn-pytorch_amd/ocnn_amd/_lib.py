@@ -32,6 +32,7 @@ SIGNATURES = {
     'ocnn_leaf_average': (_i, [_p, _i, _p, _p, _l, _i, _p, _p]),
     'ocnn_neigh_full': (_i, [_i, _i, _p, _p, _p]),
     'ocnn_neigh_from_parent': (_i, [_p, _p, _p, _l, _p, _p, _p]),
+    'ocnn_neigh_all': (_i, [_i, _i, _i, _p, _p, _p, _p, _p, _p]),
     'ocnn_host_child_slot_lut': (None, [_i, _i, POINTER(_i), POINTER(_i)]),
     'ocnn_nempty_index': (_i, [_p, _l, _p, _p, _p]),
     'ocnn_neigh_select': (_i, [_p, _p, _i, _p, POINTER(_i), _i, _l, _p, _p, _p]),

@@ -161,6 +161,34 @@ extern "C" int ocnn_neigh_from_parent(const int32_t* child_p, const int32_t* nei
   return check_launch("neigh_from_parent");
 }
 
+// All tables of an octree with one call: the launches of the shallow layers, a few microseconds
+// each, then follow each other without the host between them.
+extern "C" int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_t* h_nnum,
+                              const int64_t* h_nnum_nempty, const int32_t* const* h_children,
+                              int32_t* const* h_nempty_index, int32_t* const* h_neigh, void* stream) {
+  OCNN_REQUIRE(depth >= 1 && depth <= 16 && full_depth >= 0 && full_depth <= depth && full_depth <= 7 && batch >= 1,
+               "neigh_all: depth=%d full_depth=%d batch=%d", depth, full_depth, batch);
+  hipStream_t st = (hipStream_t)stream;
+  for (int d = 1; d <= depth; ++d) {
+    OCNN_REQUIRE(h_neigh[d] != nullptr && h_nnum[d] > 0 && h_nnum[d] * 27 < (1ll << 31), "neigh_all: layer %d", d);
+    if (d <= full_depth) {
+      const int64_t total = (int64_t)batch << (3 * d);
+      OCNN_REQUIRE(h_nnum[d] == total, "neigh_all: layer %d is not full", d);
+      hipLaunchKernelGGL(neigh_full_kernel, dim3((unsigned)cdiv(total * 27, 256)), dim3(256), 0, st, d, total,
+                         (int64_t*)nullptr, h_neigh[d]);
+      continue;
+    }
+    const int64_t n_ne = h_nnum_nempty[d - 1];
+    OCNN_REQUIRE(n_ne > 0 && 8 * n_ne == h_nnum[d] && h_children[d - 1] && h_nempty_index[d - 1],
+                 "neigh_all: layers %d and %d are inconsistent", d - 1, d);
+    hipLaunchKernelGGL(nempty_index_kernel, dim3((unsigned)cdiv(h_nnum[d - 1], 256)), dim3(256), 0, st,
+                       h_children[d - 1], h_nnum[d - 1], h_nempty_index[d - 1], (int64_t*)nullptr);
+    hipLaunchKernelGGL(neigh_from_parent_kernel, dim3((unsigned)cdiv(n_ne, kParentsPerBlock)), dim3(256), 0, st,
+                       h_children[d - 1], h_neigh[d - 1], h_nempty_index[d - 1], n_ne, (int64_t*)nullptr, h_neigh[d]);
+  }
+  return check_launch("neigh_all");
+}
+
 extern "C" int ocnn_nempty_index(const int32_t* children, int64_t n, int32_t* index32,
                                  int64_t* index64, void* stream) {
   if (n <= 0) return OCNN_OK;

@@ -421,7 +421,10 @@ class Octree:
 
   def nempty_index(self, depth: int, reset: bool = False):
     if self.nempty_indices[depth] is None or reset:
-      self._make_nempty_index(depth)
+      if not reset and self._nempty_indices32[depth] is not None:
+        self.nempty_indices[depth] = self._nempty_indices32[depth].long()
+      else:
+        self._make_nempty_index(depth)
     return self.nempty_indices[depth]
 
   def _nempty_index32(self, depth):
@@ -640,8 +643,34 @@ class Octree:
     self._drop_tables(depth)
 
   def construct_all_neigh(self):
-    for depth in range(1, self.depth + 1):
-      self.construct_neigh(depth)
+    """All tables with one library call (ocnn/octree/octree.py:443-446): the launches of the
+    shallow layers follow each other without the host in between."""
+    dev = torch.device(self.device) if isinstance(self.device, str) else self.device
+    depth = self.depth
+    nnum = [int(v) for v in self.nnum[:depth + 1].tolist()]
+    nempty = [int(v) for v in self.nnum_nempty[:depth + 1].tolist()]
+    if dev.type != 'cuda' or any(c is None for c in self.children[:depth + 1]) or min(nnum[1:] + nempty) <= 0 or \
+        any(nnum[d] != (self.batch_size << (3 * d) if d <= self.full_depth else 8 * nempty[d - 1])
+            for d in range(1, depth + 1)):
+      for d in range(1, depth + 1):                       # the layer-by-layer route says what is wrong
+        self.construct_neigh(d)
+      return
+    neigh = [None] + [torch.empty(nnum[d], 27, dtype=torch.int32, device=dev) for d in range(1, depth + 1)]
+    index = [torch.empty(nempty[d], dtype=torch.int32, device=dev) if self.full_depth <= d < depth else None
+             for d in range(depth + 1)]
+    ptrs = lambda ts: (ctypes.c_void_p * (depth + 1))(*[None if t is None else t.data_ptr() for t in ts])
+    with torch.cuda.device(dev):
+      _lib.check(_lib.lib().ocnn_neigh_all(depth, self.full_depth, self.batch_size,
+                                           (ctypes.c_int64 * (depth + 1))(*nnum),
+                                           (ctypes.c_int64 * (depth + 1))(*nempty), ptrs(self.children[:depth + 1]),
+                                           ptrs(index), ptrs(neigh), _lib.stream()))
+    for d in range(1, depth + 1):
+      self.neighs[d] = neigh[d]
+      self.nempty_neighs[d] = None
+      self._drop_tables(d)
+    for d in range(self.full_depth, depth):
+      self._nempty_indices32[d] = index[d]
+      self.nempty_indices[d] = None
 
   # ---- search (ocnn/octree/octree.py:448-488) -------------------------------
   def search_xyzb(self, query: torch.Tensor, depth: int, nempty: bool = False):
