@@ -337,21 +337,21 @@ __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles
 __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     const int32_t* __restrict__ ucount, const int32_t* __restrict__ tile_nnz, int64_t tiles, int cap,
     int32_t* __restrict__ uptr, int64_t* __restrict__ stats) {
-  __shared__ long long s_wsum[16], s_wnnz[16];
+  // the tiles in rounds of 1024, thread t on tile 1024 r + t (consecutive loads); the running
+  // offset is carried from round to round by every thread
+  __shared__ long long s_wsum[2][16], s_wnnz[16];
   __shared__ int s_wbig[16], s_wover[16], s_wmax[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t per = (tiles + 1023) / 1024;
-  const int64_t t0 = min(tiles, tid * per), t1 = min(tiles, t0 + per);
-  // sums over a wave with lane exchanges, one LDS slot per wave: 1024 threads adding to one LDS
-  // word take longer than everything else here
+  const int64_t rounds = (tiles + 1023) / 1024;
   auto wave_sum = [&](long long v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     return v;
   };
   int big = 0, over = 0;
-  for (int64_t t = t0; t < t1; ++t) {
-    const int c = ucount[t];
+  for (int64_t r = 0; r < rounds; ++r) {
+    const int64_t t = r * 1024 + tid;
+    const int c = t < tiles ? ucount[t] : 0;
     big += c > cap && c < kPlanOverflow ? 1 : 0;
     over += c >= kPlanOverflow ? 1 : 0;
   }
@@ -369,49 +369,55 @@ __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     n_over += s_wover[w];
   }
   const bool drop = n_big > 0 && n_big <= max((int64_t)1, tiles / 10);
-  long long sum = 0, nnz = 0;
+  long long base = 0, nnz = 0;
   int mx = 0;
-  for (int64_t t = t0; t < t1; ++t) {
-    const int c = ucount[t];
-    if ((drop && c > cap) || c >= kPlanOverflow) continue;
-    sum += c;
-    mx = max(mx, c);
-    nnz += tile_nnz[t];
-  }
-  // inclusive scan of `sum` over the wave, then over the 16 waves
-  long long incl = sum;
+  for (int64_t r = 0; r < rounds; ++r) {
+    const int64_t t = r * 1024 + tid;
+    int c = t < tiles ? ucount[t] : 0;
+    const bool skip = (drop && c > cap) || c >= kPlanOverflow;
+    if (skip) c = 0;
+    if (t < tiles && !skip) {
+      mx = max(mx, c);
+      nnz += tile_nnz[t];
+    }
+    long long incl = c;
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const long long v = __shfl_up(incl, o);
-    if (lane >= o) incl += v;
+    for (int o = 1; o < 64; o <<= 1) {
+      const long long v = __shfl_up(incl, o);
+      if (lane >= o) incl += v;
+    }
+    if (lane == 63) s_wsum[r & 1][wave] = incl;
+    __syncthreads();                                      // (the other set of slots is the one read a round ago)
+    long long before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const long long v = s_wsum[r & 1][w];
+      if (w < wave) before += v;
+      total += v;
+    }
+    if (t < tiles) uptr[t] = (int32_t)(base + before + incl - c);
+    base += total;
   }
   const long long wnnz = wave_sum(nnz);
   int wmx = mx;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) wmx = max(wmx, __shfl_xor(wmx, o));
-  if (lane == 63) s_wsum[wave] = incl;
-  if (lane == 0) { s_wnnz[wave] = wnnz; s_wmax[wave] = wmx; }
+  if (lane == 0) {
+    s_wnnz[wave] = wnnz;
+    s_wmax[wave] = wmx;
+  }
   __syncthreads();
-  long long before = 0, total = 0, nnz_all = 0;
-  int max_all = 0;
-#pragma unroll
-  for (int w = 0; w < 16; ++w) {
-    if (w < wave) before += s_wsum[w];
-    total += s_wsum[w];
-    nnz_all += s_wnnz[w];
-    max_all = max(max_all, s_wmax[w]);
-  }
-  long long at = before + incl - sum;
-  for (int64_t t = t0; t < t1; ++t) {
-    uptr[t] = (int32_t)at;
-    const int c = ucount[t];
-    at += ((drop && c > cap) || c >= kPlanOverflow) ? 0 : c;
-  }
-  if (tid == 1023) {
-    uptr[tiles] = (int32_t)total;
+  if (tid == 0) {
+    long long nnz_all = 0;
+    int max_all = 0;
+    for (int w = 0; w < 16; ++w) {
+      nnz_all += s_wnnz[w];
+      max_all = max(max_all, s_wmax[w]);
+    }
+    uptr[tiles] = (int32_t)base;
     stats[0] = n_big;
     stats[1] = drop ? 1 : 0;
-    stats[2] = total;
+    stats[2] = base;
     stats[3] = max_all;
     stats[4] = nnz_all;
     stats[5] = n_over;
