@@ -337,23 +337,38 @@ __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles
 __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
     const int32_t* __restrict__ ucount, const int32_t* __restrict__ tile_nnz, int64_t tiles, int cap,
     int32_t* __restrict__ uptr, int64_t* __restrict__ stats) {
-  // the tiles in rounds of 1024, thread t on tile 1024 r + t (consecutive loads); the running
-  // offset is carried from round to round by every thread
-  __shared__ long long s_wsum[2][16], s_wnnz[16];
+  // the tiles in rounds of 4096, thread t on the four tiles from 4096 r + 4 t (consecutive
+  // 16-byte loads, two rounds in flight); a round's counts fit 32 bits, the running offset is
+  // carried from round to round by every thread
+  __shared__ int s_wsum[2][16];
+  __shared__ long long s_wnnz[16];
   __shared__ int s_wbig[16], s_wover[16], s_wmax[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t rounds = (tiles + 1023) / 1024;
+  const int64_t rounds = (tiles + 4095) / 4096;
   auto wave_sum = [&](long long v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     return v;
   };
+  struct Four { int v[4]; };
+  auto load4 = [&](const int32_t* p, int64_t t) {
+    Four q;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q.v[i] = t + i < tiles ? p[t + i] : 0;
+    return q;
+  };
   int big = 0, over = 0;
-  for (int64_t r = 0; r < rounds; ++r) {
-    const int64_t t = r * 1024 + tid;
-    const int c = t < tiles ? ucount[t] : 0;
-    big += c > cap && c < kPlanOverflow ? 1 : 0;
-    over += c >= kPlanOverflow ? 1 : 0;
+  for (int64_t r = 0; r < rounds; r += 4) {               // four rounds in flight
+    Four c4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) c4[u] = load4(ucount, (r + u) * 4096 + 4 * tid);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        big += c4[u].v[i] > cap && c4[u].v[i] < kPlanOverflow ? 1 : 0;
+        over += c4[u].v[i] >= kPlanOverflow ? 1 : 0;
+      }
   }
   big = (int)wave_sum(big);
   over = (int)wave_sum(over);
@@ -371,31 +386,45 @@ __global__ __launch_bounds__(1024) void tile_plan_offsets_kernel(
   const bool drop = n_big > 0 && n_big <= max((int64_t)1, tiles / 10);
   long long base = 0, nnz = 0;
   int mx = 0;
+  Four cn = load4(ucount, 4 * tid), zn = load4(tile_nnz, 4 * tid);
   for (int64_t r = 0; r < rounds; ++r) {
-    const int64_t t = r * 1024 + tid;
-    int c = t < tiles ? ucount[t] : 0;
-    const bool skip = (drop && c > cap) || c >= kPlanOverflow;
-    if (skip) c = 0;
-    if (t < tiles && !skip) {
-      mx = max(mx, c);
-      nnz += tile_nnz[t];
+    const int64_t t = r * 4096 + 4 * tid;
+    Four c = cn;
+    const Four z = zn;
+    cn = load4(ucount, t + 4096);                         // the next round's, under this round's scan
+    zn = load4(tile_nnz, t + 4096);
+    int own = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool skip = (drop && c.v[i] > cap) || c.v[i] >= kPlanOverflow;
+      if (skip) c.v[i] = 0;
+      if (!skip) {
+        mx = max(mx, c.v[i]);
+        nnz += z.v[i];
+      }
+      own += c.v[i];
     }
-    long long incl = c;
+    int incl = own;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
-      const long long v = __shfl_up(incl, o);
+      const int v = __shfl_up(incl, o);
       if (lane >= o) incl += v;
     }
     if (lane == 63) s_wsum[r & 1][wave] = incl;
     __syncthreads();                                      // (the other set of slots is the one read a round ago)
-    long long before = 0, total = 0;
+    int before = 0, total = 0;
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
-      const long long v = s_wsum[r & 1][w];
+      const int v = s_wsum[r & 1][w];
       if (w < wave) before += v;
       total += v;
     }
-    if (t < tiles) uptr[t] = (int32_t)(base + before + incl - c);
+    long long at = base + before + incl - own;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (t + i < tiles) uptr[t + i] = (int32_t)at;
+      at += c.v[i];
+    }
     base += total;
   }
   const long long wnnz = wave_sum(nnz);
