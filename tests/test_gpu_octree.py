@@ -372,10 +372,12 @@ def test_random_octrees_vs_oracle():
 
 
 @pytest.mark.parametrize('depth,full,batch,n', [(11, 2, 1, 3000), (11, 1, 5, 4000), (12, 3, 3, 2500),
-                                                (10, 1, 2, 6000), (10, 2, 8, 6000), (16, 6, 1, 300)])
+                                                (10, 1, 2, 6000), (10, 2, 8, 6000), (16, 6, 1, 300),
+                                                (3, 3, 2, 500), (2, 2, 1, 50), (4, 3, 3, 2000)])
 def test_deep_octrees_vs_oracle(depth, full, batch, n):
-  """Depths at which batch id and Morton code pass 32 bits (the build then sorts 64-bit keys) and
-  more than seven sparse layers (the wider scan element): every layer's keys and children, the
+  """Depths at which batch id and Morton code pass 32 bits (the build then sorts 64-bit keys),
+  more than seven sparse layers (sixteen counters a point instead of eight), and octrees with no or
+  one sparse layer (depth = full_depth, full_depth + 1): every layer's keys and children, the
   counts, the point -> leaf map and the leaf signals bit exact against the oracle."""
   say('deep octree: depth', depth, 'full', full, 'batch', batch, 'points', n)
   rng = np.random.default_rng(depth * 100 + batch)
