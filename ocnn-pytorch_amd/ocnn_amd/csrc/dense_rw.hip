@@ -515,8 +515,12 @@ static int dr_wa(int ca, int cb) {
   return best;
 }
 
+// Row ranges per block of channel pairs: workgroups on three quarters of the CUs stream the rows as
+// fast as workgroups on all of them (two tiles in flight each), and every range costs a set of fp32
+// sums written and read back (64 -> 128 on 1.9 M rows: 0.300 -> 0.290 ms for the layer; twice the
+// ranges: 0.33 ms).
 static int dr_wgrad_splits(int ca, int cb, int n_cu) {
-  return std::max(1, n_cu / dr_wgrad_blocks(ca, cb, dr_wa(ca, cb)));
+  return std::max(1, n_cu * 3 / 4 / dr_wgrad_blocks(ca, cb, dr_wa(ca, cb)));
 }
 
 extern "C" int ocnn_conv_dense_wgrad_rw_supported(int dtype, int64_t rows, int ca, int cb) {
