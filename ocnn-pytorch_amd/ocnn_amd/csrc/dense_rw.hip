@@ -515,12 +515,20 @@ static int dr_wa(int ca, int cb) {
   return best;
 }
 
-// Row ranges per block of channel pairs: workgroups on three quarters of the CUs stream the rows as
-// fast as workgroups on all of them (two tiles in flight each), and every range costs a set of fp32
-// sums written and read back (64 -> 128 on 1.9 M rows: 0.300 -> 0.290 ms for the layer; twice the
-// ranges: 0.33 ms).
+// row ranges per block of channel pairs at most: a workgroup on every CU
 static int dr_wgrad_splits(int ca, int cb, int n_cu) {
-  return std::max(1, n_cu * 3 / 4 / dr_wgrad_blocks(ca, cb, dr_wa(ca, cb)));
+  return std::max(1, n_cu / dr_wgrad_blocks(ca, cb, dr_wa(ca, cb)));
+}
+
+// Every range costs a set of fp32 sums written and read back.  Where those sets weigh against the
+// operands (512 x 128 sums on 236 k rows: 128 MB against 301 MB), workgroups on three quarters of
+// the CUs do better (2x2x2 stride-2 64 -> 128 on 1.9 M rows: 0.300 -> 0.290 ms for the layer; twice
+// the ranges 0.33 ms); where they do not (96 x 96 sums on 925 k rows) every CU is needed to stream
+// the rows (70 us on all, 81 us on three quarters).
+static int dr_wgrad_ranges(int ca, int cb, int64_t rows, int n_cu) {
+  const int all = dr_wgrad_splits(ca, cb, n_cu);
+  const int64_t sums = (int64_t)all * ca * cb * 8, operands = rows * (int64_t)(ca + cb) * 2;
+  return 10 * sums >= 3 * operands ? std::max(1, all * 3 / 4) : all;
 }
 
 extern "C" int ocnn_conv_dense_wgrad_rw_supported(int dtype, int64_t rows, int ca, int cb) {
@@ -559,7 +567,7 @@ static int run_dense_wgrad(const DrOperand& x, const DrOperand& g, int64_t rows,
     return OCNN_ERR_HIP;
   }
   const int64_t tiles = cdiv(rows, 32);
-  const int nsplit = dr_wgrad_splits(ca, cb, n_cu);
+  const int nsplit = dr_wgrad_ranges(ca, cb, rows, n_cu);
   const int64_t per = std::max<int64_t>(1, cdiv(tiles, nsplit));
   const int used = (int)cdiv(tiles, per);
   if (ws_bytes < (int64_t)used * ca * cb * 4) {
