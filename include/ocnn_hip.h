@@ -416,11 +416,16 @@ int ocnn_conv_dense_wgrad_rw(int dtype, const void* x, const void* g, int64_t ro
  * index means the operand's own rows 0 .. rows - 1, as above.  This is how the stride-2 layers
  * over all nodes read the rows of the non-empty nodes out of a tensor padded to all nodes
  * without a depad pass (the reference depads first: ocnn/nn/octree_conv.py:419-420, 450-451,
- * ocnn/nn/octree_pad.py:32-39). */
+ * ocnn/nn/octree_pad.py:32-39).  The GEMM's result likewise: with out_index, row i is written to
+ * row out_index[i] of `out`, a tensor of rows_out rows (NULL: out has the `rows` rows of the
+ * result); the rows no entry names are not touched, ocnn_pad with data = NULL zeroes them: the
+ * reference's octree_pad after the product (ocnn/nn/octree_conv.py:388-389,
+ * ocnn/nn/octree_pad.py:13-29) without the copy. */
 int ocnn_conv_dense_rw_indexed(int dtype, const void* in, int64_t rows_in, const int32_t* row_index,
                                int64_t rows, const void* w, int cin, int cout, int w_transposed,
-                               const void* bias, void* out, void* workspace,
-                               int64_t workspace_bytes, void* stream);
+                               const void* bias, void* out, int64_t rows_out,
+                               const int32_t* out_index, void* workspace, int64_t workspace_bytes,
+                               void* stream);
 int ocnn_conv_dense_wgrad_rw_indexed(int dtype, const void* x, int64_t rows_x, const int32_t* x_index,
                                      const void* g, int64_t rows_g, const int32_t* g_index,
                                      int64_t rows, int ca, int cb, int out_transposed, void* gw,
@@ -585,7 +590,9 @@ int ocnn_max_gather(int dtype, const void* src, const int64_t* indices,
                     void* stream);
 
 /* ocnn/nn/octree_pad.py:13-39.  pad: out (n, c) = val except out[q] =
- * data[children[q]] where children[q] >= 0; depad: out[children[q]] = data[q]. */
+ * data[children[q]] where children[q] >= 0 (data NULL: only the rows with
+ * children[q] < 0 are written, for a result whose other rows are in place
+ * already); depad: out[children[q]] = data[q]. */
 int ocnn_pad(int dtype, const void* data, const int32_t* children, int64_t n,
              int channels, float val, void* out, void* stream);
 int ocnn_depad(int dtype, const void* data, const int32_t* children, int64_t n,

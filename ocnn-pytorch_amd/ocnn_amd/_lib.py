@@ -81,7 +81,7 @@ SIGNATURES = {
     'ocnn_conv_dense_wgrad_rw_supported': (_i, [_i, _l, _i, _i]),
     'ocnn_conv_dense_wgrad_rw_workspace_bytes': (_l, [_i, _i]),
     'ocnn_conv_dense_wgrad_rw': (_i, [_i, _p, _p, _l, _i, _i, _i, _p, _p, _l, _p]),
-    'ocnn_conv_dense_rw_indexed': (_i, [_i, _p, _l, _p, _l, _p, _i, _i, _i, _p, _p, _p, _l, _p]),
+    'ocnn_conv_dense_rw_indexed': (_i, [_i, _p, _l, _p, _l, _p, _i, _i, _i, _p, _p, _l, _p, _p, _l, _p]),
     'ocnn_conv_dense_wgrad_rw_indexed': (_i, [_i, _p, _l, _p, _p, _l, _p, _l, _i, _i, _i, _p, _p, _l, _p]),
     'ocnn_conv_wgrad_workspace_bytes': (_l, [_l, _i, _i, _i]),
     'ocnn_conv_wgrad_workspace_bytes_for': (_l, [_i, _l, _l, _i, _i, _i]),

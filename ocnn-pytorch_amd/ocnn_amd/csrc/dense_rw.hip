@@ -34,7 +34,8 @@ static __device__ __forceinline__ void dr_dma16(__amdgpu_buffer_rsrc_t rs, char*
 template <typename T, int NKS, int MB>
 __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const int32_t* __restrict__ row_index, const T* __restrict__ wpk,
-    const T* __restrict__ bias, T* __restrict__ out, int64_t rows, int cout, int64_t tiles, int64_t tiles_per_wg) {
+    const T* __restrict__ bias, T* __restrict__ out, uint32_t out_bytes, const int32_t* __restrict__ out_index,
+    int64_t rows, int cout, int64_t tiles, int64_t tiles_per_wg) {
   constexpr int RB = 2, RT = 32 * RB, NCC = NKS / 4, CIN = 16 * NKS;
   constexpr int BUF = NCC * RT * 128;
   constexpr int NBUF = NCC >= 8 ? 2 : 4;                           // tiles resident in LDS
@@ -58,8 +59,22 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
       wreg[ks][mb] = *(const u32x4*)(wpk + ((int64_t)(((ks >> 2) * ncg + cg0 + mb) * 4 + (ks & 3)) * 64 + lane) * 8);
 
   const __amdgpu_buffer_rsrc_t rs_in = make_rsrc(in, in_bytes);
-  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(out, (uint32_t)(rows * cout * 2));
+  const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(out, out_bytes);
   const int rl = lane >> 3;
+  // Output row r goes to row out_index[r] of `out` when an index is given (the compact rows of the
+  // non-empty nodes written straight into a tensor over all nodes): one entry per row block and
+  // lane, loaded NBUF - 1 tiles before its tile is stored, in registers taken in turn.
+  const bool scattered = out_index != nullptr;
+  const __amdgpu_buffer_rsrc_t rs_oidx = make_rsrc(out_index, scattered ? (uint32_t)(rows * 4) : 0u);
+  struct Odx { int32_t r[RB]; };
+  auto load_out_index = [&](int64_t tile) {
+    Odx x;
+    const uint32_t row0 = (uint32_t)min(tile, tiles) * RT;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      x.r[rb] = (int32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_oidx, (row0 + 32 * rb + r32) * 4u, 0, 0);
+    return x;
+  };
   // Row r of the operand is row row_index[r] of `in` when an index is given (the compact rows of
   // the non-empty nodes read straight from the tensor over all nodes).  A lane stages the rows
   // 8 wave + rl and 8 (wave + 4) + rl of a tile: two index entries per tile, loaded IDXD tiles
@@ -105,9 +120,9 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
   // (tiles past the range load zeros or rows of another range; rows past the end are stored
   // out of range and dropped).  NST dropped stores per prologue tile make the count right from
   // the first tile on.
-  constexpr int P = NCC * 2 + 2, NST = RB * MB * 2;                 // a tile's loads: its pieces and two index entries
-  constexpr int kWait = (NBUF - 2) * P + (NBUF - 1) * NST;
-  static_assert(kWait <= 63, "vmcnt is a 6-bit counter");
+  constexpr int P = NCC * 2 + 2 + RB, NST = RB * MB * 2;            // a tile's loads: its pieces, two + RB index entries
+  // (vmcnt is a 6-bit counter; a smaller count only waits for more)
+  constexpr int kWait = (NBUF - 2) * P + (NBUF - 1) * NST < 63 ? (NBUF - 2) * P + (NBUF - 1) * NST : 63;
   // s_waitcnt vmcnt(kWait) lgkmcnt(0) as an instruction of its own (vmcnt in bits 3:0 and 15:14,
   // lgkmcnt in bits 11:8), which the compiler's wait insertion takes into account
   constexpr int kWaitImm = 0x0070 | (kWait & 15) | ((kWait >> 4) << 14);
@@ -125,6 +140,9 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
   }
 #pragma unroll
   for (int v = 0; v < NBUF - 1; ++v) iq[v] = load_index(t_begin + NBUF - 1 + v);
+  Odx oq[NBUF - 1];                                                // oq[0]: of the tile stored next
+#pragma unroll
+  for (int v = 0; v < NBUF - 1; ++v) oq[v] = load_out_index(t_begin + v);
   for (int i = tid; i < 128 * MB; i += 256)
     s_bias[i] = bias ? to_f32(bias[(int)blockIdx.y * 128 * MB + i]) : 0.f;
   __builtin_amdgcn_s_waitcnt(0x0070);
@@ -174,8 +192,12 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
       const f32x4 bv[4] = {b4[0], b4[1], b4[4], b4[5]};
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        const uint32_t off = ((uint32_t)(tile * RT + 32 * rb + r32) * (uint32_t)cout +
-                              (uint32_t)((int)blockIdx.y * 128 * MB + cl)) * 2u;
+        const int64_t row = tile * RT + 32 * rb + r32;
+        // (with an index, rows past the end have no entry: out of range, dropped like the others)
+        const uint32_t orow = scattered ? (uint32_t)oq[U].r[rb] : (uint32_t)row;
+        const uint32_t off = scattered && row >= rows
+                                 ? 0xffffff00u                     // (+ 32 for the second store stays out of range)
+                                 : (orow * (uint32_t)cout + (uint32_t)((int)blockIdx.y * 128 * MB + cl)) * 2u;
         unsigned pk[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r)
@@ -184,6 +206,7 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
         __builtin_amdgcn_raw_buffer_store_b128(u32x4{pk[4], pk[5], pk[6], pk[7]}, rs_out, off + 32u, 0, 0);
       }
     }
+    oq[U] = load_out_index(tile + NBUF - 1);
     // the next tile has landed; every wave is done with this one
     __builtin_amdgcn_sched_barrier(0);
     // (a bare barrier: __syncthreads() would wait for every load in flight, the ring's included)
@@ -416,7 +439,8 @@ extern "C" int ocnn_conv_dense_rw_supported(int dtype, int64_t rows, int cin, in
 
 template <typename T, int NKS, int MB>
 static void launch_dense_rw(const void* in, int64_t rows_in, const int32_t* row_index, int64_t rows, int cout,
-                            const void* ws, const void* bias, void* out, int n_cu, hipStream_t st) {
+                            const void* ws, const void* bias, void* out, int64_t rows_out, const int32_t* out_index,
+                            int n_cu, hipStream_t st) {
   const int lds = ((NKS / 4) >= 8 ? 2 : 4) * (NKS / 4) * 64 * 128;
   static bool attr_set = false;
   if (!attr_set) {
@@ -431,7 +455,7 @@ static void launch_dense_rw(const void* in, int64_t rows_in, const int32_t* row_
   wgs = cdiv(tiles, per);
   hipLaunchKernelGGL((conv_dense_rw_kernel<T, NKS, MB>), dim3((unsigned)wgs, (unsigned)ny), dim3(256), lds, st,
                      (const T*)in, (uint32_t)(rows_in * NKS * 32), row_index, (const T*)ws, (const T*)bias, (T*)out,
-                     rows, cout, tiles, per);
+                     (uint32_t)(rows_out * cout * 2), out_index, rows, cout, tiles, per);
 }
 
 template <typename T>
@@ -456,7 +480,8 @@ __global__ void pack_weights_dense_kernel(const T* __restrict__ w, T* __restrict
 
 template <typename T>
 static int run_dense_rw(const void* in, int64_t rows_in, const int32_t* row_index, int64_t rows, const void* w,
-                        int cin, int cout, int w_transposed, const void* bias, void* out, void* ws, hipStream_t st) {
+                        int cin, int cout, int w_transposed, const void* bias, void* out, int64_t rows_out,
+                        const int32_t* out_index, void* ws, hipStream_t st) {
   const int n_cu = dr_cu_count();
   if (n_cu <= 0) {
     set_error("conv_dense_rw: cannot query the device");
@@ -466,7 +491,7 @@ static int run_dense_rw(const void* in, int64_t rows_in, const int32_t* row_inde
                      (const T*)w, (T*)ws, cin, cout, w_transposed);
   const int mb = dr_mb(cin, cout);
 #define OCNN_DRW(CIN_, MB_) \
-  if (cin == CIN_ && mb == MB_) { launch_dense_rw<T, CIN_ / 16, MB_>(in, rows_in, row_index, rows, cout, ws, bias, out, n_cu, st); return check_launch("conv_dense_rw"); }
+  if (cin == CIN_ && mb == MB_) { launch_dense_rw<T, CIN_ / 16, MB_>(in, rows_in, row_index, rows, cout, ws, bias, out, rows_out, out_index, n_cu, st); return check_launch("conv_dense_rw"); }
   OCNN_DRW(512, 1) OCNN_DRW(256, 1) OCNN_DRW(256, 2) OCNN_DRW(128, 1) OCNN_DRW(128, 2) OCNN_DRW(128, 4)
   OCNN_DRW(64, 1) OCNN_DRW(64, 2) OCNN_DRW(64, 4)
 #undef OCNN_DRW
@@ -476,11 +501,13 @@ static int run_dense_rw(const void* in, int64_t rows_in, const int32_t* row_inde
 
 extern "C" int ocnn_conv_dense_rw_indexed(int dtype, const void* in, int64_t rows_in, const int32_t* row_index,
                                           int64_t rows, const void* w, int cin, int cout, int w_transposed,
-                                          const void* bias, void* out, void* workspace, int64_t workspace_bytes,
-                                          void* stream) {
+                                          const void* bias, void* out, int64_t rows_out, const int32_t* out_index,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(ocnn_conv_dense_rw_supported(dtype, rows, cin, cout), "conv_dense_rw: shape not supported");
   OCNN_REQUIRE(row_index != nullptr || rows_in == rows, "conv_dense_rw: without an index the operand has `rows` rows");
+  OCNN_REQUIRE(out_index != nullptr || rows_out == rows, "conv_dense_rw: without an index the result has `rows` rows");
   OCNN_REQUIRE(rows_in >= 0 && ((int64_t)rows_in + 128) * cin * 2 <= 0xfff00000ll, "conv_dense_rw: operand too large");
+  OCNN_REQUIRE(rows_out >= 0 && ((int64_t)rows_out + 128) * cout * 2 <= 0xfff00000ll, "conv_dense_rw: result too large");
   if (rows <= 0) return OCNN_OK;
   if (workspace_bytes < (int64_t)cin * cout * 2) {
     set_error("conv_dense_rw: workspace too small");
@@ -488,15 +515,17 @@ extern "C" int ocnn_conv_dense_rw_indexed(int dtype, const void* in, int64_t row
   }
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
-    return run_dense_rw<f16>(in, rows_in, row_index, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
-  return run_dense_rw<bf16>(in, rows_in, row_index, rows, w, cin, cout, w_transposed, bias, out, workspace, st);
+    return run_dense_rw<f16>(in, rows_in, row_index, rows, w, cin, cout, w_transposed, bias, out, rows_out, out_index,
+                             workspace, st);
+  return run_dense_rw<bf16>(in, rows_in, row_index, rows, w, cin, cout, w_transposed, bias, out, rows_out, out_index,
+                            workspace, st);
 }
 
 extern "C" int ocnn_conv_dense_rw(int dtype, const void* in, int64_t rows, const void* w, int cin, int cout,
                                   int w_transposed, const void* bias, void* out, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
-  return ocnn_conv_dense_rw_indexed(dtype, in, rows, nullptr, rows, w, cin, cout, w_transposed, bias, out, workspace,
-                                    workspace_bytes, stream);
+  return ocnn_conv_dense_rw_indexed(dtype, in, rows, nullptr, rows, w, cin, cout, w_transposed, bias, out, rows, nullptr,
+                                    workspace, workspace_bytes, stream);
 }
 
 // ---- weight gradient ----

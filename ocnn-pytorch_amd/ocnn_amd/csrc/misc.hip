@@ -226,6 +226,10 @@ __global__ void pad16_kernel(const u32x4* __restrict__ data, const int32_t* __re
   int64_t q = t / chunks;
   int c = (int)(t % chunks);
   int32_t ch = children[q];
+  if (data == nullptr) {                                   // only the rows of the empty nodes
+    if (ch < 0) out[t] = fill;
+    return;
+  }
   out[t] = ch >= 0 ? data[(int64_t)ch * chunks + c] : fill;
 }
 
@@ -247,6 +251,10 @@ __global__ void pad_kernel(const T* __restrict__ data, const int32_t* __restrict
   int64_t q = t / C;
   int c = (int)(t % C);
   int32_t ch = children[q];
+  if (data == nullptr) {                                   // only the rows of the empty nodes
+    if (ch < 0) out[t] = from_f32<T>(val);
+    return;
+  }
   out[t] = ch >= 0 ? data[(int64_t)ch * C + c] : from_f32<T>(val);
 }
 

@@ -34,13 +34,20 @@ SPARSE_MIN_ROWS = 32768
 
 
 def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False,
-                in_index=None):
+                in_index=None, pad_to=None):
   """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K)).  With a
   tile plan of the same table (and a supported shape) the staged kernel runs.
   dense: the table is the one-slot identity (row i reads row i).
   in_index (int32, with dense only): row i reads row in_index[i] of `data`, which may then have
   more rows than the table (the compact rows of the non-empty nodes, read from a tensor over
-  all nodes without a depad pass)."""
+  all nodes without a depad pass).
+  pad_to = (octree, depth) (with dense only): the result comes back as octree_pad would make it,
+  a row for every node of `depth`, zeros for the empty ones: the kernel writes its rows there."""
+  if pad_to is not None:
+    if not dense:
+      return _pad_raw(conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index),
+                      *pad_to)
+    return _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, None, dense, in_index, pad_to)[0]
   out, planned = _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index)
   if planned and plan is not None and plan.overflow_rows is not None:
     # the few tiles that are too dense for the plan: plan-free kernel, results put in place
@@ -57,7 +64,7 @@ def _plan_args(plan):
   return 1, plan.umax, plan.total, float(plan.occupancy), float(plan.reuse)
 
 
-def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index=None):
+def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index=None, pad_to=None):
   """conv_gather without the overflow rows of the plan; also returns whether a kernel on
   the plan ran.  The library picks the kernel (ocnn_conv_gather_choose)."""
   _lib.require_gpu(data, table, W)
@@ -73,6 +80,9 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
   kernel = L.ocnn_conv_gather_choose(code, rows_in, rows, K, cin, cout, int(bool(dense)), *_plan_args(plan))
   if in_index is not None and kernel != _lib.GATHER_DENSE_RW:
     data, in_index = data.index_select(0, in_index.long()), None       # the other kernels take compact rows
+  if pad_to is not None and kernel != _lib.GATHER_DENSE_RW:          # the other kernels write compact rows
+    out, planned = _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense, in_index)
+    return _pad_raw(out, *pad_to), planned
   if kernel == _lib.GATHER_ZERO_PADDED:
     cin_p, cout_p = -(-cin // 32) * 32, -(-cout // 16) * 16
     Wk = W.view(K, cout, cin) if transposed else W.view(K, cin, cout)
@@ -80,13 +90,23 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
     out = conv_gather(F.pad(data, (0, cin_p - cin)), rows_in, table, F.pad(Wk, pad_w), cout_p,
                       transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), plan)
     return out[:, :cout].contiguous(), False
-  out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
   ws = _lib.workspace(L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout), data.device)
-  tail = (_lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream())
   if kernel == _lib.GATHER_DENSE_RW:
+    out_index, n_out = None, rows
+    if pad_to is not None:
+      octree, depth = pad_to
+      out_index, n_out = octree._nempty_index32(depth), int(octree.nnum[depth])
+      assert out_index.numel() == rows, 'conv_gather: one result row per non-empty node'
+    out = torch.empty((n_out, cout), dtype=data.dtype, device=data.device)
     _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(data), data.shape[0], _lib.ptr(in_index), rows,
-                                            _lib.ptr(W), cin, cout, int(transposed), *tail))
+                                            _lib.ptr(W), cin, cout, int(transposed), _lib.ptr(bias), _lib.ptr(out),
+                                            n_out, _lib.ptr(out_index), _lib.ptr(ws), ws.numel(), _lib.stream()))
+    if pad_to is not None:                                            # zeros for the empty nodes
+      _lib.check(L.ocnn_pad(code, None, _lib.ptr(octree.children[depth]), n_out, cout, 0.0, _lib.ptr(out),
+                            _lib.stream()))
     return out, False
+  out = torch.empty((rows, cout), dtype=data.dtype, device=data.device)
+  tail = (_lib.ptr(bias), _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream())
   if kernel == _lib.GATHER_DENSE:
     _lib.check(L.ocnn_conv_dense(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed), *tail))
     return out, False
@@ -308,16 +328,18 @@ class OctreeConvBase:
       cache[key] = torch.arange(rows, dtype=torch.int32, device=device).view(rows, 1)
     return cache[key]
 
-  def forward_gemm(self, data, weights, bias=None):
-    """(fine rows, in_conv) -> (table rows, out_conv)."""
+  def forward_gemm(self, data, weights, bias=None, pad_to=None):
+    """(fine rows, in_conv) -> (table rows, out_conv).  pad_to = (octree, depth): the result
+    padded to all nodes of `depth` (octree_pad of the table rows)."""
     if self.dense_children:
       P = self.neigh.shape[0]
       return conv_gather(data.view(P, 8 * self.in_conv), P, self._identity(P, data.device),
                          weights.view(1, 8 * self.in_conv, self.out_conv), self.out_conv, False,
-                         False, bias, None, dense=True)
+                         False, bias, None, dense=True, pad_to=pad_to)
     plan = self._plan(data, self.in_conv, self.out_conv)
-    return conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias,
-                       plan)
+    out = conv_gather(data, self.fine_h, self.neigh, weights, self.out_conv, False, False, bias,
+                      plan)
+    return out if pad_to is None else _pad_raw(out, *pad_to)
 
   def backward_gemm(self, grad, weights, bias=None, coarse_index=None):
     """(table rows, out_conv) -> (fine rows, in_conv).  coarse_index (int32): `grad` holds the
@@ -387,11 +409,11 @@ class OctreeConvFunction(Function):
     eng.check_and_init(data)
     data = data.contiguous()
     weights = weights.to(data.dtype).contiguous()
-    out = eng.forward_gemm(data, weights, bias)
+    out = eng.forward_gemm(data, weights, bias, pad_to=(octree, depth - 1) if padded else None)
     ctx.save_for_backward(data, weights)
     ctx.eng = eng
     ctx.pad_depth = depth - 1 if padded else None
-    return _pad_raw(out, octree, depth - 1) if padded else out
+    return out
 
   @staticmethod
   def backward(ctx, grad):
@@ -448,9 +470,8 @@ class OctreeDeconvFunction(Function):
     index = eng.octree._nempty_index32(ctx.pad_depth) if ctx.indexed else None
     grad_out = None
     if ctx.needs_input_grad[0]:
-      grad_out = eng.forward_gemm(grad, weights)
-      if ctx.pad_depth is not None:
-        grad_out = _pad_raw(grad_out, eng.octree, ctx.pad_depth)
+      grad_out = eng.forward_gemm(grad, weights,
+                                  pad_to=None if ctx.pad_depth is None else (eng.octree, ctx.pad_depth))
     # weights are (K, out_channels, in_channels): x = grad (fine side), g = data
     grad_w = eng.weight_gemm(grad, data, coarse_index=index) if ctx.needs_input_grad[1] else None
     grad_b = column_sum(grad) if ctx.needs_input_grad[10] else None

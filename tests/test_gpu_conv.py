@@ -615,10 +615,24 @@ def test_dense_rows_register_kernels_indexed(dtype, cin, cout):
                                       _lib.ptr(want), _lib.ptr(ws), ws.numel(), _lib.stream()))
       out = torch.full((rows + 1, cout), 7.0, dtype=dtype, device=DEV)
       _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(x_all), total, _lib.ptr(idx), rows, _lib.ptr(w), cin,
-                                              cout, 0, _lib.ptr(b), _lib.ptr(out), _lib.ptr(ws), ws.numel(),
-                                              _lib.stream()))
+                                              cout, 0, _lib.ptr(b), _lib.ptr(out), rows, None, _lib.ptr(ws),
+                                              ws.numel(), _lib.stream()))
       assert torch.equal(out[:rows], want) and bool((out[rows] == 7.0).all())
       assert rel_err(out[:rows], f64(x_sel) @ f64(w) + f64(b)) < TOL[dtype]
+      # the result through the index too: its rows land at the index's rows of a larger tensor,
+      # the other rows are not touched; ocnn_pad without data then zeroes the rows of the gaps
+      spread = torch.full((total, cout), 7.0, dtype=dtype, device=DEV)
+      _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(x_all), total, _lib.ptr(idx), rows, _lib.ptr(w), cin,
+                                              cout, 0, _lib.ptr(b), _lib.ptr(spread), total, _lib.ptr(idx),
+                                              _lib.ptr(ws), ws.numel(), _lib.stream()))
+      assert torch.equal(spread.index_select(0, idx.long()), want)
+      gaps = torch.ones(total, dtype=torch.bool, device=DEV)
+      gaps[idx.long()] = False
+      assert bool((spread[gaps] == 7.0).all())
+      children = torch.full((total,), -1, dtype=torch.int32, device=DEV)
+      children[idx.long()] = torch.arange(rows, dtype=torch.int32, device=DEV)
+      _lib.check(L.ocnn_pad(code, None, _lib.ptr(children), total, cout, 0.0, _lib.ptr(spread), _lib.stream()))
+      assert torch.equal(spread.index_select(0, idx.long()), want) and not bool(spread[gaps].any())
     ws = torch.empty(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(cin, cout), dtype=torch.uint8, device=DEV)
     want = torch.empty((cin, cout), dtype=dtype, device=DEV)
     _lib.check(L.ocnn_conv_dense_wgrad_rw(code, _lib.ptr(x_own), _lib.ptr(g_sel), rows, cin, cout, 0,
