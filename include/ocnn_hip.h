@@ -554,6 +554,18 @@ int ocnn_search_points(const float* pts, int64_t m, int depth, const int64_t* ke
 int ocnn_interp_linear_prepare(const float* pts, int64_t m, int depth, const int64_t* keys,
                                int64_t n, int bound_check, int32_t* idx, float* w, float* norm,
                                void* stream);
+/* ocnn_search_points and ocnn_interp_linear_prepare for the nodes of an octree layer, found by
+ * walking down the tree instead of searching the layer's keys (same results: the node's row,
+ * among all nodes of `depth` or, with nempty, among the non-empty ones, or -1): the children of
+ * the c-th non-empty node of a layer are the nodes 8 c .. 8 c + 7 of the next.  h_children: host
+ * array of depth + 1 device pointers, the octree's children arrays (layers min(depth,
+ * full_depth) .. depth are read; the last only with nempty). */
+int ocnn_locate_points(const float* pts, int64_t m, const int32_t* const* h_children, int depth,
+                       int full_depth, int batch_size, int nempty, int bound_check, int32_t* out,
+                       void* stream);
+int ocnn_interp_linear_locate(const float* pts, int64_t m, const int32_t* const* h_children,
+                              int depth, int full_depth, int batch_size, int nempty,
+                              int bound_check, int32_t* idx, float* w, float* norm, void* stream);
 int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const int32_t* col,
                   const float* val, const void* data, int channels, const float* rowdiv,
                   void* out, int64_t rows, void* stream);

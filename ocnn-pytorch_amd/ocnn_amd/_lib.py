@@ -105,6 +105,8 @@ SIGNATURES = {
     'ocnn_search_key': (_i, [_p, _l, _p, _l, _p, _p]),
     'ocnn_search_points': (_i, [_p, _l, _i, _p, _l, _i, _p, _p]),
     'ocnn_interp_linear_prepare': (_i, [_p, _l, _i, _p, _l, _i, _p, _p, _p, _p]),
+    'ocnn_locate_points': (_i, [_p, _l, _p, _i, _i, _i, _i, _i, _p, _p]),
+    'ocnn_interp_linear_locate': (_i, [_p, _l, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     'ocnn_csr_rows': (_i, [_i, _p, _i, _p, _p, _p, _i, _p, _p, _l, _p]),
     'ocnn_csr_transpose_workspace_bytes': (_l, [_l]),
     'ocnn_csr_transpose': (_i, [_p, _p, _p, _l, _i, _l, _p, _l, _p, _p, _p, _p]),

@@ -54,13 +54,52 @@ __global__ void search_points_kernel(const float* __restrict__ pts, int64_t m, i
   out[i] = (int32_t)r;
 }
 
+// ---- the same searches down the tree -------------------------------------------------------
+// A node's place in its layer follows from its parent's: the children of the c-th non-empty node
+// of a layer are the nodes 8 c .. 8 c + 7 of the next one.  Walking down from the deepest full
+// layer finds a key in depth - full_depth dependent loads, most of them in small, cache-resident
+// arrays, where the binary search over the layer's keys takes log2(nodes): the same answer, a
+// node or -1.
+constexpr int kLocateMaxDepth = 16;
+struct LocateTree {
+  const int32_t* children[kLocateMaxDepth + 1];
+  int depth, full_depth, batch_size, nempty;
+};
+
+__device__ __forceinline__ int32_t locate_key(const LocateTree& t, int64_t key) {
+  const int64_t b = key >> 48;
+  if (b < 0 || b >= t.batch_size) return -1;
+  const int64_t m = key & ((1ll << 48) - 1);
+  if ((m >> (3 * t.depth)) != 0) return -1;               // beyond the layer's keys
+  const int top = t.depth < t.full_depth ? t.depth : t.full_depth;
+  int64_t pos = (b << (3 * top)) | (m >> (3 * (t.depth - top)));
+  for (int l = top; l < t.depth; ++l) {
+    const int32_t c = t.children[l][pos];
+    if (c < 0) return -1;
+    pos = ((int64_t)c << 3) | ((m >> (3 * (t.depth - 1 - l))) & 7);
+  }
+  return t.nempty ? t.children[t.depth][pos] : (int32_t)pos;
+}
+
+__global__ void locate_points_kernel(const float* __restrict__ pts, int64_t m, LocateTree t, int bound_check,
+                                     int32_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= m) return;
+  const float x = pts[4 * i], y = pts[4 * i + 1], z = pts[4 * i + 2], b = pts[4 * i + 3];
+  int32_t r = locate_key(t, key_of(x, y, z, b, t.depth));
+  const float hi = (float)(1 << t.depth);
+  if (bound_check && !(x >= 0.f && x < hi && y >= 0.f && y < hi && z >= 0.f && z < hi)) r = -1;
+  out[i] = r;
+}
+
 // Trilinear weights: values sit at voxel centres, so f = p - 0.5, corner = floor(f), and the
 // neighbour j = (gx, gy, gz) weighs |((1 - gx) - frac_x) ((1 - gy) - frac_y) ((1 - gz) - frac_z)|.
 // One thread per (point, neighbour); the 8 threads of a point add their weights in neighbour
 // order for the normalisation.
+template <bool LOCATE>
 __global__ void interp_linear_prepare_kernel(const float* __restrict__ pts, int64_t m, int depth,
-                                             const int64_t* __restrict__ keys, int64_t n, int bound_check,
-                                             int32_t* __restrict__ idx, float* __restrict__ w,
+                                             const int64_t* __restrict__ keys, int64_t n, LocateTree tree,
+                                             int bound_check, int32_t* __restrict__ idx, float* __restrict__ w,
                                              float* __restrict__ norm) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t i = t >> 3;
@@ -72,7 +111,8 @@ __global__ void interp_linear_prepare_kernel(const float* __restrict__ pts, int6
     const float fx = pts[4 * i] - 0.5f, fy = pts[4 * i + 1] - 0.5f, fz = pts[4 * i + 2] - 0.5f;
     const float ix = floorf(fx), iy = floorf(fy), iz = floorf(fz);
     const float nx = ix + gx, ny = iy + gy, nz = iz + gz;
-    int64_t f = find_key(keys, n, key_of(nx, ny, nz, pts[4 * i + 3], depth));
+    const int64_t key = key_of(nx, ny, nz, pts[4 * i + 3], depth);
+    int64_t f = LOCATE ? (int64_t)locate_key(tree, key) : find_key(keys, n, key);
     const float hi = (float)(1 << depth);
     if (bound_check && !(nx >= 0.f && nx < hi && ny >= 0.f && ny < hi && nz >= 0.f && nz < hi)) f = -1;
     if (f >= 0) {
@@ -312,9 +352,51 @@ extern "C" int ocnn_interp_linear_prepare(const float* pts, int64_t m, int depth
   OCNN_REQUIRE(n >= 0 && n < (1ll << 31) && m >= 0 && m < (1ll << 28) && depth >= 0 && depth <= 16,
                "interp_linear_prepare: bad arguments");
   if (m == 0) return OCNN_OK;
-  hipLaunchKernelGGL(interp_linear_prepare_kernel, dim3((unsigned)cdiv(m * 8, 256)), dim3(256), 0,
-                     (hipStream_t)stream, pts, m, depth, keys, n, bound_check, idx, w, norm);
+  hipLaunchKernelGGL(interp_linear_prepare_kernel<false>, dim3((unsigned)cdiv(m * 8, 256)), dim3(256), 0,
+                     (hipStream_t)stream, pts, m, depth, keys, n, LocateTree{}, bound_check, idx, w, norm);
   return check_launch("interp_linear_prepare");
+}
+
+static int locate_tree(const int32_t* const* h_children, int depth, int full_depth, int batch_size, int nempty,
+                       LocateTree* t) {
+  OCNN_REQUIRE(depth >= 0 && depth <= kLocateMaxDepth && full_depth >= 0 && full_depth <= 8 && batch_size >= 1 &&
+                   ((int64_t)batch_size << (3 * (depth < full_depth ? depth : full_depth))) < (1ll << 31),
+               "locate: depth=%d full_depth=%d batch_size=%d out of range", depth, full_depth, batch_size);
+  for (int l = 0; l <= kLocateMaxDepth; ++l) t->children[l] = nullptr;
+  for (int l = depth < full_depth ? depth : full_depth; l <= depth; ++l) {
+    OCNN_REQUIRE(h_children[l] != nullptr || (l == depth && !nempty), "locate: no children array of layer %d", l);
+    t->children[l] = h_children[l];
+  }
+  t->depth = depth;
+  t->full_depth = full_depth;
+  t->batch_size = batch_size;
+  t->nempty = nempty;
+  return OCNN_OK;
+}
+
+extern "C" int ocnn_locate_points(const float* pts, int64_t m, const int32_t* const* h_children, int depth,
+                                  int full_depth, int batch_size, int nempty, int bound_check, int32_t* out,
+                                  void* stream) {
+  OCNN_REQUIRE(m >= 0, "locate_points: bad size");
+  LocateTree t;
+  if (int rc = locate_tree(h_children, depth, full_depth, batch_size, nempty, &t)) return rc;
+  if (m == 0) return OCNN_OK;
+  hipLaunchKernelGGL(locate_points_kernel, dim3((unsigned)cdiv(m, 256)), dim3(256), 0, (hipStream_t)stream, pts, m, t,
+                     bound_check, out);
+  return check_launch("locate_points");
+}
+
+extern "C" int ocnn_interp_linear_locate(const float* pts, int64_t m, const int32_t* const* h_children, int depth,
+                                         int full_depth, int batch_size, int nempty, int bound_check, int32_t* idx,
+                                         float* w, float* norm, void* stream) {
+  OCNN_REQUIRE(m >= 0 && m < (1ll << 28), "interp_linear_locate: bad size");
+  LocateTree t;
+  if (int rc = locate_tree(h_children, depth, full_depth, batch_size, nempty, &t)) return rc;
+  if (m == 0) return OCNN_OK;
+  hipLaunchKernelGGL(interp_linear_prepare_kernel<true>, dim3((unsigned)cdiv(m * 8, 256)), dim3(256), 0,
+                     (hipStream_t)stream, pts, m, depth, (const int64_t*)nullptr, (int64_t)0, t, bound_check, idx, w,
+                     norm);
+  return check_launch("interp_linear_locate");
 }
 
 extern "C" int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const int32_t* col, const float* val,

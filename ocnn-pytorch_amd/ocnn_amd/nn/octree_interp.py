@@ -55,6 +55,18 @@ def _keys(octree, depth, nempty):
   return octree.key(depth, nempty).contiguous()
 
 
+def _tree(octree, depth, nempty):
+  """Arguments of the library's walks down the tree (host array of the children arrays, depth,
+  full depth, batch size, nempty), or None where an array is missing or not on the device."""
+  import ctypes
+  top = min(depth, octree.full_depth)
+  need = range(top, depth + 1 if nempty else depth)
+  if any(octree.children[l] is None or not octree.children[l].is_cuda for l in need):
+    return None
+  ptrs = [None if octree.children[l] is None else octree.children[l].data_ptr() for l in range(depth + 1)]
+  return (ctypes.c_void_p * (depth + 1))(*ptrs), depth, octree.full_depth, octree.batch_size, int(bool(nempty))
+
+
 def _pts(pts):
   _lib.require_gpu(pts)
   assert pts.dim() == 2 and pts.shape[1] == 4, 'pts: (N, 4) rows of (x, y, z, batch)'
@@ -73,10 +85,15 @@ def octree_nearest_pts(data: torch.Tensor, octree, depth: int, pts: torch.Tensor
   there is none."""
   _check_rows(data, octree, depth, nempty)
   pts = _pts(pts)
-  keys = _keys(octree, depth, nempty)
   idx = torch.empty((pts.shape[0], 1), dtype=torch.int32, device=pts.device)
-  _lib.check(_lib.lib().ocnn_search_points(_lib.ptr(pts), pts.shape[0], depth, _lib.ptr(keys),
-                                           keys.numel(), int(bound_check), _lib.ptr(idx), _lib.stream()))
+  tree = _tree(octree, depth, nempty)
+  if tree is not None:
+    _lib.check(_lib.lib().ocnn_locate_points(_lib.ptr(pts), pts.shape[0], *tree, int(bound_check), _lib.ptr(idx),
+                                             _lib.stream()))
+  else:
+    keys = _keys(octree, depth, nempty)
+    _lib.check(_lib.lib().ocnn_search_points(_lib.ptr(pts), pts.shape[0], depth, _lib.ptr(keys),
+                                             keys.numel(), int(bound_check), _lib.ptr(idx), _lib.stream()))
   return _Interp.apply(data, idx, None, None)
 
 
@@ -86,14 +103,19 @@ def octree_linear_pts(data: torch.Tensor, octree, depth: int, pts: torch.Tensor,
   weight sum (ocnn/nn/octree_interp.py:49-103)."""
   _check_rows(data, octree, depth, nempty)
   pts = _pts(pts)
-  keys = _keys(octree, depth, nempty)
   m = pts.shape[0]
   idx = torch.empty((m, 8), dtype=torch.int32, device=pts.device)
   w = torch.empty((m, 8), dtype=torch.float32, device=pts.device)
   norm = torch.empty(m, dtype=torch.float32, device=pts.device)
-  _lib.check(_lib.lib().ocnn_interp_linear_prepare(_lib.ptr(pts), m, depth, _lib.ptr(keys), keys.numel(),
-                                                   int(bound_check), _lib.ptr(idx), _lib.ptr(w),
-                                                   _lib.ptr(norm), _lib.stream()))
+  tree = _tree(octree, depth, nempty)
+  if tree is not None:
+    _lib.check(_lib.lib().ocnn_interp_linear_locate(_lib.ptr(pts), m, *tree, int(bound_check), _lib.ptr(idx),
+                                                    _lib.ptr(w), _lib.ptr(norm), _lib.stream()))
+  else:
+    keys = _keys(octree, depth, nempty)
+    _lib.check(_lib.lib().ocnn_interp_linear_prepare(_lib.ptr(pts), m, depth, _lib.ptr(keys), keys.numel(),
+                                                     int(bound_check), _lib.ptr(idx), _lib.ptr(w),
+                                                     _lib.ptr(norm), _lib.stream()))
   return _Interp.apply(data, idx, w, norm)
 
 

@@ -248,3 +248,53 @@ def test_global_pool(ref_data, nempty):
   out.backward(g)
   cnt = torch.bincount(bid, minlength=2).float()
   assert torch.allclose(x.grad, (g / cnt[:, None])[bid], atol=1e-6)
+
+
+def test_walk_down_the_tree_equals_the_key_search():
+  """ocnn_locate_points / ocnn_interp_linear_locate (a node found by walking down from the
+  deepest full layer) against ocnn_search_points / ocnn_interp_linear_prepare (binary search
+  over the layer's keys, pinned by the reference's search fixture): the same rows, weights and
+  weight sums, bit for bit, for points inside, on the faces of and outside the volume, batch ids
+  that no octree has, every depth of two octrees (depths that are and are not multiples of 3,
+  above and below the full depth), all nodes and non-empty ones, with and without the bounds check."""
+  import ctypes
+  from ocnn_amd import _lib
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(23)
+  for batch, depth_max, full in ((3, 7, 2), (1, 5, 3)):
+    pts3, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, batch, 5, n=6000)
+    o = Octree(depth_max, full, batch_size=batch)
+    o.build_octree(Points(pts3.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV) if batch > 1 else None, batch_size=batch))
+    for depth in range(1, depth_max + 1):
+      scale = float(1 << depth)
+      n = 5000
+      q = torch.rand(n, 3, generator=g) * (scale + 4.0) - 2.0             # some outside on every side
+      q[:500] = torch.randint(0, (1 << depth) + 1, (500, 3), generator=g).float()      # on cell faces and corners
+      pick = torch.randint(0, pts3.shape[0], (2000,), generator=g)
+      q[500:2500] = (pts3[pick] + 1.0) * scale / 2 + torch.randn(2000, 3, generator=g) * 0.7   # around the surface
+      b = torch.randint(-1, batch + 2, (n, 1), generator=g).float()
+      b[500:2500] = bid[pick].float().view(-1, 1) if batch > 1 else 0.0
+      pts = torch.cat([q, b], 1).contiguous().to(DEV)
+      for nempty in (False, True):
+        keys = o.key(depth, nempty).contiguous()
+        children = (ctypes.c_void_p * (depth + 1))(*[o.children[l].data_ptr() for l in range(depth + 1)])
+        tree = (children, depth, full, batch, int(nempty))
+        for check in (0, 1):
+          say('walk down the tree', batch, depth, nempty, check)
+          want = torch.empty(n, dtype=torch.int32, device=DEV)
+          got = torch.empty(n, dtype=torch.int32, device=DEV)
+          _lib.check(L.ocnn_search_points(_lib.ptr(pts), n, depth, _lib.ptr(keys), keys.numel(), check,
+                                          _lib.ptr(want), _lib.stream()))
+          _lib.check(L.ocnn_locate_points(_lib.ptr(pts), n, *tree, check, _lib.ptr(got), _lib.stream()))
+          assert torch.equal(got, want)
+          assert int((want >= 0).sum()) > 100
+          outs = []
+          for fn, args in ((L.ocnn_interp_linear_prepare, (depth, _lib.ptr(keys), keys.numel())),
+                           (L.ocnn_interp_linear_locate, tree)):
+            idx = torch.empty((n, 8), dtype=torch.int32, device=DEV)
+            w = torch.empty((n, 8), dtype=torch.float32, device=DEV)
+            norm = torch.empty(n, dtype=torch.float32, device=DEV)
+            _lib.check(fn(_lib.ptr(pts), n, *args, check, _lib.ptr(idx), _lib.ptr(w), _lib.ptr(norm), _lib.stream()))
+            outs.append((idx, w, norm))
+          for a, c in zip(*outs):
+            assert torch.equal(a, c)
