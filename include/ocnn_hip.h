@@ -118,6 +118,11 @@ int ocnn_grow_layer(const int64_t* key_above, const int32_t* nempty_index, int64
 int ocnn_leaf_average(const float* src, int channels, const int32_t* perm,
                       const int32_t* seg_start, int64_t n_leaf, int mode,
                       float* out, void* stream);
+/* The two calls a cloud with normals needs (mode 0 on the scaled points, mode 1 on the normals,
+ * 3 channels each) in one pass over the leaves' points; same sums, same results. */
+int ocnn_leaf_points_normals(const float* pts, const float* normals, const int32_t* perm,
+                             const int32_t* seg_start, int64_t n_leaf, float* out_pts,
+                             float* out_normals, void* stream);
 
 /* ---- neighbour search -------------------------------------------------- */
 

@@ -30,6 +30,7 @@ SIGNATURES = {
     'ocnn_split_children': (_i, [_p, _l, _p, _l, _p, _p, _p]),
     'ocnn_grow_layer': (_i, [_p, _p, _l, _p, _p, _p]),
     'ocnn_leaf_average': (_i, [_p, _i, _p, _p, _l, _i, _p, _p]),
+    'ocnn_leaf_points_normals': (_i, [_p, _p, _p, _p, _l, _p, _p, _p]),
     'ocnn_neigh_full': (_i, [_i, _i, _p, _p, _p]),
     'ocnn_neigh_from_parent': (_i, [_p, _p, _p, _l, _p, _p, _p]),
     'ocnn_neigh_all': (_i, [_i, _i, _i, _p, _p, _p, _p, _p, _p]),

@@ -40,6 +40,35 @@ __global__ void leaf_normal_kernel(const float* src, const int32_t* perm,
   out[3 * leaf + 2] = az / d;
 }
 
+// both of them for a cloud with normals: a leaf's points are walked once
+__global__ void leaf_points_normals_kernel(const float* __restrict__ pts, const float* __restrict__ nrm,
+                                           const int32_t* __restrict__ perm, const int32_t* __restrict__ seg_start,
+                                           int64_t n_leaf, float* __restrict__ out_pts, float* __restrict__ out_nrm) {
+  int64_t leaf = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (leaf >= n_leaf) return;
+  const int32_t s = seg_start[leaf], e = seg_start[leaf + 1];
+  float px = 0.f, py = 0.f, pz = 0.f, ax = 0.f, ay = 0.f, az = 0.f;
+  for (int32_t q = s; q < e; ++q) {
+    const int64_t at = (int64_t)perm[q] * 3;
+    const float* p = pts + at;
+    const float* v = nrm + at;
+    px += p[0];
+    py += p[1];
+    pz += p[2];
+    ax += v[0];
+    ay += v[1];
+    az += v[2];
+  }
+  const float cnt = (float)(e - s);
+  out_pts[3 * leaf + 0] = px / cnt;
+  out_pts[3 * leaf + 1] = py / cnt;
+  out_pts[3 * leaf + 2] = pz / cnt;
+  const float d = fmaxf(sqrtf(ax * ax + ay * ay + az * az), 1e-12f);
+  out_nrm[3 * leaf + 0] = ax / d;
+  out_nrm[3 * leaf + 1] = ay / d;
+  out_nrm[3 * leaf + 2] = az / d;
+}
+
 // ---- regrowing an octree from split decisions (generative decoders) ----------------------
 __global__ void split_flag_kernel(const int32_t* split, int64_t n, int32_t* flag) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -424,6 +453,15 @@ extern "C" int ocnn_leaf_average(const float* src, int channels, const int32_t* 
                        channels, perm, seg_start, n_leaf, out);
   }
   return check_launch("leaf_average");
+}
+
+extern "C" int ocnn_leaf_points_normals(const float* pts, const float* normals, const int32_t* perm,
+                                        const int32_t* seg_start, int64_t n_leaf, float* out_pts, float* out_normals,
+                                        void* stream) {
+  OCNN_REQUIRE(n_leaf > 0, "leaf_points_normals: n_leaf=%lld", (long long)n_leaf);
+  hipLaunchKernelGGL(leaf_points_normals_kernel, dim3((unsigned)cdiv(n_leaf, 256)), dim3(256), 0, (hipStream_t)stream,
+                     pts, normals, perm, seg_start, n_leaf, out_pts, out_normals);
+  return check_launch("leaf_points_normals");
 }
 
 // ---- fused build ---------------------------------------------------------------------------

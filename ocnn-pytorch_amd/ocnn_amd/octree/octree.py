@@ -527,9 +527,14 @@ class Octree:
     self.nnum[:depth + 1] = torch.tensor(nnum, dtype=torch.long)
     self.nnum_nempty[:depth + 1] = torch.tensor(
         full[:-1] + [sizes[depth - d] for d in range(full_depth, depth + 1)], dtype=torch.long)
-    self.points[depth] = leaf(pts_norm, 0)
     if point_cloud.normals is not None:
-      self.normals[depth] = leaf(point_cloud.normals, 1)
+      nrm = point_cloud.normals.float().contiguous()
+      self.points[depth] = torch.empty(nleaf, 3, dtype=torch.float32, device=dev)
+      self.normals[depth] = torch.empty(nleaf, 3, dtype=torch.float32, device=dev)
+      _lib.check(L.ocnn_leaf_points_normals(_lib.ptr(pts_norm), _lib.ptr(nrm), _lib.ptr(perm), _lib.ptr(seg_start),
+                                            nleaf, _lib.ptr(self.points[depth]), _lib.ptr(self.normals[depth]), st))
+    else:
+      self.points[depth] = leaf(pts_norm, 0)
     if point_cloud.features is not None:
       self.features[depth] = leaf(point_cloud.features, 0)
 
