@@ -421,6 +421,17 @@ def main():
          'pct_mfma_peak': round(100 * r['frac_mfma_peak'], 2),
          'pct_hbm_peak': round(100 * r['frac_hbm_peak_at_algorithmic_bytes'], 1)} for r in layers]
 
+  if extras and default_workload:
+    # ---- configs[4]: the reference's segmentation U-Net end to end (bench_unet.py) ----------
+    try:
+      import bench_unet
+      u = bench_unet.run(['--steps', '10', '--warmup', '5', '--fresh', '1'])
+      result['configs4_unet'] = {k: u[k] for k in ('net', 'ms_per_step', 'ms_octree_build_and_tables',
+                                                   'ms_first_step_on_a_fresh_octree', 'dtype', 'nempty', 'batch',
+                                                   'points', 'depth', 'parameters')}
+    except Exception as e:                              # supporting figure only
+      result['configs4_unet'] = {'error': repr(e)}
+
   if not args.no_cpu:
     result['cpu_baseline'] = cpu_baseline(torch, table, rows, C, C, args.cpu_rows)
     result['cpu_baseline']['octree'] = cpu_baseline_octree(pts, pc.normals.cpu(), bid if args.batch > 1 else None,

@@ -23,7 +23,9 @@ for p in (ROOT, os.path.join(ROOT, 'ocnn-pytorch_amd')):
     sys.path.insert(0, p)
 
 
-def main():
+def run(argv=None):
+  """Runs the benchmark with the given command-line arguments (None: the process's) and returns
+  the record that main() prints."""
   ap = argparse.ArgumentParser()
   ap.add_argument('--steps', type=int, default=10)
   ap.add_argument('--warmup', type=int, default=3)
@@ -35,7 +37,7 @@ def main():
   ap.add_argument('--profile', action='store_true')
   ap.add_argument('--fresh', type=int, default=3, help='steps on a newly built octree, timed after the others')
   ap.add_argument('--torch-loss', action='store_true', help='torch.nn.functional.cross_entropy for the loss')
-  args = ap.parse_args()
+  args = ap.parse_args(argv)
   import torch
   from ocnn_amd import synthetic
   from ocnn_amd.unet import UNet
@@ -130,7 +132,11 @@ def main():
       top.append((round(t / 1e3, 3), e.count, name[:90]))
     out['device_ms_by_kind'] = {k: round(v, 3) for k, v in sorted(groups.items(), key=lambda kv: -kv[1])}
     out['top_kernels_ms_calls'] = sorted(top, reverse=True)[:24]
-  print(json.dumps(out), flush=True)
+  return out
+
+
+def main():
+  print(json.dumps(run()), flush=True)
 
 
 if __name__ == '__main__':
