@@ -298,3 +298,36 @@ def test_walk_down_the_tree_equals_the_key_search():
             outs.append((idx, w, norm))
           for a, c in zip(*outs):
             assert torch.equal(a, c)
+
+
+def test_transposed_matrix_edge_cases():
+  """ocnn_csr_transpose on matrices without any entry, with one point, with rows nobody reads and
+  with every entry on one row: row pointers, columns in point order and values against a direct
+  construction."""
+  from ocnn_amd.nn.octree_interp import _transpose
+  g = torch.Generator().manual_seed(2)
+  for points, k, rows, mode in [(5, 8, 7, 'none'), (1, 8, 3, 'some'), (300, 8, 1000, 'some'), (300, 1, 4, 'one row'),
+                                (2000, 8, 50, 'some')]:
+    say('transposed matrix', points, k, rows, mode)
+    if mode == 'none':
+      idx = torch.full((points, k), -1, dtype=torch.int32)
+    elif mode == 'one row':
+      idx = torch.full((points, k), 2, dtype=torch.int32)
+    else:
+      idx = torch.randint(-1, rows, (points, k), generator=g, dtype=torch.int32)
+    w = torch.rand(points, k, generator=g)
+    norm = torch.rand(points, generator=g) + 0.5
+    rowptr, col, val = _transpose(idx.to(DEV), w.to(DEV), norm.to(DEV), rows)
+    rowptr, col, val = rowptr.cpu().numpy(), col.cpu().numpy(), val.cpu().numpy()
+    flat = idx.numpy().reshape(-1)
+    want_rows = [np.nonzero(flat == r)[0] for r in range(rows)]          # ascending entry = point order
+    assert rowptr[0] == 0 and rowptr[-1] == sum(len(e) for e in want_rows)
+    for r, e in enumerate(want_rows):
+      assert rowptr[r + 1] - rowptr[r] == len(e), r
+      assert np.array_equal(col[rowptr[r]:rowptr[r + 1]], e // k), r
+      wantv = w.numpy().reshape(-1)[e] / (norm.numpy()[e // k] + np.float32(1e-12))
+      assert np.allclose(val[rowptr[r]:rowptr[r + 1]], wantv, rtol=1e-6), r
+    # without weights and norm: no values
+    rowptr2, col2, val2 = _transpose(idx.to(DEV), None, None, rows)
+    assert val2 is None and np.array_equal(rowptr2.cpu().numpy(), rowptr)
+    assert np.array_equal(col2.cpu().numpy()[:rowptr[-1]], col[:rowptr[-1]])

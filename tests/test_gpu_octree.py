@@ -402,6 +402,12 @@ def test_deep_octrees_vs_oracle(depth, full, batch, n):
     assert np.array_equal(np_(o.children[d]), w.children[d]), d
   assert np.array_equal(np_(o.points[depth]), w.points[depth])
   assert np.allclose(np_(o.normals[depth]), w.normals[depth], atol=1e-6)
+  if depth <= 12:                                     # the tables too (one call for all layers)
+    o.construct_all_neigh()
+    R.construct_all_neigh(w)
+    for d in range(1, depth + 1):
+      assert np.array_equal(np_(o.neighs[d]), w.neighs[d]), d
+      assert np.array_equal(np_(o.nempty_index(d)), np.nonzero(w.children[d] >= 0)[0]), d
 
 
 @pytest.mark.parametrize('depth,batch', [(8, 1), (9, 4), (6, 2)])
