@@ -432,6 +432,16 @@ def main():
     except Exception as e:                              # supporting figure only
       result['configs4_unet'] = {'error': repr(e)}
 
+  if extras and default_workload:
+    # ---- the reference's own layer benchmark (test/benchmark_conv.py), bf16 (bench_sweep.py) ----
+    try:
+      import bench_sweep
+      result['reference_benchmark_sweep'] = [
+          {k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}
+          for r in bench_sweep.run([5, 6, 7, 8, 9, 10], ['bfloat16'])]
+    except Exception as e:                              # supporting figure only
+      result['reference_benchmark_sweep'] = {'error': repr(e)}
+
   if not args.no_cpu:
     result['cpu_baseline'] = cpu_baseline(torch, table, rows, C, C, args.cpu_rows)
     result['cpu_baseline']['octree'] = cpu_baseline_octree(pts, pc.normals.cpu(), bid if args.batch > 1 else None,

@@ -77,21 +77,13 @@ def graph_replay_ms(torch, conv, x, octree, depth, gout):
   return ms
 
 
-def main():
-  ap = argparse.ArgumentParser()
-  ap.add_argument('--depths', default='5,6,7,8,9,10')
-  ap.add_argument('--dtypes', default='float32,float16,bfloat16')
-  ap.add_argument('--gpus', type=int, default=1)
-  args = ap.parse_args()
-  if args.gpus != 1:
-    sys.exit('bench_sweep.py measures one GPU; --gpus %d is not supported' % args.gpus)
+def run(depths, dtypes):
+  """The records of the sweep: one per (depth, dtype)."""
   import torch
   from ocnn_amd import synthetic
   from ocnn_amd.nn import OctreeConv
   from ocnn_amd.octree import Octree, Points
   dev = 'cuda'
-  depths = [int(d) for d in args.depths.split(',')]
-  dtypes = args.dtypes.split(',')
   records = []
   for depth in depths:
     c = CHANNELS[depth]
@@ -120,6 +112,18 @@ def main():
       del conv, x, gout
     del octree
     torch.cuda.empty_cache()
+  return records
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument('--depths', default='5,6,7,8,9,10')
+  ap.add_argument('--dtypes', default='float32,float16,bfloat16')
+  ap.add_argument('--gpus', type=int, default=1)
+  args = ap.parse_args()
+  if args.gpus != 1:
+    sys.exit('bench_sweep.py measures one GPU; --gpus %d is not supported' % args.gpus)
+  records = run([int(d) for d in args.depths.split(',')], args.dtypes.split(','))
   print('%5s %4s %9s %-9s %8s %8s %10s %10s   %s' % ('depth', 'C', 'rows', 'dtype', 'fwd ms', 'bwd ms', 'TFLOP/s',
                                                    'graph ms', 'reference (Triton, RTX 4090) fwd / bwd ms'))
   for r in records:
