@@ -6,13 +6,16 @@
 // fixed order (per-workgroup partial sums, then one thread per channel in fp64): no atomics,
 // bit-reproducible.
 #include <algorithm>
+#include <mutex>
+#include <utility>
+#include <vector>
 
 #include "common.hpp"
 
 namespace ocnn {
 
 constexpr int kBnMaxBlocks = 512;     // workgroups of a reduction (their partial sums are added by one more kernel)
-constexpr int kBnApplyBlocks = 2048;  // workgroups of an elementwise pass
+constexpr int kBnApplyBlocks = 2048;  // workgroups of an elementwise pass, at most (fewer where the device holds fewer at once)
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) BnVec { T v[VEC]; };
 
@@ -22,6 +25,39 @@ __device__ __forceinline__ float bn_param(const void* p, int dtype, int c, float
   if (dtype == OCNN_F32) return ((const float*)p)[c];
   if (dtype == OCNN_F16) return to_f32(((const f16*)p)[c]);
   return to_f32(((const bf16*)p)[c]);
+}
+
+// gamma and beta of the channels c0 .. c0 + VEC - 1 (1 and 0 where the pointer is null).  The raw
+// values of both are requested before either is converted, so that a workgroup waits for one
+// round trip to memory and not for one per channel.
+template <int VEC>
+__device__ __forceinline__ void bn_params(const void* __restrict__ gamma, const void* __restrict__ beta, int dtype,
+                                          int c0, float (&ga)[VEC], float (&be)[VEC]) {
+  if (dtype == OCNN_F32) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      ga[v] = gamma ? ((const float*)gamma)[c0 + v] : 1.f;
+      be[v] = beta ? ((const float*)beta)[c0 + v] : 0.f;
+    }
+    return;
+  }
+  // f16: 1.0 = 0x3c00; bf16: 1.0 = 0x3f80
+  unsigned short rg[VEC], rb[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    rg[v] = gamma ? ((const unsigned short*)gamma)[c0 + v] : (unsigned short)(dtype == OCNN_F16 ? 0x3c00 : 0x3f80);
+    rb[v] = beta ? ((const unsigned short*)beta)[c0 + v] : (unsigned short)0;
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    if (dtype == OCNN_F16) {
+      ga[v] = to_f32(__builtin_bit_cast(f16, rg[v]));
+      be[v] = to_f32(__builtin_bit_cast(f16, rb[v]));
+    } else {
+      ga[v] = __uint_as_float((uint32_t)rg[v] << 16);
+      be[v] = __uint_as_float((uint32_t)rb[v] << 16);
+    }
+  }
 }
 
 __device__ __forceinline__ void bn_store(void* p, int dtype, int c, float v) {
@@ -168,10 +204,14 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const T* __restrict__ x, 
   float m[VEC], sc[VEC], be[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
-    const int c = cl * VEC + v;
-    m[v] = mean[c];
-    sc[v] = invstd[c] * bn_param(gamma, pdtype, c, 1.f);
-    be[v] = bn_param(beta, pdtype, c, 0.f);
+    m[v] = mean[cl * VEC + v];
+    sc[v] = invstd[cl * VEC + v];
+  }
+  {
+    float ga[VEC];
+    bn_params<VEC>(gamma, beta, pdtype, cl * VEC, ga, be);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) sc[v] *= ga[v];
   }
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
   const int64_t r1 = min(rows, r0 + rows_per_blk);
@@ -225,19 +265,17 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
     float m[VEC], is[VEC], ga[VEC], be[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const int c = cl * VEC + v;
-      m[v] = mean[c];
-      is[v] = invstd[c];
-      ga[v] = bn_param(gamma, pdtype, c, 1.f);
-      be[v] = bn_param(beta, pdtype, c, 0.f);
+      m[v] = mean[cl * VEC + v];
+      is[v] = invstd[cl * VEC + v];
     }
+    bn_params<VEC>(gamma, beta, pdtype, cl * VEC, ga, be);
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
     const int64_t r1 = min(rows, r0 + rows_per_blk);
-    for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {          // two rows of both tensors in flight
-      V a[2], g[2], ym[2];
-      bool ok[2];
+    for (int64_t r = r0 + rl; r < r1; r += 4 * rpp) {          // four rows of both tensors in flight
+      V a[4], g[4], ym[4];
+      bool ok[4];
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < 4; ++u) {
         const int64_t ru = r + (int64_t)u * rpp;
         ok[u] = ru < r1;
         a[u] = *(const V*)(x + (ok[u] ? ru * C : 0) + cl * VEC);
@@ -245,7 +283,7 @@ __global__ __launch_bounds__(256) void bn_bwd_stats_kernel(const T* __restrict__
         if (ymask) ym[u] = *(const V*)(ymask + (ok[u] ? ru * C : 0) + cl * VEC);
       }
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           const float xc = to_f32(a[u].v[v]) - m[v];
@@ -315,14 +353,15 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__
     const int c = cl * VEC + v;
     m[v] = mean[c];
     is[v] = invstd[c];
-    sc[v] = invstd[c] * bn_param(gamma, pdtype, c, 1.f);
-    be[v] = bn_param(beta, pdtype, c, 0.f);
     db[v] = training ? dbeta[c] * inv_n : 0.f;
     dg[v] = training ? dgamma[c] * inv_n : 0.f;
   }
+  bn_params<VEC>(gamma, beta, pdtype, cl * VEC, sc, be);
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) sc[v] *= is[v];
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_blk;
   const int64_t r1 = min(rows, r0 + rows_per_blk);
-  for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {
+  for (int64_t r = r0 + rl; r < r1; r += 2 * rpp) {     // (four rows in flight cost more in occupancy than they gain)
     V a[2], g[2], ym[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -380,6 +419,26 @@ static void bn_blocks(int dtype, int64_t rows, int channels, int max_blocks, int
   *nblk = (int)cdiv(rows, *per);
 }
 
+// Workgroups of 256 threads of `kernel` that the device holds at once, kBnApplyBlocks at most:
+// an elementwise pass launched with more runs them in rounds, and the last round leaves CUs idle.
+static int bn_resident_blocks(const void* kernel) {
+  static std::mutex mu;
+  static std::vector<std::pair<const void*, int>> known;
+  std::lock_guard<std::mutex> lock(mu);
+  for (const auto& k : known)
+    if (k.first == kernel) return k.second;
+  int per_cu = 0, dev = 0, n_cu = 256;
+  (void)hipGetDevice(&dev);
+  (void)hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1) {
+    (void)hipGetLastError();
+    per_cu = 2;
+  }
+  const int cap = std::min(kBnApplyBlocks, std::max(1, per_cu * n_cu));
+  known.emplace_back(kernel, cap);
+  return cap;
+}
+
 extern "C" int64_t ocnn_batch_norm_workspace_bytes(int channels) {
   return align_up((int64_t)kBnMaxBlocks * 2 * channels * 4, 256);
 }
@@ -414,9 +473,9 @@ extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
   int nblk;
-  bn_blocks(dtype, rows, channels, kBnApplyBlocks, &per, &nblk);
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
+    bn_blocks(dtype, rows, channels, bn_resident_blocks((const void*)bn_apply_kernel<T, VEC>), &per, &nblk);
     hipLaunchKernelGGL((bn_apply_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, rows, channels, per,
                        mean, invstd, gamma, beta, param_dtype, relu, (const T*)residual, (T*)y);
   });
@@ -439,10 +498,10 @@ extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy
   int64_t per_a;
   int nblk_a;
   bn_blocks(dtype, rows, channels, kBnMaxBlocks, &per, &nblk);
-  bn_blocks(dtype, rows, channels, kBnApplyBlocks, &per_a, &nblk_a);
   float* partial = (float*)workspace;
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
+    bn_blocks(dtype, rows, channels, bn_resident_blocks((const void*)bn_bwd_apply_kernel<T, VEC>), &per_a, &nblk_a);
     hipLaunchKernelGGL((bn_bwd_stats_kernel<T, VEC>), dim3(nblk), dim3(256), 0, st, (const T*)x, (const T*)dy, rows,
                        channels, per, mean, invstd, gamma, beta, param_dtype, relu, (const T*)y, partial);
     hipLaunchKernelGGL(bn_bwd_finish_kernel, dim3((unsigned)cdiv(channels, 4)), dim3(256), 0, st, partial, nblk,
