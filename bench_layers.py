@@ -206,6 +206,11 @@ def main():
         o._table(8, '333', 1, True), bf)
     run('conv 3x3x3 s1 128->96 d9 nempty', OctreeConv(128, 96, [3], 1, nempty=True), o, 9, ne9, 128, 96,
         o._table(9, '333', 1, True), bf)
+    # the coarse levels of the same net (encoder 64 / 128 / 256 channels at depths 7 / 6 / 5, decoder 256 / 128
+    # at depths 6 / 7): few rows, many channels
+    for d, c in ((7, 64), (7, 128), (6, 128), (6, 256), (5, 256)):
+      run('conv 3x3x3 s1 %d->%d d%d nempty' % (c, c, d), OctreeConv(c, c, [3], 1, nempty=True), o, d,
+          int(o.nnum_nempty[d]), c, c, o._table(d, '333', 1, True), bf)
     run('conv 2x2x2 s2 96->96 d9->8 nempty', OctreeConv(96, 96, [2], 2, nempty=True), o, 9, ne9, 96, 96,
         o._table(9, '222', 2, True), bf)
     run('deconv 2x2x2 s2 96->96 d8->9 nempty', OctreeDeconv(96, 96, [2], 2, nempty=True), o, 8, ne8, 96, 96,
