@@ -906,15 +906,16 @@ def test_layers_on_the_sparse_kernels(medium, dtype):
   """Whole layers (module forward + backward against the oracle) with the thresholds of the
   Python layer lowered so that the pair-plan kernels run on the test octree: 3x3x3 and axis
   kernels on non-empty nodes (gather, data gradient through the mirrored slots, weight
-  gradient), 2x2x2 stride-2 conv / deconv (gathers over the table and its inverse, weight
-  gradient over the inverse table)."""
+  gradient), 2x2x2 and 3x3x3 stride-2 conv / deconv (gathers over the table and its inverse,
+  weight gradient over the inverse table)."""
   conv_mod = sys.modules['ocnn_amd.nn.octree_conv']
   keep = (conv_mod.SPARSE_MIN_ROWS, conv_mod.SPARSE_MAX_OCCUPANCY)
   conv_mod.SPARSE_MIN_ROWS, conv_mod.SPARSE_MAX_OCCUPANCY = 0, 1.0
   try:
     for kind, ks, stride, cin, cout in [('conv', [3], 1, 96, 96), ('conv', [3], 1, 128, 96), ('conv', [3, 3, 1], 1, 32, 96),
                                         ('conv', [2], 2, 96, 128), ('conv', [2], 2, 32, 64), ('deconv', [2], 2, 128, 96),
-                                        ('deconv', [2], 2, 96, 32), ('deconv', [3], 1, 96, 64)]:
+                                        ('deconv', [2], 2, 96, 32), ('deconv', [3], 1, 96, 64),
+                                        ('conv', [3], 2, 64, 64), ('conv', [3], 2, 96, 32), ('deconv', [3], 2, 32, 96)]:
       depth = 6 if kind == 'deconv' and stride == 2 else 7
       say('layers on the sparse kernels', dtype, kind, ks, stride, cin, cout)
       errs = run_layer(kind, medium, depth, ks, stride, True, cin, cout, dtype)
