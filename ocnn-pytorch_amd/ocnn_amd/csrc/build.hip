@@ -470,11 +470,16 @@ static int build_args_ok(int64_t n, int depth, int full_depth, int batch_bits) {
   OCNN_REQUIRE(depth >= 1 && depth <= kBuildMaxDepth && full_depth >= 0 && full_depth <= depth && full_depth <= 8,
                "octree_build: depth=%d full_depth=%d out of range", depth, full_depth);
   OCNN_REQUIRE(batch_bits >= 0 && batch_bits <= 15, "octree_build: batch_bits=%d out of range", batch_bits);
+  // (a point counts its node starts in depth - full_depth + 1 layers, sixteen counters at most)
+  OCNN_REQUIRE(depth - full_depth + 1 <= 16, "octree_build: %d layers below the full ones, at most 15",
+               depth - full_depth);
   return OCNN_OK;
 }
 
 extern "C" int64_t ocnn_octree_build_workspace_bytes(int64_t n, int depth, int full_depth, int batch_bits) {
-  if (n <= 0 || depth < 1 || depth > kBuildMaxDepth || full_depth < 0 || full_depth > depth) return -1;
+  if (n <= 0 || depth < 1 || depth > kBuildMaxDepth || full_depth < 0 || full_depth > depth ||
+      depth - full_depth + 1 > 16)
+    return -1;
   const int key_bits = 3 * depth, levels = depth - full_depth;
   BuildLayout L;
 #define OCNN_BUILD_BYTES(K, N) (build_layout_t<K, N>(n, &L) == OCNN_OK ? L.total : (int64_t)-1)

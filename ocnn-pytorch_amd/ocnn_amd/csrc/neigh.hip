@@ -156,6 +156,7 @@ extern "C" int ocnn_neigh_from_parent(const int32_t* child_p, const int32_t* nei
                                       const int32_t* nempty_p, int64_t n_ne, int64_t* out64,
                                       int32_t* out32, void* stream) {
   OCNN_REQUIRE(n_ne > 0 && n_ne * 8 < (1ll << 31), "neigh_from_parent: n_ne=%lld", (long long)n_ne);
+  OCNN_REQUIRE(child_p && neigh_p && nempty_p && (out64 || out32), "neigh_from_parent: a null array");
   hipLaunchKernelGGL(neigh_from_parent_kernel, dim3(cdiv(n_ne, kParentsPerBlock)), dim3(256), 0,
                      (hipStream_t)stream, child_p, neigh_p, nempty_p, n_ne, out64, out32);
   return check_launch("neigh_from_parent");
@@ -166,8 +167,11 @@ extern "C" int ocnn_neigh_from_parent(const int32_t* child_p, const int32_t* nei
 extern "C" int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_t* h_nnum,
                               const int64_t* h_nnum_nempty, const int32_t* const* h_children,
                               int32_t* const* h_nempty_index, int32_t* const* h_neigh, void* stream) {
-  OCNN_REQUIRE(depth >= 1 && depth <= 16 && full_depth >= 0 && full_depth <= depth && full_depth <= 7 && batch >= 1,
-               "neigh_all: depth=%d full_depth=%d batch=%d", depth, full_depth, batch);
+  // (the table of a layer below the full ones is made from its parents' table, and layer 0 has
+  // none: as in the reference, whose construct_neigh(1) fails on an octree with full_depth = 0)
+  OCNN_REQUIRE(depth >= 1 && depth <= 16 && full_depth >= 1 && full_depth <= depth && full_depth <= 7 && batch >= 1,
+               "neigh_all: depth=%d full_depth=%d batch=%d (full_depth >= 1: layer 1 must be full)", depth,
+               full_depth, batch);
   hipStream_t st = (hipStream_t)stream;
   for (int d = 1; d <= depth; ++d) {
     OCNN_REQUIRE(h_neigh[d] != nullptr && h_nnum[d] > 0 && h_nnum[d] * 27 < (1ll << 31), "neigh_all: layer %d", d);
@@ -179,7 +183,7 @@ extern "C" int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_
       continue;
     }
     const int64_t n_ne = h_nnum_nempty[d - 1];
-    OCNN_REQUIRE(n_ne > 0 && 8 * n_ne == h_nnum[d] && h_children[d - 1] && h_nempty_index[d - 1],
+    OCNN_REQUIRE(n_ne > 0 && 8 * n_ne == h_nnum[d] && h_children[d - 1] && h_nempty_index[d - 1] && h_neigh[d - 1],
                  "neigh_all: layers %d and %d are inconsistent", d - 1, d);
     hipLaunchKernelGGL(nempty_index_kernel, dim3((unsigned)cdiv(h_nnum[d - 1], 256)), dim3(256), 0, st,
                        h_children[d - 1], h_nnum[d - 1], h_nempty_index[d - 1], (int64_t*)nullptr);

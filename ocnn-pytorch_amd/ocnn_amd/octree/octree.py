@@ -654,7 +654,8 @@ class Octree:
     depth = self.depth
     nnum = [int(v) for v in self.nnum[:depth + 1].tolist()]
     nempty = [int(v) for v in self.nnum_nempty[:depth + 1].tolist()]
-    if dev.type != 'cuda' or any(c is None for c in self.children[:depth + 1]) or min(nnum[1:] + nempty) <= 0 or \
+    if dev.type != 'cuda' or self.full_depth < 1 or any(c is None for c in self.children[:depth + 1]) or \
+        min(nnum[1:] + nempty) <= 0 or \
         any(nnum[d] != (self.batch_size << (3 * d) if d <= self.full_depth else 8 * nempty[d - 1])
             for d in range(1, depth + 1)):
       for d in range(1, depth + 1):                       # the layer-by-layer route says what is wrong

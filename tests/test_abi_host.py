@@ -74,6 +74,20 @@ def test_octree_public_luts_and_errors():
     o.get_neigh(3, '333', stride=3)
 
 
+def test_neighbour_tables_need_a_full_first_layer():
+  """The table of a layer below the full ones is made from its parents' table, and layer 0 has
+  none: with full_depth = 0 the library refuses (an error code before any launch) instead of
+  reading a table that does not exist; the reference's construct_neigh(1) fails there too."""
+  L = _lib.lib()
+  P = lambda *v: (ctypes.c_void_p * len(v))(*v)
+  N = lambda *v: (ctypes.c_int64 * len(v))(*v)
+  assert L.ocnn_neigh_all(2, 0, 1, N(1, 8, 64), N(1, 8, 64), P(None, None, None), P(None, None, None),
+                          P(None, None, None), None) != 0
+  assert 'full_depth' in L.ocnn_last_error().decode()
+  assert L.ocnn_neigh_from_parent(None, None, None, 8, None, None, None) != 0
+  assert 'null' in L.ocnn_last_error().decode()
+
+
 def test_no_cpu_fallback():
   pts = ocnn_amd.Points(torch.rand(10, 3) * 0.5)
   o = ocnn_amd.Octree(depth=4, full_depth=2)

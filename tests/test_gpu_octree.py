@@ -410,6 +410,34 @@ def test_deep_octrees_vs_oracle(depth, full, batch, n):
       assert np.array_equal(np_(o.nempty_index(d)), np.nonzero(w.children[d] >= 0)[0]), d
 
 
+def test_octree_without_a_full_layer_below_the_root():
+  """full_depth = 0: the build equals the oracle's; the neighbour tables cannot be made (layer 1
+  would need the table of layer 0, which does not exist - the reference's construct_neigh(1) fails
+  on it too) and both routes refuse with an error instead of launching anything."""
+  rng = np.random.default_rng(3)
+  n, depth, batch = 400, 5, 2
+  pts = rng.uniform(-0.9, 0.9, (n, 3)).astype(np.float32)
+  nrm = rng.standard_normal((n, 3)).astype(np.float32)
+  bid = np.sort(np.r_[0, 1, rng.integers(0, batch, n - 2)]).astype(np.int64)
+  say('octree with full_depth 0')
+  pc = Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV),
+              batch_id=torch.from_numpy(bid).view(-1, 1).to(DEV), batch_size=batch)
+  o = Octree(depth, 0, batch_size=batch)
+  idx = o.build_octree(pc)
+  w, widx = R.build_octree(pts, nrm, None, bid, depth, 0, batch)
+  assert np.array_equal(o.nnum.numpy(), w.nnum) and np.array_equal(o.nnum_nempty.numpy(), w.nnum_nempty)
+  assert np.array_equal(np_(idx), widx)
+  for d in range(depth + 1):
+    assert np.array_equal(np_(o.keys[d]), w.keys[d]), d
+    assert np.array_equal(np_(o.children[d]), w.children[d]), d
+  with pytest.raises(AssertionError):
+    o.construct_all_neigh()
+  with pytest.raises(AssertionError):
+    o.construct_neigh(1)
+  with pytest.raises(TypeError):
+    R.construct_all_neigh(w)
+
+
 @pytest.mark.parametrize('depth,batch', [(8, 1), (9, 4), (6, 2)])
 def test_uneven_clouds_vs_oracle(depth, batch):
   """Nine points in ten of a cloud inside one small cell (thousands of points to a leaf, a few
