@@ -331,3 +331,62 @@ def test_transposed_matrix_edge_cases():
     rowptr2, col2, val2 = _transpose(idx.to(DEV), None, None, rows)
     assert val2 is None and np.array_equal(rowptr2.cpu().numpy(), rowptr)
     assert np.array_equal(col2.cpu().numpy()[:rowptr[-1]], col[:rowptr[-1]])
+
+
+def test_random_interp_and_pool_vs_oracle():
+  """Random octrees (depth 2 .. 8, one to four clouds, 1 .. 10 000 points), a random layer of
+  each, all or non-empty nodes, bounds check on or off, 1 .. 20 channels, 1 .. 5 000 query points
+  scattered around the cloud with some beyond the volume on either side: trilinear and nearest
+  interpolation, the gradient of the former, max pooling with its indices and nearest upsampling
+  against the oracle.  OCNN_TEST_CASES sets the number of cases (default 60)."""
+  from oracle import octree_ref as R
+  for case in range(int(os.environ.get('OCNN_TEST_CASES', '60'))):
+    rng = np.random.default_rng(9000 + case)
+    depth = int(rng.integers(2, 9))
+    full = max(1, min(int(rng.integers(1, 4)), depth))
+    n = int(rng.choice([1, 5, 100, 2000, 10000]))
+    batch = min(int(rng.choice([1, 1, 2, 4])), n)
+    c = rng.uniform(-0.8, 0.8, (4, 3))
+    pts = np.clip(c[rng.integers(0, 4, n)] + rng.normal(0, 0.15, (n, 3)), -1.0, 0.999999).astype(np.float32)
+    nrm = rng.standard_normal((n, 3)).astype(np.float32)
+    bid = None
+    if batch > 1:
+      bid = rng.integers(0, batch, n)
+      bid[:batch] = np.arange(batch)
+      bid = np.sort(bid).astype(np.int64)
+    d = int(rng.integers(1, depth + 1))
+    ne, bc = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    C = int(rng.choice([1, 3, 8, 16, 20]))
+    m = int(rng.choice([1, 7, 300, 5000]))
+    say('random interp', case, 'depth', depth, 'full', full, 'batch', batch, 'points', n, 'layer', d, 'nempty', ne,
+        'bound check', bc, 'channels', C, 'queries', m)
+    pc = Points(torch.from_numpy(pts).to(DEV), torch.from_numpy(nrm).to(DEV),
+                batch_id=None if bid is None else torch.from_numpy(bid).view(-1, 1).to(DEV), batch_size=batch)
+    o = Octree(depth, full, batch_size=batch)
+    o.build_octree(pc)
+    o.construct_all_neigh()
+    w, _ = R.build_octree(pts, nrm, None, bid, depth, full, batch)
+    R.construct_all_neigh(w)
+    rows = int(o.nnum_nempty[d] if ne else o.nnum[d])
+    data = rng.standard_normal((rows, C)).astype(np.float32)
+    src = rng.integers(0, n, m)
+    q = (pts[src] + 1.0) * 2.0 ** (d - 1) + rng.normal(0, 0.7, (m, 3))
+    q[rng.random(m) < 0.05] -= 2.0 ** d
+    q[rng.random(m) < 0.05] += 2.0 ** d
+    qb = (bid[src] if bid is not None else np.zeros(m)).astype(np.float32)
+    q = np.concatenate([q.astype(np.float32), qb[:, None]], 1)
+    dg = torch.from_numpy(data).to(DEV).requires_grad_()
+    qg = torch.from_numpy(q).to(DEV)
+    out = octree_linear_pts(dg, o, d, qg.clone(), ne, bc)
+    assert np.allclose(np_(out), I.linear_pts(w, data, d, q, ne, bc), atol=2e-5), case
+    grad = rng.standard_normal((m, C)).astype(np.float32)
+    out.backward(torch.from_numpy(grad).to(DEV))
+    wantg = I.linear_pts_grad(w, grad, d, q, rows, ne, bc)
+    assert np.allclose(np_(dg.grad), wantg, atol=2e-4 * max(1.0, np.abs(wantg).max())), case
+    assert np.array_equal(np_(octree_nearest_pts(dg, o, d, qg.clone(), ne, bc)), I.nearest_pts(w, data, d, q, ne, bc)), case
+    if d >= 2:
+      po, pi = octree_max_pool(dg.detach(), o, d, ne, return_indices=True)
+      wp, wi = I.max_pool(w, data, d, ne)
+      assert np.array_equal(np_(po), wp) and np.array_equal(np_(pi), wi), case
+    if d < depth:
+      assert np.array_equal(np_(octree_nearest_upsample(dg.detach(), o, d, ne)), I.nearest_upsample(w, data, d, ne)), case

@@ -2,6 +2,7 @@
 in fp64 on the CPU: outputs, running statistics, all three gradients, training and evaluation
 mode, every dtype."""
 
+import os
 import sys
 
 import numpy as np
@@ -294,3 +295,60 @@ def test_residual_block_is_its_parts(cin, cout, nempty):
     for u, v in stats:
       assert close(u.running_mean, v.running_mean) and close(u.running_var, v.running_var)
       assert int(u.num_batches_tracked) == int(v.num_batches_tracked) == 1
+
+
+def test_random_batch_norms_vs_torch():
+  """Random shapes (2 .. 200 000 rows, 4 .. 2048 channels incl. counts that are no power of two),
+  dtypes, training / evaluation, with and without ReLU and residual, against torch's batch norm in
+  fp64: output, input gradient and both parameter gradients.  The reference takes the ReLU's mask
+  from the output of the kernel (where the value before the ReLU is within rounding of zero the mask
+  is a coin toss in any arithmetic), after checking that it differs from the fp64 mask nowhere
+  else.  OCNN_TEST_CASES sets the number of cases (default 40)."""
+  for case in range(int(os.environ.get('OCNN_TEST_CASES', '40'))):
+    rng = np.random.default_rng(7000 + case)
+    rows = int(rng.choice([2, 3, 63, 64, 65, 1000, 4097, 50000, 200000]))
+    dtype = [torch.float32, torch.float16, torch.bfloat16][int(rng.integers(0, 3))]
+    c = int(rng.choice([8, 16, 24, 40, 64, 96, 128, 200, 256, 512, 1024, 2048] +
+                       ([4, 12, 36] if dtype == torch.float32 else [])))
+    if rows * c > 3e7:
+      rows = max(2, int(3e7) // c)
+    relu, training = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    res = bool(rng.integers(0, 2)) and relu
+    say('random batch norm', case, rows, c, dtype, 'relu', relu, 'training', training, 'residual', res)
+    g = torch.Generator().manual_seed(case)
+    x = (torch.randn(rows, c, generator=g) * 1.5 + 3.0).to(dtype)
+    w = (torch.rand(c, generator=g) + 0.5).to(dtype).float()
+    b = (torch.randn(c, generator=g) * 0.3).to(dtype).float()
+    rm = (torch.randn(c, generator=g) * 0.1 + 3.0).to(dtype).float()
+    rv = (torch.rand(c, generator=g) + 1.5).to(dtype).float()
+    dy = torch.randn(rows, c, generator=g).to(dtype)
+    r = torch.randn(rows, c, generator=g).to(dtype) if res else None
+    bn64 = torch.nn.BatchNorm1d(c, eps=1e-5, momentum=0.1).double()
+    with torch.no_grad():
+      bn64.weight.copy_(w.double()); bn64.bias.copy_(b.double())
+      bn64.running_mean.copy_(rm.double()); bn64.running_var.copy_(rv.double())
+    bn64.train(training)
+    xd = x.double().requires_grad_()
+    pre = bn64(xd)
+    if res:
+      pre = pre + r.double()
+    bn = BatchNormRelu1d(c, relu=relu).to(DEV)
+    with torch.no_grad():
+      bn.weight.copy_(w); bn.bias.copy_(b); bn.running_mean.copy_(rm); bn.running_var.copy_(rv)
+    bn = bn.to(dtype) if dtype != torch.float32 else bn
+    bn.train(training)
+    xg = x.to(DEV).requires_grad_()
+    y = bn(xg, r.to(DEV)) if res else bn(xg)
+    y.backward(dy.to(DEV))
+    mask = (y.detach().cpu() > 0).double() if relu else torch.ones_like(pre)
+    if relu:
+      near_zero = (4e-2 if dtype != torch.float32 else 1e-4) * (1 + (r.double().abs() if res else 0))
+      assert not bool((((pre.detach() > 0).double() != mask) & (pre.detach().abs() > near_zero)).any()), case
+    y64 = pre * mask
+    y64.backward(dy.double())
+    tol = TOL[dtype] * (8 if rows < 16 else 1)      # (statistics over a handful of rows are ill-conditioned in 16 bits)
+    sc = lambda t: max(1.0, float(t.abs().max()))
+    assert float((y.detach().double().cpu() - y64.detach()).abs().max()) <= (2 if res else 1) * tol * sc(y64.detach()), case
+    assert float((xg.grad.double().cpu() - xd.grad).abs().max()) <= 6 * tol * sc(xd.grad), case
+    assert float((bn.weight.grad.double().cpu() - bn64.weight.grad).abs().max()) <= 16 * tol * sc(bn64.weight.grad), case
+    assert float((bn.bias.grad.double().cpu() - bn64.bias.grad).abs().max()) <= 6 * tol * sc(bn64.bias.grad), case

@@ -320,8 +320,8 @@ def test_random_octrees_vs_oracle():
   """Random depth / full depth / batch size / point counts (1 .. 40 000) and point
   distributions (uniform, a sphere, clusters with duplicates, grid-aligned coordinates up to the
   box faces): keys, children, counts, point -> leaf map, leaf signals and all neighbour tables
-  bit exact against the oracle."""
-  for case in range(60):
+  bit exact against the oracle.  OCNN_TEST_CASES sets the number of cases (default 60)."""
+  for case in range(int(os.environ.get('OCNN_TEST_CASES', '60'))):
     rng = np.random.default_rng(case)
     depth = int(rng.integers(2, 10))
     full = max(1, min(int(rng.integers(1, 5)), depth - 1))
