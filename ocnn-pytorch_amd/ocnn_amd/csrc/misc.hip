@@ -203,10 +203,10 @@ __global__ __launch_bounds__(256) void dw_wgrad_rows_kernel(
 #pragma unroll
     for (int v = 0; v < 4; ++v) s_red[(rl * lpr + cl) * 4 + v] = acc[k][v];
     __syncthreads();
-    if (tid < C) {
+    for (int c = tid; c < C; c += 256) {                     // (more channels than threads from 512 on)
       float sum = 0.f;
-      for (int r = 0; r < rp; ++r) sum += s_red[(r * lpr + (tid >> 2)) * 4 + (tid & 3)];
-      dst[k * C + tid] = sum;
+      for (int r = 0; r < rp; ++r) sum += s_red[(r * lpr + (c >> 2)) * 4 + (c & 3)];
+      dst[k * C + c] = sum;
     }
   }
 }

@@ -163,6 +163,10 @@ def test_mfma_stride2_deconv_dw(medium, dtype):
     assert max(errs.values()) < TOL[dtype], errs
     errs = run_layer('dwconv', medium, 7, [2], 2, ne, 24, 24, dtype)
     assert max(errs.values()) < TOL[dtype], errs
+    # more channels than a workgroup has threads (every channel's weight gradient must be written)
+    say('dwconv s2 512', dtype, ne)
+    errs = run_layer('dwconv', medium, 6, [2], 2, ne, 512, 512, dtype)
+    assert max(errs.values()) < TOL[dtype], errs
 
 
 def test_fp32_larger(medium):
