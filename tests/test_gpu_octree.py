@@ -505,8 +505,8 @@ def test_random_octrees_regrown_from_split_masks():
   """octree_grow_full / octree_split / octree_grow (ocnn/octree/octree.py:289-402), as a
   generative decoder drives them: an octree regrown level by level from the split masks of a
   built one has the same keys, children, counts and neighbour tables (the property the
-  reference's own test checks on its one file), on 25 random octrees."""
-  for case in range(25):
+  reference's own test checks on its one file), on 25 random octrees (OCNN_TEST_CASES: another number)."""
+  for case in range(int(os.environ.get('OCNN_TEST_CASES', '25'))):
     rng = np.random.default_rng(1000 + case)
     depth = int(rng.integers(3, 8))
     full = max(1, min(int(rng.integers(1, 4)), depth - 1))
@@ -544,8 +544,9 @@ def test_random_octrees_regrown_from_split_masks():
 def test_random_merge_equals_batched_build():
   """merge_octrees of separately built octrees == build_octree on the merged cloud with batch
   ids (the identity the reference's test_octree.py:115-123 checks on its two files), on random
-  clouds of unequal sizes: keys, children, counts, leaf signals, neighbour tables, batch_nnum."""
-  for case in range(12):
+  clouds of unequal sizes: keys, children, counts, leaf signals, neighbour tables, batch_nnum
+  (12 cases, or OCNN_TEST_CASES)."""
+  for case in range(int(os.environ.get('OCNN_TEST_CASES', '12'))):
     rng = np.random.default_rng(2000 + case)
     depth = int(rng.integers(3, 8))
     full = max(1, min(int(rng.integers(1, 4)), depth - 1))
