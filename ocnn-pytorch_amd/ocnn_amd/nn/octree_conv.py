@@ -373,7 +373,10 @@ class OctreeConvBase:
       return gw.transpose(1, 2).contiguous() if out_transposed else gw
     if coarse_index is not None:
       grad = grad.index_select(0, coarse_index.long())
-    if self.stride == 2 and self.kernel in ('222', '333') and self.neigh.shape[0] >= SPARSE_MIN_ROWS // 8 and \
+    # (3x3x3 over all nodes: 20 of the 27 slots of a table row are set, and the plan-free kernel
+    # over the table is faster than the pairs of the inverse)
+    if self.stride == 2 and (self.kernel == '222' or (self.kernel == '333' and self.nempty)) and \
+        self.neigh.shape[0] >= SPARSE_MIN_ROWS // 8 and \
         _lib.lib().ocnn_conv_wgrad_sparse_supported(_lib.DTYPE_CODE.get(data.dtype, -1), grad.shape[0],
                                                     data.shape[0], self.kdim, grad.shape[1], data.shape[1], 0):
       plan_t = self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, True, self.fine_h)
