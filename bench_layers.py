@@ -16,6 +16,8 @@ MI355X (the headline number is bench.py's; these lines are supporting data).
   config f4: the rest of the kernel-shape x stride grid on the depth-8 batch of config 2, bf16,
             64 channels: 3x3x3 stride 2 (conv and deconv), the axis kernels 3x1x1 and 3x3x1 at
             stride 1 and 2, 2x2x2 at stride 1, on all nodes and on non-empty nodes.
+  config bn (not in the default set): batch norm + ReLU, forward + backward, on the tensors of
+            the U-Net of config 4.
 
 Every layer runs forward + backward through the module (autograd included); one JSON
 line per layer: ms per fwd+bwd, effective TFLOP/s over non-empty neighbours, and the
@@ -148,6 +150,21 @@ def main():
            2 * 2 * (rows * 64 + prow * 64) + 2 * 8 * prow * 64, {'rows': rows, 'parents': prow})
 
   bf = torch.bfloat16
+  if 'bn' in args.configs.split(','):
+    # batch norm + ReLU, training mode, on the tensors of the U-Net of config 4 (rows of the non-empty
+    # nodes of depths 9 .. 5 x the channels the net has there): forward 2 reads + 1 write, backward
+    # 4 reads + 1 write of the tensor
+    from ocnn_amd.nn import BatchNormRelu1d
+    for rows, c in ((925113, 32), (925113, 96), (621985, 64), (621985, 96), (280645, 128), (83376, 256),
+                    (21148, 256)):
+      bn = BatchNormRelu1d(c, relu=True).to(dev).to(bf)
+      x = torch.randn(rows, c, device=dev).to(bf).requires_grad_()
+      g = torch.randn(rows, c, device=dev).to(bf)
+
+      def step():
+        x.grad = None
+        bn(x).backward(g)
+      run_op('batch norm + relu %d x %d bfloat16' % (rows, c), step, 8 * rows * c * 2, {'rows': rows, 'channels': c})
   if '2' in args.configs.split(','):
     o, b_ms, n_ms, npts = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
     print(json.dumps({'octree': 'config 2 (batch 8, depth 8)', 'points': npts, 'build_octree_ms': b_ms,
