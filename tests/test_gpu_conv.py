@@ -112,6 +112,60 @@ def run_layer(kind, pair, depth, ks, stride, nempty, cin, cout, dtype, seed=0, u
   return errs
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_fp32_modules_on_16_bit_features(medium, dtype):
+  """Mixed precision as torch.amp leaves it (ocnn/nn/octree_conv.py:232,270: `weights.to(data.dtype)`):
+  modules with fp32 parameters on 16-bit features give the bits of the all-16-bit run on the rounded
+  parameters, and parameter gradients in fp32; the batch norm with fp32 parameters and buffers
+  likewise matches its 16-bit twin to the rounding of the parameters."""
+  from ocnn_amd.nn import BatchNormRelu1d
+  g = torch.Generator().manual_seed(5)
+  for kind, ks, stride, ne, cin, cout in [('conv', [3], 1, False, 64, 64), ('conv', [3], 1, True, 96, 96),
+                                          ('conv', [2], 2, False, 32, 64), ('deconv', [2], 2, True, 64, 32),
+                                          ('dwconv', [3], 1, False, 64, 64), ('conv', [3], 2, True, 48, 16)]:
+    say('fp32 module on', dtype, kind, ks, stride, ne, cin, cout)
+    Mod = {'conv': OctreeConv, 'deconv': OctreeDeconv}.get(kind)
+    mod = OctreeDWConv(cin, ks, stride, ne, use_bias=True) if Mod is None else Mod(cin, cout, ks, stride, ne, use_bias=True)
+    with torch.no_grad():
+      mod.weights.copy_((torch.randn(mod.weights.shape, generator=g) / 30).to(dtype).float())   # values the dtype holds
+      mod.bias.copy_(torch.randn(mod.bias.shape, generator=g).to(dtype).float())
+    mod = mod.to(DEV)
+    depth = 6 if kind == 'deconv' else 7
+    rows = rows_of(medium.ref, depth, ne)
+    x = torch.randn(rows, cin, generator=g).to(dtype).to(DEV).requires_grad_()
+    out = mod(x, medium.gpu, depth)
+    gout = torch.randn(out.shape, generator=g).to(dtype).to(DEV)
+    out.backward(gout)
+    assert out.dtype == dtype and x.grad.dtype == dtype
+    assert mod.weights.grad.dtype == torch.float32 and mod.bias.grad.dtype == torch.float32
+    import copy
+    twin = copy.deepcopy(mod).to(dtype)
+    twin.weights.grad = twin.bias.grad = None
+    x2 = x.detach().clone().requires_grad_()
+    out2 = twin(x2, medium.gpu, depth)
+    out2.backward(gout)
+    assert torch.equal(out, out2) and torch.equal(x.grad, x2.grad)
+    assert torch.equal(mod.weights.grad, twin.weights.grad.float()) and torch.equal(mod.bias.grad, twin.bias.grad.float())
+  for rows, c, relu in [(5000, 64, True), (777, 96, False)]:
+    say('fp32 batch norm on', dtype, rows, c)
+    bn = BatchNormRelu1d(c, relu=relu).to(DEV)
+    with torch.no_grad():
+      bn.weight.copy_((torch.rand(c, generator=g) + 0.5).to(dtype).float())
+      bn.bias.copy_(torch.randn(c, generator=g).to(dtype).float())
+    import copy
+    twin = copy.deepcopy(bn).to(dtype)
+    x = (torch.randn(rows, c, generator=g) + 1.0).to(dtype).to(DEV).requires_grad_()
+    x2 = x.detach().clone().requires_grad_()
+    dy = torch.randn(rows, c, generator=g).to(dtype).to(DEV)
+    y, y2 = bn(x), twin(x2)
+    y.backward(dy)
+    y2.backward(dy)
+    assert y.dtype == dtype and bn.weight.grad.dtype == torch.float32 and bn.running_mean.dtype == torch.float32
+    assert torch.equal(y, y2) and torch.equal(x.grad, x2.grad)
+    assert torch.allclose(bn.weight.grad, twin.weight.grad.float(), rtol=1e-2, atol=1e-2 * float(bn.weight.grad.abs().max()))
+    assert torch.allclose(bn.running_var, twin.running_var.float(), rtol=1e-2, atol=1e-2)
+
+
 GRID = [(k, s, ne) for k in ['333', '222', '311', '131', '113', '331', '313', '133']
         for s in (1, 2) for ne in (False, True)]
 
