@@ -242,3 +242,60 @@ def test_unet_full_size_bf16():
   cos = float((a.double() @ b.double()) / (a.double().norm() * b.double().norm()))
   say('   cosine of the full gradient vectors %.4f, norm ratio %.4f' % (cos, float(b.norm() / a.norm())))
   assert cos > 0.9
+
+
+def test_residual_blocks_replay_from_a_hip_graph():
+  """Forward + backward of a chain of residual blocks (3x3x3 convolutions, batch norm with running
+  statistics and batch counter, ReLU, 1x1 projection of the shortcut) captured in a HIP graph after
+  two eager steps: every replay gives the bits of an eager step, and the batch counters count the
+  replays (they are incremented by a kernel, not by the host)."""
+  from ocnn_amd.modules import OctreeResBlocks
+  say('residual blocks from a hip graph')
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 2, 77, n=30000)
+  o = Octree(7, 2, batch_size=2)
+  o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=2))
+  o.construct_all_neigh()
+  depth, dtype = 7, torch.bfloat16
+  torch.manual_seed(3)
+  net = OctreeResBlocks(32, 64, 2, bottleneck=1, nempty=True).to(DEV).to(dtype)
+  rows = int(o.nnum_nempty[depth])
+  x = torch.randn(rows, 32, device=DEV).to(dtype).requires_grad_()
+  gout = torch.randn(rows, 64, device=DEV).to(dtype)
+  params = [x] + list(net.parameters())
+  counters = [m.num_batches_tracked for m in net.modules() if hasattr(m, 'num_batches_tracked')]
+  assert len(counters) == 5
+
+  def step():
+    for p in params:
+      p.grad = None
+    out = net(x, o, depth)
+    out.backward(gout)
+    return out
+
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    for _ in range(2):
+      out = step()
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  want = [out.detach().clone()] + [p.grad.clone() for p in params]
+  del out
+  assert all(int(c) == 2 for c in counters)
+  graph = torch.cuda.CUDAGraph()
+  for p in params:
+    p.grad = None
+  with torch.cuda.graph(graph):
+    out_g = net(x, o, depth)
+    out_g.backward(gout)
+  for replay in range(3):
+    out_g.detach().zero_()
+    for p in params:
+      p.grad.zero_()
+    (torch.randn(500, 64, device=DEV) @ torch.randn(64, 64, device=DEV)).sum().item()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    for a, b in zip(want, [out_g] + [p.grad for p in params]):
+      assert torch.equal(a, b), replay
+  assert all(int(c) == 2 + 3 for c in counters), [int(c) for c in counters]
