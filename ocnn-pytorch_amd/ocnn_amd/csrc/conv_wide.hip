@@ -378,7 +378,9 @@ static int run_wide(const void* in, int64_t rows_in, const uint16_t* loc, const 
   const int64_t tiles = cdiv(rows_out, kWdRows);
   const int64_t per_xcd = cdiv(tiles, 8);
   const uint32_t in_bytes = (uint32_t)(rows_in * cin * 2);
-  if (cout % 256 == 0)
+  // 256 output channels per workgroup halve the LDS reads per MFMA; a launch with a handful of tiles
+  // (a quarter of the CUs or fewer) is faster with 128 per workgroup on twice as many CUs
+  if (cout % 256 == 0 && tiles * (cout / 256) > 64)
     hipLaunchKernelGGL((conv_gather_wide_kernel<T, 2>), dim3((unsigned)(per_xcd * 8), (unsigned)(cout / 256)),
                        dim3(256), 0, st, (const T*)in, in_bytes, loc, uptr, urows, (const T*)ws, (const T*)bias,
                        (T*)out, rows_out, K, cin, cout, tiles, per_xcd);
