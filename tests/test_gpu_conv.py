@@ -6,6 +6,7 @@ Tolerances (relative to the largest magnitude of the expected tensor):
   float16, bfloat16  2e-2 against the fp64 result on the same (rounded) inputs
 """
 
+import ctypes
 import os
 import sys
 
@@ -1425,3 +1426,85 @@ def test_column_sums(dtype):
     assert got.dtype == dtype and tuple(got.shape) == (C,)
     assert float((got.double() - want).abs().max()) <= tol * max(1.0, float(want.abs().max())) + tol * rows ** 0.5
     assert torch.equal(got, column_sum(x))
+
+
+def test_the_documented_call_sequence_of_the_abi():
+  """The calls a binder makes, in the order the integration notes give them, with nothing of the
+  Python layer in between: tile plan by count / offsets / fill (six statistics, one read-back),
+  the library's choice of the kernel, the register-resident gather on the plan, then the pair plan
+  (slot counts, lists on the host, count, fill) and the pair-plan gather and weight gradient -
+  against the plan-free entry points on the same table."""
+  from ctypes import byref, c_int, c_int32, c_int64
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(21)
+  rows = rows_in = 128 * 300 + 17
+  K, code, st = 27, _lib.DTYPE_CODE[torch.bfloat16], _lib.stream()
+  table = _local_table(rows, rows_in, K, g, spread=30, empty=0.8).to(DEV)
+  P = lambda t: t.data_ptr()
+  say('abi sequence: tile plan')
+  R = L.ocnn_tile_plan_rows()
+  tiles = (rows + R - 1) // R
+  ucount = torch.empty(tiles, dtype=torch.int32, device=DEV)
+  tile_nnz = torch.empty(tiles, dtype=torch.int32, device=DEV)
+  uptr = torch.empty(tiles + 1, dtype=torch.int32, device=DEV)
+  stats = torch.empty(6, dtype=torch.int64, device=DEV)
+  _lib.check(L.ocnn_tile_plan_count(P(table), rows, K, P(ucount), P(tile_nnz), st))
+  _lib.check(L.ocnn_tile_plan_offsets(P(ucount), P(tile_nnz), tiles, 415, P(uptr), P(stats), st))
+  over, dropped, total, umax, nnz, _ = stats.tolist()
+  assert over == 0 and dropped == 0 and nnz == int((table >= 0).sum()) and 0 < umax <= 415
+  urows = torch.empty(total, dtype=torch.int32, device=DEV)
+  loc = torch.empty((tiles, K, R), dtype=torch.int16, device=DEV)
+  _lib.check(L.ocnn_tile_plan_fill(P(table), rows, K, P(uptr), P(urows), P(loc), st))
+  occupancy, reuse = nnz / (rows * K), nnz / max(total, 1)
+
+  def plain(x, w, cout):
+    out = torch.empty(rows, cout, dtype=x.dtype, device=DEV)
+    ws = torch.empty(L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, x.shape[1], cout), dtype=torch.uint8, device=DEV)
+    _lib.check(L.ocnn_conv_gather(code, P(x), rows_in, P(table), rows, K, P(w), x.shape[1], cout, 0, 0, None, P(out),
+                                  P(ws), ws.numel(), st))
+    return out
+
+  say('abi sequence: 64 -> 64 on the plan')
+  x = torch.randn(rows_in, 64, generator=g).to(torch.bfloat16).to(DEV)
+  w = (torch.randn(K, 64, 64, generator=g) / 40).to(torch.bfloat16).to(DEV)
+  assert L.ocnn_conv_gather_choose(code, rows_in, rows, K, 64, 64, 0, 1, umax, total, occupancy, reuse) == _lib.GATHER_RW
+  ws = torch.empty(L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, 64, 64), dtype=torch.uint8, device=DEV)
+  out = torch.empty(rows, 64, dtype=torch.bfloat16, device=DEV)
+  _lib.check(L.ocnn_conv_gather_rw(code, P(x), rows_in, P(loc), P(uptr), P(urows), umax, total, rows, K, P(w), 64, 64,
+                                   0, 0, None, P(out), P(ws), ws.numel(), st))
+  assert rel_err(out, f64(plain(x, w, 64))) < 1e-2
+
+  say('abi sequence: pair plan, 96 -> 96')
+  counts = torch.zeros(K, dtype=torch.int64, device=DEV)
+  _lib.check(L.ocnn_pair_plan_slot_counts(P(loc), tiles, K, P(counts), st))
+  h_counts = (c_int64 * K)(*counts.tolist())
+  h_lists, h_list_count, h_bounds, n = (c_int32 * 32)(), (c_int64 * 32)(), (c_int32 * 5)(), c_int(0)
+  _lib.check(L.ocnn_pair_plan_lists(K, h_counts, h_lists, h_list_count, h_bounds, byref(n)))
+  nl = n.value
+  lists = torch.tensor(list(h_lists)[:nl], dtype=torch.int32, device=DEV)
+  nblk = torch.zeros(tiles * nl, dtype=torch.int32, device=DEV)
+  _lib.check(L.ocnn_pair_plan_count(P(loc), tiles, K, P(lists), nl, P(nblk), st))
+  cptr = torch.zeros(tiles * nl + 1, dtype=torch.int32, device=DEV)
+  cptr[1:] = nblk.cumsum(0)
+  n_blocks, max_blocks = int(cptr[-1]), int(nblk.view(tiles, nl).sum(1).max())
+  ent = torch.empty(n_blocks * 16, dtype=torch.int32, device=DEV)
+  _lib.check(L.ocnn_pair_plan_fill(P(loc), tiles, K, P(lists), nl, P(cptr), P(ent), st))
+  x = torch.randn(rows_in, 96, generator=g).to(torch.bfloat16).to(DEV)
+  w = (torch.randn(K, 96, 96, generator=g) / 50).to(torch.bfloat16).to(DEV)
+  gr = torch.randn(rows, 96, generator=g).to(torch.bfloat16).to(DEV)
+  assert L.ocnn_conv_gather_choose(code, rows_in, rows, K, 96, 96, 0, 1, umax, total, occupancy, reuse) == _lib.GATHER_SPARSE
+  ws = torch.empty(L.ocnn_conv_gather_sparse_workspace_bytes(96, 96), dtype=torch.uint8, device=DEV)
+  out = torch.empty(rows, 96, dtype=torch.bfloat16, device=DEV)
+  _lib.check(L.ocnn_conv_gather_sparse(code, P(x), rows_in, P(uptr), P(urows), umax, total, P(cptr), P(ent), n_blocks,
+                                       max_blocks, P(lists), nl, ctypes.addressof(h_bounds), rows, K, P(w), 96, 96, 0, 0,
+                                       None, P(out), P(ws), ws.numel(), st))
+  assert rel_err(out, f64(plain(x, w, 96))) < 1e-2
+  ws2 = torch.empty(L.ocnn_conv_wgrad_sparse_workspace_bytes(rows, 96, 96), dtype=torch.uint8, device=DEV)
+  gw = torch.empty(K, 96, 96, dtype=torch.bfloat16, device=DEV)
+  _lib.check(L.ocnn_conv_wgrad_sparse(code, P(x), rows_in, 96, P(gr), rows, 96, P(uptr), P(urows), umax, total, P(cptr),
+                                      P(ent), n_blocks, ctypes.addressof(h_lists), ctypes.addressof(h_list_count), nl, K, 1,
+                                      P(gw), P(ws2), ws2.numel(), st))
+  want = torch.empty(K, 96, 96, dtype=torch.bfloat16, device=DEV)
+  ws3 = torch.empty(L.ocnn_conv_wgrad_workspace_bytes_for(code, rows_in, rows, K, 96, 96), dtype=torch.uint8, device=DEV)
+  _lib.check(L.ocnn_conv_wgrad(code, P(x), rows_in, P(gr), P(table), rows, K, 96, 96, 0, P(want), P(ws3), ws3.numel(), st))
+  assert rel_err(gw, f64(want)) < 1e-2
