@@ -215,6 +215,16 @@ def test_search_key_fixture(ref_data):
   assert np.array_equal(np_(o.search_key(key, 5, True)), d['idx_ne'])
   assert np.array_equal(np_(o.search_xyzb(xyzb, 5, False)), d['idx'])
   assert np.array_equal(np_(o.search_xyzb(xyzb, 5, True)), d['idx_ne'])
+  # the same queries through the walk down the tree (ocnn_locate_points), which the point
+  # interpolation uses in place of the key search
+  from ocnn_amd import _lib
+  from ocnn_amd.nn.octree_interp import _tree
+  pts = xyzb.float().contiguous()
+  for ne, want in ((False, d['idx']), (True, d['idx_ne'])):
+    got = torch.empty(pts.shape[0], dtype=torch.int32, device=DEV)
+    _lib.check(_lib.lib().ocnn_locate_points(_lib.ptr(pts), pts.shape[0], *_tree(o, 5, ne), 0, _lib.ptr(got),
+                                             _lib.stream()))
+    assert np.array_equal(np_(got), want), ne
 
 
 def test_octree_grow_split(ref_data):
