@@ -11,6 +11,10 @@
  *   - the library never allocates device memory: outputs and workspaces are
  *     supplied by the caller (sizes from the *_workspace_bytes queries);
  *   - return value 0 = ok, negative = error (text from ocnn_last_error());
+ *   - arguments are checked on the host before anything is launched: a NULL in place of an
+ *     array that the call reads or writes (with the sizes given; an operand of zero rows may
+ *     be NULL), a negative size or an unsupported shape is OCNN_ERR_ARG, a workspace that is
+ *     too small OCNN_ERR_WORKSPACE; pointers named "may be NULL" are optional;
  *   - feature matrices are row-major (rows, channels); neighbour tables are
  *     row-major (rows, K) int32 with -1 for "no neighbour";
  *   - dtype codes: 0 = float32, 1 = float16, 2 = bfloat16 (fp32 accumulation).

@@ -404,6 +404,7 @@ extern "C" int ocnn_build_full_layer(int depth, int batch_size, int with_childre
                                      int32_t* children, void* stream) {
   OCNN_REQUIRE(depth >= 0 && depth <= 8 && batch_size >= 1 && ((int64_t)batch_size << (3 * depth)) < (1ll << 31),
                "build_full_layer: depth=%d batch_size=%d out of range", depth, batch_size);
+  OCNN_REQUIRE_PTRS("build_full_layer", keys, children);
   const int64_t total = (int64_t)batch_size << (3 * depth);
   hipLaunchKernelGGL(full_layer_kernel, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, (hipStream_t)stream, depth,
                      total, with_children ? 0 : -1, keys, children);
@@ -413,6 +414,7 @@ extern "C" int ocnn_build_full_layer(int depth, int batch_size, int with_childre
 extern "C" int ocnn_split_children(const int32_t* split, int64_t n, void* workspace, int64_t workspace_bytes,
                                    int32_t* children, int64_t* count, void* stream) {
   OCNN_REQUIRE(n > 0 && n < (1ll << 28), "split_children: n=%lld out of range", (long long)n);
+  OCNN_REQUIRE_PTRS("split_children", split, workspace, children, count);
   LevelLayout L;
   if (level_layout(n, &L) != OCNN_OK) { set_error("split_children: rocprim size query failed"); return OCNN_ERR_HIP; }
   if (workspace_bytes < L.total) { set_error("split_children: workspace %lld < %lld", (long long)workspace_bytes, (long long)L.total); return OCNN_ERR_WORKSPACE; }
@@ -433,6 +435,7 @@ extern "C" int ocnn_grow_layer(const int64_t* key_above, const int32_t* nempty_i
                                int64_t* keys, int32_t* children, void* stream) {
   OCNN_REQUIRE(n_nempty > 0 && n_nempty < (1ll << 28), "grow_layer: n_nempty=%lld out of range",
                (long long)n_nempty);
+  OCNN_REQUIRE_PTRS("grow_layer", key_above, nempty_index, keys, children);
   hipLaunchKernelGGL(grow_layer_kernel, dim3(cdiv(8 * n_nempty, 256)), dim3(256), 0, (hipStream_t)stream,
                      key_above, nempty_index, 8 * n_nempty, keys, children);
   return check_launch("grow_layer");
@@ -443,6 +446,7 @@ extern "C" int ocnn_leaf_average(const float* src, int channels, const int32_t* 
                                  void* stream) {
   OCNN_REQUIRE(channels > 0 && n_leaf > 0, "leaf_average: channels=%d n_leaf=%lld", channels,
                (long long)n_leaf);
+  OCNN_REQUIRE_PTRS("leaf_average", src, perm, seg_start, out);
   hipStream_t st = (hipStream_t)stream;
   if (mode == 1) {
     OCNN_REQUIRE(channels == 3, "leaf_average: normalise mode needs 3 channels, got %d", channels);
@@ -459,6 +463,7 @@ extern "C" int ocnn_leaf_points_normals(const float* pts, const float* normals, 
                                         const int32_t* seg_start, int64_t n_leaf, float* out_pts, float* out_normals,
                                         void* stream) {
   OCNN_REQUIRE(n_leaf > 0, "leaf_points_normals: n_leaf=%lld", (long long)n_leaf);
+  OCNN_REQUIRE_PTRS("leaf_points_normals", pts, normals, perm, seg_start, out_pts, out_normals);
   hipLaunchKernelGGL(leaf_points_normals_kernel, dim3((unsigned)cdiv(n_leaf, 256)), dim3(256), 0, (hipStream_t)stream,
                      pts, normals, perm, seg_start, n_leaf, out_pts, out_normals);
   return check_launch("leaf_points_normals");
@@ -491,6 +496,7 @@ extern "C" int ocnn_octree_build_scan(const int64_t* key, int64_t n, int depth, 
                                       void* workspace, int64_t workspace_bytes, int32_t* perm, int64_t* sizes,
                                       void* stream) {
   if (int rc = build_args_ok(n, depth, full_depth, batch_bits)) return rc;
+  OCNN_REQUIRE_PTRS("octree_build_scan", key, workspace, perm, sizes);
   const int key_bits = 3 * depth, levels = depth - full_depth;
 #define OCNN_BUILD_SCAN(K, N) \
   build_scan_t<K, N>(key, n, key_bits, batch_bits, levels, (char*)workspace, workspace_bytes, perm, sizes, (hipStream_t)stream)
@@ -506,6 +512,7 @@ extern "C" int ocnn_octree_build_fill(const void* workspace, int64_t n, int dept
   OCNN_REQUIRE(batch_size >= 1 && batch_size <= (1 << batch_bits) && ((int64_t)batch_size << (3 * full_depth)) < (1ll << 31),
                "octree_build_fill: batch_size=%d does not fit batch_bits=%d / full_depth=%d", batch_size, batch_bits,
                full_depth);
+  OCNN_REQUIRE_PTRS("octree_build_fill", workspace, h_sizes, perm, h_keys, h_children, inverse, seg_start);
   const int key_bits = 3 * depth, levels = depth - full_depth;
   BuildTree t;
   t.begin[0] = 0;

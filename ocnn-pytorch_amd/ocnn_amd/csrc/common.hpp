@@ -27,6 +27,15 @@ inline int check_launch(const char* what) {
     }                                  \
   } while (0)
 
+// Pointers that an entry point dereferences (or hands to a kernel) must not be null: a null
+// goes straight to a launch otherwise, and a kernel that reads through it takes the GPU down.
+template <typename... P>
+inline bool all_set(const P*... p) {
+  return (... && (p != nullptr));
+}
+#define OCNN_REQUIRE_PTRS(what, ...) \
+  OCNN_REQUIRE(::ocnn::all_set(__VA_ARGS__), what ": a required pointer is NULL (of " #__VA_ARGS__ ")")
+
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t align_up(int64_t a, int64_t b) { return cdiv(a, b) * b; }
 

@@ -594,6 +594,8 @@ extern "C" int ocnn_conv_gather(int dtype, const void* in, int64_t rows_in, cons
   OCNN_REQUIRE(rows_in >= 0 && rows_out >= 0 && rows_out < (1ll << 31) && rows_in < (1ll << 31),
                "conv_gather: rows out of range");
   if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_gather", table, w, out, workspace);
+  OCNN_REQUIRE(rows_in == 0 || in, "conv_gather: in is NULL");
   hipStream_t st = (hipStream_t)stream;
   GatherPlan p = plan_gather(dtype, rows_in, rows_out, cin, cout);
   if (p.mfma) {
@@ -737,6 +739,8 @@ extern "C" int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const v
   OCNN_REQUIRE(K >= 1 && K <= 27 && ca >= 1 && cb >= 1, "conv_wgrad: K=%d ca=%d cb=%d", K, ca, cb);
   OCNN_REQUIRE(rows >= 0 && rows < (1ll << 31) && rows_x >= 0 && rows_x < (1ll << 31),
                "conv_wgrad: rows out of range");
+  OCNN_REQUIRE_PTRS("conv_wgrad", gw, workspace);
+  OCNN_REQUIRE(rows == 0 || (g && table && (rows_x == 0 || x)), "conv_wgrad: a required pointer is NULL (of x, g, table)");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F32) {
     const int64_t need = f32_wgrad_workspace(rows_x, rows, K, ca, cb);

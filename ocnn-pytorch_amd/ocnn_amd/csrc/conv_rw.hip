@@ -619,8 +619,8 @@ extern "C" int ocnn_conv_gather_rw_supported(int dtype, int64_t rows_in, int K, 
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (!((cin == 64 && cout == 64) || (cin == 32 && cout == 32))) return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
-  if (plan_max_distinct > kRwCap) return 0;
-  if ((int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
+  if (plan_max_distinct < 0 || plan_max_distinct > kRwCap) return 0;
+  if (rows_in < 0 || (int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -697,6 +697,8 @@ extern "C" int ocnn_conv_gather_rw(int dtype, const void* in, int64_t rows_in, c
                    plan_total >= 0 && plan_total < (1ll << 29),
                "conv_gather_rw: rows out of range");
   if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_gather_rw", loc, uptr, urows, w, out, workspace);
+  OCNN_REQUIRE(rows_in == 0 || in, "conv_gather_rw: in is NULL");
   if (workspace_bytes < (int64_t)K * cin * cout * 2) {
     set_error("conv_gather_rw: workspace too small");
     return OCNN_ERR_WORKSPACE;
@@ -756,6 +758,10 @@ extern "C" int ocnn_conv_gather_rw_static(int dtype, const void* in, int64_t row
   OCNN_REQUIRE((int64_t)K * cin * cout * 2 <= kRwScratchBytes,
                "conv_gather_rw_static: %lld bytes of weights exceed the built-in buffer of %lld bytes",
                (long long)K * cin * cout * 2, (long long)kRwScratchBytes);
+  OCNN_REQUIRE(rows_out >= 0 && plan_total >= 0, "conv_gather_rw_static: negative row count");
+  if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_gather_rw_static", loc, uptr, urows, w, out);
+  OCNN_REQUIRE(rows_in == 0 || in, "conv_gather_rw_static: in is NULL");
   void* ws = nullptr;
   int rc = rw_scratch_of_current_device(&ws);
   if (rc != OCNN_OK) return rc;

@@ -321,8 +321,10 @@ extern "C" int ocnn_conv_gather_sparse_supported(int dtype, int64_t rows_in, int
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (cin < 32 || cin > 128 || cin % 32 != 0 || cout < 32 || cout % 32 != 0 || cout > 4096) return 0;
   if (K < 1 || K > 27) return 0;
-  if (plan_max_distinct > 511 || sp_lds_bytes(8 * kSpLists, cin, plan_max_distinct, 2) > kSpLdsLimit) return 0;
-  if ((int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
+  if (plan_max_distinct < 0 || plan_max_distinct > 511 ||
+      sp_lds_bytes(8 * kSpLists, cin, plan_max_distinct, 2) > kSpLdsLimit)
+    return 0;
+  if (rows_in < 0 || (int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -397,12 +399,15 @@ extern "C" int ocnn_conv_gather_sparse(int dtype, const void* in, int64_t rows_i
                    plan_total >= 0 && plan_total < (1ll << 29) && n_blocks >= 0 && n_blocks < (1ll << 25) &&
                    max_blocks >= 0 && max_blocks <= 8 * kSpLists && n_lists >= 1 && n_lists <= kSpLists,
                "conv_gather_sparse: rows or lists out of range");
+  OCNN_REQUIRE_PTRS("conv_gather_sparse", group_bounds);
   SpGroups groups;
   for (int g = 0; g < 5; ++g) groups.gb[g] = group_bounds[g];
   bool ok = groups.gb[0] == 0 && groups.gb[4] == n_lists;
   for (int g = 0; g < 4; ++g) ok = ok && groups.gb[g + 1] >= groups.gb[g] && groups.gb[g + 1] - groups.gb[g] <= 8;
   OCNN_REQUIRE(ok, "conv_gather_sparse: the four groups must split the lists into ranges of at most 8");
   if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_gather_sparse", uptr, urows, cptr, ent, lists, w, out, workspace);
+  OCNN_REQUIRE(rows_in == 0 || in, "conv_gather_sparse: in is NULL");
   if (workspace_bytes < (int64_t)n_lists * cin * cout * 2) {
     set_error("conv_gather_sparse: workspace too small");
     return OCNN_ERR_WORKSPACE;

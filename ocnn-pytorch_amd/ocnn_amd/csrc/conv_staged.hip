@@ -209,8 +209,8 @@ using namespace ocnn;
 
 extern "C" int ocnn_conv_gather_planned_supported(int dtype, int64_t rows_in, int cin, int cout) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (cin % 64 != 0 || cout % 64 != 0) return 0;
-  if ((int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;       // 32-bit buffer offsets
+  if (cin <= 0 || cout <= 0 || cin % 64 != 0 || cout % 64 != 0) return 0;
+  if (rows_in < 0 || (int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;       // 32-bit buffer offsets
   return 1;
 }
 
@@ -244,6 +244,8 @@ extern "C" int ocnn_conv_gather_planned(int dtype, const void* in, int64_t rows_
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows_out >= 0 && rows_out < (1ll << 31),
                "conv_gather_planned: bad shape");
   if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_gather_planned", loc, uptr, urows, w, out, workspace);
+  OCNN_REQUIRE(rows_in == 0 || in, "conv_gather_planned: in is NULL");
   if (workspace_bytes < (int64_t)K * cin * cout * 2) {
     set_error("conv_gather_planned: workspace too small");
     return OCNN_ERR_WORKSPACE;

@@ -363,8 +363,8 @@ extern "C" int ocnn_conv_gather_wide_supported(int dtype, int64_t rows_in, int K
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (cin < 64 || cin % 32 != 0 || cout < 96 || cout % 32 != 0 || cin > 2048 || cout > 2048) return 0;
   if (K < 1 || K > 27) return 0;
-  if (plan_max_distinct > kWdCap) return 0;
-  if ((int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
+  if (plan_max_distinct < 0 || plan_max_distinct > kWdCap) return 0;
+  if (rows_in < 0 || (int64_t)rows_in * cin * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -401,6 +401,8 @@ extern "C" int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in,
   OCNN_REQUIRE(rows_out >= 0 && rows_out < (1ll << 31) && plan_total >= 0 && plan_total < (1ll << 29),
                "conv_gather_wide: rows out of range");
   if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_gather_wide", loc, uptr, urows, w, out, workspace);
+  OCNN_REQUIRE(rows_in == 0 || in, "conv_gather_wide: in is NULL");
   if (workspace_bytes < (int64_t)K * align_up(cin, 64) * cout * 2) {
     set_error("conv_gather_wide: workspace too small");
     return OCNN_ERR_WORKSPACE;
@@ -428,7 +430,7 @@ static DensePlan dense_plan(int cin, int cout) {
 extern "C" int ocnn_conv_dense_supported(int dtype, int64_t rows, int cin, int cout) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (cin < 64 || cin % 64 != 0 || cin > 1024 || cout < 128 || cout % 128 != 0 || cout > 4096) return 0;
-  if (((int64_t)rows + 128) * cin * 2 > 0xfff00000ll) return 0;
+  if (rows < 0 || ((int64_t)rows + 128) * cin * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -467,7 +469,8 @@ extern "C" int ocnn_conv_dense(int dtype, const void* in, int64_t rows, const vo
                                int w_transposed, const void* bias, void* out, void* workspace,
                                int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(ocnn_conv_dense_supported(dtype, rows, cin, cout), "conv_dense: shape not supported");
-  if (rows <= 0) return OCNN_OK;
+  if (rows == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_dense", in, w, out, workspace);
   if (workspace_bytes < (int64_t)cin * cout * 2) {
     set_error("conv_dense: workspace too small");
     return OCNN_ERR_WORKSPACE;

@@ -432,8 +432,8 @@ static int dr_mb(int cin, int cout) {
 
 extern "C" int ocnn_conv_dense_rw_supported(int dtype, int64_t rows, int cin, int cout) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
-  if (dr_mb(cin, cout) == 0 || cout > 4096) return 0;
-  if (((int64_t)rows + 128) * std::max(cin, cout) * 2 > 0xfff00000ll) return 0;
+  if (cin <= 0 || cout <= 0 || dr_mb(cin, cout) == 0 || cout > 4096) return 0;
+  if (rows < 0 || ((int64_t)rows + 128) * std::max(cin, cout) * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -508,7 +508,8 @@ extern "C" int ocnn_conv_dense_rw_indexed(int dtype, const void* in, int64_t row
   OCNN_REQUIRE(out_index != nullptr || rows_out == rows, "conv_dense_rw: without an index the result has `rows` rows");
   OCNN_REQUIRE(rows_in >= 0 && ((int64_t)rows_in + 128) * cin * 2 <= 0xfff00000ll, "conv_dense_rw: operand too large");
   OCNN_REQUIRE(rows_out >= 0 && ((int64_t)rows_out + 128) * cout * 2 <= 0xfff00000ll, "conv_dense_rw: result too large");
-  if (rows <= 0) return OCNN_OK;
+  if (rows == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("conv_dense_rw", in, w, out, workspace);
   if (workspace_bytes < (int64_t)cin * cout * 2) {
     set_error("conv_dense_rw: workspace too small");
     return OCNN_ERR_WORKSPACE;
@@ -563,7 +564,7 @@ static int dr_wgrad_ranges(int ca, int cb, int64_t rows, int n_cu) {
 extern "C" int ocnn_conv_dense_wgrad_rw_supported(int dtype, int64_t rows, int ca, int cb) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (dr_wa(ca, cb) == 0 || ca > 4096 || cb > 4096) return 0;
-  if (((int64_t)rows + 128) * std::max(ca, cb) * 2 > 0xfff00000ll) return 0;
+  if (rows < 0 || ((int64_t)rows + 128) * std::max(ca, cb) * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -624,6 +625,8 @@ extern "C" int ocnn_conv_dense_wgrad_rw_indexed(int dtype, const void* x, int64_
   OCNN_REQUIRE(rows_x >= 0 && rows_g >= 0 && ((int64_t)rows_x + 128) * ca * 2 <= 0xfff00000ll &&
                    ((int64_t)rows_g + 128) * cb * 2 <= 0xfff00000ll,
                "conv_dense_wgrad_rw: operand too large");
+  OCNN_REQUIRE_PTRS("conv_dense_wgrad_rw", gw, workspace);
+  OCNN_REQUIRE(rows == 0 || (x && g), "conv_dense_wgrad_rw: a required pointer is NULL (of x, g)");
   hipStream_t st = (hipStream_t)stream;
   const DrOperand xo{x, rows_x, x_index}, go{g, rows_g, g_index};
   if (dtype == OCNN_F16)

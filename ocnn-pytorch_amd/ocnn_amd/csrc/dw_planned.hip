@@ -499,8 +499,8 @@ extern "C" int ocnn_dwconv_gather_planned_supported(int dtype, int64_t rows_in, 
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (channels < 64 || channels % 64 != 0 || channels > 4096) return 0;
   if (!dp_slots_ok(K)) return 0;
-  if (plan_max_distinct > kDpCap) return 0;
-  if ((int64_t)rows_in * channels * 2 > 0xfff00000ll) return 0;
+  if (plan_max_distinct < 0 || plan_max_distinct > kDpCap) return 0;
+  if (rows_in < 0 || (int64_t)rows_in * channels * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -541,6 +541,8 @@ extern "C" int ocnn_dwconv_gather_planned(int dtype, const void* in, int64_t row
                    (int64_t)rows_out * channels * 2 <= 0xfff00000ll,
                "dwconv_gather_planned: rows out of range");
   if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("dwconv_gather_planned", loc, uptr, urows, w, out);
+  OCNN_REQUIRE(rows_in == 0 || in, "dwconv_gather_planned: in is NULL");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
     return run_dp_gather<f16>(in, rows_in, loc, uptr, urows, rows_out, K, w, channels, reverse_slots, bias, out, st);
@@ -550,7 +552,7 @@ extern "C" int ocnn_dwconv_gather_planned(int dtype, const void* in, int64_t row
 extern "C" int ocnn_dwconv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K,
                                                    int channels, int plan_max_distinct) {
   if (!ocnn_dwconv_gather_planned_supported(dtype, rows_x, K, channels, plan_max_distinct)) return 0;
-  if ((int64_t)rows * channels * 2 > 0xfff00000ll) return 0;
+  if (rows < 0 || (int64_t)rows * channels * 2 > 0xfff00000ll) return 0;
   return 1;
 }
 
@@ -603,6 +605,9 @@ extern "C" int ocnn_dwconv_wgrad_planned(int dtype, const void* x, int64_t rows_
                "dwconv_wgrad_planned: shape not supported");
   OCNN_REQUIRE(rows >= 0 && rows < (1ll << 31) && plan_total >= 0 && plan_total < (1ll << 29),
                "dwconv_wgrad_planned: rows out of range");
+  OCNN_REQUIRE_PTRS("dwconv_wgrad_planned", gw, workspace);
+  OCNN_REQUIRE(rows == 0 || (g && loc && uptr && urows && (rows_x == 0 || x)),
+               "dwconv_wgrad_planned: a required pointer is NULL (of x, g, loc, uptr, urows)");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
     return run_dp_wgrad<f16>(x, rows_x, g, loc, uptr, urows, rows, K, channels, gw, workspace, workspace_bytes, st);

@@ -333,6 +333,7 @@ extern "C" int ocnn_search_key(const int64_t* keys, int64_t n, const int64_t* qu
                                void* stream) {
   OCNN_REQUIRE(n >= 0 && m >= 0, "search_key: bad sizes");
   if (m == 0) return OCNN_OK;
+  OCNN_REQUIRE(query && out && (n == 0 || keys), "search_key: a required pointer is NULL");
   hipLaunchKernelGGL(search_key_kernel, dim3((unsigned)cdiv(m, 256)), dim3(256), 0, (hipStream_t)stream, keys, n,
                      query, m, out);
   return check_launch("search_key");
@@ -342,6 +343,7 @@ extern "C" int ocnn_search_points(const float* pts, int64_t m, int depth, const 
                                   int bound_check, int32_t* out, void* stream) {
   OCNN_REQUIRE(n >= 0 && n < (1ll << 31) && m >= 0 && depth >= 0 && depth <= 16, "search_points: bad arguments");
   if (m == 0) return OCNN_OK;
+  OCNN_REQUIRE(pts && out && (n == 0 || keys), "search_points: a required pointer is NULL");
   hipLaunchKernelGGL(search_points_kernel, dim3((unsigned)cdiv(m, 256)), dim3(256), 0, (hipStream_t)stream, pts, m,
                      depth, keys, n, bound_check, out);
   return check_launch("search_points");
@@ -352,6 +354,7 @@ extern "C" int ocnn_interp_linear_prepare(const float* pts, int64_t m, int depth
   OCNN_REQUIRE(n >= 0 && n < (1ll << 31) && m >= 0 && m < (1ll << 28) && depth >= 0 && depth <= 16,
                "interp_linear_prepare: bad arguments");
   if (m == 0) return OCNN_OK;
+  OCNN_REQUIRE(pts && idx && w && norm && (n == 0 || keys), "interp_linear_prepare: a required pointer is NULL");
   hipLaunchKernelGGL(interp_linear_prepare_kernel<false>, dim3((unsigned)cdiv(m * 8, 256)), dim3(256), 0,
                      (hipStream_t)stream, pts, m, depth, keys, n, LocateTree{}, bound_check, idx, w, norm);
   return check_launch("interp_linear_prepare");
@@ -362,6 +365,7 @@ static int locate_tree(const int32_t* const* h_children, int depth, int full_dep
   OCNN_REQUIRE(depth >= 0 && depth <= kLocateMaxDepth && full_depth >= 0 && full_depth <= 8 && batch_size >= 1 &&
                    ((int64_t)batch_size << (3 * (depth < full_depth ? depth : full_depth))) < (1ll << 31),
                "locate: depth=%d full_depth=%d batch_size=%d out of range", depth, full_depth, batch_size);
+  OCNN_REQUIRE_PTRS("locate", h_children);
   for (int l = 0; l <= kLocateMaxDepth; ++l) t->children[l] = nullptr;
   for (int l = depth < full_depth ? depth : full_depth; l <= depth; ++l) {
     OCNN_REQUIRE(h_children[l] != nullptr || (l == depth && !nempty), "locate: no children array of layer %d", l);
@@ -381,6 +385,7 @@ extern "C" int ocnn_locate_points(const float* pts, int64_t m, const int32_t* co
   LocateTree t;
   if (int rc = locate_tree(h_children, depth, full_depth, batch_size, nempty, &t)) return rc;
   if (m == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("locate_points", pts, out);
   hipLaunchKernelGGL(locate_points_kernel, dim3((unsigned)cdiv(m, 256)), dim3(256), 0, (hipStream_t)stream, pts, m, t,
                      bound_check, out);
   return check_launch("locate_points");
@@ -393,6 +398,7 @@ extern "C" int ocnn_interp_linear_locate(const float* pts, int64_t m, const int3
   LocateTree t;
   if (int rc = locate_tree(h_children, depth, full_depth, batch_size, nempty, &t)) return rc;
   if (m == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("interp_linear_locate", pts, idx, w, norm);
   hipLaunchKernelGGL(interp_linear_prepare_kernel<true>, dim3((unsigned)cdiv(m * 8, 256)), dim3(256), 0,
                      (hipStream_t)stream, pts, m, depth, (const int64_t*)nullptr, (int64_t)0, t, bound_check, idx, w,
                      norm);
@@ -405,6 +411,7 @@ extern "C" int ocnn_csr_rows(int dtype, const int32_t* rowptr, int kfixed, const
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && rows >= 0 && (rowptr || kfixed >= 1),
                "csr_rows: bad arguments");
   if (rows == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("csr_rows", col, data, out);
   hipStream_t st = (hipStream_t)stream;
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
@@ -452,6 +459,8 @@ extern "C" int ocnn_csr_transpose(const int32_t* idx, const float* w, const floa
                "csr_transpose: points=%lld k=%d rows=%lld out of range", (long long)points, k, (long long)rows);
   OCNN_REQUIRE((w != nullptr || norm != nullptr) == (val != nullptr),
                "csr_transpose: values are written exactly when weights or a norm are given");
+  OCNN_REQUIRE_PTRS("csr_transpose", workspace, rowptr);
+  OCNN_REQUIRE(n == 0 || (idx && col), "csr_transpose: a required pointer is NULL (of idx, col)");
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   TransposeLayout L;
@@ -480,6 +489,7 @@ extern "C" int ocnn_max_pool(int dtype, const void* data, const int32_t* fine_ch
                              int64_t out_rows, int channels, void* out, int64_t* indices, void* stream) {
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && out_rows >= 0, "max_pool: bad arguments");
   if (out_rows == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("max_pool", data, out, indices);
   hipStream_t st = (hipStream_t)stream;
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
@@ -497,6 +507,7 @@ extern "C" int ocnn_max_unpool(int dtype, const void* src, const int64_t* indice
                                const int32_t* src_row, int64_t out_rows, int channels, void* out, void* stream) {
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && out_rows >= 0, "max_unpool: bad arguments");
   if (out_rows == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("max_unpool", src, indices, out);
   hipStream_t st = (hipStream_t)stream;
   OCNN_DISPATCH_DTYPE(dtype, {
     constexpr int VEC = 16 / sizeof(T);
@@ -514,6 +525,7 @@ extern "C" int ocnn_max_gather(int dtype, const void* src, const int64_t* indice
                                int64_t parents, int channels, void* out, void* stream) {
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && parents >= 0, "max_gather: bad arguments");
   if (parents == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("max_gather", src, indices, out);
   hipStream_t st = (hipStream_t)stream;
   OCNN_DISPATCH_DTYPE(dtype, {
     hipLaunchKernelGGL(max_gather_kernel<T>, dim3((unsigned)cdiv(parents * channels, 256)), dim3(256), 0, st,

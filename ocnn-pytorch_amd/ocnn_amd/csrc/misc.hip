@@ -425,7 +425,9 @@ extern "C" int ocnn_dwconv_gather(int dtype, const void* in, int64_t rows_in,
                                   void* stream) {
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2, "dwconv_gather: dtype %d", dtype);
   OCNN_REQUIRE(K >= 1 && K <= 27 && channels >= 1, "dwconv_gather: K=%d channels=%d", K, channels);
-  if (rows_out <= 0) return OCNN_OK;
+  OCNN_REQUIRE(rows_out >= 0 && rows_in >= 0, "dwconv_gather: negative row count");
+  if (rows_out == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("dwconv_gather", in, table, w, out);
   hipStream_t st = (hipStream_t)stream;
   const int C = channels;
   if (dw_rows_ok(K, C, std::max(rows_in, rows_out), dtype_size(dtype))) {
@@ -471,6 +473,9 @@ extern "C" int ocnn_dwconv_wgrad(int dtype, const void* x, int64_t rows_x, const
                                  void* workspace, int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(dtype >= 0 && dtype <= 2, "dwconv_wgrad: dtype %d", dtype);
   OCNN_REQUIRE(K >= 1 && K <= 27 && channels >= 1, "dwconv_wgrad: K=%d channels=%d", K, channels);
+  OCNN_REQUIRE(rows >= 0 && rows_x >= 0, "dwconv_wgrad: negative row count");
+  OCNN_REQUIRE_PTRS("dwconv_wgrad", gw, workspace);
+  OCNN_REQUIRE(rows == 0 || (x && g && table), "dwconv_wgrad: a required pointer is NULL (of x, g, table)");
   hipStream_t st = (hipStream_t)stream;
   int64_t splits = 0, rps = 0;
   if (rows > 0) split_rows(rows, K, &splits, &rps);
@@ -512,8 +517,9 @@ extern "C" int ocnn_dwconv_wgrad(int dtype, const void* x, int64_t rows_x, const
 
 extern "C" int ocnn_pad(int dtype, const void* data, const int32_t* children, int64_t n,
                         int channels, float val, void* out, void* stream) {
-  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1, "pad: bad arguments");
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && n >= 0, "pad: bad arguments");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("pad", children, out);      // (data may be NULL: only the empty nodes' rows are written)
   hipStream_t st = (hipStream_t)stream;
   const int64_t row_bytes = (int64_t)channels * dtype_size(dtype);
   if (row_bytes % 16 == 0 && ((uintptr_t)data % 16 == 0) && ((uintptr_t)out % 16 == 0)) {
@@ -542,8 +548,9 @@ extern "C" int ocnn_pad(int dtype, const void* data, const int32_t* children, in
 
 extern "C" int ocnn_depad(int dtype, const void* data, const int32_t* children, int64_t n,
                           int channels, void* out, void* stream) {
-  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1, "depad: bad arguments");
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && n >= 0, "depad: bad arguments");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("depad", data, children, out);
   hipStream_t st = (hipStream_t)stream;
   const int64_t row_bytes = (int64_t)channels * dtype_size(dtype);
   if (row_bytes % 16 == 0 && ((uintptr_t)data % 16 == 0) && ((uintptr_t)out % 16 == 0)) {
@@ -565,7 +572,9 @@ extern "C" int64_t ocnn_colsum_workspace_bytes(int64_t rows, int channels) {
 
 extern "C" int ocnn_colsum(int dtype, const void* g, int64_t rows, int channels, void* out,
                            void* workspace, int64_t workspace_bytes, void* stream) {
-  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1, "colsum: bad arguments");
+  OCNN_REQUIRE(dtype >= 0 && dtype <= 2 && channels >= 1 && rows >= 0, "colsum: bad arguments");
+  OCNN_REQUIRE_PTRS("colsum", out, workspace);
+  OCNN_REQUIRE(rows == 0 || g, "colsum: g is NULL");
   hipStream_t st = (hipStream_t)stream;
   int64_t splits = 0, rps = 0;
   if (rows > 0) split_rows(rows, 1, &splits, &rps);

@@ -82,7 +82,9 @@ extern "C" int ocnn_xyz2key(const int64_t* x, const int64_t* y, const int64_t* z
                             const int64_t* b, int64_t n, int depth, int64_t* key,
                             void* stream) {
   OCNN_REQUIRE(depth >= 0 && depth <= 16, "xyz2key: depth %d not in [0,16]", depth);
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(n >= 0, "xyz2key: negative count");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("xyz2key", x, y, z, key);
   hipLaunchKernelGGL(xyz2key_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, x, y,
                      z, b, n, depth, key);
   return check_launch("xyz2key");
@@ -91,7 +93,9 @@ extern "C" int ocnn_xyz2key(const int64_t* x, const int64_t* y, const int64_t* z
 extern "C" int ocnn_key2xyz(const int64_t* key, int64_t n, int depth, int64_t* x, int64_t* y,
                             int64_t* z, int64_t* b, void* stream) {
   OCNN_REQUIRE(depth >= 0 && depth <= 16, "key2xyz: depth %d not in [0,16]", depth);
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(n >= 0, "key2xyz: negative count");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("key2xyz", key, x, y, z, b);
   int nbits = 9 * ((depth + 2) / 3);
   hipLaunchKernelGGL(key2xyz_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, key,
                      n, nbits, x, y, z, b);
@@ -102,7 +106,9 @@ extern "C" int ocnn_points2key(const float* pts, int64_t n, const float* h_bbmin
                                const void* batch, int batch_is_float, int depth,
                                float* pts_out, int64_t* key, void* stream) {
   OCNN_REQUIRE(depth >= 1 && depth <= 16, "points2key: depth %d not in [1,16]", depth);
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(n >= 0, "points2key: negative count");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("points2key", pts, h_bbmin, pts_out, key);
   hipLaunchKernelGGL(points2key_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream,
                      pts, n, h_bbmin[0], h_bbmin[1], h_bbmin[2], factor, batch, batch_is_float,
                      depth, pts_out, key);

@@ -147,6 +147,7 @@ extern "C" int ocnn_neigh_full(int depth, int batch, int64_t* out64, int32_t* ou
   OCNN_REQUIRE(depth >= 0 && depth <= 7 && batch >= 1, "neigh_full: depth=%d batch=%d", depth, batch);
   int64_t total = (int64_t)batch << (3 * depth);
   OCNN_REQUIRE(total * 27 < (1ll << 31), "neigh_full: table too large for a full layer");
+  OCNN_REQUIRE(out64 || out32, "neigh_full: both outputs are NULL");
   hipLaunchKernelGGL(neigh_full_kernel, dim3(cdiv(total * 27, 256)), dim3(256), 0,
                      (hipStream_t)stream, depth, total, out64, out32);
   return check_launch("neigh_full");
@@ -172,6 +173,7 @@ extern "C" int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_
   OCNN_REQUIRE(depth >= 1 && depth <= 16 && full_depth >= 1 && full_depth <= depth && full_depth <= 7 && batch >= 1,
                "neigh_all: depth=%d full_depth=%d batch=%d (full_depth >= 1: layer 1 must be full)", depth,
                full_depth, batch);
+  OCNN_REQUIRE_PTRS("neigh_all", h_nnum, h_nnum_nempty, h_children, h_nempty_index, h_neigh);
   hipStream_t st = (hipStream_t)stream;
   for (int d = 1; d <= depth; ++d) {
     OCNN_REQUIRE(h_neigh[d] != nullptr && h_nnum[d] > 0 && h_nnum[d] * 27 < (1ll << 31), "neigh_all: layer %d", d);
@@ -195,7 +197,9 @@ extern "C" int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_
 
 extern "C" int ocnn_nempty_index(const int32_t* children, int64_t n, int32_t* index32,
                                  int64_t* index64, void* stream) {
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(n >= 0, "nempty_index: negative count");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE(children && (index32 || index64), "nempty_index: a required pointer is NULL");
   hipLaunchKernelGGL(nempty_index_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream,
                      children, n, index32, index64);
   return check_launch("nempty_index");
@@ -205,7 +209,9 @@ extern "C" int ocnn_neigh_select(const int32_t* neigh, const int32_t* row_index,
                                  const int32_t* children, const int* h_cols, int K, int64_t rows,
                                  int64_t* out64, int32_t* out32, void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27, "neigh_select: K=%d", K);
-  if (rows <= 0) return OCNN_OK;
+  OCNN_REQUIRE(rows >= 0, "neigh_select: negative row count");
+  if (rows == 0) return OCNN_OK;
+  OCNN_REQUIRE(neigh && (out64 || out32), "neigh_select: a required pointer is NULL");
   Cols cols;
   for (int c = 0; c < 27; ++c) cols.c[c] = c;
   if (h_cols)
@@ -220,13 +226,17 @@ extern "C" int ocnn_neigh_select(const int32_t* neigh, const int32_t* row_index,
 }
 
 extern "C" int ocnn_table_to_i64(const int32_t* in, int64_t n, int64_t* out, void* stream) {
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(n >= 0, "table_to_i64: negative count");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("table_to_i64", in, out);
   hipLaunchKernelGGL(widen_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, in, n, out);
   return check_launch("table_to_i64");
 }
 
 extern "C" int ocnn_table_to_i32(const int64_t* in, int64_t n, int32_t* out, void* stream) {
-  if (n <= 0) return OCNN_OK;
+  OCNN_REQUIRE(n >= 0, "table_to_i32: negative count");
+  if (n == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("table_to_i32", in, out);
   hipLaunchKernelGGL(narrow_kernel, dim3(cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream, in, n, out);
   return check_launch("table_to_i32");
 }
@@ -234,6 +244,7 @@ extern "C" int ocnn_table_to_i32(const int64_t* in, int64_t n, int32_t* out, voi
 extern "C" int ocnn_table_transpose(const int32_t* table, int64_t rows, int K, int64_t rows_in,
                                     int32_t* out, void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows >= 0 && rows_in >= 0, "table_transpose: bad shape");
+  OCNN_REQUIRE((rows_in == 0 || out) && (rows == 0 || (table && out)), "table_transpose: a required pointer is NULL");
   hipStream_t st = (hipStream_t)stream;
   if (rows_in > 0)
     hipLaunchKernelGGL(fill_i32_kernel, dim3(cdiv(rows_in * K, 256)), dim3(256), 0, st, out,

@@ -449,6 +449,7 @@ extern "C" int ocnn_batch_norm_stats(int dtype, const void* x, int64_t rows, int
                                      int64_t* batches_tracked, void* workspace, int64_t workspace_bytes,
                                      void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_stats: shape not supported");
+  OCNN_REQUIRE_PTRS("batch_norm_stats", x, mean, var, invstd, workspace);
   OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels), "batch_norm_stats: workspace too small");
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
@@ -470,6 +471,7 @@ extern "C" int ocnn_batch_norm_apply(int dtype, const void* x, int64_t rows, int
                                      const float* invstd, const void* gamma, const void* beta, int param_dtype,
                                      int relu, const void* residual, void* y, void* stream) {
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_apply: shape not supported");
+  OCNN_REQUIRE_PTRS("batch_norm_apply", x, mean, invstd, y);
   hipStream_t st = (hipStream_t)stream;
   int64_t per;
   int nblk;
@@ -490,6 +492,7 @@ extern "C" int ocnn_batch_norm_backward(int dtype, const void* x, const void* dy
                                         int64_t workspace_bytes, void* stream) {
   OCNN_REQUIRE(!d_residual || dx, "batch_norm_backward: d_residual needs dx");
   OCNN_REQUIRE(ocnn_batch_norm_supported(dtype, rows, channels), "batch_norm_backward: shape not supported");
+  OCNN_REQUIRE_PTRS("batch_norm_backward", x, dy, mean, invstd, dgamma, dbeta, workspace);
   OCNN_REQUIRE(workspace_bytes >= ocnn_batch_norm_workspace_bytes(channels),
                "batch_norm_backward: workspace too small");
   hipStream_t st = (hipStream_t)stream;

@@ -514,6 +514,9 @@ static int plan_launch(const int32_t* table, int64_t rows, int K, int mode, int3
                        void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && rows >= 0 && rows < (1ll << 31), "tile_plan: bad shape");
   if (rows == 0) return OCNN_OK;
+  // count: the table and the counts; fill: the offsets, the lists and the positions; build: all but the offsets
+  OCNN_REQUIRE(table && (mode == 1 ? (uptr && urows && loc) : ucount != nullptr) && (mode != 2 || (urows && loc)),
+               "tile_plan: a required pointer is NULL");
   int64_t tiles = cdiv(rows, kPlanRows);
   if (mode == 2)
     hipLaunchKernelGGL(tile_plan_kernel<kPlanHashQuick>, dim3((unsigned)tiles), dim3(kPlanThreads), 0,
@@ -536,6 +539,7 @@ extern "C" int ocnn_tile_plan_compact(const int32_t* ucount, const int32_t* uptr
   OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 31) && cap >= 0 && cap <= pad,
                "tile_plan_compact: bad shape");
   if (tiles == 0) return OCNN_OK;
+  OCNN_REQUIRE_PTRS("tile_plan_compact", ucount, uptr, stats, ulist, urows, loc);
   hipLaunchKernelGGL(tile_plan_compact_kernel, dim3((unsigned)cdiv(tiles, 4)), dim3(256), 0, (hipStream_t)stream,
                      ucount, uptr, stats, cap, pad, ulist, urows, loc, K, tiles);
   return check_launch("tile_plan_compact");
@@ -549,6 +553,8 @@ extern "C" int ocnn_tile_plan_count(const int32_t* table, int64_t rows, int K, i
 extern "C" int ocnn_tile_plan_offsets(const int32_t* ucount, const int32_t* tile_nnz, int64_t tiles, int cap,
                                       int32_t* uptr, int64_t* stats, void* stream) {
   OCNN_REQUIRE(tiles >= 0 && tiles < (1ll << 31) && cap >= 0, "tile_plan_offsets: bad shape");
+  OCNN_REQUIRE_PTRS("tile_plan_offsets", uptr, stats);
+  OCNN_REQUIRE(tiles == 0 || (ucount && tile_nnz), "tile_plan_offsets: a required pointer is NULL (of ucount, tile_nnz)");
   hipLaunchKernelGGL(tile_plan_offsets_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ucount, tile_nnz,
                      tiles, cap, uptr, stats);
   return check_launch("tile_plan_offsets");
@@ -562,6 +568,7 @@ extern "C" int ocnn_tile_plan_fill(const int32_t* table, int64_t rows, int K, co
 extern "C" int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,
                                           void* stream) {
   OCNN_REQUIRE(K >= 1 && K <= 27 && tiles >= 0 && tiles < (1ll << 24), "pair_plan: bad shape");
+  OCNN_REQUIRE(slot_count && (tiles == 0 || loc), "pair_plan_slot_counts: a required pointer is NULL");
   hipLaunchKernelGGL(pair_plan_zero_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream,
                      (unsigned long long*)slot_count, K);
   const unsigned gy = (unsigned)std::max<int64_t>(1, std::min<int64_t>(64, cdiv(tiles, 16)));
@@ -573,6 +580,7 @@ extern "C" int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, in
 extern "C" int ocnn_pair_plan_lists(int K, const int64_t* slot_count, int32_t* lists, int64_t* list_count,
                                     int32_t* group_bounds, int* n_lists) {
   OCNN_REQUIRE(K >= 1 && K <= 27, "pair_plan_lists: bad slot count");
+  OCNN_REQUIRE_PTRS("pair_plan_lists", slot_count, lists, list_count, group_bounds, n_lists);
   struct List { int k, r0, r1; int64_t load; };
   std::vector<List> all;
   int64_t total = 0;
@@ -624,6 +632,7 @@ static int pair_plan_launch(const uint16_t* loc, int64_t tiles, int K, const int
   OCNN_REQUIRE(K >= 1 && K <= 27 && nl >= 1 && nl <= 32 && tiles >= 0 && tiles < (1ll << 24),
                "pair_plan: bad shape");
   if (tiles == 0) return OCNN_OK;
+  OCNN_REQUIRE(loc && lists && (mode == 0 ? nblk != nullptr : (cptr && ent)), "pair_plan: a required pointer is NULL");
   hipLaunchKernelGGL(pair_plan_kernel, dim3((unsigned)cdiv(tiles * nl, 4)), dim3(256), 0, (hipStream_t)stream, loc,
                      tiles, K, lists, nl, mode, nblk, cptr, ent);
   return check_launch("pair_plan");

@@ -403,7 +403,8 @@ extern "C" int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int6
   if (!(ca == 32 && cb == 32) && !(ca >= 64 && cb >= 64 && ca % 32 == 0 && cb % 32 == 0 && ca <= 1024 && cb <= 1024))
     return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
-  if (plan_max_distinct > kWpCap) return 0;
+  if (plan_max_distinct < 0 || plan_max_distinct > kWpCap) return 0;
+  if (rows_x < 0 || rows < 0) return 0;
   if ((int64_t)rows_x * ca * 2 > 0xfff00000ll || ((int64_t)rows + kWpRows) * cb * 2 > 0xfff00000ll) return 0;
   return 1;
 }
@@ -479,6 +480,9 @@ extern "C" int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x,
   OCNN_REQUIRE(rows >= 0 && (int64_t)rows * K * 2 < 0xfff00000ll && plan_total >= 0 &&
                    plan_total < (1ll << 29),
                "conv_wgrad_planned: rows out of range");
+  OCNN_REQUIRE_PTRS("conv_wgrad_planned", gw, workspace);
+  OCNN_REQUIRE(rows == 0 || (g && loc && uptr && urows && (rows_x == 0 || x)),
+               "conv_wgrad_planned: a required pointer is NULL (of x, g, loc, uptr, urows)");
   hipStream_t st = (hipStream_t)stream;
   if (dtype == OCNN_F16)
     return run_wp<f16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, cb, out_transposed, gw, workspace,

@@ -270,7 +270,8 @@ extern "C" int ocnn_conv_wgrad_sparse_supported(int dtype, int64_t rows_a, int64
                                                 int plan_max_distinct) {
   if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
   if (ca < 32 || ca % 32 != 0 || ca > 1024 || cb < 32 || cb % 32 != 0 || cb > 96) return 0;
-  if (K < 1 || K > 27 || plan_max_distinct > kWsCap) return 0;
+  if (K < 1 || K > 27 || plan_max_distinct < 0 || plan_max_distinct > kWsCap) return 0;
+  if (rows_a < 0 || rows_b < 0) return 0;
   if ((int64_t)rows_a * ca * 2 > 0xfff00000ll || ((int64_t)rows_b + 128) * cb * 2 > 0xfff00000ll) return 0;
   return 1;
 }
@@ -369,6 +370,9 @@ extern "C" int ocnn_conv_wgrad_sparse(int dtype, const void* a, int64_t rows_a, 
   OCNN_REQUIRE(rows_b >= 0 && rows_b < (1ll << 31) && plan_total >= 0 && plan_total < (1ll << 29) &&
                    n_blocks >= 0 && n_blocks < (1ll << 25) && n_lists >= 1 && n_lists <= 32,
                "conv_wgrad_sparse: rows or lists out of range");
+  OCNN_REQUIRE_PTRS("conv_wgrad_sparse", out);
+  OCNN_REQUIRE(rows_b == 0 || (b && uptr && urows && cptr && ent && lists && list_count && workspace && (rows_a == 0 || a)),
+               "conv_wgrad_sparse: a required pointer is NULL");
   hipStream_t st = (hipStream_t)stream;
   if (rows_b == 0) {                                   // nothing to add up: zeros
     WsUnits none;

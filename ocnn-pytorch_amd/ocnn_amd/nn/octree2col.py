@@ -7,13 +7,14 @@ summation order here too."""
 import torch
 
 from .. import _lib
+from ..octree.contract import tables_of
 
 
 def octree2col(data: torch.Tensor, octree, depth: int, kernel_size: str = '333', stride: int = 1,
                nempty: bool = False):
   """(rows_in, C) -> (rows, K, C): entry (i, k) is the row of `data` that slot k of table row i
   names, zeros where it names none."""
-  table = octree._table(depth, kernel_size, stride, nempty)
+  table = tables_of(octree)._table(depth, kernel_size, stride, nempty)
   _lib.require_gpu(data, table)
   hit = table >= 0
   col = data[table.clamp_min(0).long()]                  # (rows, K, C)
@@ -26,7 +27,7 @@ def col2octree(data: torch.Tensor, octree, depth: int, kernel_size: str = '333',
   entries (i, k) whose slot names j.  Every (j, k) has at most one such i (the inverse
   table), so the sum over k is taken in slot order."""
   rows_in = int(octree.nnum_nempty[depth] if nempty else octree.nnum[depth])
-  inverse = octree._table_t(depth, kernel_size, stride, nempty, rows_in)     # (rows_in, K)
+  inverse = tables_of(octree)._table_t(depth, kernel_size, stride, nempty, rows_in)     # (rows_in, K)
   _lib.require_gpu(data, inverse)
   K = inverse.shape[1]
   slot = torch.arange(K, device=data.device).expand_as(inverse)

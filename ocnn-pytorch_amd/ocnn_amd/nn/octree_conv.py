@@ -20,6 +20,7 @@ import torch.nn
 from torch.autograd import Function
 
 from .. import _lib
+from ..octree.contract import tables_of
 from ..utils import list2str, resize_with_last_val, xavier_uniform_
 from .octree2col import col2octree, octree2col
 from .octree_pad import _depad_raw, _pad_raw, octree_depad, octree_pad
@@ -78,6 +79,15 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
     bias = bias.to(data.dtype).contiguous()
   code = _lib.dtype_code(data)
   kernel = L.ocnn_conv_gather_choose(code, rows_in, rows, K, cin, cout, int(bool(dense)), *_plan_args(plan))
+  if kernel == _lib.GATHER_DENSE_RW and (in_index is not None or pad_to is not None):
+    # the indexed form also addresses the tensors over all nodes with 32-bit offsets: past that
+    # range the rows are copied out (depad) / in (pad) around the kernel on the compact rows
+    n_all = max(data.shape[0], rows if pad_to is None else int(pad_to[0].nnum[pad_to[1]]))
+    if not L.ocnn_conv_dense_rw_supported(code, n_all, cin, cout):
+      if in_index is not None:
+        data, in_index = data.index_select(0, in_index.long()), None
+      out, planned = _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan, dense)
+      return (out if pad_to is None else _pad_raw(out, *pad_to)), planned
   if in_index is not None and kernel != _lib.GATHER_DENSE_RW:
     data, in_index = data.index_select(0, in_index.long()), None       # the other kernels take compact rows
   if pad_to is not None and kernel != _lib.GATHER_DENSE_RW:          # the other kernels write compact rows
@@ -160,8 +170,10 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense, g_index=None):
   ca, cb = x.shape[1], g.shape[1]
   code = _lib.dtype_code(x)
   kernel = L.ocnn_conv_wgrad_choose(code, x.shape[0], rows, K, ca, cb, int(bool(dense)), *_plan_args(plan)[:4])
-  if g_index is not None and kernel != _lib.WGRAD_DENSE_RW:
-    g, g_index = g.index_select(0, g_index.long()), None                # the other kernels take compact rows
+  if g_index is not None and (kernel != _lib.WGRAD_DENSE_RW or
+                              not L.ocnn_conv_dense_wgrad_rw_supported(code, max(rows, g.shape[0]), ca, cb)):
+    # (the other kernels take compact rows, and so does the dense one past its 32-bit offset range)
+    g, g_index = g.index_select(0, g_index.long()), None
   assert (g_index is not None or g.shape[0] == rows) and x.dtype == g.dtype and table.dtype == torch.int32
   if kernel == _lib.WGRAD_ZERO_PADDED:
     ca_p, cb_p = -(-ca // 32) * 32, -(-cb // 32) * 32
@@ -264,6 +276,8 @@ class OctreeConvBase:
 
   def setup(self, octree, depth: int):
     """Heights of input/output and the table (ocnn/nn/octree_conv.py:51-100)."""
+    # (an octree of another class gets its tables from its public members, octree/contract.py)
+    octree = tables_of(octree)
     self.in_depth = self.out_depth = self.neigh_depth = depth
     if self.stride == 2:
       if self.is_conv_layer():
@@ -409,6 +423,7 @@ class OctreeConvFunction(Function):
               max_buffer: int = int(2e8), bias=None, padded: bool = False):
     eng = _OctreeConv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
+    octree = eng.octree
     eng.check_and_init(data)
     data = data.contiguous()
     weights = weights.to(data.dtype).contiguous()
@@ -447,6 +462,7 @@ class OctreeDeconvFunction(Function):
               max_buffer: int = int(2e8), bias=None, padded: bool = False):
     eng = _OctreeDeconv(in_channels, out_channels, kernel_size, stride, nempty, max_buffer)
     eng.setup(octree, depth)
+    octree = eng.octree
     index = None
     data = data.contiguous()
     if padded:
@@ -524,7 +540,7 @@ class OctreeConv(OctreeConvBase, torch.nn.Module):
 
   def explicit_gemm(self, data: torch.Tensor, octree, depth: int):
     """im2col, then one matrix product (autograd differentiates the torch ops)."""
-    col = octree2col(data, octree, depth, self.kernel, self.stride, self.nempty)
+    col = octree2col(data, tables_of(octree), depth, self.kernel, self.stride, self.nempty)
     return torch.mm(col.flatten(1), self.weights.to(data.dtype).flatten(0, 1))
 
   def reset_parameters(self):
@@ -575,7 +591,7 @@ class OctreeDeconv(OctreeConv):
     if self.method == 'explicit_gemm':
       # one product for all slots, then the adjoint of im2col (ocnn/nn/octree_conv.py:453-457)
       col = torch.mm(data, self.weights.to(data.dtype).flatten(0, 1).t())
-      out = col2octree(col.view(col.shape[0], self.kdim, -1), octree, depth + (self.stride == 2), self.kernel,
+      out = col2octree(col.view(col.shape[0], self.kdim, -1), tables_of(octree), depth + (self.stride == 2), self.kernel,
                        self.stride, self.nempty)
     else:
       out = octree_deconv(data, self.weights, octree, depth, self.in_channels, self.out_channels,

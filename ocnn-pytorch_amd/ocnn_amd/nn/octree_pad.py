@@ -5,8 +5,16 @@ import torch
 from .. import _lib
 
 
-def _pad_raw(data: torch.Tensor, octree, depth: int, val: float = 0.0):
+def _children32(octree, depth):
+  """children[depth] as the kernels read it: int32, contiguous (the reference's own dtype,
+  ocnn/octree/octree.py:59; another integer type is converted)."""
   children = octree.children[depth]
+  _lib.require_gpu(children)
+  return children if children.dtype == torch.int32 and children.is_contiguous() else children.int().contiguous()
+
+
+def _pad_raw(data: torch.Tensor, octree, depth: int, val: float = 0.0):
+  children = _children32(octree, depth)
   _lib.require_gpu(data, children)
   data = data.contiguous()
   assert data.shape[0] == int(octree.nnum_nempty[depth]), 'octree_pad: wrong number of rows'
@@ -18,7 +26,7 @@ def _pad_raw(data: torch.Tensor, octree, depth: int, val: float = 0.0):
 
 
 def _depad_raw(data: torch.Tensor, octree, depth: int):
-  children = octree.children[depth]
+  children = _children32(octree, depth)
   _lib.require_gpu(data, children)
   data = data.contiguous()
   assert data.shape[0] == int(octree.nnum[depth]), 'octree_depad: wrong number of rows'

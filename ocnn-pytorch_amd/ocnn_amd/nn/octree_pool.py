@@ -7,6 +7,7 @@ import torch
 import torch.nn
 
 from .. import _lib
+from ..octree.contract import tables_of
 from ..utils import list2str, resize_with_last_val
 from .octree_pad import octree_pad
 
@@ -44,6 +45,7 @@ def _unpool_raw(data, indices, octree, depth, nempty):
   out = torch.empty((out_rows, c), dtype=data.dtype, device=data.device)
   # non-empty form: out row r is node nempty_index[r] of the fine level, source row = parent;
   # all-nodes form: out row = node, source row = the parent's node at the coarse level
+  octree = tables_of(octree)
   out_node = octree._nempty_index32(depth + 1) if nempty else None
   src_row = None if nempty else octree._nempty_index32(depth)
   _lib.check(_lib.lib().ocnn_max_unpool(_lib.dtype_code(data), _lib.ptr(data), _lib.ptr(indices),
@@ -145,7 +147,7 @@ def octree_avg_pool(data: torch.Tensor, octree, depth: int, kernel: str, stride:
   row-gather kernel of the interpolation with unit weights, divided by the neighbour count;
   the gradient runs over the transposed table (no atomics)."""
   from .octree_interp import _Interp
-  table = octree._table(depth, kernel, stride, nempty)
+  table = tables_of(octree)._table(depth, kernel, stride, nempty)
   count = (table >= 0).sum(1).to(torch.float32)
   return _Interp.apply(data, table, None, count)
 

@@ -23,6 +23,48 @@ def declared_symbols():
   return sorted(set(re.findall(r'\b(ocnn_[a-z0-9_]+)\s*\(', text)))
 
 
+def _launching_entry_points():
+  """Entry points that return a status and take a pointer: everything but the size queries, the
+  *_supported / *_choose predicates and the host evaluations of kernel arithmetic."""
+  names = set()
+  for name, (res, args) in _lib.SIGNATURES.items():
+    if res is ctypes.c_int and any(a is ctypes.c_void_p or hasattr(a, '_type_') and not isinstance(a._type_, str)
+                                   for a in args):
+      names.add(name)
+  return names
+
+
+def test_entry_points_refuse_bad_pointers_and_sizes_before_any_launch():
+  """Every launching entry point, called with valid sizes, refuses a NULL in place of each array it
+  reads or writes, a negative size and a missing workspace with an error code, before anything is
+  launched.  The calls are made by a child process to which no GPU is visible, so an entry point
+  that let one through would fail to launch there, not fault."""
+  import json
+  import subprocess
+  import sys
+  sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+  import abi_null_cases
+  assert set(abi_null_cases.CASES) == _launching_entry_points()
+  env = dict(os.environ, HIP_VISIBLE_DEVICES='-1', ROCR_VISIBLE_DEVICES='-1', CUDA_VISIBLE_DEVICES='-1')
+  res = subprocess.run([sys.executable, os.path.join(ROOT, 'tests', 'abi_null_cases.py')], env=env,
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+  assert res.returncode == 0, res.stderr[-2000:]
+  got = json.loads(res.stdout.strip().splitlines()[-1])
+  if 'skipped' in got:
+    pytest.skip(got['skipped'])
+  ERR_ARG, ERR_HIP, ERR_WS = -1, -2, -3
+  for name, r in got.items():
+    assert r['all_null'][0] == ERR_ARG, (name, r['all_null'])
+    for i, (rc, msg) in r['one_null'].items():
+      assert rc == ERR_ARG and 'null' in msg.lower(), (name, 'argument', i, rc, msg)
+    for i, (rc, msg) in r['negative'].items():
+      assert rc in (ERR_ARG, ERR_WS), (name, 'argument', i, rc, msg)
+    if r['no_workspace'] is not None:
+      assert r['no_workspace'][0] < 0, (name, r['no_workspace'])
+    # the sizes of the case are valid: with every pointer set the call gets as far as the device
+    assert r['good'][0] == (0 if name in abi_null_cases.HOST_ONLY else ERR_HIP), (name, r['good'])
+
+
 def test_library_exports_every_declared_symbol():
   names = declared_symbols()
   assert len(names) >= 30
