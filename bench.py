@@ -230,12 +230,17 @@ def main():
     t_gather.reset()
     t_wgrad.reset()
     t_gather.enabled = t_wgrad.enabled = True
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
       step()
+      marks[i + 1].record()
     torch.cuda.synchronize()
     dt_s = time.perf_counter() - t0
     t_gather.enabled = t_wgrad.enabled = False
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    run_steps.median_ms = per_step[len(per_step) // 2] if per_step else float('nan')
     return dt_s * 1e3 / steps, t_gather.mean_ms(), t_wgrad.mean_ms(), t_gather.count()
 
   def timed_steps(dt, steps, warmup, oct=octree, only='all'):
@@ -272,6 +277,7 @@ def main():
 
   # ---- the headline step: W warm-up steps, K timed steps ---------------------------
   ms, gather_ms, wgrad_ms, n_gather = run_steps(headline, args.steps, args.warmup)
+  median_ms = run_steps.median_ms
   gather_ms = gather_ms or float('nan')
   wgrad_ms = wgrad_ms or float('nan')
   flops_step = 6.0 * nnz * C * C
@@ -291,6 +297,10 @@ def main():
       'steps': args.steps,
       'warmup': args.warmup,
       'ms_per_step': ms,
+      'ms_per_step_median': median_ms,
+      # every untimed step of the layer before the timed ones: the first call, the cold-start series and
+      # the W warm-up steps (the timed steps follow them without a gap: a fully ramped figure)
+      'untimed_steps_before_timing': (41 if extras else 0) + args.warmup,
       'higher_is_better': True,
       'scaling': 'weak',
       'vs_baseline': None,
@@ -356,7 +366,7 @@ def main():
 
     # ---- what the part sustains: v_mfma_f32_32x32x16 alone, all CUs ----------
     try:
-      from ocnn_amd import probe
+      import bench_probe as probe
       sustained = {k: probe.mfma_rate(dtype, k, 20000)['tflops'] for k in ('constant', 'normal')}
       alone, mixed = probe.mfma_mix(False), probe.mfma_mix(True)
       result['mfma_sustained'] = {

@@ -1,24 +1,58 @@
-"""ctypes binding of libocnn_probe.so: what the GPU itself sustains (MFMA rate with given
-operand statistics, LDS read / write rate for a given address pattern).  Used by bench.py to
-put the kernels' figures next to the part's; not part of the operator library."""
+"""ctypes binding of libbench_probe.so (bench_probe.hip): what the GPU itself sustains (MFMA rate
+with given operand statistics, LDS read / write rate for a given address pattern).  Used by
+bench.py to put the kernels' figures next to the part's; not part of the operator library."""
 
 import ctypes
+import hashlib
 import os
+import subprocess
+import sys
 from ctypes import c_double, c_int, c_void_p, POINTER, byref
 
 import torch
 
-from . import build as _build
+ROOT = os.path.dirname(os.path.abspath(__file__))
+SOURCE = os.path.join(ROOT, 'bench_probe.hip')
+LIB_PATH = os.path.join(ROOT, 'libbench_probe.so')
+STAMP_PATH = LIB_PATH + '.sha256'
 
 _lib = None
+
+
+def _source_hash():
+  with open(SOURCE, 'rb') as f:
+    return hashlib.sha256(f.read()).hexdigest()
+
+
+def is_current():
+  try:
+    with open(STAMP_PATH) as f:
+      return os.path.exists(LIB_PATH) and f.read().strip() == _source_hash()
+  except OSError:
+    return False
+
+
+def build_library(verbose=False):
+  """Compiles the probes for gfx950 (the operator library's compiler and flags)."""
+  sys.path.insert(0, os.path.join(ROOT, 'ocnn-pytorch_amd'))
+  from ocnn_amd import build as b
+  cmd = [b._hipcc()] + b.COMMON + ['-shared', SOURCE, '-o', LIB_PATH]
+  res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+  if res.returncode != 0:
+    raise RuntimeError('command failed: {}\n{}'.format(' '.join(cmd), res.stdout))
+  with open(STAMP_PATH, 'w') as f:
+    f.write(_source_hash() + '\n')
+  if verbose:
+    print('built', LIB_PATH)
+  return LIB_PATH
 
 
 def lib():
   global _lib
   if _lib is None:
-    if not _build.is_current():
-      _build.build_library()
-    h = ctypes.CDLL(_build.PROBE_LIB_PATH)
+    if not is_current():
+      build_library()
+    h = ctypes.CDLL(LIB_PATH)
     h.ocnn_probe_mfma_rate.restype = c_int
     h.ocnn_probe_mfma_rate.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, POINTER(c_double),
                                        POINTER(c_double)]

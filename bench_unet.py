@@ -2,7 +2,8 @@
 channels 32-32-64-128-256 with 2/3/4/6 residual blocks, decoder 256-256-128-96-96 with 2 each,
 2x2x2 stride-2 (de)convolutions between levels, trilinear interpolation of the last features at
 the query points, a 1x1 head) as this package assembles it (ocnn_amd/unet.py), on one MI355X.  Supporting data for the pieces around the convolutions (the headline number is
-bench.py's): synthetic batch of 8 clouds x 150 000 points at depth 9, input signal 'ND'
+bench.py's): synthetic batch of 8 clouds x 150 000 points at depth 9 (indoor-like scenes: a floor,
+walls and 10 - 20 boxes each; --scene mixed: 3 spheres and 2 boxes), input signal 'ND'
 (normals + displacement), 10 classes, random weights, cross-entropy against random labels.
 
 One JSON line: ms per forward + backward, and the share of the step spent in each kind of
@@ -36,6 +37,9 @@ def run(argv=None):
   ap.add_argument('--nempty', type=int, default=1)
   ap.add_argument('--profile', action='store_true')
   ap.add_argument('--fresh', type=int, default=3, help='steps on a newly built octree, timed after the others')
+  ap.add_argument('--scene', default='indoor', choices=['indoor', 'mixed'],
+                  help='indoor: floor, walls and 10 - 20 boxes per cloud (the configuration\'s scene); '
+                       'mixed: 3 spheres and 2 boxes')
   ap.add_argument('--torch-loss', action='store_true', help='torch.nn.functional.cross_entropy for the loss')
   args = ap.parse_args(argv)
   import torch
@@ -48,7 +52,8 @@ def run(argv=None):
   dtype = getattr(torch, args.dtype)
   nempty = bool(args.nempty)
 
-  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, args.batch, 1004, n=args.points)
+  maker = synthetic.indoor_cloud if args.scene == 'indoor' else synthetic.mixed_cloud
+  pts, nrm, bid = synthetic.batch_clouds(maker, args.batch, 1004, n=args.points)
   pc = Points(pts.to(dev), nrm.to(dev), batch_id=bid.to(dev), batch_size=args.batch)
   def build():
     o = Octree(args.depth, 2, batch_size=args.batch)
@@ -99,7 +104,7 @@ def run(argv=None):
   mid = fresh[len(fresh) // 2] if fresh else (None, None)
   out = {'net': 'U-Net (ocnn/models/unet.py), forward + backward', 'ms_per_step': ms,
          'ms_octree_build_and_tables': mid[0], 'ms_first_step_on_a_fresh_octree': mid[1],
-         'dtype': args.dtype,
+         'dtype': args.dtype, 'scene': args.scene,
          'nempty': nempty, 'batch': args.batch, 'points': int(pts.shape[0]), 'depth': args.depth,
          'rows_per_depth': (octree.nnum_nempty if nempty else octree.nnum).tolist(),
          'parameters': sum(p.numel() for p in params)}

@@ -10,8 +10,6 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(HERE, 'csrc')
 LIB_DIR = os.path.join(HERE, 'lib')
 LIB_PATH = os.path.join(LIB_DIR, 'libocnn_hip.so')
-# measurement probes (MFMA and LDS rates of the part), used by bench.py only: a library of their own
-PROBE_LIB_PATH = os.path.join(LIB_DIR, 'libocnn_probe.so')
 INCLUDE = os.path.join(ROOT, 'include')
 
 # file -> extra flags.  The key/build kernels must round every fp32 operation
@@ -44,7 +42,7 @@ STAMP_PATH = os.path.join(LIB_DIR, 'sources.sha256')
 
 
 def source_hash():
-  """Hash of everything the libraries are built from (sources, headers, flags)."""
+  """Hash of everything the library is built from (sources, headers, flags)."""
   h = hashlib.sha256()
   names = sorted(os.listdir(CSRC))
   for path in [os.path.join(CSRC, n) for n in names] + [os.path.join(INCLUDE, n) for n in sorted(os.listdir(INCLUDE))]:
@@ -57,13 +55,13 @@ def source_hash():
 
 
 def is_current():
-  """True when both libraries exist and were built from the sources as they are now."""
+  """True when the library exists and was built from the sources as they are now."""
   try:
     with open(STAMP_PATH) as f:
       stamp = f.read().strip()
   except OSError:
     return False
-  return os.path.exists(LIB_PATH) and os.path.exists(PROBE_LIB_PATH) and stamp == source_hash()
+  return os.path.exists(LIB_PATH) and stamp == source_hash()
 
 
 def _hipcc():
@@ -96,7 +94,6 @@ def build_library(verbose=False):
   with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
     objs = list(pool.map(compile_one, SOURCES.items()))
   _run([hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-o', LIB_PATH] + objs)
-  _run([hipcc] + COMMON + ['-shared', os.path.join(CSRC, 'probe.hip'), '-o', PROBE_LIB_PATH])
   with open(STAMP_PATH, 'w') as f:
     f.write(source_hash() + '\n')
   if verbose:

@@ -102,6 +102,58 @@ def planes_cloud(n=250000, seed=1003, n_planes=4, n_spheres=3):
   return torch.cat(pts), torch.cat(nrm)
 
 
+def rect_points(n, g, axis, level, lo, hi, sign):
+  """Uniform on the axis-aligned rectangle {x[axis] = level, lo <= x <= hi on the other two axes};
+  normal = sign along the axis."""
+  lo = torch.tensor(lo, dtype=torch.float32)
+  hi = torch.tensor(hi, dtype=torch.float32)
+  p = lo + torch.rand(n, 3, generator=g) * (hi - lo)
+  p[:, axis] = level
+  nrm = torch.zeros(n, 3)
+  nrm[:, axis] = float(sign)
+  return p, nrm
+
+
+def indoor_cloud(n=150000, seed=1004, min_boxes=10, max_boxes=20):
+  """Config 4: an indoor-like scene: the floor of a room, two to four of its walls, and 10 - 20
+  random axis-aligned boxes standing on the floor (furniture).  Points are spread over the
+  surfaces in proportion to their areas; normals point into the room (floor, walls) or out of
+  the boxes."""
+  g = _gen(seed)
+  u = lambda: torch.rand(1, generator=g).item()
+  half, floor = 0.95, -0.9
+  top = floor + 0.9 + 0.8 * u()                           # height of the walls
+  parts = [('rect', (2, floor, (-half, -half, floor), (half, half, floor), 1.0), (2 * half) ** 2)]
+  walls = [(0, -half, 1.0), (0, half, -1.0), (1, -half, 1.0), (1, half, -1.0)]
+  order = torch.randperm(4, generator=g).tolist()
+  for w in order[:2 + int(u() * 3) % 3]:
+    axis, level, sign = walls[w]
+    lo = [-half, -half, floor]
+    hi = [half, half, top]
+    lo[axis] = hi[axis] = level
+    parts.append(('rect', (axis, level, tuple(lo), tuple(hi), sign), 2 * half * (top - floor)))
+  n_boxes = min_boxes + int(u() * (max_boxes - min_boxes + 1)) % (max_boxes - min_boxes + 1)
+  for _ in range(n_boxes):
+    ext = [0.08 + 0.4 * u(), 0.08 + 0.4 * u(), 0.08 + 0.6 * u()]
+    cx = (u() * 2 - 1) * (half - 0.02 - ext[0] / 2)
+    cy = (u() * 2 - 1) * (half - 0.02 - ext[1] / 2)
+    lo = (cx - ext[0] / 2, cy - ext[1] / 2, floor)
+    hi = (cx + ext[0] / 2, cy + ext[1] / 2, min(floor + ext[2], 0.97))
+    e = [h - l for l, h in zip(lo, hi)]
+    parts.append(('box', (lo, hi), 2 * (e[0] * e[1] + e[1] * e[2] + e[0] * e[2])))
+  area = torch.tensor([a for _, _, a in parts])
+  which = torch.multinomial(area / area.sum(), n, replacement=True, generator=g)
+  counts = torch.bincount(which, minlength=len(parts)).tolist()
+  pts, nrm = [], []
+  for (kind, args, _), c in zip(parts, counts):
+    if c == 0:
+      continue
+    p, m = rect_points(c, g, *args) if kind == 'rect' else box_points(c, g, *args)
+    pts.append(p)
+    nrm.append(m)
+  return torch.cat(pts), torch.cat(nrm)
+
+
 def shell_voxels(depth, device='cpu', thickness=1.25):
   """Integer coordinates of the cells of the 2^depth grid whose centre lies within `thickness` cells
   inside the sphere inscribed in the grid: the octree of the reference's layer benchmark

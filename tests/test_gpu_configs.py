@@ -6,6 +6,11 @@
   configs[1]  batch 8 x 100 000 points, depth 8, 64 -> 64 in fp16 / bf16: every slot of the
               weight gradient and sampled rows of the output and of the data gradient against
               the fp64 definition (the adjoint scalars alone would let a few wrong rows pass)
+  configs[2]  the same batch in bf16: OctreeConv 2x2x2 stride 2 64 -> 128 (depth 8 -> 7),
+              OctreeDeconv 2x2x2 stride 2 128 -> 64 (depth 7 -> 8) and OctreeDWConv 3x3x3 on 128
+              channels at depth 7, each through its module: every slot of the weight gradient,
+              sampled rows of the output and of the data gradient against the fp64 definition,
+              and the rows of the empty nodes of the padded tensors exactly zero
   configs[3]  batch 4 x 250 000 points (planes + spheres), depth 9: integer invariants of
               the build and the tables, then 32 -> 32 at depth 9 and 256 -> 256 at depth 6 in
               bf16 the same way
@@ -26,7 +31,7 @@ import pytest
 import torch
 
 from ocnn_amd import synthetic
-from ocnn_amd.nn import OctreeConv
+from ocnn_amd.nn import OctreeConv, OctreeDeconv, OctreeDWConv
 from ocnn_amd.octree import Octree, Points, xyz2key
 from oracle import conv_ref as C
 from oracle import octree_ref as R
@@ -152,7 +157,110 @@ def definition_checks(o, depth, ch, dtype, nempty, seed, samples=512):
   assert err_g < tol and err_g_row < 4 * tol
 
 
+def table_definition_checks(t, fine, coarse, fwd, bwd, outer, got_gather, got_scatter, got_w, dtype, g,
+                            samples=512):
+  """The three passes of a layer over the table t (rows, K), whose entries index the rows of
+  `fine`, against their fp64 definitions:
+    gather   rows i:  sum_k [t_ik >= 0] fwd(k, fine[t_ik])            (sampled rows of got_gather)
+    scatter  rows j:  sum over the entries (i, k) that hold j of bwd(k, coarse[i])
+                                                                    (sampled rows of got_scatter)
+    weights  slot k:  outer(fine[t_ik], coarse[i]) over the rows with t_ik >= 0   (all of got_w)
+  """
+  rows, K = t.shape
+  tol = TOL[dtype]
+  want_w = []
+  for k in range(K):
+    v = torch.nonzero(t[:, k] >= 0).squeeze(1)
+    want_w.append(outer(fine[t[v, k].long()].double(), coarse[v].double()))
+  want_w = torch.stack(want_w)
+  err_w = rel(got_w.reshape(want_w.shape), want_w)
+  err_w_slot = max(rel(got_w.reshape(want_w.shape)[k], want_w[k]) for k in range(K))
+
+  sel = torch.randint(0, rows, (samples,), generator=g).to(DEV)
+  ts = t[sel].long()
+  want_o = None
+  for k in range(K):
+    v = ts[:, k] >= 0
+    term = fwd(k, fine[ts[:, k].clamp_min(0)].double()) * v.unsqueeze(1)
+    want_o = term if want_o is None else want_o + term
+  err_o, err_o_row = rel(got_gather[sel], want_o), rel_rows(got_gather[sel], want_o)
+
+  n_fine = fine.shape[0]
+  sel = torch.unique(torch.randint(0, n_fine, (samples,), generator=g)).to(DEV)
+  where = torch.full((n_fine,), -1, dtype=torch.long, device=DEV)
+  where[sel] = torch.arange(sel.numel(), device=DEV)
+  want_g = torch.zeros(sel.numel(), got_scatter.shape[1], dtype=torch.float64, device=DEV)
+  for k in range(K):
+    tk = t[:, k].long()
+    pos = torch.where(tk >= 0, where[tk.clamp_min(0)], torch.full_like(tk, -1))
+    i = torch.nonzero(pos >= 0).squeeze(1)
+    want_g.index_add_(0, pos[i], bwd(k, coarse[i].double()))
+  err_g, err_g_row = rel(got_scatter[sel], want_g), rel_rows(got_scatter[sel], want_g)
+  say('   table %d x %d, %.2f entries a row: rel err weights %.2e (worst slot %.2e)  gather %.2e (worst row %.2e)  '
+      'scatter %.2e (worst row %.2e)' % (rows, K, float((t >= 0).sum()) / rows, err_w, err_w_slot, err_o,
+                                         err_o_row, err_g, err_g_row))
+  assert err_w < tol and err_w_slot < tol
+  assert err_o < tol and err_o_row < 4 * tol
+  assert err_g < tol and err_g_row < 4 * tol
+
+
 # ---------------------------------------------------------------------------------------------
+
+def test_config2_stride2_conv_deconv_and_depthwise_bf16():
+  dtype = torch.bfloat16
+  say('configs[2]: 8 x 100 000 points, depth 8, bf16')
+  o, _, _, _, _ = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
+  g = torch.Generator().manual_seed(41)
+  n8, n7, p7 = int(o.nnum[8]), int(o.nnum[7]), int(o.nnum_nempty[7])
+  assert n8 == 8 * p7
+  t = o._table(8, '222', 2, False)                          # (non-empty nodes of depth 7, 8) -> rows of depth 8
+  node7 = o.nempty_index(7)                                 # their rows among all nodes of depth 7
+  empty7 = o.children[7] < 0
+
+  say('  OctreeConv 2x2x2 stride 2, 64 -> 128, depth 8 -> 7')
+  conv = OctreeConv(64, 128, [2], 2)
+  with torch.no_grad():
+    conv.weights.copy_(torch.randn(conv.weights.shape, generator=g) / (8 * 64) ** 0.5)
+  conv = conv.to(DEV).to(dtype)
+  x = torch.randn(n8, 64, generator=g).to(dtype).to(DEV).requires_grad_()
+  gout = torch.randn(n7, 128, generator=g).to(dtype).to(DEV)      # (the rows of the empty nodes must not count)
+  out = conv(x, o, 8)
+  out.backward(gout)
+  assert out.shape == (n7, 128) and out.dtype == dtype
+  assert not bool(out[empty7].any())                        # octree_pad: zeros for the empty nodes
+  W = conv.weights.detach().double()
+  table_definition_checks(t, x.detach(), gout[node7], lambda k, r: r @ W[k], lambda k, r: r @ W[k].T,
+                          lambda a, b: a.T @ b, out[node7], x.grad, conv.weights.grad, dtype, g)
+
+  say('  OctreeDeconv 2x2x2 stride 2, 128 -> 64, depth 7 -> 8')
+  deconv = OctreeDeconv(128, 64, [2], 2)
+  with torch.no_grad():
+    deconv.weights.copy_(torch.randn(deconv.weights.shape, generator=g) / (8 * 128) ** 0.5)
+  deconv = deconv.to(DEV).to(dtype)
+  x = torch.randn(n7, 128, generator=g).to(dtype).to(DEV).requires_grad_()   # a row for every node of depth 7
+  gout = torch.randn(n8, 64, generator=g).to(dtype).to(DEV)
+  out = deconv(x, o, 7)
+  out.backward(gout)
+  assert out.shape == (n8, 64) and x.grad.shape == (n7, 128)
+  assert not bool(x.grad[empty7].any())                     # the rows the depad dropped get no gradient
+  W = deconv.weights.detach().double()                      # (8, 64, 128)
+  table_definition_checks(t, gout, x.detach()[node7], lambda k, r: r @ W[k], lambda k, r: r @ W[k].T,
+                          lambda a, b: a.T @ b, x.grad[node7], out, deconv.weights.grad, dtype, g)
+
+  say('  OctreeDWConv 3x3x3, 128 channels, depth 7')
+  dw = OctreeDWConv(128, [3], 1)
+  with torch.no_grad():
+    dw.weights.copy_(torch.randn(dw.weights.shape, generator=g) / 27 ** 0.5)
+  dw = dw.to(DEV).to(dtype)
+  t7 = o._table(7, '333', 1, False)
+  x = torch.randn(n7, 128, generator=g).to(dtype).to(DEV).requires_grad_()
+  gout = torch.randn(n7, 128, generator=g).to(dtype).to(DEV)
+  out = dw(x, o, 7)
+  out.backward(gout)
+  w = dw.weights.detach().double().view(27, 128)
+  table_definition_checks(t7, x.detach(), gout, lambda k, r: r * w[k], lambda k, r: r * w[k],
+                          lambda a, b: (a * b).sum(0), out, x.grad, dw.weights.grad, dtype, g)
+
 
 @pytest.mark.parametrize('nempty', [False, True])
 def test_config0_sphere_depth6_fp32(nempty):

@@ -1187,6 +1187,41 @@ def test_dwconv_planned_kernels(dtype, K, ch):
     assert torch.equal(gw, dw_wgrad(x.to(DEV), gr.to(DEV), tg, plan))
 
 
+def test_dwconv_planned_non_finite_values_stay_in_their_group_of_four():
+  """The planned depth-wise gather multiplies on the 4x4x4 matrix instruction with diag(w) as one
+  operand, so 0 x inf of one channel reaches the other three channels of its group of four as
+  NaN; the per-channel kernel (and the reference) keeps it in its own channel.  Fixed here: an
+  infinite input value makes non-finite outputs only in rows that read its row, and there only
+  in the channels 4 * (c / 4) .. + 3; every other value equals the result on the finite input."""
+  from ocnn_amd.nn.octree_dwconv import dw_gather
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(99)
+  K, ch, rows = 27, 64, 1000
+  table = _local_table(rows, rows, K, g)
+  tg = table.to(DEV)
+  plan = TilePlan(tg)
+  plan.reuse = 10.0
+  for dtype in (torch.float16, torch.bfloat16):
+    x = torch.randn(rows, ch, generator=g).to(dtype).to(DEV)
+    w = torch.randn(K, 1, ch, generator=g).to(dtype).to(DEV)
+    clean = dw_gather(x, rows, tg, w, False, None, plan)
+    bad_row, bad_ch = 321, 13
+    x2 = x.clone()
+    x2[bad_row, bad_ch] = float('inf')
+    got = dw_gather(x2, rows, tg, w, False, None, plan)
+    readers = (tg == bad_row).any(1)                       # rows that gather the bad row
+    group = torch.zeros(ch, dtype=torch.bool, device=DEV)
+    group[4 * (bad_ch // 4):4 * (bad_ch // 4) + 4] = True
+    touched = readers.unsqueeze(1) & group.unsqueeze(0)
+    assert bool(readers.any())
+    assert torch.equal(got[~touched], clean[~touched])
+    assert not bool(torch.isfinite(got[readers][:, bad_ch]).any())     # its own channel: inf (or NaN), as it must be
+    # the plan-free kernel keeps the value in its channel
+    plain = dw_gather(x2, rows, tg, w, False, None, None)
+    own = readers.unsqueeze(1) & (torch.arange(ch, device=DEV) == bad_ch).unsqueeze(0)
+    assert bool(torch.isfinite(plain[~own]).all())
+
+
 def test_dwconv_all_slot_kernels(medium):
   """Depth-wise kernels that keep all slots of a row in one thread (power-of-two channel
   counts), every slot count, fp32 and 16-bit, against the oracle."""
@@ -1452,7 +1487,7 @@ def test_the_documented_call_sequence_of_the_abi():
   _lib.check(L.ocnn_tile_plan_offsets(P(ucount), P(tile_nnz), tiles, 415, P(uptr), P(stats), st))
   over, dropped, total, umax, nnz, _ = stats.tolist()
   assert over == 0 and dropped == 0 and nnz == int((table >= 0).sum()) and 0 < umax <= 415
-  urows = torch.empty(total, dtype=torch.int32, device=DEV)
+  urows = torch.empty(max(total, 1), dtype=torch.int32, device=DEV)
   loc = torch.empty((tiles, K, R), dtype=torch.int16, device=DEV)
   _lib.check(L.ocnn_tile_plan_fill(P(table), rows, K, P(uptr), P(urows), P(loc), st))
   occupancy, reuse = nnz / (rows * K), nnz / max(total, 1)
@@ -1487,7 +1522,7 @@ def test_the_documented_call_sequence_of_the_abi():
   cptr = torch.zeros(tiles * nl + 1, dtype=torch.int32, device=DEV)
   cptr[1:] = nblk.cumsum(0)
   n_blocks, max_blocks = int(cptr[-1]), int(nblk.view(tiles, nl).sum(1).max())
-  ent = torch.empty(n_blocks * 16, dtype=torch.int32, device=DEV)
+  ent = torch.empty(max(n_blocks, 1) * 16, dtype=torch.int32, device=DEV)
   _lib.check(L.ocnn_pair_plan_fill(P(loc), tiles, K, P(lists), nl, P(cptr), P(ent), st))
   x = torch.randn(rows_in, 96, generator=g).to(torch.bfloat16).to(DEV)
   w = (torch.randn(K, 96, 96, generator=g) / 50).to(torch.bfloat16).to(DEV)

@@ -3,9 +3,10 @@
 Small octree, fp32: logits, loss and the gradient of EVERY parameter against a composition,
 in fp64 on the CPU, of the oracle's layers (conv / deconv definitions, trilinear
 interpolation) with torch's batch norm, ReLU and linear — the same parameters, same inputs.
-Full size (8 x 150 000 points, depth 9), bf16: one forward + backward; loss and all gradients
-finite, loss equal to the fp32 run of the same net within 16-bit rounding, gradients pointing
-the same way as the fp32 ones.
+Full size (8 x 150 000 points of indoor-like scenes, depth 9): the first block's output on all
+rows against its fp64 definition in fp32 and bf16; then one forward + backward in bf16: loss and
+all gradients finite, loss equal to the fp32 run of the same net within 16-bit rounding,
+gradients pointing the same way as the fp32 ones.
 """
 
 import sys
@@ -206,10 +207,31 @@ def test_unet_small_fp32_against_oracle_layers(nempty, training):
   assert e < (1e-1 if training else 1e-2)
 
 
+def _first_block_definition(net, feat, table, dtype):
+  """conv1 of the net (3x3x3 convolution on the table, batch norm with the statistics of the batch,
+  ReLU) in fp64 with plain torch indexing on the device, from the parameters and the input as the
+  run in `dtype` sees them (rounded to it)."""
+  W = net.conv1.conv.weights.detach().to(dtype).double()                  # (27, cin, cout)
+  x = feat.to(dtype).double()
+  rows = table.shape[0]
+  z = torch.zeros(rows, W.shape[2], dtype=torch.float64, device=DEV)
+  for r0 in range(0, rows, 1 << 18):
+    ts = table[r0:r0 + (1 << 18)].long()
+    for k in range(27):
+      z[r0:r0 + ts.shape[0]] += (x[ts[:, k].clamp_min(0)] * (ts[:, k] >= 0).unsqueeze(1)) @ W[k]
+  bn = net.conv1.bn
+  mean, var = z.mean(0), z.var(0, unbiased=False)
+  y = (z - mean) / torch.sqrt(var + bn.eps) * bn.weight.detach().to(dtype).double() + bn.bias.detach().to(dtype).double()
+  return y.clamp_min(0)
+
+
 def test_unet_full_size_bf16():
+  """configs[4] at full size on its own kind of scene (floor, walls, 10 - 20 boxes per cloud): the
+  output of the first block (all rows) against its fp64 definition in fp32 (1e-4) and bf16 (2e-2),
+  then the whole net in bf16 against its fp32 run."""
   depth, batch, n = 9, 8, 150000
-  say('U-Net, 8 x 150 000 points, depth 9, non-empty nodes: bf16 against fp32 of the same net')
-  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, batch, 1004, n=n)
+  say('U-Net, 8 x 150 000 points of indoor-like scenes, depth 9, non-empty nodes')
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.indoor_cloud, batch, 1004, n=n)
   o = Octree(depth, 2, batch_size=batch)
   o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=batch))
   o.construct_all_neigh()
@@ -218,11 +240,23 @@ def test_unet_full_size_bf16():
   labels = torch.randint(0, 10, (query.shape[0],), generator=torch.Generator().manual_seed(5)).to(DEV)
   torch.manual_seed(0)
   net = UNet(feat.shape[1], 10, 'linear', True).to(DEV)
+  say('   rows per depth', o.nnum_nempty.tolist())
+  table = o._table(depth, '333', 1, True)
   res = {}
   for dtype in (torch.float32, torch.bfloat16):
     say('  ', dtype)
     net.zero_grad(set_to_none=True)
     m = net.to(dtype)
+    with torch.no_grad():
+      got = m.conv1(feat.to(dtype), o, depth).double()
+      want = _first_block_definition(net, feat, table, dtype)
+      scale = float(want.abs().max())
+      err = float((got - want).abs().max()) / scale
+      row = (got - want).abs().amax(1) / want.abs().amax(1).clamp_min(0.05 * scale)
+      say('   first block, %d rows: rel err %.2e, worst row %.2e' % (got.shape[0], err, float(row.max())))
+      tol = 1e-4 if dtype == torch.float32 else 2e-2
+      assert err < tol and float(row.max()) < 4 * tol
+      del got, want, row
     logits = m(feat.to(dtype), o, depth, query.clone())
     loss = _loss(logits.float(), labels)
     loss.backward()

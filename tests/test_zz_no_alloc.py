@@ -47,12 +47,14 @@ def _both(dtype, rows, rows_in, K, ch, g, transposed, reverse, with_bias):
       _lib.ptr(ws), ws.numel(), _lib.stream()))
   # everything the second entry point touches exists by now: it may not allocate
   before = torch.cuda.memory_allocated()
+  free_before = torch.cuda.mem_get_info()[0]             # hipMemGetInfo: sees a hipMalloc inside the library too
   _lib.check(L.ocnn_conv_gather_rw_static(
       code, _lib.ptr(x), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax,
       plan.total, rows, K, _lib.ptr(w), ch, ch, int(transposed), int(reverse), _lib.ptr(b), _lib.ptr(got),
       _lib.stream()))
   torch.cuda.synchronize()
   assert torch.cuda.memory_allocated() == before
+  assert torch.cuda.mem_get_info()[0] >= free_before
   assert torch.isfinite(want.float()).all()
   assert torch.equal(got, want)
 
