@@ -30,6 +30,7 @@ from .octree_pad import _depad_raw, _pad_raw, octree_depad, octree_pad
 # the layer level needs: when odd channel counts run zero-padded, and from how many rows on the
 # pair-plan kernels pay for loading their weights)
 PAD_MIN_ROWS = 16384
+_CHOICES = {}            # kernel choices of the calls without a plan, by shape (see _conv_gather)
 SPARSE_MAX_OCCUPANCY = 0.3
 SPARSE_MIN_ROWS = 32768
 
@@ -78,7 +79,17 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
   if bias is not None:
     bias = bias.to(data.dtype).contiguous()
   code = _lib.dtype_code(data)
-  kernel = L.ocnn_conv_gather_choose(code, rows_in, rows, K, cin, cout, int(bool(dense)), *_plan_args(plan))
+  # (the choice and the workspace size depend on the shapes and the plan only: asked once per plan)
+  memo = _CHOICES if plan is None else plan.__dict__.setdefault('_choices', {})
+  key = ('g', code, rows_in, rows, K, cin, cout, bool(dense))
+  picked = memo.get(key)
+  if picked is None:
+    if len(memo) > 256:
+      memo.clear()
+    picked = memo[key] = (L.ocnn_conv_gather_choose(code, rows_in, rows, K, cin, cout, int(bool(dense)),
+                                                     *_plan_args(plan)),
+                          L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout))
+  kernel, ws_bytes = picked
   if kernel == _lib.GATHER_DENSE_RW and (in_index is not None or pad_to is not None):
     # the indexed form also addresses the tensors over all nodes with 32-bit offsets: past that
     # range the rows are copied out (depad) / in (pad) around the kernel on the compact rows
@@ -100,7 +111,7 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
     out = conv_gather(F.pad(data, (0, cin_p - cin)), rows_in, table, F.pad(Wk, pad_w), cout_p,
                       transposed, reverse, None if bias is None else F.pad(bias, (0, cout_p - cout)), plan)
     return out[:, :cout].contiguous(), False
-  ws = _lib.workspace(L.ocnn_conv_gather_workspace_bytes(code, rows_in, K, cin, cout), data.device)
+  ws = _lib.workspace(ws_bytes, data.device)
   if kernel == _lib.GATHER_DENSE_RW:
     out_index, n_out = None, rows
     if pad_to is not None:
@@ -169,7 +180,14 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense, g_index=None):
   rows, K = table.shape
   ca, cb = x.shape[1], g.shape[1]
   code = _lib.dtype_code(x)
-  kernel = L.ocnn_conv_wgrad_choose(code, x.shape[0], rows, K, ca, cb, int(bool(dense)), *_plan_args(plan)[:4])
+  memo = _CHOICES if plan is None else plan.__dict__.setdefault('_choices', {})
+  key = ('w', code, x.shape[0], rows, K, ca, cb, bool(dense))
+  kernel = memo.get(key)
+  if kernel is None:
+    if len(memo) > 256:
+      memo.clear()
+    kernel = memo[key] = L.ocnn_conv_wgrad_choose(code, x.shape[0], rows, K, ca, cb, int(bool(dense)),
+                                                  *_plan_args(plan)[:4])
   if g_index is not None and (kernel != _lib.WGRAD_DENSE_RW or
                               not L.ocnn_conv_dense_wgrad_rw_supported(code, max(rows, g.shape[0]), ca, cb)):
     # (the other kernels take compact rows, and so does the dense one past its 32-bit offset range)
@@ -323,6 +341,16 @@ class OctreeConvBase:
     """Tile plan for the staged kernel, when the shape can use it."""
     L, code = _lib.lib(), _lib.DTYPE_CODE.get(data.dtype, -1)
     rows = data.shape[0]
+    # (asked by every pass of every step: the answer is kept with the table it belongs to and
+    # goes when the octree drops that table)
+    memo = self.neigh.__dict__.setdefault('_plan_memo', {}) if hasattr(self.neigh, '__dict__') else None
+    key = (code, rows, cin, cout, bool(inverse), self.fine_h)
+    octree = self.octree
+    ck = ((self.neigh_depth, self.kernel, self.stride, bool(self.nempty)), bool(inverse))
+    if memo is not None and key in memo:
+      plan = memo[key]
+      if plan is None or octree._plans.get(ck) is plan:
+        return plan
     if self.neigh.shape[0] >= PAD_MIN_ROWS:               # odd channel counts run zero-padded
       cin, cout = -(-cin // 32) * 32, -(-cout // 32) * 32
     if not (L.ocnn_conv_gather_planned_supported(code, rows, cin, cout) or
@@ -330,9 +358,12 @@ class OctreeConvBase:
             L.ocnn_conv_gather_wide_supported(code, rows, self.kdim, cin, cout, 0) or
             L.ocnn_conv_gather_sparse_supported(code, rows, self.kdim, cin, cout, 0) or
             L.ocnn_conv_wgrad_planned_supported(code, rows, rows, self.kdim, cin, cout, 0)):
-      return None
-    return self.octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse,
-                             self.fine_h)
+      plan = None
+    else:
+      plan = octree._plan(self.neigh_depth, self.kernel, self.stride, self.nempty, inverse, self.fine_h)
+    if memo is not None:
+      memo[key] = plan
+    return plan
 
   def _identity(self, rows, device):
     """(rows, 1) table [0, 1, ..]: the one-slot 'gather' of the dense form."""
