@@ -41,6 +41,8 @@ def main():
   ap.add_argument('--steps', type=int, default=30)
   ap.add_argument('--warmup', type=int, default=5)
   ap.add_argument('--configs', default='2,3,4,f4')
+  ap.add_argument('--scene', default='indoor', choices=['indoor', 'mixed'],
+                  help="clouds of config 4: indoor-like scenes (the configuration's), or 3 spheres + 2 boxes")
   args = ap.parse_args()
   import torch
   from ocnn_amd import synthetic
@@ -213,8 +215,9 @@ def main():
   if '4' in args.configs.split(','):
     # the U-Net's octree (config 4: batch 8, 150k points each, depth 9), layers on the non-empty
     # nodes of depths 9 and 8, where 14 % / 25 % of the table entries hold a neighbour
-    o, b_ms, n_ms, npts = build(synthetic.mixed_cloud, 8, 1004, 150000, 9)
-    print(json.dumps({'octree': 'config 4 (batch 8, depth 9)', 'points': npts, 'build_octree_ms': b_ms,
+    o, b_ms, n_ms, npts = build(synthetic.indoor_cloud if args.scene == 'indoor' else synthetic.mixed_cloud, 8, 1004,
+                                150000, 9)
+    print(json.dumps({'octree': 'config 4 (batch 8, depth 9, %s scenes)' % args.scene, 'points': npts, 'build_octree_ms': b_ms,
                       'construct_all_neigh_ms': n_ms, 'nnum_nempty': o.nnum_nempty.tolist()}), flush=True)
     ne9, ne8 = int(o.nnum_nempty[9]), int(o.nnum_nempty[8])
     run('conv 3x3x3 s1 96->96 d9 nempty', OctreeConv(96, 96, [3], 1, nempty=True), o, 9, ne9, 96, 96,

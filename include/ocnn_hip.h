@@ -347,7 +347,7 @@ int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint
  *          device copy of the array);
  *   fill : cptr (tiles * n_lists + 1) = exclusive prefix sum of nblk, made by the caller;
  *          ent (16 entries per block): position of the pair's input row in the tile's list
- *          of rows + 1, | (128 r + 16 (r & 7)) << 16 for row r of the tile; the last block
+ *          of rows + 1, | r << 16 for row r of the tile; the last block
  *          of a list is filled up with position 0, r = 128. */
 int ocnn_pair_plan_slot_counts(const uint16_t* loc, int64_t tiles, int K, int64_t* slot_count,
                                void* stream);

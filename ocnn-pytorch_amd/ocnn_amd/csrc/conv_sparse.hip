@@ -13,8 +13,8 @@
 //     centre of a 3x3x3 table holds a third of them), so that the groups carry equal loads;
 //   * per tile and list the pair plan names the rows that have a neighbour, in blocks of 16
 //     pairs (entry = position p of the input row among the tile's staged rows, 0 = the zero
-//     row, | byte offset of the output row's accumulators << 16, 128 r + 16 (r & 7) for row r
-//     of the tile; a block is filled up with entries for (0, 128): zeros added to a spare row);
+//     row, | row r of the tile << 16; a block is filled up with entries for (0, 128): zeros
+//     added to a spare row);
 //   * the distinct input rows of the tile are staged in LDS once (global->LDS loads, row
 //     pitch cin * 2 + 16 bytes so that 16 rows spread over the banks);
 //   * a block is one v_mfma_f32_16x16x32 chain (M = 16 pairs, N = 16 channels, K = cin) whose
@@ -33,8 +33,9 @@
 namespace ocnn {
 
 constexpr int kSpRows = 128;              // rows per tile (the plan's tile size)
-constexpr int kSpAccPitch = 32;           // floats per accumulator row; the 16-byte piece c of row r
-                                          // lies at piece c ^ (r & 7) (bank spread)
+constexpr int kSpAccPitch = 36;           // floats per accumulator row: 144 bytes, so that the same 16-byte
+                                          // piece of 16 rows falls on 16 different groups of four banks when
+                                          // the rows differ mod 16 (9 r mod 16 is one to one)
 constexpr int kSpAccRows = kSpRows + 1;   // + a spare row that the filling entries of a block go to
 constexpr int kSpAccCopy = kSpAccRows * kSpAccPitch * 4;   // bytes of the sums of one group
 constexpr int kSpLists = 32;              // lists of a plan at most
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(128 * NG, WPC) void conv_gather_sparse_kernel(
     const int blast = max(bend - 1, 0);
     u32x4 Ac[NKS], An[NKS];
     f32x4 dp = {0.f, 0.f, 0.f, 0.f};                                      // result of the block before
-    char* ap = acc_w + ((kSpRows * kSpAccPitch * 4) ^ acc_c);             // and where it goes (spare row)
+    char* ap = acc_w + (kSpRows * kSpAccPitch * 4 + acc_c);               // and where it goes (spare row)
     uint32_t ec, en;
     {
       ec = s_ent[min(b, blast) * 16 + em];
@@ -250,7 +251,7 @@ __global__ __launch_bounds__(128 * NG, WPC) void conv_gather_sparse_kernel(
           av += dp;
           *(f32x4*)ap = av;
           dp = d;
-          ap = acc_w + ((ec >> 16) ^ acc_c);
+          ap = acc_w + ((ec >> 16) * (uint32_t)(kSpAccPitch * 4) + acc_c);
           ec = en;
           en = e2;
 #pragma unroll
@@ -276,7 +277,7 @@ __global__ __launch_bounds__(128 * NG, WPC) void conv_gather_sparse_kernel(
       float v[CH];
 #pragma unroll
       for (int q4 = 0; q4 < CH / 4; ++q4) {
-        const int pc = 4 * (((CH / 4) * wh + q4) ^ (wr & 7));
+        const int pc = 4 * ((CH / 4) * wh + q4);
         f32x4 x = *(const f32x4*)(a0 + pc);
         *(f32x4*)(a0 + pc) = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(kPlanThreads) void tile_plan_kernel(
 
 // Pair plan of a table, on top of its tile plan: per tile and LIST the rows that have a
 // neighbour, in blocks of 16 entries (position of the neighbour in the tile's list of rows
-// | where the row's sums live in the pair-plan gather kernel << 16).  A list is a slot, or
+// | row of the tile << 16).  A list is a slot, or
 // the rows r0 .. r1 - 1 of the tiles of a slot that holds many pairs (list = slot |
 // r0 << 8 | (r1 - 1) << 16).  One wave per (tile, list); mode 0 counts the blocks, mode 1
 // writes the entries and fills the last block up.
@@ -321,7 +321,7 @@ __global__ void pair_plan_kernel(const uint16_t* __restrict__ loc, int64_t tiles
   }
   uint32_t* e = ent + (int64_t)cptr[item] * 16;
   const unsigned long long below = (1ull << lane) - 1ull;
-  auto entry = [](uint32_t pos, int r) { return pos | ((uint32_t)(128 * r + 16 * (r & 7)) << 16); };
+  auto entry = [](uint32_t pos, int r) { return pos | ((uint32_t)r << 16); };
   if (l0 != 0) e[__popcll(m0 & below)] = entry(l0, lane);
   if (l1 != 0) e[n0 + __popcll(m1 & below)] = entry(l1, lane + 64);
   const int padded = (n + 15) & ~15;

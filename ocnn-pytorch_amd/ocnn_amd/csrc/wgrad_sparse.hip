@@ -96,7 +96,7 @@ static __device__ __forceinline__ void ws_tile(const char* __restrict__ sa, cons
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh) {
         const uint32_t e = se[b * 16 + erow + 4 * hh];
-        const uint32_t pos = e & 0xffffu, r = min(e >> 23, (uint32_t)(kWsRows - 1));   // filling: zero row x any row
+        const uint32_t pos = e & 0xffffu, r = min(e >> 16, (uint32_t)(kWsRows - 1));   // filling: zero row x any row
         av[hh] = Mma<T>::read_tr((const T*)(sa + (pos << 6) + byte0));
 #pragma unroll
         for (int bh = 0; bh < HB; ++bh)

@@ -830,7 +830,7 @@ def _gather_sparse(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
 def test_pair_plan_lists(K):
   """The pair plan against its definition, from the tile plan's positions: per tile and list
   (slot, or rows r0 .. r1 - 1 of a heavy slot) the rows with a neighbour in ascending order,
-  entry = position | (128 r + 16 (r & 7)) << 16, filled up to whole blocks of 16 with
+  entry = position | r << 16, filled up to whole blocks of 16 with
   position 0 and r = 128."""
   from ocnn_amd.octree.octree import TilePlan
   g = torch.Generator().manual_seed(K)
@@ -850,7 +850,7 @@ def test_pair_plan_lists(K):
     assert nl > K                                              # the full slot is cut by rows
   cptr = pp.cptr.cpu().numpy()
   ent = pp.ent.cpu().numpy().astype(np.int64) & 0xffffffff
-  filler = (128 * 128) << 16
+  filler = 128 << 16
   at = 0
   most = 0
   for t in range(tiles):
@@ -859,7 +859,7 @@ def test_pair_plan_lists(K):
       assert cptr[t * nl + j] == at
       k, r0, r1 = lists[j] & 255, (lists[j] >> 8) & 255, ((lists[j] >> 16) & 255) + 1
       rows = [r for r in range(r0, r1) if loc[t, k, r] > 0]
-      want = [int(loc[t, k, r]) | ((128 * r + 16 * (r & 7)) << 16) for r in rows]
+      want = [int(loc[t, k, r]) | (r << 16) for r in rows]
       want += [filler] * (-len(want) % 16)
       assert ent[16 * at:16 * at + len(want)].tolist() == want
       at += len(want) // 16
