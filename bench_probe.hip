@@ -54,9 +54,11 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(const u32x4* __restri
 
 // The MFMA loop again, now with what a wave of the register-resident gather-GEMM kernel issues
 // around its MFMAs, in that kernel's proportions per 8 MFMAs: NV independent VALU operations
-// per MFMA, NR 16-byte LDS reads, NW 16-byte LDS writes, NU 2-byte LDS reads (all conflict-free,
-// results awaited half an iteration later).  Two accumulator chains, as in that kernel.
-template <int NV, int NR, int NW, int NU>
+// per MFMA, NR 16-byte LDS reads, NW 16-byte LDS writes, NU 2-byte LDS reads (results awaited
+// half an iteration later).  STRIDE: bytes between the 16-byte chunks of consecutive lanes (16:
+// conflict-free, 32: two lanes per bank group).  NB > 0: an s_barrier every NB iterations.  Two
+// accumulator chains, as in that kernel.
+template <int NV, int NR, int NW, int NU, int STRIDE = 16, int NB = 0>
 __global__ __launch_bounds__(256, 1) void mfma_mix_kernel(const u32x4* __restrict__ src, float* __restrict__ out,
                                                           int iters, long long* __restrict__ ticks) {
   __shared__ __attribute__((aligned(16))) char lds[65536];
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(256, 1) void mfma_mix_kernel(const u32x4* __restric
 #pragma unroll
   for (int i = 0; i < 8; ++i) r[i] = u32x4{0u, 0u, 0u, 0u};
   const unsigned wave = threadIdx.x >> 6;
-  const unsigned off = (threadIdx.x & 63) * 16 + wave * 8192, offw = off + 32768;
+  const unsigned off = ((threadIdx.x & 63) * STRIDE + wave * 8192) & 0x7ff0, offw = off + 32768;
   constexpr int kWait = (NR + NW + NU) / 2 > 15 ? 15 : (NR + NW + NU) / 2;
   const long long t0 = clock64();
   for (int it = 0; it < iters; ++it) {
@@ -98,6 +100,7 @@ __global__ __launch_bounds__(256, 1) void mfma_mix_kernel(const u32x4* __restric
       for (int k = (i * NU) / 8; k < ((i + 1) * NU) / 8; ++k)
         asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(u[k & 3]) : "v"(off), "n"(64 * (k & 7)) : "memory");
       if (i == 3 || i == 7) asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(kWait) : "memory");
+      if (NB > 0 && i == 7 && (it % (NB > 0 ? NB : 1)) == 0) asm volatile("s_barrier" ::: "memory");
     }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -225,22 +228,45 @@ extern "C" int ocnn_probe_lds_rate(int write, int threads, const void* addr, voi
   }, ms);
 }
 
-// The same count of MFMAs as ocnn_probe_mfma_rate per iteration would be 14; here an iteration
-// is 8 MFMAs (bf16) with the gather-GEMM kernel's side work when mix != 0 (per 8 MFMAs: 16
-// VALU operations, six 16-byte LDS reads, one 16-byte LDS write, two 2-byte LDS reads), none
-// when mix == 0.  flops = CUs x 4 waves x iters x 8 x 32768.
+// An iteration is 8 bf16 MFMAs of one wave (ocnn_probe_mfma_rate: 14) with side work chosen by
+// `mix` (per 8 MFMAs; V = VALU operations, R = 16-byte LDS reads, W = 16-byte LDS writes, U =
+// 2-byte LDS reads):
+//   0 none                     1 the gather-GEMM kernel's: 16 V, 6 R, 1 W, 2 U
+//   2 16 V      3 32 V         4 4 R     5 6 R     6 8 R     7 8 R, two lanes per bank group
+//   8 1 W       9 2 W          10 2 U
+//   11 as 1, two lanes per bank group    12 as 1 without the write
+//   13 16 V, 8 R, 2 U (a wave that owns its outputs: one operand read per MFMA, no exchange)
+//   14 as 1 with an s_barrier every 32 MFMAs
+// flops = CUs x 4 waves x iters x 8 x 32768.
 extern "C" int ocnn_probe_mfma_mix(int mix, const void* operands, void* out, void* ticks, int iters, void* stream,
                                    double* ms, double* flops) {
   const int n_cu = cu_count();
-  if (n_cu <= 0 || iters <= 0 || iters > (1 << 22)) return -1;
+  if (n_cu <= 0 || iters <= 0 || iters > (1 << 22) || mix < 0 || mix > 14) return -1;
   hipStream_t st = (hipStream_t)stream;
   *flops = (double)n_cu * 4.0 * iters * 8.0 * 32768.0;
+#define OCNN_MIX_CASE(id, ...)                                                                                  \
+  case id:                                                                                                      \
+    hipLaunchKernelGGL((mfma_mix_kernel<__VA_ARGS__>), dim3(n_cu), dim3(256), 0, st, (const u32x4*)operands,    \
+                       (float*)out, iters, (long long*)ticks);                                                  \
+    break;
   return timed(st, [&]() {
-    if (mix)
-      hipLaunchKernelGGL((mfma_mix_kernel<2, 6, 1, 2>), dim3(n_cu), dim3(256), 0, st, (const u32x4*)operands,
-                         (float*)out, iters, (long long*)ticks);
-    else
-      hipLaunchKernelGGL((mfma_mix_kernel<0, 0, 0, 0>), dim3(n_cu), dim3(256), 0, st, (const u32x4*)operands,
-                         (float*)out, iters, (long long*)ticks);
+    switch (mix) {
+      OCNN_MIX_CASE(0, 0, 0, 0, 0)
+      OCNN_MIX_CASE(1, 2, 6, 1, 2)
+      OCNN_MIX_CASE(2, 2, 0, 0, 0)
+      OCNN_MIX_CASE(3, 4, 0, 0, 0)
+      OCNN_MIX_CASE(4, 0, 4, 0, 0)
+      OCNN_MIX_CASE(5, 0, 6, 0, 0)
+      OCNN_MIX_CASE(6, 0, 8, 0, 0)
+      OCNN_MIX_CASE(7, 0, 8, 0, 0, 32)
+      OCNN_MIX_CASE(8, 0, 0, 1, 0)
+      OCNN_MIX_CASE(9, 0, 0, 2, 0)
+      OCNN_MIX_CASE(10, 0, 0, 0, 2)
+      OCNN_MIX_CASE(11, 2, 6, 1, 2, 32)
+      OCNN_MIX_CASE(12, 2, 6, 0, 2)
+      OCNN_MIX_CASE(13, 2, 8, 0, 2)
+      OCNN_MIX_CASE(14, 2, 6, 1, 2, 16, 4)
+    }
   }, ms);
+#undef OCNN_MIX_CASE
 }

@@ -91,10 +91,10 @@ def mfma_rate(dtype=torch.bfloat16, operands='normal', iters=20000, device='cuda
 
 
 def mfma_mix(mix=True, operands='normal', iters=30000, device='cuda'):
-  """The bf16 MFMA loop with two accumulator chains, alone (mix=False) or with the side work of
-  the register-resident gather-GEMM kernel in its proportions (per 8 MFMAs: 16 VALU operations,
-  six 16-byte LDS reads, one 16-byte write, two 2-byte reads).  Returns dict(tflops, ms,
-  ticks_per_mfma, ns_per_mfma, ghz)."""
+  """The bf16 MFMA loop with two accumulator chains, alone (mix=False / 0), with the side work of
+  the register-resident gather-GEMM kernel in its proportions (mix=True / 1; per 8 MFMAs: 16 VALU
+  operations, six 16-byte LDS reads, one 16-byte write, two 2-byte reads), or with one of
+  MIX_VARIANTS.  Returns dict(tflops, ms, ticks_per_mfma, ns_per_mfma, ghz)."""
   g = torch.Generator().manual_seed(1)
   n = 9 * 256 * 8
   src = {'zero': torch.zeros(n), 'constant': torch.full((n,), 0.5),
@@ -103,7 +103,7 @@ def mfma_mix(mix=True, operands='normal', iters=30000, device='cuda'):
   out = torch.empty(_cus(device) * 256, dtype=torch.float32, device=device)
   ticks = torch.zeros(_cus(device), dtype=torch.int64, device=device)
   ms, flops = c_double(), c_double()
-  rc = lib().ocnn_probe_mfma_mix(int(bool(mix)), src.data_ptr(), out.data_ptr(), ticks.data_ptr(), iters,
+  rc = lib().ocnn_probe_mfma_mix(int(mix), src.data_ptr(), out.data_ptr(), ticks.data_ptr(), iters,
                                  torch.cuda.current_stream().cuda_stream, byref(ms), byref(flops))
   if rc != 0:
     raise RuntimeError('ocnn_probe_mfma_mix failed')
@@ -111,6 +111,26 @@ def mfma_mix(mix=True, operands='normal', iters=30000, device='cuda'):
   t, ns = float(ticks.double().mean()) / per, ms.value * 1e6 / per
   return {'tflops': flops.value / ms.value / 1e9, 'ms': ms.value, 'ticks_per_mfma': t, 'ns_per_mfma': ns,
           'ghz': t / ns}
+
+
+# side work per 8 MFMAs, by the variant number of ocnn_probe_mfma_mix
+MIX_VARIANTS = [
+    (0, 'no side work'),
+    (2, '16 VALU'),
+    (3, '32 VALU'),
+    (4, '4 ds_read_b128'),
+    (5, '6 ds_read_b128'),
+    (6, '8 ds_read_b128'),
+    (7, '8 ds_read_b128, two lanes per bank group'),
+    (8, '1 ds_write_b128'),
+    (9, '2 ds_write_b128'),
+    (10, '2 ds_read_u16'),
+    (1, 'the gather-GEMM kernel\'s: 16 VALU, 6 ds_read_b128, 1 ds_write_b128, 2 ds_read_u16'),
+    (11, 'the same, two lanes per bank group'),
+    (12, 'the same without the write'),
+    (13, 'a wave that owns its outputs: 16 VALU, 8 ds_read_b128, 2 ds_read_u16'),
+    (14, 'the kernel\'s with an s_barrier every 32 MFMAs'),
+]
 
 
 def lds_rate(offsets, write=False, iters=4000, device='cuda'):
@@ -157,11 +177,11 @@ def main():
       print('  %-9s operands %-9s %7.1f TFLOP/s  %5.2f ticks/MFMA  %5.2f ns/MFMA  (%.2f GHz)' % (
           str(dt)[6:], ops, r['tflops'], r['ticks_per_mfma'], r['ns_per_mfma'], r['ticks_per_mfma'] / r['ns_per_mfma']))
   print('\nbf16 MFMA loop, two accumulator chains, N(0,1) operands:')
-  for mix, name in ((False, 'alone'), (True, 'with the gather-GEMM kernel\'s side work (per 8 MFMAs: 16 VALU, 6 ds_read_b128, '
-                                            '1 ds_write_b128, 2 ds_read_u16)')):
-    r = mfma_mix(mix)
-    print('  %-8s %7.1f TFLOP/s  %5.2f ticks/MFMA  %5.2f ns/MFMA  (%.2f GHz)  %s' % (
-        'alone' if not mix else 'mixed', r['tflops'], r['ticks_per_mfma'], r['ns_per_mfma'], r['ghz'], '' if not mix else name))
+  print('  (side work per 8 MFMAs of a wave)')
+  for mix, name in MIX_VARIANTS:
+    r = mfma_mix(mix, iters=20000)
+    print('  %7.1f TFLOP/s  %5.2f ticks/MFMA  %5.2f ns/MFMA  (%.2f GHz)  %s' % (
+        r['tflops'], r['ticks_per_mfma'], r['ns_per_mfma'], r['ghz'], name))
   print('\nLDS, 16 bytes per lane and access, one workgroup of 256 threads per CU (B / tick / CU):')
   lanes = torch.arange(256)
   patterns = [
