@@ -606,6 +606,16 @@ __global__ __launch_bounds__(256, 1) void conv_gather_rw32_kernel(
     tile_body(std::integral_constant<int, 0>{}, tile);
     if (tile + 1 < t_end) tile_body(std::integral_constant<int, 1>{}, tile + 1);
   }
+  // The waits above COUNT operations, so every tile must issue all kOps of them - also the last
+  // tiles of the range, whose list entries and list boundaries nobody reads any more: without a
+  // reader the compiler drops those loads, the count of the tile comes out short and the wait
+  // at its end no longer covers the rows of the tile after it.  These empty statements are
+  // that reader.
+#pragma unroll
+  for (int b = 0; b < 3; ++b)
+#pragma unroll
+    for (int i = 0; i < kRowPieces; ++i) asm volatile("" ::"v"(ids[b][i]));
+  asm volatile("" ::"s"(p_a), "s"(p_b), "s"(p_c), "s"(p_d));
   __builtin_amdgcn_s_waitcnt(0x0070);                            // loads past the range still write LDS
 }
 

@@ -231,6 +231,15 @@ __global__ __launch_bounds__(256, 1) void conv_dense_rw_kernel(
     static_assert(NBUF == 2 || NBUF == 4, "index registers are taken in turn");
     for (; tile < t_end; ++tile) tile_step(std::integral_constant<int, 0>{}, tile);
   }
+  // The waits count operations: the index entries loaded by the last tiles of the range have no
+  // reader, and without one the compiler drops those loads and a tile's count comes out short.
+  // These empty statements are that reader.
+#pragma unroll
+  for (int v = 0; v < NBUF - 1; ++v) {
+    asm volatile("" ::"v"(iq[v].r[0]), "v"(iq[v].r[1]));
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) asm volatile("" ::"v"(oq[v].r[rb]));
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
 }
 
@@ -389,6 +398,10 @@ __global__ __launch_bounds__(256, 1) void conv_dense_wgrad_rw_kernel(
     step(std::integral_constant<int, 0>{}, tile);
     if (tile + 1 < t_end) step(std::integral_constant<int, 1>{}, tile + 1);
   }
+  // (a reader for the index entries that the last steps load: the waits count operations, and the
+  // compiler drops a load whose result nobody reads)
+#pragma unroll
+  for (int v = 0; v < 3; ++v) asm volatile("" ::"v"(iq[v].x), "v"(iq[v].g));
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 // loads past the range still write LDS
 
   // ---- per-range sums -> partial[split][a][b] ----

@@ -1111,6 +1111,35 @@ def test_planned_kernels_at_the_staging_limit(ch):
     assert rel_err(gw, C.weight_gemm(f64(x), f64(gr), t64)) < 2e-2
 
 
+@pytest.mark.parametrize('K,ch', [(3, 32), (27, 32), (8, 32), (3, 64), (27, 64)])
+def test_persistent_kernels_on_every_tile_count_per_workgroup(K, ch):
+  """EVERY row of the persistent gather kernels against the plan-free kernel on tables whose
+  workgroups get 3 m + 1, 3 m + 2 and 3 m tiles each (a ring of three tiles in LDS: the last one
+  or two tiles of a range run outside the ring's loop).  The 32 -> 32 kernel waits for its loads
+  by counting operations: the list entries the last tiles of a range load have no reader, the
+  compiler dropped those loads, and the wait at the end of the tile before the last no longer
+  covered the last tile's rows - a handful of wrong rows in some runs, found by the random
+  layers at K = 3, where a tile is much shorter than a load."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(31 + K)
+  wgs = torch.cuda.get_device_properties(0).multi_processor_count
+  for per in (4, 5, 6, 11):
+    rows = 128 * wgs * per - 37
+    table = _local_table(rows, rows, K, g, spread=60, empty=0.4).to(DEV)
+    plan = TilePlan(table)
+    assert L.ocnn_conv_gather_rw_supported(2, rows, K, ch, ch, plan.umax)
+    x = torch.randn(rows, ch, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(K, ch, ch, generator=g) / (K * ch) ** 0.5).bfloat16().to(DEV)
+    want = ocnn_amd.nn.conv_gather(x, rows, table, w, ch, False, False, None, None).float()
+    scale = float(want.abs().max())
+    for rep in range(3):
+      say('persistent gather, all rows', 'K', K, 'ch', ch, 'tiles per workgroup', per, 'run', rep)
+      got = ocnn_amd.nn.conv_gather(x, rows, table, w, ch, False, False, None, plan).float()
+      bad = ((got - want).abs().max(1).values > 2e-2 * scale).nonzero().view(-1)
+      assert bad.numel() == 0, (K, ch, per, rep, bad[:8].tolist(), (bad // 128)[:8].tolist())
+
+
 def test_planned_kernels_non_finite_rows():
   """Rows past the end of the table and empty entries must not pick up values of
   staged rows: NaN / Inf rows that no valid entry refers to stay out of the result."""
