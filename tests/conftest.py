@@ -19,3 +19,10 @@ def pytest_configure(config):
 @pytest.fixture(scope='session')
 def ref_data():
   return REF_DATA
+
+
+def random_cases(default):
+  """The case numbers (= seeds) of a random parity test: `default` of them from 0 on, or
+  OCNN_TEST_CASES of them from OCNN_TEST_FIRST on (a sweep continues where another one ended)."""
+  first = int(os.environ.get('OCNN_TEST_FIRST', '0'))
+  return range(first, first + int(os.environ.get('OCNN_TEST_CASES', str(default))))

@@ -101,9 +101,10 @@ def integer_invariants(o, idx, pts, bid, depth):
   assert torch.equal(leaf_key[idx], xyz2key(p[:, 0], p[:, 1], p[:, 2], b, depth))
 
 
-def definition_checks(o, depth, ch, dtype, nempty, seed, samples=512):
+def definition_checks(o, depth, ch, dtype, nempty, seed):
   """One OctreeConv 3x3x3 ch -> ch forward + backward through the module; every slot of the
-  weight gradient, `samples` rows of the output and of the data gradient against fp64."""
+  weight gradient, every row of the output and of the data gradient against fp64 (a row's error
+  over its own largest expected magnitude, or over a twentieth of the tensor's if that is larger)."""
   g = torch.Generator().manual_seed(seed)
   t = o._table(depth, '333', 1, nempty)
   rows = t.shape[0]
@@ -128,27 +129,37 @@ def definition_checks(o, depth, ch, dtype, nempty, seed, samples=512):
   err_w = rel(conv.weights.grad, want_w)
   err_w_slot = max(rel(conv.weights.grad[k], want_w[k]) for k in range(27))
 
-  # sampled rows of the output: out[i] = sum_k [t_ik >= 0] x[t_ik] @ W[k]
-  sel = torch.randint(0, rows, (samples,), generator=g).to(DEV)
-  ts = t[sel].long()
-  want_o = torch.zeros(samples, ch, dtype=torch.float64, device=DEV)
-  for k in range(27):
-    v = ts[:, k] >= 0
-    want_o[v] += xd[ts[v, k]].double() @ W[k]
-  err_o, err_o_row = rel(out[sel], want_o), rel_rows(out[sel], want_o)
+  # EVERY row of the output: out[i] = sum_k [t_ik >= 0] x[t_ik] @ W[k] (in pieces of 2^18 rows)
+  err_o = err_o_row = 0.0
+  scale_o = None
+  piece = 1 << 18
+  want_all = []
+  for r0 in range(0, rows, piece):
+    ts = t[r0:r0 + piece].long()
+    want_o = torch.zeros(ts.shape[0], ch, dtype=torch.float64, device=DEV)
+    for k in range(27):
+      v = ts[:, k] >= 0
+      want_o[v] += xd[ts[v, k]].double() @ W[k]
+    want_all.append(want_o)
+  scale_o = max(float(w.abs().max()) for w in want_all)
+  for r0, want_o in zip(range(0, rows, piece), want_all):
+    d = (out[r0:r0 + piece].detach().double() - want_o).abs()
+    err_o = max(err_o, float(d.max()) / scale_o)
+    err_o_row = max(err_o_row, float((d.amax(1) / want_o.abs().amax(1).clamp_min(0.05 * scale_o)).max()))
+  del want_all
 
-  # sampled rows of the data gradient, scatter form: gin[j] = sum over the entries (i, k) of
-  # the WHOLE table that hold j of g[i] @ W[k]^T
-  sel = torch.unique(torch.randint(0, rows, (samples,), generator=g)).to(DEV)
-  where = torch.full((rows,), -1, dtype=torch.long, device=DEV)
-  where[sel] = torch.arange(sel.numel(), device=DEV)
-  want_g = torch.zeros(sel.numel(), ch, dtype=torch.float64, device=DEV)
+  # EVERY row of the data gradient, scatter form: gin[j] = sum over the entries (i, k) of the
+  # table that hold j of g[i] @ W[k]^T
+  want_g = torch.zeros(rows, ch, dtype=torch.float64, device=DEV)
   for k in range(27):
     tk = t[:, k].long()
-    pos = torch.where(tk >= 0, where[tk.clamp_min(0)], torch.full_like(tk, -1))
-    i = torch.nonzero(pos >= 0).squeeze(1)
-    want_g.index_add_(0, pos[i], gout[i].double() @ W[k].T)
-  err_g, err_g_row = rel(x.grad[sel], want_g), rel_rows(x.grad[sel], want_g)
+    i = torch.nonzero(tk >= 0).squeeze(1)
+    want_g.index_add_(0, tk[i], gout[i].double() @ W[k].T)
+  d = (x.grad.double() - want_g).abs()
+  scale_g = float(want_g.abs().max())
+  err_g = float(d.max()) / scale_g
+  err_g_row = float((d.amax(1) / want_g.abs().amax(1).clamp_min(0.05 * scale_g)).max())
+  del want_g, d
   say('   rows %d  nnz/row %.2f  rel err: gW %.2e (worst slot %.2e)  out %.2e (worst row %.2e)  '
       'gdata %.2e (worst row %.2e)' % (rows, float((t >= 0).sum()) / rows, err_w, err_w_slot, err_o,
                                        err_o_row, err_g, err_g_row))
@@ -157,13 +168,12 @@ def definition_checks(o, depth, ch, dtype, nempty, seed, samples=512):
   assert err_g < tol and err_g_row < 4 * tol
 
 
-def table_definition_checks(t, fine, coarse, fwd, bwd, outer, got_gather, got_scatter, got_w, dtype, g,
-                            samples=512):
+def table_definition_checks(t, fine, coarse, fwd, bwd, outer, got_gather, got_scatter, got_w, dtype, g):
   """The three passes of a layer over the table t (rows, K), whose entries index the rows of
   `fine`, against their fp64 definitions:
-    gather   rows i:  sum_k [t_ik >= 0] fwd(k, fine[t_ik])            (sampled rows of got_gather)
+    gather   rows i:  sum_k [t_ik >= 0] fwd(k, fine[t_ik])            (every row of got_gather)
     scatter  rows j:  sum over the entries (i, k) that hold j of bwd(k, coarse[i])
-                                                                    (sampled rows of got_scatter)
+                                                                    (every row of got_scatter)  
     weights  slot k:  outer(fine[t_ik], coarse[i]) over the rows with t_ik >= 0   (all of got_w)
   """
   rows, K = t.shape
@@ -176,26 +186,34 @@ def table_definition_checks(t, fine, coarse, fwd, bwd, outer, got_gather, got_sc
   err_w = rel(got_w.reshape(want_w.shape), want_w)
   err_w_slot = max(rel(got_w.reshape(want_w.shape)[k], want_w[k]) for k in range(K))
 
-  sel = torch.randint(0, rows, (samples,), generator=g).to(DEV)
-  ts = t[sel].long()
-  want_o = None
-  for k in range(K):
-    v = ts[:, k] >= 0
-    term = fwd(k, fine[ts[:, k].clamp_min(0)].double()) * v.unsqueeze(1)
-    want_o = term if want_o is None else want_o + term
-  err_o, err_o_row = rel(got_gather[sel], want_o), rel_rows(got_gather[sel], want_o)
+  def row_errors(got, want):
+    d = (got.detach().double() - want).abs()
+    scale = float(want.abs().max())
+    return float(d.max()) / scale, float((d.amax(1) / want.abs().amax(1).clamp_min(0.05 * scale)).max())
 
+  # every row of the gather, in pieces of 2^18 rows
+  err_o = err_o_row = 0.0
+  wants = []
+  for r0 in range(0, rows, 1 << 18):
+    ts = t[r0:r0 + (1 << 18)].long()
+    want_o = None
+    for k in range(K):
+      v = ts[:, k] >= 0
+      term = fwd(k, fine[ts[:, k].clamp_min(0)].double()) * v.unsqueeze(1)
+      want_o = term if want_o is None else want_o + term
+    wants.append(want_o)
+  err_o, err_o_row = row_errors(got_gather, torch.cat(wants))
+  del wants
+
+  # every row of the scatter
   n_fine = fine.shape[0]
-  sel = torch.unique(torch.randint(0, n_fine, (samples,), generator=g)).to(DEV)
-  where = torch.full((n_fine,), -1, dtype=torch.long, device=DEV)
-  where[sel] = torch.arange(sel.numel(), device=DEV)
-  want_g = torch.zeros(sel.numel(), got_scatter.shape[1], dtype=torch.float64, device=DEV)
+  want_g = torch.zeros(n_fine, got_scatter.shape[1], dtype=torch.float64, device=DEV)
   for k in range(K):
     tk = t[:, k].long()
-    pos = torch.where(tk >= 0, where[tk.clamp_min(0)], torch.full_like(tk, -1))
-    i = torch.nonzero(pos >= 0).squeeze(1)
-    want_g.index_add_(0, pos[i], bwd(k, coarse[i].double()))
-  err_g, err_g_row = rel(got_scatter[sel], want_g), rel_rows(got_scatter[sel], want_g)
+    i = torch.nonzero(tk >= 0).squeeze(1)
+    want_g.index_add_(0, tk[i], bwd(k, coarse[i].double()))
+  err_g, err_g_row = row_errors(got_scatter, want_g)
+  del want_g
   say('   table %d x %d, %.2f entries a row: rel err weights %.2e (worst slot %.2e)  gather %.2e (worst row %.2e)  '
       'scatter %.2e (worst row %.2e)' % (rows, K, float((t >= 0).sum()) / rows, err_w, err_w_slot, err_o,
                                          err_o_row, err_g, err_g_row))
@@ -314,3 +332,52 @@ def test_config3_depth9_build_and_layers():
   say('configs[3]: the same layers on non-empty nodes')
   definition_checks(o, 9, 32, torch.bfloat16, True, 35)
   definition_checks(o, 6, 256, torch.bfloat16, True, 36)
+
+
+def test_layers_give_the_same_bits_on_every_run():
+  """No kernel of the path sums in an order that depends on timing, and none may read a row
+  before its load has landed: every layer shape of the benchmark configurations and of the
+  kernel-shape x stride grid, at full size (8 x 100 000 points, depth 8), run four times on the
+  same inputs - output, data gradient and weight gradient are the same bits every time.  (A
+  wait that comes too early shows as a few differing rows in some runs; the oracle tests on
+  small octrees, whose tiles are few, may never see it.)"""
+  say('same bits on every run: 8 x 100 000 points, depth 8, bf16')
+  o, _, _, _, _ = build(synthetic.mixed_cloud, 8, 1001, 100000, 8)
+  rows = {(d, ne): int((o.nnum_nempty if ne else o.nnum)[d]) for d in (6, 7, 8) for ne in (False, True)}
+  layers = [('conv', ks, 1, ne, ch, ch, 8) for ks in ([3], [3, 1, 1], [1, 3, 1], [3, 3, 1], [2])
+            for ne in (False, True) for ch in (32, 64)]
+  layers += [(kind, ks, 2, ne, 64, 64, 8 if kind == 'conv' else 7) for kind in ('conv', 'deconv')
+             for ks in ([3], [3, 1, 1], [3, 3, 1], [2]) for ne in (False, True)]
+  layers += [('conv', [2], 2, False, 64, 128, 8), ('deconv', [2], 2, False, 128, 64, 7), ('dwconv', [3], 1, False, 128, 128, 7),
+             ('dwconv', [3], 1, True, 64, 64, 8), ('conv', [3], 1, True, 96, 96, 8), ('conv', [3], 1, True, 128, 96, 8),
+             ('conv', [3], 1, True, 128, 128, 7), ('conv', [3], 1, False, 256, 256, 6), ('conv', [2], 2, True, 96, 96, 8),
+             ('deconv', [2], 2, True, 96, 96, 7)]
+  g = torch.Generator().manual_seed(77)
+  for kind, ks, stride, ne, cin, cout, depth in layers:
+    if kind == 'dwconv':
+      mod = OctreeDWConv(cin, ks, stride, ne)
+    else:
+      mod = (OctreeConv if kind == 'conv' else OctreeDeconv)(cin, cout, ks, stride, ne)
+    mod = mod.to(DEV).to(torch.bfloat16)
+    n_in = rows[(depth, ne)]
+    x = torch.randn(n_in, cin, generator=g).bfloat16().to(DEV).requires_grad_()
+    first = None
+    for run in range(4):
+      x.grad = None
+      mod.weights.grad = None
+      out = mod(x, o, depth)
+      if first is None:
+        gout = torch.randn(out.shape, generator=g).bfloat16().to(DEV)
+      out.backward(gout)
+      now = (out.detach().clone(), x.grad.clone(), mod.weights.grad.clone())
+      if first is None:
+        first = now
+        continue
+      for name, a, b in zip(('output', 'data gradient', 'weight gradient'), first, now):
+        if not torch.equal(a, b):
+          d = (a.float() - b.float()).abs().view(a.shape[0], -1).amax(1)
+          bad = d.nonzero().view(-1)
+          raise AssertionError('%s of %s %s stride %d nempty %s %d -> %d differs in run %d: %d rows, first %s' % (
+              name, kind, ks, stride, ne, cin, cout, run, bad.numel(), bad[:8].tolist()))
+    say('   %s %s stride %d nempty %s %d -> %d depth %d: %d rows in, same bits 4 times' % (kind, ks, stride, ne, cin, cout, depth, n_in))
+

@@ -12,6 +12,7 @@ import sys
 
 import numpy as np
 import pytest
+from conftest import random_cases
 import torch
 
 import ocnn_amd
@@ -1358,12 +1359,12 @@ def test_random_layers_vs_oracle():
   """Random module configurations (conv / deconv / depth-wise, all eight kernel shapes, both
   strides, all or non-empty nodes, channel counts incl. 4 / 10 / 16 / 48, f16 / bf16 / fp32, with
   and without bias) on octrees of depth 5 to 8: forward and all gradients against the oracle.
-  OCNN_TEST_CASES sets the number of cases (default 48)."""
+  OCNN_TEST_CASES sets the number of cases (default 48), OCNN_TEST_FIRST the first one."""
   octs = [(5, 2, 3000, 1), (6, 3, 8000, 2), (7, 2, 30000, 3), (7, 1, 60000, 4), (8, 2, 50000, 5)]
   kerns = ['333', '222', '311', '131', '113', '331', '313', '133']
   chans = [32, 64, 96, 128, 48, 16, 4, 10, 160, 256]
   pairs = {}
-  for case in range(int(os.environ.get('OCNN_TEST_CASES', '48'))):
+  for case in random_cases(48):
     rng = np.random.default_rng(case)
     kind = ['conv', 'deconv', 'dwconv'][int(rng.integers(0, 3))]
     depth, batch, n, seed = octs[int(rng.integers(0, len(octs)))]

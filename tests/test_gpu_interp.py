@@ -6,6 +6,7 @@ import sys
 
 import numpy as np
 import pytest
+from conftest import random_cases
 import torch
 
 import ocnn_amd
@@ -340,7 +341,7 @@ def test_random_interp_and_pool_vs_oracle():
   interpolation, the gradient of the former, max pooling with its indices and nearest upsampling
   against the oracle.  OCNN_TEST_CASES sets the number of cases (default 60)."""
   from oracle import octree_ref as R
-  for case in range(int(os.environ.get('OCNN_TEST_CASES', '60'))):
+  for case in random_cases(60):
     rng = np.random.default_rng(9000 + case)
     depth = int(rng.integers(2, 9))
     full = max(1, min(int(rng.integers(1, 4)), depth))

@@ -7,6 +7,7 @@ import sys
 
 import numpy as np
 import pytest
+from conftest import random_cases
 import torch
 
 from ocnn_amd.nn import BatchNormRelu1d
@@ -304,7 +305,7 @@ def test_random_batch_norms_vs_torch():
   from the output of the kernel (where the value before the ReLU is within rounding of zero the mask
   is a coin toss in any arithmetic), after checking that it differs from the fp64 mask nowhere
   else.  OCNN_TEST_CASES sets the number of cases (default 40)."""
-  for case in range(int(os.environ.get('OCNN_TEST_CASES', '40'))):
+  for case in random_cases(40):
     rng = np.random.default_rng(7000 + case)
     rows = int(rng.choice([2, 3, 63, 64, 65, 1000, 4097, 50000, 200000]))
     dtype = [torch.float32, torch.float16, torch.bfloat16][int(rng.integers(0, 3))]

@@ -6,6 +6,7 @@ import sys
 
 import numpy as np
 import pytest
+from conftest import random_cases
 import torch
 
 import ocnn_amd
@@ -331,7 +332,7 @@ def test_random_octrees_vs_oracle():
   distributions (uniform, a sphere, clusters with duplicates, grid-aligned coordinates up to the
   box faces): keys, children, counts, point -> leaf map, leaf signals and all neighbour tables
   bit exact against the oracle.  OCNN_TEST_CASES sets the number of cases (default 60)."""
-  for case in range(int(os.environ.get('OCNN_TEST_CASES', '60'))):
+  for case in random_cases(60):
     rng = np.random.default_rng(case)
     depth = int(rng.integers(2, 10))
     full = max(1, min(int(rng.integers(1, 5)), depth - 1))
@@ -516,7 +517,7 @@ def test_random_octrees_regrown_from_split_masks():
   generative decoder drives them: an octree regrown level by level from the split masks of a
   built one has the same keys, children, counts and neighbour tables (the property the
   reference's own test checks on its one file), on 25 random octrees (OCNN_TEST_CASES: another number)."""
-  for case in range(int(os.environ.get('OCNN_TEST_CASES', '25'))):
+  for case in random_cases(25):
     rng = np.random.default_rng(1000 + case)
     depth = int(rng.integers(3, 8))
     full = max(1, min(int(rng.integers(1, 4)), depth - 1))
@@ -556,7 +557,7 @@ def test_random_merge_equals_batched_build():
   ids (the identity the reference's test_octree.py:115-123 checks on its two files), on random
   clouds of unequal sizes: keys, children, counts, leaf signals, neighbour tables, batch_nnum
   (12 cases, or OCNN_TEST_CASES)."""
-  for case in range(int(os.environ.get('OCNN_TEST_CASES', '12'))):
+  for case in random_cases(12):
     rng = np.random.default_rng(2000 + case)
     depth = int(rng.integers(3, 8))
     full = max(1, min(int(rng.integers(1, 4)), depth - 1))

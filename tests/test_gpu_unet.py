@@ -228,7 +228,7 @@ def _first_block_definition(net, feat, table, dtype):
 def test_unet_full_size_bf16():
   """configs[4] at full size on its own kind of scene (floor, walls, 10 - 20 boxes per cloud): the
   output of the first block (all rows) against its fp64 definition in fp32 (1e-4) and bf16 (2e-2),
-  then the whole net in bf16 against its fp32 run."""
+  then the whole net in bf16 against its fp32 run, and twice on the same inputs (same bits)."""
   depth, batch, n = 9, 8, 150000
   say('U-Net, 8 x 150 000 points of indoor-like scenes, depth 9, non-empty nodes')
   pts, nrm, bid = synthetic.batch_clouds(synthetic.indoor_cloud, batch, 1004, n=n)
@@ -266,6 +266,17 @@ def test_unet_full_size_bf16():
     for k, gk in grads.items():
       assert torch.isfinite(gk).all(), k
     res[dtype] = (float(loss), grads)
+    if dtype == torch.bfloat16:
+      # No kernel of the path sums in an order that depends on timing: the same step again gives
+      # the same bits, logits and every parameter gradient (a load waited for too early, the
+      # kind of defect a handful of wrong rows comes from, shows here as a difference).
+      m.zero_grad(set_to_none=True)
+      again = m(feat.to(dtype), o, depth, query.clone())
+      _loss(again.float(), labels).backward()
+      assert torch.equal(again, logits), 'logits differ between two runs'
+      diff = [k for k, p in m.named_parameters() if not torch.equal(p.grad.float(), grads[k])]
+      assert not diff, ('gradients differ between two runs', diff[:6])
+      del again
     net = m.float()
   l32, g32 = res[torch.float32]
   l16, g16 = res[torch.bfloat16]
