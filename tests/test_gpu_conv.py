@@ -1141,6 +1141,57 @@ def test_persistent_kernels_on_every_tile_count_per_workgroup(K, ch):
       assert bad.numel() == 0, (K, ch, per, rep, bad[:8].tolist(), (bad // 128)[:8].tolist())
 
 
+def test_other_planned_kernels_on_many_tile_counts():
+  """The other kernels on the plan (weight gradient, wide gather, pair-plan gather and weight
+  gradient, depth-wise gather and weight gradient) against the plan-free kernels on EVERY row,
+  on tables of 4 .. 7 tiles per CU: ranges of tiles that end inside a ring of buffers, tails of
+  every length."""
+  from ocnn_amd.nn.octree_dwconv import dw_gather, dw_wgrad
+  from ocnn_amd.octree.octree import TilePlan
+  g = torch.Generator().manual_seed(5)
+  wgs = torch.cuda.get_device_properties(0).multi_processor_count
+  bf = torch.bfloat16
+
+  def close(tag, got, want, per):
+    got, want = got.float(), want.float()
+    scale = float(want.abs().max())
+    bad = ((got - want).abs().reshape(got.shape[0], -1).amax(1) > 2e-2 * scale).nonzero().view(-1)
+    assert bad.numel() == 0, (tag, per, bad[:8].tolist())
+
+  for per in (4, 5, 6, 7):
+    rows = 128 * wgs * per - 61
+    say('planned kernels, all rows, tiles per CU', per, 'rows', rows)
+    table = _local_table(rows, rows, 27, g, spread=60, empty=0.4).to(DEV)
+    plan = TilePlan(table)
+    for ch in (32, 64):
+      x = torch.randn(rows, ch, generator=g).to(bf).to(DEV)
+      gr = torch.randn(rows, ch, generator=g).to(bf).to(DEV)
+      close('weight gradient %d' % ch, ocnn_amd.nn.conv_wgrad(x, gr, table, False, plan),
+            ocnn_amd.nn.conv_wgrad(x, gr, table, False, None), per)
+    x = torch.randn(rows, 128, generator=g).to(bf).to(DEV)
+    w = (torch.randn(27, 128, 128, generator=g) / (27 * 128) ** 0.5).to(bf).to(DEV)
+    close('wide gather', _gather_wide(x, rows, table, plan, w, 128, False, False, None),
+          ocnn_amd.nn.conv_gather(x, rows, table, w, 128, False, False, None, None), per)
+    gr = torch.randn(rows, 128, generator=g).to(bf).to(DEV)
+    close('weight gradient 128', ocnn_amd.nn.conv_wgrad(x, gr, table, False, plan),
+          ocnn_amd.nn.conv_wgrad(x, gr, table, False, None), per)
+    xd = torch.randn(rows, 64, generator=g).to(bf).to(DEV)
+    wd = torch.randn(27, 1, 64, generator=g).to(bf).to(DEV)
+    grd = torch.randn(rows, 64, generator=g).to(bf).to(DEV)
+    plan.reuse = 10.0
+    close('depth-wise gather', dw_gather(xd, rows, table, wd, False, None, plan), dw_gather(xd, rows, table, wd, False, None, None), per)
+    close('depth-wise weight gradient', dw_wgrad(xd, grd, table, plan), dw_wgrad(xd, grd, table, None), per)
+    sparse = _local_table(rows, rows, 27, g, spread=60, empty=0.85).to(DEV)
+    splan = TilePlan(sparse)
+    x = torch.randn(rows, 96, generator=g).to(bf).to(DEV)
+    w = (torch.randn(27, 96, 96, generator=g) / (27 * 96 * 0.15) ** 0.5).to(bf).to(DEV)
+    gr = torch.randn(rows, 96, generator=g).to(bf).to(DEV)
+    close('pair-plan gather', _gather_sparse(x, rows, sparse, splan, w, 96, False, False, None),
+          ocnn_amd.nn.conv_gather(x, rows, sparse, w, 96, False, False, None, None), per)
+    close('pair-plan weight gradient', _wgrad_sparse(x, gr, sparse, splan, False),
+          ocnn_amd.nn.conv_wgrad(x, gr, sparse, False, None), per)
+
+
 def test_planned_kernels_non_finite_rows():
   """Rows past the end of the table and empty entries must not pick up values of
   staged rows: NaN / Inf rows that no valid entry refers to stay out of the result."""
