@@ -463,10 +463,15 @@ int ocnn_conv_wgrad(int dtype, const void* x, int64_t rows_x, const void* g,
  * reference lines, same result up to the fp32 summation order, which is fixed).
  * Per tile the distinct x rows and the g rows are staged once in LDS; persistent
  * workgroups keep the sums of all K slots in accumulator registers over a range
- * of tiles.  plan_max_distinct must be <= 415; ..._supported() tells. */
+ * of tiles.  plan_max_distinct must be <= 415; ..._supported() tells.
+ * fp32 tensors run as two bf16 pieces each (x = hi + lo): three passes of the bf16
+ * kernel (hi hi, hi lo, lo hi) into three sets of sums and one reduction, about 1e-5
+ * relative; the workspace then also holds the pieces: ..._workspace_bytes_for(). */
 int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
                                       int cb, int plan_max_distinct);
-int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K, int ca, int cb);
+int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K, int ca, int cb);   /* f16 / bf16 */
+int64_t ocnn_conv_wgrad_planned_workspace_bytes_for(int dtype, int64_t rows_x, int64_t rows, int K,
+                                                    int ca, int cb);
 int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x, const void* g,
                             const uint16_t* loc, const int32_t* uptr, const int32_t* urows,
                             int plan_max_distinct, int64_t plan_total, int64_t rows, int K,

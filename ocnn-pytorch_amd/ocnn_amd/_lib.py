@@ -89,6 +89,7 @@ SIGNATURES = {
     'ocnn_conv_wgrad': (_i, [_i, _p, _l, _p, _p, _l, _i, _i, _i, _i, _p, _p, _l, _p]),
     'ocnn_conv_wgrad_planned_supported': (_i, [_i, _l, _l, _i, _i, _i, _i]),
     'ocnn_conv_wgrad_planned_workspace_bytes': (_l, [_i, _i, _i]),
+    'ocnn_conv_wgrad_planned_workspace_bytes_for': (_l, [_i, _l, _l, _i, _i, _i]),
     'ocnn_conv_wgrad_planned': (_i, [_i, _p, _l, _p, _p, _p, _p, _i, _l, _l, _i, _i, _i, _i, _p, _p,
                                      _l, _p]),
     'ocnn_dwconv_gather': (_i, [_i, _p, _l, _p, _l, _i, _p, _i, _i, _p, _p, _p]),

@@ -237,15 +237,6 @@ __global__ void split3_weights_kernel(const float* __restrict__ w, int K, int ci
   }
 }
 
-__global__ void split2_kernel(const float* __restrict__ x, int64_t n, bf16* __restrict__ hi,
-                              bf16* __restrict__ lo) {
-  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= n) return;
-  float v = x[e];
-  bf16 h = (bf16)v;
-  hi[e] = h;
-  lo[e] = (bf16)(v - (float)h);
-}
 
 // --------------------------------------------------------------------------
 // gather-GEMM, plain (any dtype, any channel count)

@@ -55,6 +55,18 @@ __global__ void wgrad_reduce4_kernel(const float* __restrict__ partial, int spli
   }
 }
 
+// fp32 values as two bf16 pieces: x = hi + lo (+ 2^-17 |x|); a product of two such values is
+// hi_a hi_b + hi_a lo_b + lo_a hi_b to about 1e-5 relative
+static __global__ void split2_kernel(const float* __restrict__ x, int64_t n, bf16* __restrict__ hi,
+                              bf16* __restrict__ lo) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n) return;
+  float v = x[e];
+  bf16 h = (bf16)v;
+  hi[e] = h;
+  lo[e] = (bf16)(v - (float)h);
+}
+
 // launches the reduction that fits
 template <typename T>
 inline void launch_wgrad_reduce(const float* partial, int splits, int K, int ca, int cb,

@@ -399,7 +399,7 @@ static int wp_cu_count() {
 
 extern "C" int ocnn_conv_wgrad_planned_supported(int dtype, int64_t rows_x, int64_t rows, int K, int ca,
                                                  int cb, int plan_max_distinct) {
-  if (dtype != OCNN_F16 && dtype != OCNN_BF16) return 0;
+  if (dtype != OCNN_F16 && dtype != OCNN_BF16 && dtype != OCNN_F32) return 0;   // (fp32: as bf16 pieces)
   if (!(ca == 32 && cb == 32) && !(ca >= 64 && cb >= 64 && ca % 32 == 0 && cb % 32 == 0 && ca <= 1024 && cb <= 1024))
     return 0;
   if (K != 27 && K != 9 && K != 8 && K != 3) return 0;
@@ -413,6 +413,15 @@ extern "C" int64_t ocnn_conv_wgrad_planned_workspace_bytes(int K, int ca, int cb
   const int n_cu = wp_cu_count();
   const int64_t splits = n_cu > 0 ? wp_splits(K, ca, cb, n_cu) : 256;
   return align_up(splits * K * ca * cb * 4, 256);
+}
+
+// fp32: three sets of per-range sums (hi_x hi_g, hi_x lo_g, lo_x hi_g) after the bf16 pieces
+// of both tensors
+extern "C" int64_t ocnn_conv_wgrad_planned_workspace_bytes_for(int dtype, int64_t rows_x, int64_t rows, int K,
+                                                               int ca, int cb) {
+  const int64_t sums = ocnn_conv_wgrad_planned_workspace_bytes(K, ca, cb);
+  if (dtype != OCNN_F32 || rows_x < 0 || rows < 0) return sums;
+  return 2 * align_up(rows_x * ca * 2, 256) + 2 * align_up(rows * cb * 2, 256) + 3 * sums;
 }
 
 template <typename T, int C, int KK, int NFULL, int NHALF, int GROUPS>
@@ -432,10 +441,34 @@ static void launch_wp(const void* x, int64_t rows_x, const void* g, const uint16
                        gb, loc, lb, uptr, urows, ub, tiles, per, nsplit, ca, cb, partial);
 }
 
+// the launches of one pass over the plan: per-range sums of x^T g into `partial`
+template <typename T>
+static void launch_wp_pass(const void* x, int64_t rows_x, const void* g, const uint16_t* loc, const int32_t* uptr,
+                           const int32_t* urows, int64_t plan_total, int64_t rows, int K, int ca, int cb,
+                           int nsplit, int64_t per, float* partial, hipStream_t st) {
+#define OCNN_WP_LAUNCH(CC, KK, NF, NH, GR) \
+  launch_wp<T, CC, KK, NF, NH, GR>(x, rows_x, g, loc, uptr, urows, plan_total, rows, ca, cb, nsplit, per, partial, st)
+  if (ca >= 64) {
+    if (K == 27) OCNN_WP_LAUNCH(64, 27, 3, 1, 2);
+    else if (K == 9) OCNN_WP_LAUNCH(64, 9, 2, 1, 1);
+    else if (K == 8) OCNN_WP_LAUNCH(64, 8, 2, 0, 1);
+    else OCNN_WP_LAUNCH(64, 3, 1, 0, 1);
+  } else {
+    if (K == 27) OCNN_WP_LAUNCH(32, 27, 7, 0, 1);
+    else if (K == 9) OCNN_WP_LAUNCH(32, 9, 3, 0, 1);
+    else if (K == 8) OCNN_WP_LAUNCH(32, 8, 2, 0, 1);
+    else OCNN_WP_LAUNCH(32, 3, 1, 0, 1);
+  }
+#undef OCNN_WP_LAUNCH
+}
+
+// T: the type of x, g and gw (float: x and g go through the kernels as two bf16 pieces each,
+// three passes into three sets of sums, one reduction over all of them)
 template <typename T>
 static int run_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* loc, const int32_t* uptr,
                   const int32_t* urows, int64_t plan_total, int64_t rows, int K, int ca, int cb,
                   int out_transposed, void* gw, void* ws, int64_t ws_bytes, hipStream_t st) {
+  constexpr bool kPieces = std::is_same<T, float>::value;
   const int n_cu = wp_cu_count();
   if (n_cu <= 0) {
     set_error("conv_wgrad_planned: cannot query the device");
@@ -445,28 +478,36 @@ static int run_wp(const void* x, int64_t rows_x, const void* g, const uint16_t* 
   const int64_t tiles = cdiv(rows, kWpRows);
   const int64_t per = std::max<int64_t>(1, cdiv(tiles, nsplit));
   const int used = (int)cdiv(tiles, per);                 // ranges that hold tiles
-  if (ws_bytes < (int64_t)used * K * ca * cb * 4) {
+  const int64_t set = (int64_t)used * K * ca * cb;         // floats of one set of sums
+  const int64_t xb = kPieces ? align_up(rows_x * ca * 2, 256) : 0, gb = kPieces ? align_up(rows * cb * 2, 256) : 0;
+  if (ws_bytes < 2 * xb + 2 * gb + (kPieces ? 3 : 1) * set * 4) {
     set_error("conv_wgrad_planned: workspace too small");
     return OCNN_ERR_WORKSPACE;
   }
-  float* partial = (float*)ws;
-  if (rows > 0) {
-#define OCNN_WP_LAUNCH(CC, KK, NF, NH, GR) \
-  launch_wp<T, CC, KK, NF, NH, GR>(x, rows_x, g, loc, uptr, urows, plan_total, rows, ca, cb, nsplit, per, partial, st)
-    if (ca >= 64) {
-      if (K == 27) OCNN_WP_LAUNCH(64, 27, 3, 1, 2);
-      else if (K == 9) OCNN_WP_LAUNCH(64, 9, 2, 1, 1);
-      else if (K == 8) OCNN_WP_LAUNCH(64, 8, 2, 0, 1);
-      else OCNN_WP_LAUNCH(64, 3, 1, 0, 1);
-    } else {
-      if (K == 27) OCNN_WP_LAUNCH(32, 27, 7, 0, 1);
-      else if (K == 9) OCNN_WP_LAUNCH(32, 9, 3, 0, 1);
-      else if (K == 8) OCNN_WP_LAUNCH(32, 8, 2, 0, 1);
-      else OCNN_WP_LAUNCH(32, 3, 1, 0, 1);
+  float* partial = (float*)((char*)ws + 2 * xb + 2 * gb);
+  if constexpr (kPieces) {
+    if (rows > 0) {
+      bf16* xh = (bf16*)ws;
+      bf16* xl = (bf16*)((char*)ws + xb);
+      bf16* gh = (bf16*)((char*)ws + 2 * xb);
+      bf16* gl = (bf16*)((char*)ws + 2 * xb + gb);
+      if (rows_x > 0)
+        hipLaunchKernelGGL(split2_kernel, dim3((unsigned)cdiv(rows_x * ca, 256)), dim3(256), 0, st, (const float*)x,
+                           rows_x * ca, xh, xl);
+      hipLaunchKernelGGL(split2_kernel, dim3((unsigned)cdiv(rows * cb, 256)), dim3(256), 0, st, (const float*)g,
+                         rows * cb, gh, gl);
+      const bf16* xs[3] = {xh, xh, xl};
+      const bf16* gs[3] = {gh, gl, gh};
+      for (int i = 0; i < 3; ++i)
+        launch_wp_pass<bf16>(xs[i], rows_x, gs[i], loc, uptr, urows, plan_total, rows, K, ca, cb, nsplit, per,
+                             partial + i * set, st);
     }
-#undef OCNN_WP_LAUNCH
+    launch_wgrad_reduce<float>(partial, rows > 0 ? 3 * used : 0, K, ca, cb, out_transposed, (float*)gw, st);
+  } else {
+    if (rows > 0)
+      launch_wp_pass<T>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, cb, nsplit, per, partial, st);
+    launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, ca, cb, out_transposed, (T*)gw, st);
   }
-  launch_wgrad_reduce<T>(partial, rows > 0 ? used : 0, K, ca, cb, out_transposed, (T*)gw, st);
   return check_launch("conv_wgrad_planned");
 }
 
@@ -484,6 +525,9 @@ extern "C" int ocnn_conv_wgrad_planned(int dtype, const void* x, int64_t rows_x,
   OCNN_REQUIRE(rows == 0 || (g && loc && uptr && urows && (rows_x == 0 || x)),
                "conv_wgrad_planned: a required pointer is NULL (of x, g, loc, uptr, urows)");
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == OCNN_F32)
+    return run_wp<float>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, cb, out_transposed, gw, workspace,
+                         workspace_bytes, st);
   if (dtype == OCNN_F16)
     return run_wp<f16>(x, rows_x, g, loc, uptr, urows, plan_total, rows, K, ca, cb, out_transposed, gw, workspace,
                        workspace_bytes, st);

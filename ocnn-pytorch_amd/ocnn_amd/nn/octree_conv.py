@@ -215,7 +215,7 @@ def _conv_wgrad(x, g, table, out_transposed, plan, dense, g_index=None):
         int(not out_transposed), _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
     return gw, True
   if kernel == _lib.WGRAD_PLANNED:
-    ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes(K, ca, cb), x.device)
+    ws = _lib.workspace(L.ocnn_conv_wgrad_planned_workspace_bytes_for(code, x.shape[0], rows, K, ca, cb), x.device)
     _lib.check(L.ocnn_conv_wgrad_planned(
         code, _lib.ptr(x), x.shape[0], _lib.ptr(g), _lib.ptr(plan.loc), _lib.ptr(plan.uptr),
         _lib.ptr(plan.urows), plan.umax, plan.total, rows, K, ca, cb, int(out_transposed),

@@ -623,6 +623,32 @@ def test_planned_64x64_kernels(dtype, K, ch):
     assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
 
 
+@pytest.mark.parametrize('K,ca,cb', [(27, 32, 32), (27, 64, 64), (9, 64, 128), (8, 128, 64), (3, 32, 32), (27, 96, 160)])
+def test_planned_weight_gradient_fp32(K, ca, cb):
+  """fp32 tensors on the planned weight-gradient kernel (two bf16 pieces per value, three passes,
+  one reduction): 1e-4 of the fp64 sums, the same bits on a second run, both output layouts,
+  and the selection takes it."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  g = torch.Generator().manual_seed(200 + K + ca)
+  for rows, rows_in in [(1000, 1000), (4133, 2300), (128 * 300 + 1, 128 * 300 + 1)]:
+    say('planned weight gradient, fp32', 'K', K, ca, cb, 'rows', rows, 'rows_in', rows_in)
+    table = _local_table(rows, rows_in, K, g)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    assert L.ocnn_conv_wgrad_planned_supported(0, rows_in, rows, K, ca, cb, plan.umax)
+    assert L.ocnn_conv_wgrad_choose(0, rows_in, rows, K, ca, cb, 0, 1, plan.umax, plan.total,
+                                    float(plan.occupancy)) == _lib.WGRAD_PLANNED
+    x = torch.randn(rows_in, ca, generator=g)
+    gr = torch.randn(rows, cb, generator=g)
+    want = C.weight_gemm(f64(x), f64(gr), table.numpy().astype(np.int64))
+    gw = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan)
+    assert gw.dtype == torch.float32 and rel_err(gw, want) < 1e-4, rel_err(gw, want)
+    assert torch.equal(gw, ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, False, plan))
+    gwt = ocnn_amd.nn.conv_wgrad(x.to(DEV), gr.to(DEV), tg, True, plan)
+    assert torch.equal(gwt, gw.transpose(1, 2).contiguous())
+
+
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('cin,cout', [(64, 128), (128, 512), (512, 128), (256, 256), (1024, 384), (192, 1024)])
 def test_dense_rows_kernel(dtype, cin, cout):
