@@ -240,11 +240,14 @@ __global__ __launch_bounds__(128 * NG, WPC) void conv_gather_sparse_kernel(
         const int be = __builtin_amdgcn_readfirstlane(cp[jbase + i + 1]);
         while (b < be) {
           // rows of the next block, entry of the one after, accumulators of the one before
+          // (LDS reads come back in the order of their issue: the sums first, so that their
+          // read - add - write does not wait for the gathered rows)
+          f32x4 av = *(const f32x4*)ap;
+          const uint32_t e2 = s_ent[min(b + 2, blast) * 16 + em];
           const char* a = a_base + (en & 0xffffu) * PITCH;
 #pragma unroll
           for (int s = 0; s < NKS; ++s) An[s] = *(const u32x4*)(a + s * 64);
-          const uint32_t e2 = s_ent[min(b + 2, blast) * 16 + em];
-          f32x4 av = *(const f32x4*)ap;
+          __builtin_amdgcn_sched_barrier(0);
           f32x4 d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < NKS; ++s) d = Mma<T>::run(W[i][s], Ac[s], d);
