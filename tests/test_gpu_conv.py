@@ -1218,6 +1218,68 @@ def test_other_planned_kernels_on_many_tile_counts():
           ocnn_amd.nn.conv_wgrad(x, gr, sparse, False, None), per)
 
 
+@pytest.mark.parametrize('ch,empty,kernel', [(64, 0.3, 'GATHER_RW'), (32, 0.3, 'GATHER_RW'), (128, 0.3, 'GATHER_WIDE'),
+                                             (96, 0.85, 'GATHER_SPARSE')])
+def test_tables_at_the_end_of_32_bit_offsets(ch, empty, kernel):
+  """The kernels on the plan address their tensors with 32-bit byte offsets.  A table just
+  under that range runs on them (the selection says so), one just over it on another
+  kernel; either way the first, the last and 2000 random rows of output, data gradient and
+  the whole weight gradient equal their fp64 definitions (rows near 2^32 bytes are where an
+  offset that wraps would show)."""
+  from ocnn_amd.octree.octree import TilePlan
+  L = _lib.lib()
+  K, dtype = 3, torch.bfloat16
+  limit = 0xfff00000 // (ch * 2)                       # rows of `ch` bf16 channels in the range
+  for rows, planned in ((limit - 4096 - 77, True), (limit + 4096 + 77, False)):
+    say('tables at the end of 32-bit offsets:', ch, 'channels,', rows, 'rows,', kernel if planned else 'another kernel')
+    g = torch.Generator(device=DEV).manual_seed(rows % 1000)
+    base = torch.arange(rows, device=DEV).view(-1, 1)
+    if kernel == 'GATHER_WIDE':                          # (that kernel is for tables whose tiles reuse their rows)
+      table = (base + torch.arange(-1, K - 1, device=DEV).view(1, -1)).clamp_(0, rows - 1).to(torch.int32)
+    else:
+      table = (base + torch.randint(-40, 41, (rows, K), device=DEV, generator=g)).clamp_(0, rows - 1).to(torch.int32)
+    table[torch.rand(rows, K, device=DEV, generator=g) < empty] = -1
+    del base
+    plan = TilePlan(table)
+    code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+    took = L.ocnn_conv_gather_choose(code, rows, rows, K, ch, ch, 0, 1, plan.umax, plan.total, float(plan.occupancy),
+                                     float(plan.reuse))
+    assert (took == getattr(_lib, kernel)) == planned, (took, kernel)
+    x = torch.randn(rows, ch, device=DEV, generator=g).to(dtype)
+    gr = torch.randn(rows, ch, device=DEV, generator=g).to(dtype)
+    w = (torch.randn(K, ch, ch, device=DEV, generator=g) / (K * ch) ** 0.5).to(dtype)
+    sel = torch.cat([torch.arange(0, 1000, device=DEV), torch.arange(rows - 1000, rows, device=DEV),
+                     torch.randint(0, rows, (2000,), device=DEV, generator=g)])
+    ts = table[sel].long()
+
+    def rows_of_definition(src, wk):                   # sum_k [t_ik >= 0] src[t_ik] @ wk(k), rows `sel`
+      want = torch.zeros(sel.numel(), ch, dtype=torch.float64, device=DEV)
+      for k in range(K):
+        v = ts[:, k] >= 0
+        want[v] += src[ts[v, k]].double() @ wk(k)
+      return want
+
+    out = ocnn_amd.nn.conv_gather(x, rows, table, w, ch, False, False, None, plan)
+    assert rel_err(out[sel], rows_of_definition(x, lambda k: w[k].double()).cpu().numpy()) < TOL[dtype]
+    del out
+    # the mirrored form (data gradient of a symmetric table)
+    out = ocnn_amd.nn.conv_gather(gr, rows, table, w, ch, True, True, None, plan)
+    assert rel_err(out[sel], rows_of_definition(gr, lambda k: w[K - 1 - k].double().T).cpu().numpy()) < TOL[dtype]
+    del out
+    gw = ocnn_amd.nn.conv_wgrad(x, gr, table, False, plan)
+    want = torch.empty(K, ch, ch, dtype=torch.float64, device=DEV)
+    for k in range(K):
+      v = torch.nonzero(table[:, k] >= 0).squeeze(1)
+      acc = torch.zeros(ch, ch, dtype=torch.float64, device=DEV)
+      for r0 in range(0, v.numel(), 1 << 22):            # (pieces: the fp64 copies of the rows are large)
+        vv = v[r0:r0 + (1 << 22)]
+        acc += x[table[vv, k].long()].double().T @ gr[vv].double()
+      want[k] = acc
+    assert rel_err(gw, want.cpu().numpy()) < TOL[dtype]
+    del x, gr, table, plan, gw, want
+    torch.cuda.empty_cache()
+
+
 def test_planned_kernels_non_finite_rows():
   """Rows past the end of the table and empty entries must not pick up values of
   staged rows: NaN / Inf rows that no valid entry refers to stay out of the result."""
