@@ -17,7 +17,15 @@
  *     too small OCNN_ERR_WORKSPACE; pointers named "may be NULL" are optional;
  *   - feature matrices are row-major (rows, channels); neighbour tables are
  *     row-major (rows, K) int32 with -1 for "no neighbour";
- *   - dtype codes: 0 = float32, 1 = float16, 2 = bfloat16 (fp32 accumulation).
+ *   - dtype codes: 0 = float32, 1 = float16, 2 = bfloat16 (fp32 accumulation);
+ *   - sizes the reference does not limit and this library does (OCNN_ERR_ARG beyond them):
+ *     a neighbour table has fewer than 2^31 entries (79.5 M rows of 27 slots), a layer
+ *     and a point cloud fewer than 2^31 nodes / points, full layers reach depth 8 in the
+ *     build and depth 7 in the neighbour search (batch x 8^depth x 27 < 2^31), octrees
+ *     depth 16 (what 48-bit keys hold); the kernels on a tile plan address their tensors
+ *     with 32-bit byte offsets (rows x channels x 2 bytes below 0xfff00000: their
+ *     ..._supported() and the ..._choose() functions tell, and the plan-free entry points
+ *     take what is larger).
  */
 #ifndef OCNN_HIP_H_
 #define OCNN_HIP_H_

@@ -171,12 +171,14 @@ extern "C" int ocnn_neigh_all(int depth, int full_depth, int batch, const int64_
   // (the table of a layer below the full ones is made from its parents' table, and layer 0 has
   // none: as in the reference, whose construct_neigh(1) fails on an octree with full_depth = 0)
   OCNN_REQUIRE(depth >= 1 && depth <= 16 && full_depth >= 1 && full_depth <= depth && full_depth <= 7 && batch >= 1,
-               "neigh_all: depth=%d full_depth=%d batch=%d (full_depth >= 1: layer 1 must be full)", depth,
-               full_depth, batch);
+               "neigh_all: depth=%d full_depth=%d batch=%d (1 <= full_depth <= min(depth, 7): layer 1 must be "
+               "full, and the table of a full layer has batch x 8^depth x 27 < 2^31 entries)",
+               depth, full_depth, batch);
   OCNN_REQUIRE_PTRS("neigh_all", h_nnum, h_nnum_nempty, h_children, h_nempty_index, h_neigh);
   hipStream_t st = (hipStream_t)stream;
   for (int d = 1; d <= depth; ++d) {
-    OCNN_REQUIRE(h_neigh[d] != nullptr && h_nnum[d] > 0 && h_nnum[d] * 27 < (1ll << 31), "neigh_all: layer %d", d);
+    OCNN_REQUIRE(h_neigh[d] != nullptr && h_nnum[d] > 0 && h_nnum[d] * 27 < (1ll << 31),
+                 "neigh_all: layer %d: no table, or no nodes, or 2^31 table entries and more", d);
     if (d <= full_depth) {
       const int64_t total = (int64_t)batch << (3 * d);
       OCNN_REQUIRE(h_nnum[d] == total, "neigh_all: layer %d is not full", d);

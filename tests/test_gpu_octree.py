@@ -593,3 +593,47 @@ def test_random_merge_equals_batched_build():
         assert np.array_equal(np_(merged.neighs[d]), np_(whole.neighs[d])), d
     for name in ('points', 'normals', 'features'):
       assert np.array_equal(np_(getattr(merged, name)[depth]), np_(getattr(whole, name)[depth])), name
+
+
+def test_octree_with_a_table_of_more_than_a_billion_entries():
+  """8 x 1.1 M points at depth 11: 50 M nodes in the deepest layer, 1.35 G table entries (the
+  library takes tables of up to 2^31).  Too large for the oracle; what must hold of any octree
+  holds: keys sorted and unique per layer, eight children per non-empty parent, children
+  numbered in order, the centre slot of every row is the row, central symmetry of the tables
+  (the first and last 100 000 rows and 400 000 random ones per layer), and every point's leaf
+  carries the point's key."""
+  from ocnn_amd import synthetic
+  depth = 11
+  pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 8, 77, n=1100000)
+  o = Octree(depth, 2, batch_size=8)
+  idx = o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=8))
+  o.construct_all_neigh()
+  say('large octree: nodes per layer', o.nnum.tolist())
+  assert int(o.nnum[depth]) * 27 > 1 << 30
+  g = torch.Generator(device=DEV).manual_seed(3)
+  for d in range(3, depth + 1):
+    k = o.keys[d]
+    assert bool((k[1:] > k[:-1]).all())
+    assert int(o.nnum[d]) == 8 * int(o.nnum_nempty[d - 1])
+    c = o.children[d]
+    assert torch.equal(c[c >= 0].long(), torch.arange(int(o.nnum_nempty[d]), device=DEV))
+    t = o._table(d, '333', 1, False)
+    rows = t.shape[0]
+    assert torch.equal(t[:, 13], torch.arange(rows, device=DEV, dtype=torch.int32))
+    sel = torch.cat([torch.arange(0, min(rows, 100000), device=DEV), torch.arange(max(0, rows - 100000), rows, device=DEV),
+                     torch.randint(0, rows, (400000,), device=DEV, generator=g)])
+    ts = t[sel].long()
+    at, slot = torch.nonzero(ts >= 0, as_tuple=True)
+    assert torch.equal(t[ts[at, slot], 26 - slot].long(), sel[at]), d
+    assert torch.equal(k >> 3 & ((1 << 45) - 1),
+                       (o.keys[d - 1][o.nempty_index(d - 1)] & ((1 << 48) - 1)).repeat_interleave(8))
+  leaf_key = o.keys[depth][o.nempty_index(depth)]
+  p = (pts.to(DEV) + 1.0) * float(2 ** (depth - 1))
+  assert torch.equal(leaf_key[idx], xyz2key(p[:, 0], p[:, 1], p[:, 2], bid.to(DEV).view(-1), depth))
+  # one layer further the table would pass 2^31 entries: refused, not truncated
+  big = Octree(depth + 1, 2, batch_size=8)
+  big.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=8))
+  if int(big.nnum[depth + 1]) * 27 >= 1 << 31:
+    with pytest.raises(Exception):
+      big.construct_all_neigh()
+
