@@ -381,3 +381,92 @@ def test_layers_give_the_same_bits_on_every_run():
               name, kind, ks, stride, ne, cin, cout, run, bad.numel(), bad[:8].tolist()))
     say('   %s %s stride %d nempty %s %d -> %d depth %d: %d rows in, same bits 4 times' % (kind, ks, stride, ne, cin, cout, depth, n_in))
 
+
+def test_the_ops_around_the_convolutions_on_more_than_2_31_elements():
+  """Batch norm + ReLU (training mode, forward and backward), pad / depad, max pooling and the
+  depth-wise convolution on the deepest layer of an octree of 8 x 1.1 M points at depth 11:
+  49.9 M nodes x 64 channels = 3.2 G elements per tensor, where a 32-bit element index wraps.
+  Against fp64 torch on the first, the last and random rows (and the rows around element
+  2^31 and 2^32)."""
+  from ocnn_amd.nn import BatchNormRelu1d, octree_pad, octree_depad, octree_max_pool
+  say('ops on tensors of more than 2^31 elements')
+  o, _, _, _, _ = build(synthetic.mixed_cloud, 8, 77, 1100000, 11)
+  d, C = 11, 64
+  n_all, n_ne = int(o.nnum[d]), int(o.nnum_nempty[d])
+  assert n_all * C > 1 << 31
+  g = torch.Generator(device=DEV).manual_seed(1)
+  piece = 1 << 22
+  sel = torch.cat([torch.arange(0, 1000, device=DEV), torch.arange(n_all - 1000, n_all, device=DEV),
+                   torch.arange((1 << 31) // C - 500, (1 << 31) // C + 500, device=DEV),
+                   torch.arange((1 << 32) // C - 500, (1 << 32) // C + 500, device=DEV).clamp_(max=n_all - 1),
+                   torch.randint(0, n_all, (5000,), device=DEV, generator=g)])
+
+  def close(got, want, tol=2e-2):
+    err = float((got.double() - want).abs().max() / want.abs().max())
+    assert err < tol, err
+    return err
+
+  # ---- batch norm + ReLU ----
+  x = torch.randn(n_all, C, device=DEV, generator=g).bfloat16().requires_grad_()
+  gy = torch.randn(n_all, C, device=DEV, generator=g).bfloat16()
+  bn = BatchNormRelu1d(C, relu=True).to(DEV).bfloat16()
+  with torch.no_grad():
+    bn.weight.copy_(torch.rand(C, device=DEV, generator=g) + 0.5)
+    bn.bias.copy_(torch.randn(C, device=DEV, generator=g) * 0.1)
+  y = bn(x)
+  y.backward(gy)
+  xd = x.detach()
+  mean = torch.zeros(C, device=DEV, dtype=torch.float64)
+  sq = torch.zeros(C, device=DEV, dtype=torch.float64)
+  for r0 in range(0, n_all, piece):
+    xx = xd[r0:r0 + piece].double()
+    mean += xx.sum(0)
+    sq += (xx * xx).sum(0)
+  mean /= n_all
+  inv = 1.0 / torch.sqrt(sq / n_all - mean * mean + bn.eps)
+  scale = bn.weight.detach().double() * inv
+  shift = bn.bias.detach().double() - mean * scale
+  e_fwd = close(y.detach()[sel], torch.relu(xd[sel].double() * scale + shift))
+  s1 = torch.zeros(C, device=DEV, dtype=torch.float64)
+  s2 = torch.zeros(C, device=DEV, dtype=torch.float64)
+  for r0 in range(0, n_all, piece):
+    xx = xd[r0:r0 + piece].double()
+    gg = gy[r0:r0 + piece].double() * ((xx * scale + shift) > 0)
+    s1 += gg.sum(0)
+    s2 += (gg * (xx - mean) * inv).sum(0)
+  xx = xd[sel].double()
+  gg = gy[sel].double() * ((xx * scale + shift) > 0)
+  e_bwd = close(x.grad[sel], scale * (gg - s1 / n_all - (xx - mean) * inv * s2 / n_all))
+  close(bn.weight.grad, s2)
+  close(bn.bias.grad, s1)
+  say('   batch norm + ReLU, %d x %d: forward %.1e, backward %.1e' % (n_all, C, e_fwd, e_bwd))
+  del x, y, gy, bn, xd
+  torch.cuda.empty_cache()
+
+  # ---- pad / depad, max pooling ----
+  xn = torch.randn(n_ne, C, device=DEV, generator=g).bfloat16()
+  p = octree_pad(xn, o, d)
+  assert p.shape[0] == n_all and torch.equal(p[o.nempty_index(d)], xn) and torch.equal(octree_depad(p, o, d), xn)
+  assert int(torch.count_nonzero(p)) == int(torch.count_nonzero(xn))                               # zeros elsewhere
+  del p, xn
+  xa = torch.randn(n_all, C, device=DEV, generator=g).bfloat16()
+  pooled = octree_max_pool(xa, o, d, nempty=False)
+  assert torch.equal(octree_depad(pooled, o, d - 1), xa.view(-1, 8, C).max(1).values)
+  del xa, pooled
+  torch.cuda.empty_cache()
+
+  # ---- depth-wise convolution on the non-empty nodes ----
+  dw = OctreeDWConv(C, [3], 1, nempty=True).to(DEV).bfloat16()
+  xd = torch.randn(n_ne, C, device=DEV, generator=g).bfloat16()
+  out = dw(xd, o, d)
+  t = o._table(d, '333', 1, True)
+  rows = torch.cat([torch.arange(0, 1000, device=DEV), torch.arange(n_ne - 1000, n_ne, device=DEV),
+                    torch.randint(0, n_ne, (3000,), device=DEV, generator=g)])
+  ts = t[rows].long()
+  w = dw.weights.detach().double().view(27, C)
+  want = torch.zeros(rows.numel(), C, dtype=torch.float64, device=DEV)
+  for k in range(27):
+    v = ts[:, k] >= 0
+    want[v] += xd[ts[v, k]].double() * w[k]
+  say('   depth-wise convolution on %d rows: %.1e' % (n_ne, close(out.detach()[rows], want)))
+
