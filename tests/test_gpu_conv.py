@@ -1494,6 +1494,60 @@ def test_random_shapes_through_the_dispatch(first):
     assert rel_err(ocnn_amd.nn.conv_wgrad(xd, gd, td, True, plan).transpose(1, 2), want) < TOL[dtype]
 
 
+def test_random_large_tables_planned_against_plan_free():
+  """Large random tables (80 k .. 1.5 M rows, 3 .. 27 slots, 32 .. 256 channels, 5 % .. 100 % of the
+  entries set, narrow to wide neighbourhoods): the kernels the selection takes with a plan
+  against the plan-free kernels on EVERY row of output and mirrored gather, on the weight
+  gradient, and (64-channel multiples) on the depth-wise pair.  No oracle at these sizes: the
+  plan-free kernels are held to it elsewhere; this is about row ranges, tails and tile counts
+  per workgroup that small tables do not reach.  3 x OCNN_TEST_CASES cases (default 120) from
+  OCNN_TEST_FIRST on."""
+  from ocnn_amd.nn.octree_dwconv import dw_gather, dw_wgrad
+  from ocnn_amd.octree.octree import TilePlan
+  chans = [32, 64, 96, 128, 160, 192, 256]
+  cases = random_cases(40)
+  for case in range(3 * cases.start, 3 * cases.stop):
+    rng = np.random.default_rng(case)
+    g = torch.Generator(device=DEV).manual_seed(case)
+    dtype = [torch.float16, torch.bfloat16][case % 2]
+    K = int(rng.choice([3, 8, 9, 27, 27, 27]))
+    cin = int(rng.choice(chans))
+    cout = cin if rng.random() < 0.6 else int(rng.choice(chans))
+    rows = int(rng.integers(80_000, 1_500_000))
+    rows_in = rows if rng.random() < 0.6 else int(rng.integers(40_000, 1_500_000))
+    p = float(rng.choice([0.05, 0.1, 0.15, 0.25, 0.35, 0.6, 1.0]))
+    spread = int(rng.choice([3, 10, 40, 150]))
+    base = (torch.arange(rows, device=DEV, dtype=torch.float64) * (rows_in / rows)).long().view(-1, 1)
+    t = (base + torch.randint(-spread, spread + 1, (rows, K), device=DEV, generator=g)).clamp_(0, rows_in - 1).to(torch.int32)
+    t[torch.rand(rows, K, device=DEV, generator=g) >= p] = -1
+    plan = TilePlan(t)
+    x = torch.randn(rows_in, cin, device=DEV, generator=g).to(dtype)
+    w = (torch.randn(K, cin, cout, device=DEV, generator=g) / (K * cin * p) ** 0.5).to(dtype)
+    gr = torch.randn(rows, cout, device=DEV, generator=g).to(dtype)
+    tag = 'large random table %d: %s K %d %d -> %d rows %d rows_in %d set %.2f spread %d, %d distinct rows a tile at most' % (
+        case, str(dtype)[6:], K, cin, cout, rows, rows_in, p, spread, plan.umax)
+    say(tag)
+
+    def close(name, got, want):
+      got, want = got.float(), want.float()
+      scale = float(want.abs().max()) + 1e-30
+      d = (got - want).abs().reshape(got.shape[0], -1).amax(1)
+      wrong = (d > 2e-2 * scale).nonzero().view(-1)
+      assert wrong.numel() == 0, (tag, name, wrong.numel(), wrong[:8].tolist(), float(d.max()) / scale)
+
+    close('gather', ocnn_amd.nn.conv_gather(x, rows_in, t, w, cout, False, False, None, plan),
+          ocnn_amd.nn.conv_gather(x, rows_in, t, w, cout, False, False, None, None))
+    if rows_in == rows:
+      close('mirrored gather', ocnn_amd.nn.conv_gather(gr, rows, t, w, cin, True, True, None, plan),
+            ocnn_amd.nn.conv_gather(gr, rows, t, w, cin, True, True, None, None))
+    close('weight gradient', ocnn_amd.nn.conv_wgrad(x, gr, t, False, plan), ocnn_amd.nn.conv_wgrad(x, gr, t, False, None))
+    if cin == cout and cin % 64 == 0 and case % 3 == 0:
+      wd = torch.randn(K, 1, cin, device=DEV, generator=g).to(dtype)
+      close('depth-wise gather', dw_gather(x, rows_in, t, wd, False, None, plan), dw_gather(x, rows_in, t, wd, False, None, None))
+      close('depth-wise weight gradient', dw_wgrad(x, gr, t, plan), dw_wgrad(x, gr, t, None))
+    del x, w, gr, t, plan, base
+
+
 def test_random_layers_vs_oracle():
   """Random module configurations (conv / deconv / depth-wise, all eight kernel shapes, both
   strides, all or non-empty nodes, channel counts incl. 4 / 10 / 16 / 48, f16 / bf16 / fp32, with
