@@ -1548,6 +1548,56 @@ def test_random_large_tables_planned_against_plan_free():
     del x, w, gr, t, plan, base
 
 
+def test_random_sizes_of_the_dense_kernels_against_torch():
+  """The persistent one-slot kernels (the form of the 2x2x2 stride-2 layers) on random row
+  counts up to 2 M, operands read and results written through a row index, against torch's
+  matmul in fp32 on every row.  OCNN_TEST_CASES cases (default 40) from OCNN_TEST_FIRST on."""
+  L = _lib.lib()
+  for case in random_cases(40):
+    rng = np.random.default_rng(case)
+    g = torch.Generator(device=DEV).manual_seed(case)
+    dtype = [torch.float16, torch.bfloat16][case % 2]
+    code = _lib.dtype_code(torch.zeros(1, dtype=dtype))
+    cin, cout = int(rng.choice([64, 128, 256, 512])), int(rng.choice([128, 256, 384, 512]))
+    rows = int(rng.integers(1000, 2_000_000)) if rng.random() < 0.8 else int(rng.integers(1, 3000))
+    n_all = rows + int(rng.integers(0, rows + 10))
+    say('dense kernels, random sizes', case, dtype, cin, cout, 'rows', rows, 'of', n_all)
+    x_all = torch.randn(n_all, cin, device=DEV, generator=g).to(dtype)
+    gr_all = torch.randn(n_all, cout, device=DEV, generator=g).to(dtype)
+    idx = torch.sort(torch.randperm(n_all, device=DEV, generator=g)[:rows]).values.to(torch.int32)
+    w = (torch.randn(cin, cout, device=DEV, generator=g) / cin ** 0.5).to(dtype)
+    b = torch.randn(cout, device=DEV, generator=g).to(dtype)
+    xc = x_all[:rows].contiguous()
+
+    def close(name, got, want):
+      got, want = got.float(), want.float()
+      scale = float(want.abs().max()) + 1e-30
+      d = (got - want).abs().reshape(got.shape[0], -1).amax(1)
+      wrong = (d > 2e-2 * scale).nonzero().view(-1)
+      assert wrong.numel() == 0, (case, name, wrong.numel(), wrong[:8].tolist(), float(d.max()) / scale)
+
+    if L.ocnn_conv_dense_rw_supported(code, n_all, cin, cout):
+      ws = torch.empty(cin * cout * 2, dtype=torch.uint8, device=DEV)
+      out = torch.empty(rows, cout, dtype=dtype, device=DEV)
+      _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(x_all), n_all, _lib.ptr(idx), rows, _lib.ptr(w), cin, cout, 0,
+                                              _lib.ptr(b), _lib.ptr(out), rows, None, _lib.ptr(ws), ws.numel(), _lib.stream()))
+      close('rows read through an index', out, x_all[idx.long()].float() @ w.float() + b.float())
+      out = torch.zeros(n_all, cout, dtype=dtype, device=DEV)
+      _lib.check(L.ocnn_conv_dense_rw_indexed(code, _lib.ptr(xc), rows, None, rows, _lib.ptr(w), cin, cout, 0,
+                                              _lib.ptr(b), _lib.ptr(out), n_all, _lib.ptr(idx), _lib.ptr(ws), ws.numel(),
+                                              _lib.stream()))
+      want = torch.zeros(n_all, cout, device=DEV)
+      want[idx.long()] = xc.float() @ w.float() + b.float()
+      close('rows written through an index', out, want)
+    if L.ocnn_conv_dense_wgrad_rw_supported(code, n_all, cin, cout):
+      ws = torch.empty(L.ocnn_conv_dense_wgrad_rw_workspace_bytes(cin, cout), dtype=torch.uint8, device=DEV)
+      gw = torch.empty(cin, cout, dtype=dtype, device=DEV)
+      _lib.check(L.ocnn_conv_dense_wgrad_rw_indexed(code, _lib.ptr(xc), rows, None, _lib.ptr(gr_all), n_all, _lib.ptr(idx), rows,
+                                                    cin, cout, 0, _lib.ptr(gw), _lib.ptr(ws), ws.numel(), _lib.stream()))
+      close('weight gradient, g through an index', gw, xc.float().T @ gr_all[idx.long()].float())
+    del x_all, gr_all, idx, xc
+
+
 def test_random_layers_vs_oracle():
   """Random module configurations (conv / deconv / depth-wise, all eight kernel shapes, both
   strides, all or non-empty nodes, channel counts incl. 4 / 10 / 16 / 48, f16 / bf16 / fp32, with
