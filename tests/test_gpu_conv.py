@@ -1218,8 +1218,7 @@ def test_other_planned_kernels_on_many_tile_counts():
           ocnn_amd.nn.conv_wgrad(x, gr, sparse, False, None), per)
 
 
-@pytest.mark.parametrize('ch,empty,kernel', [(64, 0.3, 'GATHER_RW'), (32, 0.3, 'GATHER_RW'), (128, 0.3, 'GATHER_WIDE'),
-                                             (96, 0.85, 'GATHER_SPARSE')])
+@pytest.mark.parametrize('ch,empty,kernel', [(64, 0.3, 'GATHER_RW'), (128, 0.3, 'GATHER_WIDE'), (96, 0.85, 'GATHER_SPARSE')])
 def test_tables_at_the_end_of_32_bit_offsets(ch, empty, kernel):
   """The kernels on the plan address their tensors with 32-bit byte offsets.  A table just
   under that range runs on them (the selection says so), one just over it on another
