@@ -35,6 +35,38 @@ SPARSE_MAX_OCCUPANCY = 0.3
 SPARSE_MIN_ROWS = 32768
 
 
+# Stride 2 over all nodes, seen from the coarse side.  Row q of such a table is the first child
+# of the non-empty coarse node q with its neighbours at the fine offsets delta in {-1, 0, 1}^3
+# (ocnn/octree/octree.py:502-506).  The fine node at child c (bits x y z) of the coarse node q'
+# is therefore named by the coarse nodes q = q' + e, e in {0, 1}^3 with e <= c per axis, in slot
+# delta = c - 2 e: the data gradient of the fine rows, (parents, 8 children x channels) since
+# the children of a non-empty node are eight consecutive rows, is a 2x2x2 stride-1 gather over the
+# NON-EMPTY COARSE nodes (slots e, the octree's own '222' table) with block weights
+# Wb[e][:, c] = W[slot(c - 2 e)]^T, zero where e > c.  That gather issues 8 x 8 blocks of
+# matrix work per coarse row, of which 27 are real, where the gather over the inverse table
+# (fine rows x all slots of the kernel) issues 8 x 27 for 27.
+_BLOCK_MAPS = {}
+
+
+def _block_map(kernel, device):
+  """(index (64,), mask (8, 8, 1, 1)): the kernel's slot for (e, c), e and c as 4 x + 2 y + z."""
+  key = (kernel, str(device))
+  if key not in _BLOCK_MAPS:
+    from ..octree.octree import LUT_KERNEL
+    slots = list(range(27)) if kernel == '333' else LUT_KERNEL[kernel]
+    m = torch.full((8, 8), -1, dtype=torch.long)
+    for e in range(8):
+      for c in range(8):
+        d = [((c >> a) & 1) - 2 * ((e >> a) & 1) for a in (2, 1, 0)]
+        k27 = 9 * (d[0] + 1) + 3 * (d[1] + 1) + (d[2] + 1)
+        if min(d) >= -1 and k27 in slots:
+          m[e, c] = slots.index(k27)
+    m = m.to(device)
+    _BLOCK_MAPS[key] = (m.clamp_min(0).view(-1), (m >= 0).view(8, 8, 1, 1))
+  return _BLOCK_MAPS[key]
+
+
+
 def conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias=None, plan=None, dense=False,
                 in_index=None, pad_to=None):
   """out (rows, cout) = gather-GEMM over `table` (int32, (rows, K)).  With a
@@ -327,6 +359,10 @@ class OctreeConvBase:
     # so the layer is a dense GEMM on the (P, 8 * C) view of the fine side: no gather at all
     self.dense_children = (self.kernel == '222' and self.stride == 2 and not self.nempty and
                            self.fine_h == 8 * self.neigh.shape[0])
+    # the other kernels at stride 2 over all nodes: the data gradient in block form (_block_map)
+    self.coarse_depth = self.out_depth if self.is_conv_layer() else self.in_depth
+    self.block_children = (self.kernel != '222' and self.stride == 2 and not self.nempty and
+                           self.fine_h == 8 * self.neigh.shape[0])
 
   def check_and_init(self, data: torch.Tensor):
     check = tuple(data.shape) == self.in_shape
@@ -400,6 +436,10 @@ class OctreeConvBase:
       return out.view(8 * P, self.in_conv)
     if coarse_index is not None:
       grad = grad.index_select(0, coarse_index.long())
+    if self.block_children:
+      out = self._backward_blocks(grad, weights, bias)
+      if out is not None:
+        return out
     if self.symmetric:
       plan = self._plan(grad, self.out_conv, self.in_conv)
       return conv_gather(grad, grad.shape[0], self.neigh, weights, self.in_conv, True, True, bias,
@@ -407,6 +447,52 @@ class OctreeConvBase:
     plan = self._plan(grad, self.out_conv, self.in_conv, inverse=True)
     return conv_gather(grad, grad.shape[0], self._inverse_table(), weights, self.in_conv, True,
                        False, bias, plan)
+
+  def _backward_blocks(self, grad, weights, bias):
+    """backward_gemm of a stride-2 layer over all nodes as a 2x2x2 stride-1 gather over the
+    non-empty coarse nodes into the (parents, 8 x in_conv) view of the fine rows (_block_map).
+    None where the kernels for wide layers do not take the shape (the caller then goes over
+    the inverse table)."""
+    L, code = _lib.lib(), _lib.DTYPE_CODE.get(grad.dtype, -1)
+    P, wide = self.neigh.shape[0], 8 * self.in_conv
+    octree = self.octree
+    plan = octree._plan(self.coarse_depth, '222', 1, True)
+    if L.ocnn_conv_gather_choose(code, P, P, 8, self.out_conv, wide, 0, *_plan_args(plan)) != _lib.GATHER_WIDE:
+      return None
+    index, valid = _block_map(self.kernel, grad.device)
+    blocks = weights.view(self.kdim, self.in_conv, self.out_conv).index_select(0, index)
+    blocks = blocks.view(8, 8, self.in_conv, self.out_conv) * valid.to(weights.dtype)          # e, c, in, out
+    blocks = blocks.permute(0, 3, 1, 2).reshape(8, self.out_conv, wide)                        # e, out, (c, in)
+    out = conv_gather(grad, P, octree._table(self.coarse_depth, '222', 1, True), blocks, wide, False, False,
+                      None if bias is None else bias.repeat(8), plan)
+    return out.view(8 * P, self.in_conv)
+
+  def _weight_blocks(self, data, grad, out_transposed):
+    """weight_gemm of a stride-2 layer over all nodes on the planned kernel: the fine rows as
+    (parents, 8 x in_conv), the table of the eight coarse nodes whose children a row's slots
+    reach (offsets {-1, 0}^3: slot delta of coarse node q reads child c = delta mod 2 of the node
+    at e = floor(delta / 2)), sums (8, 8 x in_conv, out_conv) of which the kernel's slots are 27
+    blocks at most.  None where the planned kernel does not take the shape."""
+    L, code = _lib.lib(), _lib.DTYPE_CODE.get(data.dtype, -1)
+    P, wide = self.neigh.shape[0], 8 * self.in_conv
+    octree = self.octree
+    plan = octree._plan(self.coarse_depth, '222m', 1, True)
+    if L.ocnn_conv_wgrad_choose(code, P, P, 8, wide, self.out_conv, 0, *_plan_args(plan)[:4]) != _lib.WGRAD_PLANNED:
+      return None
+    sums = conv_wgrad(data.view(P, wide), grad, octree._table(self.coarse_depth, '222m', 1, True), False, plan)
+    key = ('w', self.kernel, str(data.device))
+    if key not in _BLOCK_MAPS:
+      from ..octree.octree import LUT_KERNEL
+      slots = list(range(27)) if self.kernel == '333' else LUT_KERNEL[self.kernel]
+      e, c = [], []
+      for k27 in slots:
+        d = [k27 // 9 - 1, (k27 // 3) % 3 - 1, k27 % 3 - 1]
+        e.append(sum((0 if v == -1 else 1) << (2 - a) for a, v in enumerate(d)))      # '222m' slot: offsets -1 -> 0, 0 -> 1
+        c.append(sum((v & 1) << (2 - a) for a, v in enumerate(d)))                    # child bit: 1 for delta = +-1
+      _BLOCK_MAPS[key] = (torch.tensor(e, device=data.device), torch.tensor(c, device=data.device))
+    e, c = _BLOCK_MAPS[key]
+    gw = sums.view(8, 8, self.in_conv, self.out_conv)[e, c]                             # (K, in_conv, out_conv)
+    return gw.transpose(1, 2).contiguous() if out_transposed else gw
 
   def weight_gemm(self, data, grad, out_transposed=False, coarse_index=None):
     """data: fine rows; grad: table rows -> (K, in_conv, out_conv).  coarse_index: as in
@@ -418,6 +504,10 @@ class OctreeConvBase:
       return gw.transpose(1, 2).contiguous() if out_transposed else gw
     if coarse_index is not None:
       grad = grad.index_select(0, coarse_index.long())
+    if self.block_children and self.kernel == '333':      # (8 x 8 blocks issued: a loss for 3 or 9 slots)
+      gw = self._weight_blocks(data, grad, out_transposed)
+      if gw is not None:
+        return gw
     # (3x3x3 over all nodes: 20 of the 27 slots of a table row are set, and the plan-free kernel
     # over the table is faster than the pairs of the inverse)
     if self.stride == 2 and (self.kernel == '222' or (self.kernel == '333' and self.nempty)) and \

@@ -19,7 +19,7 @@ import weakref
 import torch
 
 from .. import _lib
-from .octree import Octree, PlanHistory
+from .octree import LUT_INTERNAL, Octree, PlanHistory
 
 _ADAPTERS = weakref.WeakKeyDictionary()
 _ATTR = '_ocnn_amd_contract'
@@ -118,6 +118,10 @@ class ContractOctree:
     self._check(depth)
     ck = (depth, kernel, stride, bool(nempty))
     if ck not in self._tables:
+      if kernel in LUT_INTERNAL:          # (not a kernel of the contract: columns of its 3x3x3 table)
+        cols = torch.tensor(LUT_INTERNAL[kernel], device=self._table(depth, '333', stride, nempty).device)
+        self._tables[ck] = self._table(depth, '333', stride, nempty).index_select(1, cols).contiguous()
+        return self._tables[ck]
       t = self._o.get_neigh(depth, kernel, stride, nempty)
       _lib.require_gpu(t)
       t = t.contiguous()

@@ -32,6 +32,11 @@ LUT_KERNEL = {
     '313': [3, 4, 5, 12, 13, 14, 21, 22, 23],
     '133': [9, 10, 11, 12, 13, 14, 15, 16, 17],
 }
+# tables the layers ask for on top of the reference's kernels: '222m', the mirror image of '222'
+# (offsets {-1, 0}^3: where the fine neighbours of a first child live, seen from the coarse side)
+LUT_INTERNAL = {
+    '222m': [0, 1, 3, 4, 9, 10, 12, 13],
+}
 
 
 class _NeighTables:
@@ -697,7 +702,7 @@ class Octree:
     """int32 table of get_neigh(depth, kernel, stride, nempty), cached."""
     if stride not in (1, 2):
       raise ValueError('Unsupported stride {}'.format(stride))
-    if kernel != '333' and kernel not in LUT_KERNEL:
+    if kernel != '333' and kernel not in LUT_KERNEL and kernel not in LUT_INTERNAL:
       raise ValueError('Unsupported kernel {}'.format(kernel))
     ck = (depth, kernel, stride, bool(nempty))
     if ck in self._tables:
@@ -708,7 +713,7 @@ class Octree:
       self._tables[ck] = base
       return base
     _lib.require_gpu(base)
-    cols = LUT_KERNEL.get(kernel)
+    cols = LUT_KERNEL.get(kernel, LUT_INTERNAL.get(kernel))
     K = 27 if cols is None else len(cols)
     h_cols = None if cols is None else (ctypes.c_int * K)(*cols)
     row_index, row_stride, rows = None, 1, base.shape[0]

@@ -1279,6 +1279,49 @@ def test_tables_at_the_end_of_32_bit_offsets(ch, empty, kernel):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize('kernel', ['333', '331', '313', '133', '311', '131', '113'])
+def test_stride2_data_gradient_in_block_form(medium, kernel):
+  """backward_gemm of the stride-2 layers over all nodes as a 2x2x2 stride-1 gather over the
+  non-empty coarse nodes with block weights: the path is taken (64 and 96 channels, f16 and bf16,
+  with and without bias) and gives the oracle's scatter over the layer's own table, rows of all
+  fine nodes; fp32 and 32 output channels take the inverse table and give the same.  Likewise
+  the weight gradient on the planned kernel over the mirror image of that table."""
+  import importlib
+  OC = importlib.import_module('ocnn_amd.nn.octree_conv')
+  o, ref, depth = medium.gpu, medium.ref, 7
+  ks = [int(c) for c in kernel]
+  g = torch.Generator().manual_seed(17)
+  table = ref.get_neigh(depth, kernel, 2, False).astype(np.int64)
+  P, fine = table.shape[0], int(ref.nnum[depth])
+  assert fine == 8 * P
+  for cin, cout, dtype, blocks in ((64, 64, torch.bfloat16, True), (96, 64, torch.float16, True), (32, 128, torch.bfloat16, True),
+                                   (64, 32, torch.bfloat16, False), (64, 64, torch.float32, False)):
+    eng = OC._OctreeConv(cin, cout, ks, 2, False, int(2e8))
+    eng.setup(o, depth)
+    assert eng.block_children and eng.coarse_depth == depth - 1
+    grad = torch.randn(P, cout, generator=g).to(dtype)
+    w = (torch.randn(len(table[0]), cin, cout, generator=g) / (len(table[0]) * cout) ** 0.5).to(dtype)
+    b = torch.randn(cin, generator=g).to(dtype)
+    want = C.backward_gemm(f64(grad), f64(w), table, fine)
+    say('stride-2 data gradient', kernel, cin, cout, dtype, 'block form' if blocks else 'inverse table')
+    got = eng._backward_blocks(grad.to(DEV), w.to(DEV), None)
+    assert (got is not None) == blocks
+    tol = 1e-4 if dtype == torch.float32 else TOL[dtype]
+    if blocks:
+      assert got.shape == (fine, cin) and rel_err(got, want) < tol
+      assert rel_err(eng._backward_blocks(grad.to(DEV), w.to(DEV), b.to(DEV)), want + f64(b)) < tol
+    assert rel_err(eng.backward_gemm(grad.to(DEV), w.to(DEV)), want) < tol
+    # the weight gradient on the planned kernel over the mirror table, or as before
+    x = torch.randn(fine, cin, generator=g).to(dtype)
+    want = C.weight_gemm(f64(x), f64(grad), table)
+    gw = eng._weight_blocks(x.to(DEV), grad.to(DEV), False)
+    assert (gw is not None) == (cout >= 64), (cin, cout, dtype)       # (fp32: as bf16 pieces on the same kernel)
+    if gw is not None:
+      assert gw.shape == want.shape and rel_err(gw, want) < tol
+      assert torch.equal(eng._weight_blocks(x.to(DEV), grad.to(DEV), True), gw.transpose(1, 2).contiguous())
+    assert rel_err(eng.weight_gemm(x.to(DEV), grad.to(DEV)), want) < tol
+
+
 def test_planned_kernels_non_finite_rows():
   """Rows past the end of the table and empty entries must not pick up values of
   staged rows: NaN / Inf rows that no valid entry refers to stay out of the result."""
