@@ -38,6 +38,11 @@ extern "C" int ocnn_conv_gather_choose(int dtype, int64_t rows_in, int64_t rows_
     if (ocnn_conv_gather_rw_supported(dtype, rows_in, K, cin, cout, plan_max_distinct) &&
         rows_out * K * 2 < kOffsetLimit && (rows_out + 128) * cout * 2 < kOffsetLimit)
       return OCNN_GATHER_RW;
+    // (eight slots - the 2x2x2 tables and their inverses - stream a third of the weights of 27 per
+    // tile: there the kernel for wide layers beats the pair plan also at one slot in eight set,
+    // 0.84 -> 0.67 ms for 96 -> 96 between depths 9 and 8, and without rows shared inside a tile)
+    if (K == 8 && ocnn_conv_gather_wide_supported(dtype, rows_in, K, cin, cout, plan_max_distinct))
+      return OCNN_GATHER_WIDE;
     if (plan_occupancy <= kSparseMaxOccupancy && rows_out >= kSparseMinRows &&
         rows_out * cout * 2 <= kOffsetLimit &&
         ocnn_conv_gather_sparse_supported(dtype, rows_in, K, cin, cout, plan_max_distinct))

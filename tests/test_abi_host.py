@@ -245,7 +245,7 @@ def test_kernel_selection_is_consistent_with_the_predicates():
               assert L.ocnn_conv_gather_sparse_supported(BF, rows, K, cin, cout, umax)
               assert rows * cout * 2 <= lim and occ <= 0.3 and rows >= 32768
             elif k == _lib.GATHER_WIDE:
-              assert L.ocnn_conv_gather_wide_supported(BF, rows, K, cin, cout, umax) and reuse >= 2
+              assert L.ocnn_conv_gather_wide_supported(BF, rows, K, cin, cout, umax) and (reuse >= 2 or K == 8)
             elif k == _lib.GATHER_PLANNED:
               assert L.ocnn_conv_gather_planned_supported(BF, rows, cin, cout) and reuse >= 2
             elif k == _lib.GATHER_ZERO_PADDED:
