@@ -437,7 +437,8 @@ def main():
       import bench_unet
       u = bench_unet.run(['--steps', '10', '--warmup', '5', '--fresh', '1'])
       result['configs4_unet'] = {k: u[k] for k in ('net', 'ms_per_step', 'ms_octree_build_and_tables',
-                                                   'ms_first_step_on_a_fresh_octree', 'dtype', 'nempty', 'batch',
+                                                   'ms_first_step_on_a_fresh_octree',
+                                                   'ms_per_step_new_octree_built_on_a_side_stream', 'dtype', 'nempty', 'batch',
                                                    'points', 'depth', 'parameters')}
     except Exception as e:                              # supporting figure only
       result['configs4_unet'] = {'error': repr(e)}

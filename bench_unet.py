@@ -9,7 +9,9 @@ walls and 10 - 20 boxes each; --scene mixed: 3 spheres and 2 boxes), input signa
 One JSON line: ms per forward + backward, and the share of the step spent in each kind of
 kernel when --profile is given (torch profiler, device time).  ms_per_step is the step on a
 resident octree; ms_octree_build_and_tables + ms_first_step_on_a_fresh_octree is what a step costs
-when every batch brings a new octree (the plans of its tables are built inside that step).
+when every batch brings a new octree (the plans of its tables are built inside that step);
+ms_per_step_new_octree_built_on_a_side_stream is the step of a loop that builds the next octree and
+its plans on a second stream while the device runs the step before (Octree.prepare).
 """
 
 import argparse
@@ -37,6 +39,9 @@ def run(argv=None):
   ap.add_argument('--nempty', type=int, default=1)
   ap.add_argument('--profile', action='store_true')
   ap.add_argument('--fresh', type=int, default=3, help='steps on a newly built octree, timed after the others')
+  ap.add_argument('--prefetch', type=int, default=6,
+                  help='steps that each run on a new octree built (with its plans) on a side stream while '
+                       'the step before is running')
   ap.add_argument('--scene', default='indoor', choices=['indoor', 'mixed'],
                   help='indoor: floor, walls and 10 - 20 boxes per cloud (the configuration\'s scene); '
                        'mixed: 3 spheres and 2 boxes')
@@ -102,8 +107,40 @@ def run(argv=None):
     fresh.append(((t1 - t0) * 1e3, (time.perf_counter() - t1) * 1e3))
   fresh.sort(key=lambda v: v[0] + v[1])
   mid = fresh[len(fresh) // 2] if fresh else (None, None)
+  # the same with the next octree built ahead: the host has queued the whole step long before the
+  # device is through with it, so the build of the next octree, on a stream of its own, runs
+  # beside the step's kernels (its read-backs wait for that stream only)
+  ms_prefetch = None
+  if args.prefetch > 0:
+    side, main = torch.cuda.Stream(), torch.cuda.current_stream()
+    torch.cuda.synchronize()                      # (the points are on the device by now: the side stream need not wait for main's queue)
+
+    def ahead():
+      with torch.cuda.stream(side):
+        o = build().prepare()
+        f = o.get_input_feature('ND', nempty).to(dtype)
+      return o, f
+
+    def prefetch_steps(n, nxt):
+      nonlocal feat
+      for _ in range(n):
+        main.wait_stream(side)
+        o, feat = nxt
+        o.record_stream(main)
+        feat.record_stream(main)
+        step(o)
+        nxt = ahead()
+      torch.cuda.synchronize()
+      return nxt
+
+    nxt = prefetch_steps(2, ahead())
+    t0 = time.perf_counter()
+    prefetch_steps(args.prefetch, nxt)
+    ms_prefetch = (time.perf_counter() - t0) / args.prefetch * 1e3
+    feat = octree.get_input_feature('ND', nempty).to(dtype)
   out = {'net': 'U-Net (ocnn/models/unet.py), forward + backward', 'ms_per_step': ms,
          'ms_octree_build_and_tables': mid[0], 'ms_first_step_on_a_fresh_octree': mid[1],
+         'ms_per_step_new_octree_built_on_a_side_stream': ms_prefetch,
          'dtype': args.dtype, 'scene': args.scene,
          'nempty': nempty, 'batch': args.batch, 'points': int(pts.shape[0]), 'depth': args.depth,
          'rows_per_depth': (octree.nnum_nempty if nempty else octree.nnum).tolist(),

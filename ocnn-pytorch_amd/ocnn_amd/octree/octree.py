@@ -770,6 +770,53 @@ class Octree:
           plan._on_pairs = lambda: history.note(kind, ck, pairs=True)
     return self._plans[ck]
 
+  def prepare(self):
+    """Builds now, together, the tables and plans that earlier octrees of the same (depth,
+    full_depth) were asked for (`plan_history`): what the first layer's request would otherwise
+    set off in the middle of a step.  A training loop calls it on a side stream while the step
+    before is still running,
+
+      with torch.cuda.stream(side):
+        nxt = Octree(...); nxt.build_octree(points); nxt.construct_all_neigh(); nxt.prepare()
+      ...
+      torch.cuda.current_stream().wait_stream(side)
+      nxt.record_stream(torch.cuda.current_stream())
+
+    so that a new octree every step costs the step nothing but the compute units its kernels
+    take.  (No counterpart in the reference, whose data loader builds octrees on the CPU in
+    worker processes: ocnn/dataset.py:61-67.)"""
+    requests = self.plan_history.requests((self.depth, self.full_depth))
+    if Octree.PREBUILD_PLANS and requests and not self._plans_prebuilt:
+      self._plans_prebuilt = True
+      self._prebuild_plans(requests)
+    return self
+
+  def record_stream(self, stream):
+    """Tells torch's allocator that `stream` uses every device tensor this octree holds now
+    (keys, children, tables, plans, leaf signals): for an octree built on another stream, so
+    that its memory is not handed out again on that stream while work queued on `stream`
+    still reads it."""
+    seen = set()
+
+    def walk(v):
+      if id(v) in seen:
+        return
+      seen.add(id(v))
+      if isinstance(v, torch.Tensor):
+        if v.is_cuda:
+          v.record_stream(stream)
+      elif isinstance(v, (list, tuple)):
+        for x in v:
+          walk(x)
+      elif isinstance(v, dict):
+        for x in v.values():
+          walk(x)
+      elif isinstance(v, (TilePlan, PairPlan, _NeighTables)):
+        walk(vars(v))
+
+    walk(vars(self))
+    return self
+
   def _fine_rows(self, depth, nempty):
     """Rows on the side of a table that its entries index (all tables of this class: the
     nodes of `depth`, or the non-empty ones)."""

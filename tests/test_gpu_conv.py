@@ -541,6 +541,53 @@ def test_fresh_octree_builds_the_plans_of_its_predecessors(medium):
     Octree.plan_history = saved
 
 
+def test_octree_prepared_on_a_side_stream():
+  say('plans: an octree built and prepared on a second stream while the first one works')
+  def fresh():
+    o = Octree(7, 2, batch_size=3)
+    pts, nrm, bid = synthetic.batch_clouds(synthetic.mixed_cloud, 3, 11, n=40000)
+    o.build_octree(Points(pts.to(DEV), nrm.to(DEV), batch_id=bid.to(DEV), batch_size=3))
+    o.construct_all_neigh()
+    return o
+  from ocnn_amd.octree.octree import PlanHistory
+  saved = Octree.plan_history
+  Octree.plan_history = PlanHistory()
+  try:
+    torch.manual_seed(3)
+    layers = [ocnn_amd.nn.OctreeConv(64, 64, [3], 1, nempty=True).to(DEV).bfloat16(),
+              ocnn_amd.nn.OctreeConv(64, 96, [2], 2, nempty=True).to(DEV).bfloat16(),
+              ocnn_amd.nn.OctreeDeconv(96, 64, [2], 2, nempty=True).to(DEV).bfloat16()]
+    def run(o, x):
+      x = x.clone().requires_grad_()
+      y = layers[0](x, o, 7)
+      z = layers[2](layers[1](y, o, 7), o, 6)
+      for l in layers:
+        l.weights.grad = None
+      (y + z).float().square().sum().backward()
+      return [z.detach().clone(), x.grad.clone()] + [l.weights.grad.clone() for l in layers]
+    first = fresh()
+    x = torch.randn(int(first.nnum_nempty[7]), 64, device=DEV).bfloat16()
+    want = run(first, x)
+    assert first.prepare() is first and len(first._plans) >= 3      # (nothing left to build)
+    side, main = torch.cuda.Stream(), torch.cuda.current_stream()
+    torch.cuda.synchronize()
+    for rep in range(3):
+      # main gets a queue of work; the next octree is built beside it
+      for _ in range(4):
+        run(first, x)
+      with torch.cuda.stream(side):
+        nxt = fresh().prepare()
+      assert set(nxt._plans) == set(first._plans)
+      main.wait_stream(side)
+      nxt.record_stream(main)
+      got = run(nxt, x)
+      del nxt
+      for a, b in zip(want, got):
+        assert torch.equal(a, b), rep
+  finally:
+    Octree.plan_history = saved
+
+
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 def test_staged_kernel_many_passes(dtype):
   """A table with no locality: tiles need far more distinct rows than fit in
