@@ -713,6 +713,11 @@ class Octree:
       self._tables[ck] = base
       return base
     _lib.require_gpu(base)
+    if kernel == '222' and stride == 2 and nempty and self.children[depth].numel() == base.shape[0]:
+      # the 2x2x2 window of a parent's first child is its eight children, and the non-empty
+      # numbering of node 8 p + c is children[8 p + c]: the table is a view of that array
+      self._tables[ck] = self.children[depth].view(-1, 8)
+      return self._tables[ck]
     cols = LUT_KERNEL.get(kernel, LUT_INTERNAL.get(kernel))
     K = 27 if cols is None else len(cols)
     h_cols = None if cols is None else (ctypes.c_int * K)(*cols)
