@@ -566,6 +566,7 @@ def test_octree_prepared_on_a_side_stream():
       (y + z).float().square().sum().backward()
       return [z.detach().clone(), x.grad.clone()] + [l.weights.grad.clone() for l in layers]
     first = fresh()
+    assert first.prepare() is first and not first._plans          # nothing asked for yet: nothing built
     x = torch.randn(int(first.nnum_nempty[7]), 64, device=DEV).bfloat16()
     want = run(first, x)
     assert first.prepare() is first and len(first._plans) >= 3      # (nothing left to build)
