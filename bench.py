@@ -436,10 +436,16 @@ def main():
     try:
       import bench_unet
       u = bench_unet.run(['--steps', '10', '--warmup', '5', '--fresh', '1'])
-      result['configs4_unet'] = {k: u[k] for k in ('net', 'ms_per_step', 'ms_octree_build_and_tables',
+      result['configs4_unet'] = {k: u[k] for k in ('net', 'scene', 'ms_per_step', 'ms_octree_build_and_tables',
                                                    'ms_first_step_on_a_fresh_octree',
                                                    'ms_per_step_new_octree_built_on_a_side_stream', 'dtype', 'nempty', 'batch',
-                                                   'points', 'depth', 'parameters')}
+                                                   'points', 'depth', 'rows_per_depth', 'parameters')}
+      result['configs4_unet']['scene_note'] = ('indoor: floor, walls and 10 - 20 boxes per cloud, the scene the '
+                                               'configuration names; earlier records of this benchmark ran it on '
+                                               'spheres and boxes, the figure below')
+      # the same net on the clouds of the earlier records (3 spheres + 2 boxes): fewer rows per level
+      v = bench_unet.run(['--steps', '10', '--warmup', '5', '--fresh', '0', '--prefetch', '0', '--scene', 'mixed'])
+      result['configs4_unet']['spheres_and_boxes'] = {k: v[k] for k in ('scene', 'ms_per_step', 'rows_per_depth')}
     except Exception as e:                              # supporting figure only
       result['configs4_unet'] = {'error': repr(e)}
 
