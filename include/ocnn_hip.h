@@ -331,14 +331,20 @@ int ocnn_conv_gather_rw_static(int dtype, const void* in, int64_t rows_in, const
  * channels at a time, the weights stream from L2 into registers in the MFMA operand
  * layout, the four waves of a workgroup split the output channels.  Same arguments and
  * result as ocnn_conv_gather_rw; plan_max_distinct <= 416; workspace K * cin64 * cout * 2 bytes
- * with cin64 = cin rounded up to a multiple of 64. */
+ * with cin64 = cin rounded up to a multiple of 64.  plan_occupancy: the share of the table's
+ * entries that are set (as for ocnn_conv_gather_choose), negative if unknown: from 40 % down
+ * (other than 2x2x2 tables) the kernel tests, per slot and 32-row block of a tile, whether any
+ * row has an entry there and leaves the block's products out otherwise: the rows of empty
+ * entries are zeros (as in the reference's buffer, ocnn/nn/octree_conv.py:133-137), so the
+ * result is the same. */
 int ocnn_conv_gather_wide_supported(int dtype, int64_t rows_in, int K, int cin, int cout,
                                     int plan_max_distinct);
 int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,
                           const int32_t* uptr, const int32_t* urows, int plan_max_distinct,
-                          int64_t plan_total, int64_t rows_out, int K, const void* w, int cin, int cout,
-                          int w_transposed, int reverse_slots, const void* bias, void* out,
-                          void* workspace, int64_t workspace_bytes, void* stream);
+                          int64_t plan_total, double plan_occupancy, int64_t rows_out, int K,
+                          const void* w, int cin, int cout, int w_transposed, int reverse_slots,
+                          const void* bias, void* out, void* workspace, int64_t workspace_bytes,
+                          void* stream);
 
 /* Pair plan of a table, on top of its tile plan (loc: tiles x K x ocnn_tile_plan_rows()):
  * what ocnn_conv_gather_sparse and ocnn_conv_wgrad_sparse walk over.  It holds, per tile and

@@ -73,7 +73,7 @@ SIGNATURES = {
     'ocnn_conv_gather_sparse_workspace_bytes': (_l, [_i, _i]),
     'ocnn_conv_gather_sparse': (_i, [_i, _p, _l, _p, _p, _i, _l, _p, _p, _l, _i, _p, _i, _p, _l, _i, _p, _i, _i, _i,
                                      _i, _p, _p, _p, _l, _p]),
-    'ocnn_conv_gather_wide': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _l, _i, _p, _i, _i, _i, _i, _p, _p,
+    'ocnn_conv_gather_wide': (_i, [_i, _p, _l, _p, _p, _p, _i, _l, _d, _l, _i, _p, _i, _i, _i, _i, _p, _p,
                                    _p, _l, _p]),
     'ocnn_conv_dense_supported': (_i, [_i, _l, _i, _i]),
     'ocnn_conv_dense': (_i, [_i, _p, _l, _p, _i, _i, _i, _p, _p, _p, _l, _p]),

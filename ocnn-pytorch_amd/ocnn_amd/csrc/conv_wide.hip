@@ -20,6 +20,10 @@ namespace ocnn {
 constexpr int kWdRows = 128;   // rows per tile (the plan's tile size)
 constexpr int kWdCap = 416;    // staged rows; plans with a larger tile use another kernel
 constexpr int kWdRowsAlloc = (kWdCap + 8) / 8 * 8;   // LDS rows 0..kWdCap in whole 8-row groups
+// share of a table's entries that are set up to which the kernel tests for empty (32-row block,
+// slot) units: at 32 - 38 % (the non-empty nodes of depths 7 and 6 of a depth-9 octree) a quarter
+// to a half of the units are empty and the launches are 3 - 14 % faster, at 41 - 50 % 0 - 7 % slower
+constexpr double kWdSkipMaxOccupancy = 0.40;
 
 // (Not in the kernel template: the arguments of the global->LDS load builtin must not be
 // type-dependent expressions.)
@@ -60,7 +64,13 @@ __global__ void pack_weights_wide_kernel(const T* __restrict__ w, T* __restrict_
 // the output channels 32 MB w .. of that block.  Channel counts are multiples of 32: the
 // last 64-channel chunk of the input may be half a chunk (its other half is staged as zeros
 // and meets zero weights), and waves whose output channels lie past the end idle.
-template <typename T, int MB>
+//
+// SKIP: per slot and 32-row block of the tile a wave asks whether any row has an entry there (a
+// ballot over the positions it reads anyway) and leaves the block's MFMAs out otherwise.  The
+// kernel is bound by the power its MFMAs draw (also those on zero rows), and the branches cost
+// 2 - 7 % where nothing is empty: it pays from about a quarter of the (block, slot) units empty -
+// the non-empty nodes of coarse levels -, which the launch decides from the table's occupancy.
+template <typename T, int MB, bool SKIP>
 __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
     const T* __restrict__ in, uint32_t in_bytes, const uint16_t* __restrict__ loc,
     const int32_t* __restrict__ uptr, const int32_t* __restrict__ urows, const T* __restrict__ wpk,
@@ -124,12 +134,15 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   const uint16_t* lcw = s_loc + r32;
   uint32_t pvc[4], pvn[4];
   u32x4 Bb[2][4];
-  auto load_pos = [&](int k, uint32_t (&pv)[4]) {
+  // (SKIP) which 32-row blocks of the tile have an entry in the slot at all, wave-uniform
+  bool nzc[4] = {true, true, true, true}, nzn[4] = {true, true, true, true};
+  auto load_pos = [&](int k, uint32_t (&pv)[4], bool (&nz)[4]) {
     const uint16_t* p = lcw + k * kWdRows;
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
       const uint32_t l = p[32 * rb];                         // 0 = empty = the zero row
       pv[rb] = (l << 7) | (((l << 3) & 0x70u) ^ ((uint32_t)q << 4));
+      if constexpr (SKIP) nz[rb] = __builtin_amdgcn_ballot_w64(l != 0u) != 0ull;
     }
   };
   auto read_b = [&](const uint32_t (&pv)[4], int s, u32x4 (&b)[4]) {
@@ -164,27 +177,32 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
   load_a(0, 1, A[1]);
   for (int cc = 0; cc < nfull; ++cc) {
     stage_chunk(cc);
-    load_pos(0, pvc);
+    load_pos(0, pvc, nzc);
     read_b(pvc, 0, Bb[0]);
     for (int k = 0; k < K; ++k) {
       const int kk = cc * K + k;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         // fetches: positions of the next slot, weights two k-steps ahead, rows one k-step ahead
-        if (s == 0) load_pos(k + 1 < K ? k + 1 : 0, pvn);
+        if (s == 0) load_pos(k + 1 < K ? k + 1 : 0, pvn, nzn);
         load_a(kk + (s >= 2 ? 1 : 0), (s + 2) & 3, A[(s + 2) & 3]);
         if (s < 3) read_b(pvc, s + 1, Bb[(s + 1) & 1]);
         else read_b(pvn, 0, Bb[0]);                          // (past the last slot: unused)
         if (active) {
 #pragma unroll
           for (int rb = 0; rb < 4; ++rb)
+            if (!SKIP || nzc[rb]) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[s][mb], Bb[s & 1][rb], acc[rb][mb]);
+              for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[s][mb], Bb[s & 1][rb], acc[rb][mb]);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int rb = 0; rb < 4; ++rb) pvc[rb] = pvn[rb];
+      for (int rb = 0; rb < 4; ++rb) {
+        pvc[rb] = pvn[rb];
+        if constexpr (SKIP) nzc[rb] = nzn[rb];
+      }
     }
   }
   if (nfull < ncc) {
@@ -193,27 +211,32 @@ __global__ __launch_bounds__(256, 2) void conv_gather_wide_kernel(
     // so the slots are taken two at a time (the chunk before left the first pair filled).
     const int cc = nfull;
     stage_chunk(cc);
-    load_pos(0, pvc);
+    load_pos(0, pvc, nzc);
     read_b(pvc, 0, Bb[0]);
     auto half_slot = [&](int k, auto ring) {
       constexpr int r = decltype(ring)::value;               // this slot's pair of the ring: 0 or 2
       const int kk = cc * K + k;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        if (s == 0) load_pos(k + 1 < K ? k + 1 : 0, pvn);
+        if (s == 0) load_pos(k + 1 < K ? k + 1 : 0, pvn, nzn);
         load_a(kk + 1, s, A[(r ^ 2) + s]);
         if (s == 0) read_b(pvc, 1, Bb[1]);
         else read_b(pvn, 0, Bb[0]);                          // (past the last slot: unused)
         if (active) {
 #pragma unroll
           for (int rb = 0; rb < 4; ++rb)
+            if (!SKIP || nzc[rb]) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[r + s][mb], Bb[s][rb], acc[rb][mb]);
+              for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = Mma32<T>::run(A[r + s][mb], Bb[s][rb], acc[rb][mb]);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int rb = 0; rb < 4; ++rb) pvc[rb] = pvn[rb];
+      for (int rb = 0; rb < 4; ++rb) {
+        pvc[rb] = pvn[rb];
+        if constexpr (SKIP) nzc[rb] = nzn[rb];
+      }
     };
     for (int k = 0; k < K; k += 2) {
       half_slot(k, std::integral_constant<int, 0>{});
@@ -371,7 +394,8 @@ extern "C" int ocnn_conv_gather_wide_supported(int dtype, int64_t rows_in, int K
 template <typename T>
 static int run_wide(const void* in, int64_t rows_in, const uint16_t* loc, const int32_t* uptr,
                     const int32_t* urows, int64_t rows_out, int K, int cin, int cout, const void* w,
-                    int w_transposed, int reverse, const void* bias, void* out, void* ws, hipStream_t st) {
+                    int w_transposed, int reverse, const void* bias, void* out, void* ws, bool skip,
+                    hipStream_t st) {
   const int64_t total = (int64_t)K * align_up(cin, 64) * cout;
   hipLaunchKernelGGL(pack_weights_wide_kernel<T>, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, st,
                      (const T*)w, (T*)ws, K, cin, cout, w_transposed, reverse);
@@ -380,22 +404,29 @@ static int run_wide(const void* in, int64_t rows_in, const uint16_t* loc, const 
   const uint32_t in_bytes = (uint32_t)(rows_in * cin * 2);
   // 256 output channels per workgroup halve the LDS reads per MFMA; a launch with a handful of tiles
   // (a quarter of the CUs or fewer) is faster with 128 per workgroup on twice as many CUs
-  if (cout % 256 == 0 && tiles * (cout / 256) > 64)
-    hipLaunchKernelGGL((conv_gather_wide_kernel<T, 2>), dim3((unsigned)(per_xcd * 8), (unsigned)(cout / 256)),
-                       dim3(256), 0, st, (const T*)in, in_bytes, loc, uptr, urows, (const T*)ws, (const T*)bias,
-                       (T*)out, rows_out, K, cin, cout, tiles, per_xcd);
-  else
-    hipLaunchKernelGGL((conv_gather_wide_kernel<T, 1>), dim3((unsigned)(per_xcd * 8), (unsigned)cdiv(cout, 128)),
-                       dim3(256), 0, st, (const T*)in, in_bytes, loc, uptr, urows, (const T*)ws, (const T*)bias,
-                       (T*)out, rows_out, K, cin, cout, tiles, per_xcd);
+  const bool mb2 = cout % 256 == 0 && tiles * (cout / 256) > 64;
+  const dim3 grid((unsigned)(per_xcd * 8), (unsigned)(mb2 ? cout / 256 : cdiv(cout, 128)));
+#define OCNN_WIDE_LAUNCH(MB_, SKIP_)                                                                          \
+  hipLaunchKernelGGL((conv_gather_wide_kernel<T, MB_, SKIP_>), grid, dim3(256), 0, st, (const T*)in, in_bytes, \
+                     loc, uptr, urows, (const T*)ws, (const T*)bias, (T*)out, rows_out, K, cin, cout, tiles,   \
+                     per_xcd)
+  if (mb2) {
+    if (skip) OCNN_WIDE_LAUNCH(2, true);
+    else OCNN_WIDE_LAUNCH(2, false);
+  } else {
+    if (skip) OCNN_WIDE_LAUNCH(1, true);
+    else OCNN_WIDE_LAUNCH(1, false);
+  }
+#undef OCNN_WIDE_LAUNCH
   return check_launch("conv_gather_wide");
 }
 
 extern "C" int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in, const uint16_t* loc,
                                      const int32_t* uptr, const int32_t* urows, int plan_max_distinct,
-                                     int64_t plan_total, int64_t rows_out, int K, const void* w, int cin,
-                                     int cout, int w_transposed, int reverse_slots, const void* bias,
-                                     void* out, void* workspace, int64_t workspace_bytes, void* stream) {
+                                     int64_t plan_total, double plan_occupancy, int64_t rows_out, int K,
+                                     const void* w, int cin, int cout, int w_transposed, int reverse_slots,
+                                     const void* bias, void* out, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
   OCNN_REQUIRE(ocnn_conv_gather_wide_supported(dtype, rows_in, K, cin, cout, plan_max_distinct),
                "conv_gather_wide: shape not supported");
   OCNN_REQUIRE(rows_out >= 0 && rows_out < (1ll << 31) && plan_total >= 0 && plan_total < (1ll << 29),
@@ -408,11 +439,13 @@ extern "C" int ocnn_conv_gather_wide(int dtype, const void* in, int64_t rows_in,
     return OCNN_ERR_WORKSPACE;
   }
   hipStream_t st = (hipStream_t)stream;
+  // (a 2x2x2 table has an entry in every slot of every 32 rows, whatever its occupancy)
+  const bool skip = K != 8 && plan_occupancy >= 0.0 && plan_occupancy <= kWdSkipMaxOccupancy;
   if (dtype == OCNN_F16)
     return run_wide<f16>(in, rows_in, loc, uptr, urows, rows_out, K, cin, cout, w, w_transposed, reverse_slots,
-                         bias, out, workspace, st);
+                         bias, out, workspace, skip, st);
   return run_wide<bf16>(in, rows_in, loc, uptr, urows, rows_out, K, cin, cout, w, w_transposed, reverse_slots,
-                        bias, out, workspace, st);
+                        bias, out, workspace, skip, st);
 }
 
 // ---- dense rows ----

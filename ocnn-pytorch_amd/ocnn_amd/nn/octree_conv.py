@@ -163,10 +163,16 @@ def _conv_gather(data, rows_in, table, W, cout, transposed, reverse, bias, plan,
   if kernel == _lib.GATHER_DENSE:
     _lib.check(L.ocnn_conv_dense(code, _lib.ptr(data), rows, _lib.ptr(W), cin, cout, int(transposed), *tail))
     return out, False
-  if kernel in (_lib.GATHER_RW, _lib.GATHER_WIDE):
-    fn = L.ocnn_conv_gather_rw if kernel == _lib.GATHER_RW else L.ocnn_conv_gather_wide
-    _lib.check(fn(code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
-                  plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse), *tail))
+  if kernel == _lib.GATHER_RW:
+    _lib.check(L.ocnn_conv_gather_rw(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
+        plan.umax, plan.total, rows, K, _lib.ptr(W), cin, cout, int(transposed), int(reverse), *tail))
+    return out, True
+  if kernel == _lib.GATHER_WIDE:
+    _lib.check(L.ocnn_conv_gather_wide(
+        code, _lib.ptr(data), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows),
+        plan.umax, plan.total, float(plan.occupancy), rows, K, _lib.ptr(W), cin, cout, int(transposed),
+        int(reverse), *tail))
     return out, True
   if kernel == _lib.GATHER_SPARSE:
     pp = plan.pairs()

@@ -48,8 +48,8 @@ CASES = {
     'ocnn_conv_gather_planned': [2, 'P', 200, 'P', 'P', 'P', 200, 27, 'P', 64, 64, 0, 0, 'O', 'P', 'P', 'W', 'O'],
     'ocnn_conv_gather_rw': [2, 'P', 200, 'P', 'P', 'P', 100, 150, 200, 27, 'P', 64, 64, 0, 0, 'O', 'P', 'P', 'W', 'O'],
     'ocnn_conv_gather_rw_static': [2, 'P', 200, 'P', 'P', 'P', 100, 150, 200, 27, 'P', 64, 64, 0, 0, 'O', 'P', 'O'],
-    'ocnn_conv_gather_wide': [2, 'P', 200, 'P', 'P', 'P', 100, 150, 200, 27, 'P', 128, 128, 0, 0, 'O', 'P', 'P', 'W',
-                              'O'],
+    'ocnn_conv_gather_wide': [2, 'P', 200, 'P', 'P', 'P', 100, 150, 0.3, 200, 27, 'P', 128, 128, 0, 0, 'O', 'P', 'P',
+                              'W', 'O'],
     'ocnn_pair_plan_slot_counts': ['P', 2, 27, 'P', 'O'],
     'ocnn_pair_plan_lists': [27, [5] * 27, [0] * 32, [0] * 32, [0] * 5, [0]],
     'ocnn_pair_plan_count': ['P', 2, 27, 'P', 27, 'P', 'O'],

@@ -832,9 +832,10 @@ def test_dense_rows_register_kernels(dtype, cin, cout):
       assert torch.equal(got[0], got[1].contiguous()) and torch.equal(got[0], got[2])
 
 
-def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
+def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias, occupancy=-1.0):
   """ocnn_conv_gather_wide through the C ABI (the Python layer picks it only for plans with
-  enough reuse)."""
+  enough reuse).  occupancy: the share of entries set as the entry point is told it (from 40 %
+  down it leaves out the products of 32-row blocks without an entry in a slot)."""
   L = _lib.lib()
   rows, K = table.shape
   cin = x.shape[1]
@@ -844,7 +845,7 @@ def _gather_wide(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
   ws = torch.empty(K * (-(-cin // 64) * 64) * cout * 2, dtype=torch.uint8, device=x.device)   # whole 64-channel chunks
   _lib.check(L.ocnn_conv_gather_wide(
       code, _lib.ptr(x), rows_in, _lib.ptr(plan.loc), _lib.ptr(plan.uptr), _lib.ptr(plan.urows), plan.umax,
-      plan.total, rows, K, _lib.ptr(w), cin, cout, int(transposed), int(reverse), _lib.ptr(bias),
+      plan.total, occupancy, rows, K, _lib.ptr(w), cin, cout, int(transposed), int(reverse), _lib.ptr(bias),
       _lib.ptr(out), _lib.ptr(ws), ws.numel(), _lib.stream()))
   return out
 
@@ -879,6 +880,43 @@ def test_wide_gather_kernel(dtype, K, cin, cout):
       got = _gather_wide(gr.to(DEV), rows_in, tg, plan, w.to(DEV), cin, True, True, None)
       want = C.forward_gemm(f64(gr), np.ascontiguousarray(f64(w)[::-1].transpose(0, 2, 1)), t64)
       assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize('K,cin,cout', [(27, 128, 128), (27, 128, 256), (9, 96, 160), (3, 256, 256), (8, 128, 128)])
+def test_wide_gather_leaves_out_blocks_without_entries(K, cin, cout):
+  """Told an occupancy of 40 % or less, the kernel for wide layers tests every (32-row block,
+  slot) of a tile for entries and leaves the products of the empty ones out: tables where
+  whole blocks, whole slots and whole tiles are empty, against the oracle and - bit for bit -
+  against the same kernel without the test (occupancy unknown)."""
+  from ocnn_amd.octree.octree import TilePlan
+  dtype = torch.bfloat16
+  g = torch.Generator().manual_seed(31 * K + cin)
+  for rows, rows_in in [(128 * 9 + 77, 1400), (128 * 3, 500), (100, 90)]:
+    say('wide gather with empty blocks', K, cin, cout, rows, rows_in)
+    table = _local_table(rows, rows_in, K, g)
+    blk = torch.arange(rows) // 32
+    for k in range(K):
+      table[(blk + k) % 3 == 0, k] = -1                  # a third of the (block, slot) units
+    table[:, K // 2] = -1                                # a slot without entries
+    if rows > 256:
+      table[128:256] = -1                                # a tile without entries
+      table[300:310, 0] = 5                              # (and a block with a few)
+    tg = table.to(DEV)
+    plan = TilePlan(tg)
+    t64 = table.numpy().astype(np.int64)
+    x = torch.randn(rows_in, cin, generator=g).to(dtype)
+    w = (torch.randn(K, cin, cout, generator=g) / (K * cin) ** 0.5).to(dtype)
+    b = torch.randn(cout, generator=g).to(dtype)
+    want = C.forward_gemm(f64(x), f64(w), t64) + f64(b)
+    plain = _gather_wide(x.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV))
+    skipping = _gather_wide(x.to(DEV), rows_in, tg, plan, w.to(DEV), cout, False, False, b.to(DEV), occupancy=0.2)
+    assert rel_err(plain, want) < TOL[dtype] and rel_err(skipping, want) < TOL[dtype]
+    assert torch.equal(plain, skipping)
+    gr = torch.randn(rows_in, cout, generator=g).to(dtype)
+    if cin >= 96:
+      a = _gather_wide(gr.to(DEV), rows_in, tg, plan, w.to(DEV), cin, True, True, None)
+      c = _gather_wide(gr.to(DEV), rows_in, tg, plan, w.to(DEV), cin, True, True, None, occupancy=0.39)
+      assert torch.equal(a, c)
 
 
 def _gather_sparse(x, rows_in, table, plan, w, cout, transposed, reverse, bias):
